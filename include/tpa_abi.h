@@ -1,0 +1,159 @@
+/*
+ * C ABI of libtpa_gfx950.so: Tensor Product Attention forward (prefill + decode) and a
+ * same-shape dense multi-head flash attention, as hand-written HIP kernels for gfx950.
+ *
+ * The reference has no native ABI.  Its operator boundary for this path is the Pallas call
+ *   pl.pallas_call(_fwd_kernel, ...)(qa, qb, ka, kb, va, vb, q_segment_ids, kv_segment_ids) -> [o, l]
+ * at tpa/tpa.py:492-543 (statics sm_scale, causal bound at tpa/tpa.py:493-500), reached from
+ * tpa()/_tpa_fwd() (tpa/tpa.py:73-165) once per batch element through jax.vmap.  The entry
+ * points below are what a jax.ffi / ctypes binding for that seam binds: plain pointers and
+ * sizes, no torch or jax types.
+ *
+ * Common rules for every entry point
+ *   - all pointers are device pointers owned by the caller; they must stay valid until the
+ *     work enqueued on `stream` has completed;
+ *   - calls only enqueue work on `stream` (a hipStream_t passed as void*; NULL = the null
+ *     stream); they never synchronise, allocate or free device memory, throw or abort;
+ *   - return 0 on success or a negative TPA_ERR_* code, with nothing enqueued on error;
+ *   - re-entrant: may be called concurrently from several host threads.
+ */
+#ifndef TPA_ABI_H_
+#define TPA_ABI_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TPA_ABI_VERSION 1
+
+/* element types of the factor / output arrays */
+enum { TPA_DTYPE_F32 = 0, TPA_DTYPE_BF16 = 1 };
+
+/* error codes (tpa_strerror gives text) */
+enum {
+  TPA_OK = 0,
+  TPA_ERR_NULL = -1,        /* a required pointer is NULL */
+  TPA_ERR_SHAPE = -2,       /* a dimension is <= 0 or exceeds what the kernels support */
+  TPA_ERR_DTYPE = -3,       /* unknown dtype */
+  TPA_ERR_ALIGN = -4,       /* pointer or stride not aligned as the selected kernel needs */
+  TPA_ERR_WORKSPACE = -5,   /* workspace missing or too small */
+  TPA_ERR_UNSUPPORTED = -6, /* the requested kernel cannot run this problem */
+  TPA_ERR_LAUNCH = -7       /* the HIP runtime refused the launch */
+};
+
+/* which kernel family to use */
+enum {
+  TPA_KERNEL_AUTO = 0,    /* MFMA kernels when the problem qualifies, else the generic kernel */
+  TPA_KERNEL_GENERIC = 1, /* any-shape fp32-math kernel */
+  TPA_KERNEL_MFMA = 2     /* MFMA kernels only; TPA_ERR_UNSUPPORTED if the problem does not qualify */
+};
+
+/*
+ * One factor array: A factors a[b, l, r, h] or B factors b[b, l, r, d].  The innermost
+ * dimension is contiguous; the other three have ELEMENT strides, so both the split arrays
+ * qa[lq, rq, h] / qb[lq, rq, dk] of tpa/tpa.py:246-251 and the concatenated q[b, lq, rq, h+dk]
+ * of tpa/tpa.py:75-77 (A = base, B = base + h, rank stride h+dk) are read in place.
+ */
+typedef struct TpaFactor {
+  const void* ptr;
+  int64_t stride_b; /* elements between batch entries */
+  int64_t stride_l; /* elements between tokens */
+  int64_t stride_r; /* elements between ranks */
+} TpaFactor;
+
+/*
+ * tpa_fwd / tpa_decode arguments.  Replaces the operand list and statics of the pallas_call at
+ * tpa/tpa.py:492-543.  Semantics (tpa/tpa.py:245-443):
+ *   Q = (1/rq) sum_r qa_r (x) qb_r, K, V likewise with 1/rk           (tpa/tpa.py:317,364,417)
+ *   x = sm_scale * Q K^T                                              (tpa/tpa.py:365-367)
+ *   masked (-inf) where segment ids differ or, if causal, key index > query index
+ *                                                                      (tpa/tpa.py:369-386)
+ *   lse = logsumexp_k x ; o = softmax_k(x) V                          (tpa/tpa.py:389-424)
+ *   rows with every key masked: o = NaN, lse = -inf                   (tpa/tpa.py:437-439)
+ */
+typedef struct TpaFwdArgs {
+  TpaFactor qa; /* [B, lq, rq, H]  */
+  TpaFactor qb; /* [B, lq, rq, dk] */
+  TpaFactor ka; /* [B, lk, rk, H]  */
+  TpaFactor kb; /* [B, lk, rk, dk] */
+  TpaFactor va; /* [B, lk, rk, H]  */
+  TpaFactor vb; /* [B, lk, rk, dv] */
+  const int32_t* q_segment_ids;  /* [B, lq] contiguous, or NULL (then kv_segment_ids must be NULL) */
+  const int32_t* kv_segment_ids; /* [B, lk] contiguous, or NULL */
+  void* o;      /* [B, lq, H, dv] contiguous, element type = dtype (tpa/tpa.py:529) */
+  float* lse;   /* [B, H, lq] contiguous fp32 natural-log logsumexp, or NULL to skip it.
+                   The reference's l[lq, h] (tpa/tpa.py:530) is the transpose of one batch entry. */
+  int32_t B, lq, lk, H, dk, dv, rq, rk;
+  int32_t dtype;  /* TPA_DTYPE_*: element type of the six factor arrays and of o */
+  float sm_scale; /* multiplies the logits after the dot product (tpa/tpa.py:367) */
+  int32_t causal; /* non-zero: key index <= query index, top-left aligned (tpa/tpa.py:377-379) */
+  int32_t kernel; /* TPA_KERNEL_* */
+  void* workspace;        /* tpa_decode only: scratch for split partials, else ignored */
+  size_t workspace_bytes; /* size of workspace */
+  int32_t num_splits;     /* tpa_decode only: 0 = choose; otherwise the number of key ranges */
+} TpaFwdArgs;
+
+/*
+ * mha_fwd arguments: dense attention with the layouts of mha() at tpa/mha.py:11-17,
+ *   q[B, lq, H, dk]  k[B, lk, H, dk]  v[B, lk, H, dv]  ->  o[B, lq, H, dv],
+ * x = sm_scale * q k^T (+ bias[b, lq, lk] broadcast over heads, tpa/mha.py:31-34), softmax, p v.
+ * `causal` is an addition: the reference expresses causality as a dense -inf bias
+ * (tpa/tpa_test.py:52-54).  A dense bias is honoured by the generic kernel only.
+ */
+typedef struct MhaFwdArgs {
+  const void* q; /* token stride = H*dk, batch stride = lq*H*dk (contiguous) */
+  const void* k;
+  const void* v;
+  const float* bias; /* [B, lq, lk] fp32 additive, or NULL */
+  void* o;
+  float* lse; /* [B, H, lq] fp32 or NULL */
+  int32_t B, lq, lk, H, dk, dv;
+  int32_t dtype;
+  float sm_scale;
+  int32_t causal;
+  int32_t kernel;
+  void* workspace;        /* used when lq is small (split over keys), else ignored */
+  size_t workspace_bytes;
+  int32_t num_splits;
+} MhaFwdArgs;
+
+/* ABI version of the loaded library (TPA_ABI_VERSION it was built with). */
+int tpa_abi_version(void);
+
+/* Text for an error code returned by the functions below. */
+const char* tpa_strerror(int code);
+
+/*
+ * Forward pass for any lq (prefill).  Replaces pl.pallas_call(..., name="tpa_fwd") at
+ * tpa/tpa.py:492-543 for all batch entries at once (the reference vmaps it, tpa/tpa.py:144-163).
+ */
+int tpa_fwd(const TpaFwdArgs* args, void* stream);
+
+/*
+ * Forward pass for few query tokens over a long factored cache (the reference reaches this as
+ * the same call with lq = 1: block_q = min(128, lq), tpa/tpa.py:485).  Keys are split into
+ * ranges whose partial (o, lse) are merged with the rule of _lse_accum (tpa/tpa.py:228-242).
+ * Needs `workspace` of at least tpa_decode_workspace_bytes(...) bytes.  Masks are not
+ * supported (causal must be 0 and segment ids NULL): TPA_ERR_UNSUPPORTED otherwise.
+ */
+int tpa_decode(const TpaFwdArgs* args, void* stream);
+
+/* Bytes of workspace tpa_decode needs for this problem (num_splits = 0: the default choice). */
+size_t tpa_decode_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dv, int32_t num_splits);
+
+/* Number of key ranges tpa_decode uses when args->num_splits == 0. */
+int32_t tpa_decode_default_splits(int32_t B, int32_t lq, int32_t lk, int32_t H);
+
+/* Dense attention forward with the layouts of tpa/mha.py:11-17 (see MhaFwdArgs). */
+int mha_fwd(const MhaFwdArgs* args, void* stream);
+
+/* Bytes of workspace mha_fwd needs (0 unless lq is small enough for the split-key kernel). */
+size_t mha_fwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dv, int32_t num_splits);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TPA_ABI_H_ */

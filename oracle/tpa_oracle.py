@@ -1,0 +1,158 @@
+"""CPU oracle for the Tensor Product Attention forward path.  TEST INFRASTRUCTURE ONLY.
+
+This file restates, in plain numpy, the arithmetic of the reference's jnp oracle so that
+the HIP kernels can be checked against it.  Only tests, the smoke check and the benchmark's
+`cpu_baseline` leg may import it; the product package never does.
+
+What follows what (reference file:line):
+  * `split_factors`      - tpa/tpa_test.py:35-37  (A factor = first `num_heads` columns)
+  * `reconstruct`        - tpa/tpa_test.py:42-44  (X = (1/R) * sum_r a_r (x) b_r)
+  * `attention_bias`     - tpa/tpa_test.py:46-55  (segment equality, then top-left tril; additive -inf)
+  * `mha_forward`        - tpa/mha.py:23-37       (dot, scale AFTER the dot, + bias broadcast over heads,
+                                                   softmax over keys, p @ v, output [b, lq, h, dv])
+  * `lse` / `lse_accum`  - tpa/tpa.py:220-242     (-inf safe logsumexp and its pairwise merge)
+  * empty rows           - tpa/tpa.py:437-439     (O = NaN, LSE = -inf), same as softmax of an all -inf row
+  * shape rules          - tpa/tpa.py:474-479
+
+The reference returns LSE as l[b, lq, h] (tpa/tpa.py:255,443); this oracle returns it in that
+layout too (`lse_blh`); callers transpose when they compare with the kernels' [b, h, lq].
+
+How this oracle is pinned (tests/test_oracle.py): brute-force float64 loops on tiny shapes,
+torch's scaled_dot_product_attention and scipy's softmax/logsumexp as independent library
+routines, closed forms (zero queries -> running mean of V and LSE = ln(count); lk = 1), rank
+invariances (duplicated / permuted ranks, a*c with b/c), the causal prefix property, and the
+only literal known-answer the reference holds (tpa/mha_test.py:44-118, forward part).
+Parity against the bit-stream of jax itself is unpinned (jax is not installable here); the
+mathematical contract is pinned by the checks above.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+__all__ = [
+    "split_factors",
+    "reconstruct",
+    "attention_bias",
+    "mha_forward",
+    "tpa_reference",
+    "tpa_reference_rows",
+    "lse",
+    "lse_accum",
+]
+
+
+def split_factors(x: np.ndarray, num_heads: int):
+    """x[b, l, r, h + d] -> (a[b, l, r, h], b[b, l, r, d]).  tpa/tpa_test.py:35-37."""
+    return x[..., :num_heads], x[..., num_heads:]
+
+
+def reconstruct(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """(1/R) * sum_r a[b,l,r,h] * b[b,l,r,d] -> [b, l, h, d].  tpa/tpa_test.py:42-44."""
+    rank = a.shape[2]
+    return np.einsum("blrh,blrd->blhd", a, b) / rank
+
+
+def attention_bias(batch, lq, lk, q_segment_ids, kv_segment_ids, causal, dtype=np.float64):
+    """Additive bias [b, lq, lk] of 0 / -inf.  tpa/tpa_test.py:46-55."""
+    bias = np.zeros((batch, lq, lk), dtype=dtype)
+    if q_segment_ids is not None:
+        assert kv_segment_ids is not None
+        same = np.asarray(q_segment_ids)[:, :, None] == np.asarray(kv_segment_ids)[:, None, :]
+        bias = bias + np.where(same, 0.0, -np.inf)
+    if causal:
+        tril = np.tril(np.ones((lq, lk), dtype=bool))
+        bias = bias + np.where(tril, 0.0, -np.inf)[None]
+    return bias
+
+
+def lse(x: np.ndarray) -> np.ndarray:
+    """-inf safe logsumexp over the last axis.  tpa/tpa.py:220-226."""
+    m = np.max(x, axis=-1)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        val = m + np.log(np.sum(np.exp(x - m[..., None]), axis=-1))
+    return np.where(np.isneginf(m), -np.inf, val)
+
+
+def lse_accum(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """log(exp(a) + exp(b)), -inf safe.  tpa/tpa.py:228-242."""
+    assert a.shape == b.shape
+    hi = np.maximum(a, b)
+    lo = np.minimum(a, b)
+    with np.errstate(invalid="ignore"):
+        val = hi + np.log(1 + np.exp(lo - hi))
+    return np.where(np.isneginf(hi), -np.inf, val)
+
+
+def mha_forward(q, k, v, bias=None, sm_scale=1.0):
+    """Dense attention, tpa/mha.py:23-37, plus the logsumexp the kernels also emit.
+
+    q[b,lq,h,dk] k[b,lk,h,dk] v[b,lk,h,dv] bias[b,lq,lk] -> (o[b,lq,h,dv], lse[b,lq,h]).
+    A row whose logits are all -inf gives o = NaN and lse = -inf.
+    """
+    x = np.einsum("bqhd,bkhd->bhqk", q, k)
+    x = sm_scale * x
+    if bias is not None:
+        x = x + bias[:, None, :, :]
+    m = np.max(x, axis=-1, keepdims=True)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        e = np.exp(x - m)  # all -inf row: -inf - -inf = NaN, as jax.nn.softmax gives
+        s = np.sum(e, axis=-1, keepdims=True)
+        p = e / s
+        l_ = np.where(np.isneginf(m[..., 0]), -np.inf, m[..., 0] + np.log(s[..., 0]))
+    o = np.einsum("bhqk,bkhd->bqhd", p, v)
+    return o, np.transpose(l_, (0, 2, 1))
+
+
+def tpa_reference(
+    q, k, v, q_segment_ids, kv_segment_ids, num_heads, sm_scale=1.0, causal=False, dtype=np.float64
+):
+    """The reference's `reference()` (tpa/tpa_test.py:22-57) on concatenated factors.
+
+    q[b,lq,rq,h+dk] k[b,lk,rk,h+dk] v[b,lk,rk,h+dv] -> (o[b,lq,h,dv], lse[b,lq,h]), computed in `dtype`.
+    """
+    q = np.asarray(q, dtype=dtype)
+    k = np.asarray(k, dtype=dtype)
+    v = np.asarray(v, dtype=dtype)
+    qa, qb = split_factors(q, num_heads)
+    ka, kb = split_factors(k, num_heads)
+    va, vb = split_factors(v, num_heads)
+    b, lq = qa.shape[:2]
+    lk = ka.shape[1]
+    assert k.shape[:3] == v.shape[:3], (k.shape, v.shape)  # tpa/tpa.py:474-475
+    q_ = reconstruct(qa, qb)
+    k_ = reconstruct(ka, kb)
+    v_ = reconstruct(va, vb)
+    bias = attention_bias(b, lq, lk, q_segment_ids, kv_segment_ids, causal, dtype=dtype)
+    return mha_forward(q_, k_, v_, bias=bias, sm_scale=sm_scale)
+
+
+def tpa_reference_rows(
+    q, k, v, q_segment_ids, kv_segment_ids, num_heads, rows, sm_scale=1.0, causal=False, dtype=np.float64
+):
+    """Same result as `tpa_reference(...)[:, rows]`, computed for the listed query rows only.
+
+    Each output row depends only on its own row of logits, so this is exact; it lets long
+    sequences be checked without materialising [b, h, lq, lk].  The causal mask uses the
+    absolute row index (top-left aligned tril, tpa/tpa_test.py:53).
+    """
+    rows = np.asarray(rows)
+    q = np.asarray(q)[:, rows].astype(dtype)
+    k = np.asarray(k, dtype=dtype)
+    v = np.asarray(v, dtype=dtype)
+    qa, qb = split_factors(q, num_heads)
+    ka, kb = split_factors(k, num_heads)
+    va, vb = split_factors(v, num_heads)
+    b = q.shape[0]
+    lk = k.shape[1]
+    q_ = reconstruct(qa, qb)
+    k_ = reconstruct(ka, kb)
+    v_ = reconstruct(va, vb)
+    bias = np.zeros((b, len(rows), lk), dtype=dtype)
+    if q_segment_ids is not None:
+        same = np.asarray(q_segment_ids)[:, rows][:, :, None] == np.asarray(kv_segment_ids)[:, None, :]
+        bias = bias + np.where(same, 0.0, -np.inf)
+    if causal:
+        keep = rows[:, None] >= np.arange(lk)[None, :]
+        bias = bias + np.where(keep, 0.0, -np.inf)[None]
+    return mha_forward(q_, k_, v_, bias=bias, sm_scale=sm_scale)

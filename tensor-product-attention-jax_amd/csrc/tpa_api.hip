@@ -1,0 +1,87 @@
+// extern "C" entry points of libtpa_gfx950.so: argument validation and kernel selection.
+#include "tpa_common.h"
+
+namespace {
+
+int check_factor(const TpaFactor& f) { return f.ptr == nullptr ? TPA_ERR_NULL : TPA_OK; }
+
+int validate_tpa(const TpaFwdArgs* a) {
+  if (!a) return TPA_ERR_NULL;
+  if (a->dtype != TPA_DTYPE_F32 && a->dtype != TPA_DTYPE_BF16) return TPA_ERR_DTYPE;
+  if (a->B <= 0 || a->lq <= 0 || a->lk <= 0 || a->H <= 0 || a->dk <= 0 || a->dv <= 0 || a->rq <= 0 || a->rk <= 0)
+    return TPA_ERR_SHAPE;
+  if (a->dk > 256 || a->dv > 256) return TPA_ERR_SHAPE;
+  const TpaFactor* fs[6] = {&a->qa, &a->qb, &a->ka, &a->kb, &a->va, &a->vb};
+  for (const TpaFactor* f : fs)
+    if (check_factor(*f) != TPA_OK) return TPA_ERR_NULL;
+  if (!a->o) return TPA_ERR_NULL;
+  // segment ids come in pairs (tpa/tpa.py:369-371)
+  if ((a->q_segment_ids == nullptr) != (a->kv_segment_ids == nullptr)) return TPA_ERR_NULL;
+  if (a->kernel != TPA_KERNEL_AUTO && a->kernel != TPA_KERNEL_GENERIC && a->kernel != TPA_KERNEL_MFMA)
+    return TPA_ERR_UNSUPPORTED;
+  return TPA_OK;
+}
+
+int validate_mha(const MhaFwdArgs* a) {
+  if (!a) return TPA_ERR_NULL;
+  if (a->dtype != TPA_DTYPE_F32 && a->dtype != TPA_DTYPE_BF16) return TPA_ERR_DTYPE;
+  if (a->B <= 0 || a->lq <= 0 || a->lk <= 0 || a->H <= 0 || a->dk <= 0 || a->dv <= 0) return TPA_ERR_SHAPE;
+  if (a->dk > 256 || a->dv > 256) return TPA_ERR_SHAPE;
+  if (!a->q || !a->k || !a->v || !a->o) return TPA_ERR_NULL;
+  if (a->kernel != TPA_KERNEL_AUTO && a->kernel != TPA_KERNEL_GENERIC && a->kernel != TPA_KERNEL_MFMA)
+    return TPA_ERR_UNSUPPORTED;
+  return TPA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int tpa_abi_version(void) { return TPA_ABI_VERSION; }
+
+const char* tpa_strerror(int code) {
+  switch (code) {
+    case TPA_OK: return "ok";
+    case TPA_ERR_NULL: return "a required pointer is NULL (or only one of the two segment-id arrays was given)";
+    case TPA_ERR_SHAPE: return "a dimension is not positive or exceeds what the kernels support";
+    case TPA_ERR_DTYPE: return "unknown dtype";
+    case TPA_ERR_ALIGN: return "pointer or stride not aligned for the selected kernel";
+    case TPA_ERR_WORKSPACE: return "workspace missing or too small";
+    case TPA_ERR_UNSUPPORTED: return "the requested kernel cannot run this problem";
+    case TPA_ERR_LAUNCH: return "the HIP runtime refused the launch";
+    default: return "unknown error code";
+  }
+}
+
+int tpa_fwd(const TpaFwdArgs* a, void* stream) {
+  const int rc = validate_tpa(a);
+  if (rc != TPA_OK) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (a->kernel != TPA_KERNEL_GENERIC && tpa_prefill_mfma_supported(a)) return tpa_prefill_mfma_launch(a, s);
+  if (a->kernel == TPA_KERNEL_MFMA) return TPA_ERR_UNSUPPORTED;
+  return tpa_generic_launch(a, s);
+}
+
+int tpa_decode(const TpaFwdArgs* a, void* stream) {
+  const int rc = validate_tpa(a);
+  if (rc != TPA_OK) return rc;
+  if (a->causal || a->q_segment_ids) return TPA_ERR_UNSUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (a->kernel != TPA_KERNEL_GENERIC && tpa_decode_mfma_supported(a)) return tpa_decode_mfma_launch(a, s);
+  if (a->kernel == TPA_KERNEL_MFMA) return TPA_ERR_UNSUPPORTED;
+  return tpa_generic_launch(a, s);
+}
+
+int mha_fwd(const MhaFwdArgs* a, void* stream) {
+  const int rc = validate_mha(a);
+  if (rc != TPA_OK) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (a->kernel != TPA_KERNEL_GENERIC) {
+    if (mha_decode_supported(a)) return mha_decode_launch(a, s);
+    if (mha_prefill_mfma_supported(a)) return mha_prefill_mfma_launch(a, s);
+  }
+  if (a->kernel == TPA_KERNEL_MFMA) return TPA_ERR_UNSUPPORTED;
+  return mha_generic_launch(a, s);
+}
+
+}  // extern "C"

@@ -1,0 +1,85 @@
+// Shared device/host helpers for the gfx950 TPA kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "tpa_abi.h"
+
+namespace tpa {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// bf16 bit pattern (in the low or high half of a dword) -> fp32
+__device__ __forceinline__ float bf16lo_to_f32(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16hi_to_f32(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+__device__ __forceinline__ float bf16bits_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+
+// two fp32 -> packed bf16 pair (round to nearest even), lo in bits 0..15
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  bf16x2 r;
+  r[0] = (__bf16)lo;
+  r[1] = (__bf16)hi;
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+template <typename T>
+__device__ __forceinline__ float load_as_f32(const T* p);
+template <>
+__device__ __forceinline__ float load_as_f32<float>(const float* p) {
+  return *p;
+}
+template <>
+__device__ __forceinline__ float load_as_f32<uint16_t>(const uint16_t* p) {
+  return bf16bits_to_f32(*p);
+}
+
+template <typename T>
+__device__ __forceinline__ void store_from_f32(T* p, float v);
+template <>
+__device__ __forceinline__ void store_from_f32<float>(float* p, float v) {
+  *p = v;
+}
+template <>
+__device__ __forceinline__ void store_from_f32<uint16_t>(uint16_t* p, float v) {
+  __bf16 b = (__bf16)v;
+  *p = __builtin_bit_cast(uint16_t, b);
+}
+
+// Combine a value with the one held by lane ^ 32.  v_permlane32_swap hands every lane both its
+// own value and its partner's (which of the two results holds which depends on the half the
+// lane is in), so order-independent reductions need no select.
+__device__ __forceinline__ float halves_max(float x) {
+  uint32_t u = __float_as_uint(x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float halves_sum(float x) {
+  uint32_t u = __float_as_uint(x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+}  // namespace tpa
+
+// host-side entry points of the individual kernel files (launchers return TPA_* codes)
+int tpa_generic_launch(const TpaFwdArgs* a, hipStream_t stream);
+int mha_generic_launch(const MhaFwdArgs* a, hipStream_t stream);
+int tpa_prefill_mfma_supported(const TpaFwdArgs* a);
+int tpa_prefill_mfma_launch(const TpaFwdArgs* a, hipStream_t stream);
+int mha_prefill_mfma_supported(const MhaFwdArgs* a);
+int mha_prefill_mfma_launch(const MhaFwdArgs* a, hipStream_t stream);
+int tpa_decode_mfma_supported(const TpaFwdArgs* a);
+int tpa_decode_mfma_launch(const TpaFwdArgs* a, hipStream_t stream);
+int mha_decode_supported(const MhaFwdArgs* a);
+int mha_decode_launch(const MhaFwdArgs* a, hipStream_t stream);

@@ -1,0 +1,413 @@
+// Decode over the factored KV cache for gfx950: a few query tokens against a long cache, split
+// over key ranges, built to be bound by HBM bandwidth.
+//
+// The cache is never expanded to per-head K/V.  With Qm[h, :] = (c / (Rq Rk)) sum_i qa[i, h] qb[i, :]
+// the logits are  s[h, t] = sum_j a_k[t, j, h] * (Qm[h, :] . b_k[t, j, :])  and the output is
+// o[h, :] = (1/Rk) sum_t sum_j (p[h, t] a_v[t, j, h]) b_v[t, j, :]  (the rank-shared products of
+// the non-materialising form, tpa/tpa.py:333-359,398-413), so the rows b_k[(t, j), :] and
+// b_v[(t, j), :] are plain row-major matrices that feed two skinny MFMA contractions with the
+// heads as the N dimension.  Every cache byte is read from HBM exactly once for all heads.
+//
+// A workgroup has 4 independent waves; each streams its own range of 32-row blocks
+// (32 / Rk tokens) with fully coalesced 16-byte loads that stay in flight in registers one
+// block ahead, stages the block in its private LDS region (XOR-swizzled so that both the
+// 16-byte operand reads and the transposed reads are bank-conflict free), and keeps a private
+// online softmax (tpa/tpa.py:389-424).  The waves are merged through LDS, the key ranges
+// through a workspace and a small second kernel, both with the rule of _lse_accum
+// (tpa/tpa.py:228-242).
+#include "tpa_common.h"
+
+namespace tpa {
+namespace {
+
+constexpr int kWaves = 4;
+constexpr int kRowsPerBlock = 32;
+
+struct DecodeParams {
+  TpaFactor qa, qb, ka, kb, va, vb;
+  float* part_o;  // [B, lq, S, H, D] fp32, unnormalised
+  float* part_m;  // [B, lq, S, H] running max (log2 domain)
+  float* part_l;  // [B, lq, S, H] sum of exp2
+  int B, lq, lk, H, rq;
+  int S;           // key ranges
+  int nblocks;     // 32-row blocks in the cache: ceil(lk * rk / 32)
+  float qscale;    // sm_scale * log2(e) / (rq * rk)
+};
+
+template <int D>
+struct DecodeLds {
+  static constexpr int kB = kRowsPerBlock * D;       // elements of one B tile
+  static constexpr int kA = kRowsPerBlock * 32;      // elements of one A tile (32 heads)
+  static constexpr int kWave = 2 * kB + 2 * kA;      // elements per wave
+  static constexpr int kReduce = 32 * D * 2 + 128;   // fp32 O^T + m + l, in uint16 units
+  static constexpr int kPerWave = kWave > kReduce ? kWave : kReduce;
+  static constexpr size_t kBytes = (size_t)kWaves * kPerWave * sizeof(uint16_t);
+};
+
+template <int D, int RK>
+__global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
+  constexpr int CPR = D / 8;               // 16-byte chunks per B row
+  constexpr int RPI = 64 / CPR;            // B rows per load instruction
+  constexpr int NLB = kRowsPerBlock / RPI; // load instructions per B tile
+  constexpr int NKS = D / 16;
+  constexpr int NDB = D / 32;
+  constexpr int TPQ = 4 / RK;              // tokens per 4-row group
+  static_assert(RK == 1 || RK == 2 || RK == 4, "rank must divide 4");
+
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+
+  const int S = p.S;
+  const int b = blockIdx.x / S, split = blockIdx.x % S;
+  const int qi = blockIdx.y;
+  const int h0 = blockIdx.z * 32;
+  const int tid = threadIdx.x;
+  const int w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
+  const int hl = min(h0 + i, p.H - 1);  // this lane's head (clamped: lanes past H idle along)
+
+  uint16_t* lds = smem + w * DecodeLds<D>::kPerWave;
+  uint16_t* lds_bk = lds;
+  uint16_t* lds_bv = lds + DecodeLds<D>::kB;
+  uint16_t* lds_ak = lds + 2 * DecodeLds<D>::kB;
+  uint16_t* lds_av = lds_ak + DecodeLds<D>::kA;
+
+  // ---- Qm^T fragments (B operand of S'^T = B_k Qm^T): lane (h, g) holds Qm[h][16ks + 8g + 0..7]
+  bf16x8 qf[NKS];
+  {
+    const uint16_t* ap = static_cast<const uint16_t*>(p.qa.ptr) + b * p.qa.stride_b + (int64_t)qi * p.qa.stride_l + hl;
+    const uint16_t* bp = static_cast<const uint16_t*>(p.qb.ptr) + b * p.qb.stride_b + (int64_t)qi * p.qb.stride_l + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      float acc[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+      for (int r = 0; r < p.rq; ++r) {
+        const float a = bf16bits_to_f32(ap[r * p.qa.stride_r]);
+        const u32x4 bv = *reinterpret_cast<const u32x4*>(bp + r * p.qb.stride_r + 16 * ks);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[2 * j] += a * bf16lo_to_f32(bv[j]);
+          acc[2 * j + 1] += a * bf16hi_to_f32(bv[j]);
+        }
+      }
+      u32x4 packed;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) packed[j] = pack_bf16(acc[2 * j] * p.qscale, acc[2 * j + 1] * p.qscale);
+      qf[ks] = __builtin_bit_cast(bf16x8, packed);
+    }
+  }
+
+  // ---- this wave's block range
+  const int nparts = S * kWaves;
+  const int part = split * kWaves + w;
+  const int per = (p.nblocks + nparts - 1) / nparts;
+  const int blk_begin = min(part * per, p.nblocks);
+  const int blk_end = min(blk_begin + per, p.nblocks);
+  const int last_row = p.lk * RK - 1;
+
+  // rows of the cache matrices: row = token * RK + rank, row stride = stride_r
+  const uint16_t* kb_base = static_cast<const uint16_t*>(p.kb.ptr) + b * p.kb.stride_b;
+  const uint16_t* vb_base = static_cast<const uint16_t*>(p.vb.ptr) + b * p.vb.stride_b;
+  const uint16_t* ka_base = static_cast<const uint16_t*>(p.ka.ptr) + b * p.ka.stride_b + h0;
+  const uint16_t* va_base = static_cast<const uint16_t*>(p.va.ptr) + b * p.va.stride_b + h0;
+  const int a_chunks = min(4, (p.H - h0) / 8);  // valid 16-byte chunks of an A row in this head block
+
+  // loader lane roles
+  const int lb_row = l / CPR, lb_c = l % CPR;             // B tiles: row within the instruction, chunk
+  const int la_row = l >> 2, la_c = min(l & 3, a_chunks - 1);  // A tiles: 16 rows per instruction
+
+  u32x4 rbk[NLB], rbv[NLB], rak[2], rav[2];
+  auto issue = [&](int blk) {
+    const int row0 = blk * kRowsPerBlock;
+#pragma unroll
+    for (int n = 0; n < NLB; ++n) {
+      const int row = min(row0 + n * RPI + lb_row, last_row);
+      rbk[n] = *reinterpret_cast<const u32x4*>(kb_base + (int64_t)row * p.kb.stride_r + 8 * lb_c);
+      rbv[n] = *reinterpret_cast<const u32x4*>(vb_base + (int64_t)row * p.vb.stride_r + 8 * lb_c);
+    }
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+      const int row = min(row0 + 16 * n + la_row, last_row);
+      rak[n] = *reinterpret_cast<const u32x4*>(ka_base + (int64_t)row * p.ka.stride_r + 8 * la_c);
+      rav[n] = *reinterpret_cast<const u32x4*>(va_base + (int64_t)row * p.va.stride_r + 8 * la_c);
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int n = 0; n < NLB; ++n) {
+      const int row = n * RPI + lb_row;
+      const int pos = lb_c ^ (row & (CPR - 1));
+      *reinterpret_cast<u32x4*>(lds_bk + row * D + 8 * pos) = rbk[n];
+      *reinterpret_cast<u32x4*>(lds_bv + row * D + 8 * pos) = rbv[n];
+    }
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+      const int row = 16 * n + la_row;
+      *reinterpret_cast<u32x4*>(lds_ak + row * 32 + 8 * (l & 3)) = rak[n];
+      *reinterpret_cast<u32x4*>(lds_av + row * 32 + 8 * (l & 3)) = rav[n];
+    }
+  };
+
+  f32x16 o[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
+  float m = -INFINITY, lsum = 0.f;
+
+  const int lp = l & 15, dhalf = (l >> 4) & 1;
+
+  if (blk_begin < blk_end) issue(blk_begin);
+  for (int blk = blk_begin; blk < blk_end; ++blk) {
+    stage();  // waits for this block's loads, then the registers are free again
+    if (blk + 1 < blk_end) issue(blk + 1);
+
+    // ---- S'^T[row, h] = sum_d B_k[row, d] Qm[h, d]
+    f32x16 sp;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) sp[v] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      const int pos = (2 * ks + g) ^ (i & (CPR - 1));
+      const bf16x8 kf = *reinterpret_cast<const bf16x8*>(lds_bk + i * D + 8 * pos);
+      sp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sp, 0, 0, 0);
+    }
+
+    // ---- a_k / a_v of this lane's head for its 16 rows (rows 8q + 4g + 0..3, q = 0..3)
+    float ak[16], av[16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int arow = 8 * q + 4 * g + (lp >> 2);
+      const s16x4 tk = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (s16x4 __attribute__((address_space(3)))*)(lds_ak + arow * 32 + 16 * dhalf + 4 * (lp & 3)));
+      const s16x4 tv = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (s16x4 __attribute__((address_space(3)))*)(lds_av + arow * 32 + 16 * dhalf + 4 * (lp & 3)));
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        ak[4 * q + j] = bf16bits_to_f32((uint16_t)tk[j]);
+        av[4 * q + j] = bf16bits_to_f32((uint16_t)tv[j]);
+      }
+    }
+
+    // ---- logits per token (log2 domain), masked past the end of the cache
+    float st[4 * TPQ];
+    float tmax = -INFINITY;
+    const int row0 = blk * kRowsPerBlock;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int e = 0; e < TPQ; ++e) {
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < RK; ++j) acc += ak[4 * q + e * RK + j] * sp[4 * q + e * RK + j];
+        const int row = row0 + 8 * q + 4 * g + e * RK;
+        if (row > last_row) acc = -INFINITY;
+        st[q * TPQ + e] = acc;
+        tmax = fmaxf(tmax, acc);
+      }
+    tmax = halves_max(tmax);
+    const float m_new = fmaxf(m, tmax);  // finite: row0 itself is always inside the cache
+    if (__any(m_new > m)) {
+      const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+      lsum *= alpha;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+      m = m_new;
+    }
+
+    // ---- P'^T[row, h] = p[h, token(row)] * a_v[row, h], packed as the B operand of the PV product
+    float pp[16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int e = 0; e < TPQ; ++e) {
+        const float pt = __builtin_amdgcn_exp2f(st[q * TPQ + e] - m);
+        lsum += pt;
+#pragma unroll
+        for (int j = 0; j < RK; ++j) pp[4 * q + e * RK + j] = pt * av[4 * q + e * RK + j];
+      }
+    bf16x8 pf[2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      u32x4 pk;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pk[j] = pack_bf16(pp[8 * kk + 2 * j], pp[8 * kk + 2 * j + 1]);
+      pf[kk] = __builtin_bit_cast(bf16x8, pk);
+    }
+
+    // ---- O^T[d, h] += sum_row B_v[row, d] P'^T[row, h]; slot (g, j) = row 16kk + 8(j/4) + 4g + j%4
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      const int r_lo = 16 * kk + 4 * g + (lp >> 2);
+      const int r_hi = r_lo + 8;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) {
+        const int chunk = 4 * db + 2 * dhalf + ((lp & 3) >> 1);
+        const int sub = 4 * (lp & 1);
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (s16x4 __attribute__((address_space(3)))*)(lds_bv + r_lo * D + 8 * (chunk ^ (r_lo & (CPR - 1))) + sub));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (s16x4 __attribute__((address_space(3)))*)(lds_bv + r_hi * D + 8 * (chunk ^ (r_hi & (CPR - 1))) + sub));
+        const bf16x8 vf = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kk], o[db], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- merge the 4 waves through LDS (each wave reuses its own staging region)
+  const float ltot = halves_sum(lsum);
+  float* red_o = reinterpret_cast<float*>(lds);  // [32 heads][D]
+  float* red_m = red_o + 32 * D;
+  float* red_l = red_m + 32;
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red_o[i * D + 32 * db + 8 * (v >> 2) + 4 * g + (v & 3)] = o[db][v];
+  if (g == 0) {
+    red_m[i] = m;
+    red_l[i] = ltot;
+  }
+  __syncthreads();
+
+  const int nh = min(32, p.H - h0);
+  const int64_t pbase = (((int64_t)b * p.lq + qi) * S + split) * p.H + h0;
+  for (int idx = tid; idx < nh * D; idx += kWaves * 64) {
+    const int hh = idx / D, d = idx % D;
+    float mw[kWaves], mmax = -INFINITY;
+#pragma unroll
+    for (int ww = 0; ww < kWaves; ++ww) {
+      mw[ww] = reinterpret_cast<const float*>(smem + ww * DecodeLds<D>::kPerWave)[32 * D + hh];
+      mmax = fmaxf(mmax, mw[ww]);
+    }
+    float acc = 0.f, lacc = 0.f;
+#pragma unroll
+    for (int ww = 0; ww < kWaves; ++ww) {
+      const float* ro = reinterpret_cast<const float*>(smem + ww * DecodeLds<D>::kPerWave);
+      const float f = mw[ww] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw[ww] - mmax);
+      acc += f * ro[hh * D + d];
+      lacc += f * ro[32 * D + 32 + hh];
+    }
+    p.part_o[(pbase + hh) * D + d] = acc;
+    if (d == 0) {
+      p.part_m[pbase + hh] = mmax;
+      p.part_l[pbase + hh] = lacc;
+    }
+  }
+}
+
+// Merge the key ranges: o = sum_s f_s O_s / (Rk sum_s f_s l_s), f_s = 2^(m_s - max m); lse = ln of the total.
+template <int D>
+__global__ __launch_bounds__(D) void decode_merge_kernel(const float* part_o, const float* part_m, const float* part_l,
+                                                         uint16_t* o, float* lse, int S, int H, int lq, float inv_rk) {
+  const int bq = blockIdx.x;  // b * lq + qi
+  const int h = blockIdx.y;
+  const int d = threadIdx.x;
+  float mmax = -INFINITY;
+  for (int s = 0; s < S; ++s) mmax = fmaxf(mmax, part_m[((int64_t)bq * S + s) * H + h]);
+  float acc = 0.f, lacc = 0.f;
+  for (int s = 0; s < S; ++s) {
+    const int64_t idx = ((int64_t)bq * S + s) * H + h;
+    const float ms = part_m[idx];
+    const float f = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - mmax);
+    acc += f * part_o[idx * D + d];
+    lacc += f * part_l[idx];
+  }
+  store_from_f32(o + ((int64_t)bq * H + h) * D + d, acc * inv_rk / lacc);
+  if (lse && d == 0) {
+    const int b = bq / lq, qi = bq % lq;
+    lse[((int64_t)b * H + h) * lq + qi] = (mmax + __builtin_amdgcn_logf(lacc)) * kLn2;
+  }
+}
+
+size_t workspace_bytes(int B, int lq, int H, int D, int S) {
+  return (size_t)B * lq * S * H * (D + 2) * sizeof(float);
+}
+
+template <int D, int RK>
+int launch_decode(const TpaFwdArgs* a, int S, hipStream_t stream) {
+  DecodeParams p{};
+  p.qa = a->qa; p.qb = a->qb; p.ka = a->ka; p.kb = a->kb; p.va = a->va; p.vb = a->vb;
+  float* ws = static_cast<float*>(a->workspace);
+  const size_t no = (size_t)a->B * a->lq * S * a->H * D;
+  const size_t nm = (size_t)a->B * a->lq * S * a->H;
+  p.part_o = ws; p.part_m = ws + no; p.part_l = ws + no + nm;
+  p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.S = S;
+  p.nblocks = (int)(((int64_t)a->lk * RK + kRowsPerBlock - 1) / kRowsPerBlock);
+  p.qscale = a->sm_scale * kLog2e / ((float)a->rq * (float)RK);
+  auto kern = decode_kernel<D, RK>;
+  static bool configured = false;
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)DecodeLds<D>::kBytes) != hipSuccess)
+      return TPA_ERR_LAUNCH;
+    configured = true;
+  }
+  dim3 grid(a->B * S, a->lq, (a->H + 31) / 32);
+  hipLaunchKernelGGL(kern, grid, dim3(kWaves * 64), DecodeLds<D>::kBytes, stream, p);
+  if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
+  hipLaunchKernelGGL(decode_merge_kernel<D>, dim3(a->B * a->lq, a->H), dim3(D), 0, stream, p.part_o, p.part_m, p.part_l,
+                     static_cast<uint16_t*>(a->o), a->lse, S, a->H, a->lq, 1.f / (float)RK);
+  return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
+}
+
+bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
+
+int default_splits(int B, int lq, int lk, int H) {
+  // one workgroup per CU is resident (the kernel keeps a block of loads in flight in registers),
+  // so aim for a whole number of waves of 256 workgroups and at least 4 blocks per wave
+  const int groups = B * lq * ((H + 31) / 32);
+  int S = (256 + groups - 1) / groups;
+  if (groups >= 256) S = 1;
+  const int max_s = (lk + 4 * kWaves * 16 - 1) / (4 * kWaves * 16);
+  if (S > max_s) S = max_s;
+  if (S < 1) S = 1;
+  return S;
+}
+
+}  // namespace
+}  // namespace tpa
+
+extern "C" int32_t tpa_decode_default_splits(int32_t B, int32_t lq, int32_t lk, int32_t H) {
+  if (B <= 0 || lq <= 0 || lk <= 0 || H <= 0) return 0;
+  return tpa::default_splits(B, lq, lk, H);
+}
+
+extern "C" size_t tpa_decode_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dv, int32_t num_splits) {
+  if (B <= 0 || lq <= 0 || lk <= 0 || H <= 0 || dv <= 0) return 0;
+  const int S = num_splits > 0 ? num_splits : tpa::default_splits(B, lq, lk, H);
+  return tpa::workspace_bytes(B, lq, H, dv, S);
+}
+
+int tpa_decode_mfma_supported(const TpaFwdArgs* a) {
+  using namespace tpa;
+  if (a->dtype != TPA_DTYPE_BF16) return 0;
+  if (a->dk != a->dv || (a->dk != 64 && a->dk != 128)) return 0;
+  if (a->rk != 1 && a->rk != 2 && a->rk != 4) return 0;
+  if (a->H % 8 != 0) return 0;
+  if (a->lq > 64) return 0;
+  if (a->causal || a->q_segment_ids || a->kv_segment_ids) return 0;
+  // rows (token, rank) must be uniformly strided: stride_l == rk * stride_r
+  const TpaFactor* fs[4] = {&a->ka, &a->kb, &a->va, &a->vb};
+  for (const TpaFactor* f : fs) {
+    if (f->stride_l != (int64_t)a->rk * f->stride_r) return 0;
+    if (!aligned16(f->ptr) || f->stride_r % 8 != 0 || f->stride_b % 8 != 0) return 0;
+  }
+  if (!aligned16(a->qb.ptr) || a->qb.stride_r % 8 != 0 || a->qb.stride_l % 8 != 0 || a->qb.stride_b % 8 != 0) return 0;
+  return 1;
+}
+
+int tpa_decode_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
+  using namespace tpa;
+  const int S = a->num_splits > 0 ? a->num_splits : default_splits(a->B, a->lq, a->lk, a->H);
+  if (S > 65535 || (int64_t)a->B * S > 2147483647LL) return TPA_ERR_SHAPE;
+  if (!a->workspace || a->workspace_bytes < workspace_bytes(a->B, a->lq, a->H, a->dv, S)) return TPA_ERR_WORKSPACE;
+  if (!aligned16(a->workspace)) return TPA_ERR_ALIGN;
+  if (a->dk == 128) {
+    if (a->rk == 1) return launch_decode<128, 1>(a, S, stream);
+    if (a->rk == 2) return launch_decode<128, 2>(a, S, stream);
+    return launch_decode<128, 4>(a, S, stream);
+  }
+  if (a->rk == 1) return launch_decode<64, 1>(a, S, stream);
+  if (a->rk == 2) return launch_decode<64, 2>(a, S, stream);
+  return launch_decode<64, 4>(a, S, stream);
+}

@@ -1,0 +1,257 @@
+"""Tensor Product Attention forward: the operator API of the reference's tpa/tpa.py.
+
+Same names, argument meaning and error behaviour as tpa/tpa.py:35-165,220-242,446-543; the
+work is done by the gfx950 HIP kernels behind the C ABI (include/tpa_abi.h).  Arrays are torch
+tensors that live on the GPU (numpy arrays are copied there and back).  Differences from the
+reference, all on purpose:
+
+  * accumulation is always fp32 (the reference accumulates in the input dtype, tpa/tpa.py:433-434);
+  * the logsumexp residual is fp32 (the reference keeps it in the input dtype, tpa/tpa.py:530);
+  * sequence lengths need not be multiples of the block sizes (tpa/tpa.py:489-490 asserts that);
+    `block_sizes` is accepted and ignored because the kernels fix their own tiles;
+  * `nomat` does not change results in the reference (it picks an evaluation order,
+    tpa/tpa.py:333-359) and is ignored here: prefill rebuilds K/V tiles in LDS, decode uses the
+    non-materialising form;
+  * `interpret=True` (the Pallas CPU interpreter upstream) selects the plain fp32-arithmetic
+    kernel instead of the MFMA kernels; `debug` is ignored;
+  * the backward pass is not implemented: differentiating raises NotImplementedError (the
+    reference's own backward test skips on exactly that, tpa/tpa_test.py:198-201).
+"""
+
+from __future__ import annotations
+
+import dataclasses
+
+import numpy as np
+import torch
+
+from . import _dispatch as _d
+
+__all__ = ["BlockSizes", "tpa", "tpa_factors", "tpa_decode", "_tpa_fwd", "_fwd", "_lse", "_lse_accum"]
+
+
+@dataclasses.dataclass
+class BlockSizes:
+    """Tile configuration of the reference kernels (tpa/tpa.py:35-70).  Kept for signature
+    compatibility; the HIP kernels use fixed tiles and ignore it."""
+
+    block_q: int = 128
+    block_kv: int = 128
+    block_h: int = 4
+
+
+def _lse(x: torch.Tensor) -> torch.Tensor:
+    """Logsumexp over the last dimension, -inf for all -inf input (tpa/tpa.py:220-226)."""
+    m = torch.amax(x, dim=-1)
+    safe = torch.where(torch.isneginf(m), torch.zeros_like(m), m)
+    l_ = safe + torch.log(torch.sum(torch.exp(x - safe[..., None]), dim=-1))
+    return torch.where(torch.isneginf(m), m, l_)
+
+
+def _lse_accum(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """log(exp(a) + exp(b)), -inf safe (tpa/tpa.py:228-242)."""
+    assert a.shape == b.shape, f"mismatching shapes: {a.shape}, {b.shape}"
+    hi = torch.maximum(a, b)
+    lo = torch.minimum(a, b)
+    safe = torch.where(torch.isneginf(hi), torch.zeros_like(hi), hi)
+    lse = safe + torch.log(1 + torch.exp(lo - safe))
+    return torch.where(torch.isneginf(hi), hi, lse)
+
+
+def _as_device_tensor(x, device):
+    """torch GPU tensors pass through; numpy arrays / CPU tensors are copied to `device`."""
+    if isinstance(x, torch.Tensor):
+        return x if x.is_cuda else x.to(device)
+    return torch.as_tensor(np.asarray(x)).to(device)
+
+
+def _pick_device(*xs) -> torch.device:
+    for x in xs:
+        if isinstance(x, torch.Tensor) and x.is_cuda:
+            return x.device
+    if not torch.cuda.is_available():
+        raise RuntimeError("tpa needs an AMD GPU: no HIP device is visible and there is no CPU fallback")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def _segment_ids(ids, batch: int, length: int, device) -> torch.Tensor | None:
+    if ids is None:
+        return None
+    t = _as_device_tensor(ids, device).to(torch.int32)
+    if t.dim() == 1:  # the reference vmaps with in_axes=None for unbatched ids (tpa/tpa.py:144-163)
+        t = t[None].expand(batch, length)
+    if tuple(t.shape) != (batch, length):
+        raise ValueError(f"segment ids must have shape {(batch, length)}, got {tuple(t.shape)}")
+    return t.contiguous()
+
+
+def tpa_factors(
+    qa, qb, ka, kb, va, vb,
+    q_segment_ids=None,
+    kv_segment_ids=None,
+    sm_scale: float = 1.0,
+    causal: bool = False,
+    kernel: int = _d.KERNEL_AUTO,
+    return_lse: bool = True,
+):
+    """Forward pass on the six split factor arrays, the operands of the reference's kernel
+    launch (tpa/tpa.py:246-251,543) with a leading batch dimension:
+
+        qa[b,lq,rq,h] qb[b,lq,rq,dk] ka[b,lk,rk,h] kb[b,lk,rk,dk] va[b,lk,rk,h] vb[b,lk,rk,dv]
+
+    Returns (o[b,lq,h,dv] in the input dtype, lse[b,h,lq] fp32 or None).  The arrays may be
+    views (e.g. slices of the concatenated tensors); only the last dimension must be contiguous.
+    """
+    device = _pick_device(qa, qb, ka, kb, va, vb)
+    qa, qb, ka, kb, va, vb = (_as_device_tensor(x, device) for x in (qa, qb, ka, kb, va, vb))
+    dtype = qa.dtype
+    for name, t in (("qb", qb), ("ka", ka), ("kb", kb), ("va", va), ("vb", vb)):
+        if t.dtype != dtype:
+            raise TypeError(f"{name} has dtype {t.dtype}, expected {dtype}")
+    b, lq, rq, h = qa.shape
+    _, lk, rk, dv = vb.shape
+    dk = qb.shape[-1]
+    # shape rules of tpa/tpa.py:474-475: k and v share length and rank, q and k share h + dk
+    assert tuple(qb.shape) == (b, lq, rq, dk), qb.shape
+    assert tuple(ka.shape) == (b, lk, rk, h), ka.shape
+    assert tuple(kb.shape) == (b, lk, rk, dk), kb.shape
+    assert tuple(va.shape) == (b, lk, rk, h), va.shape
+    qseg = _segment_ids(q_segment_ids, b, lq, device)
+    kvseg = _segment_ids(kv_segment_ids, b, lk, device)
+    if (qseg is None) != (kvseg is None):
+        raise ValueError("q_segment_ids and kv_segment_ids must be given together")
+
+    o = torch.empty((b, lq, h, dv), dtype=dtype, device=device)
+    lse = torch.empty((b, h, lq), dtype=torch.float32, device=device) if return_lse else None
+    args = _d.TpaFwdArgs(
+        qa=_d.factor(qa), qb=_d.factor(qb), ka=_d.factor(ka), kb=_d.factor(kb), va=_d.factor(va), vb=_d.factor(vb),
+        q_segment_ids=qseg.data_ptr() if qseg is not None else None,
+        kv_segment_ids=kvseg.data_ptr() if kvseg is not None else None,
+        o=o.data_ptr(), lse=lse.data_ptr() if lse is not None else None,
+        B=b, lq=lq, lk=lk, H=h, dk=dk, dv=dv, rq=rq, rk=rk,
+        dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=int(bool(causal)), kernel=int(kernel),
+        workspace=None, workspace_bytes=0, num_splits=0,
+    )
+    lib = _d.load_library()
+    with torch.cuda.device(device):
+        _d.check("tpa_fwd", lib.tpa_fwd(args, _d.current_stream_ptr(device)))
+    return o, lse
+
+
+def tpa_decode(
+    qa, qb, ka, kb, va, vb,
+    sm_scale: float = 1.0,
+    num_splits: int = 0,
+    workspace: torch.Tensor | None = None,
+    kernel: int = _d.KERNEL_AUTO,
+):
+    """Few query tokens against a long factored KV cache (no mask), split over key ranges.
+
+    The reference has no separate entry point for this: it is tpa() with lq = 1
+    (block_q = min(128, lq), tpa/tpa.py:485).  Same operands as `tpa_factors`; the cache is
+    ka/kb/va/vb.  `workspace` (uint8, at least `decode_workspace_bytes(...)`) may be passed to
+    avoid the allocation.  Returns (o[b,lq,h,dv], lse[b,h,lq]).
+    """
+    device = _pick_device(qa, qb, ka, kb, va, vb)
+    qa, qb, ka, kb, va, vb = (_as_device_tensor(x, device) for x in (qa, qb, ka, kb, va, vb))
+    dtype = qa.dtype
+    b, lq, rq, h = qa.shape
+    _, lk, rk, dv = vb.shape
+    dk = qb.shape[-1]
+    assert tuple(kb.shape) == (b, lk, rk, dk), kb.shape
+    assert tuple(ka.shape) == (b, lk, rk, h) and tuple(va.shape) == (b, lk, rk, h)
+    lib = _d.load_library()
+    need = lib.tpa_decode_workspace_bytes(b, lq, lk, h, dv, num_splits)
+    if workspace is None:
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
+    o = torch.empty((b, lq, h, dv), dtype=dtype, device=device)
+    lse = torch.empty((b, h, lq), dtype=torch.float32, device=device)
+    args = _d.TpaFwdArgs(
+        qa=_d.factor(qa), qb=_d.factor(qb), ka=_d.factor(ka), kb=_d.factor(kb), va=_d.factor(va), vb=_d.factor(vb),
+        q_segment_ids=None, kv_segment_ids=None, o=o.data_ptr(), lse=lse.data_ptr(),
+        B=b, lq=lq, lk=lk, H=h, dk=dk, dv=dv, rq=rq, rk=rk,
+        dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=0, kernel=int(kernel),
+        workspace=workspace.data_ptr(), workspace_bytes=workspace.numel() * workspace.element_size(),
+        num_splits=int(num_splits),
+    )
+    with torch.cuda.device(device):
+        _d.check("tpa_decode", lib.tpa_decode(args, _d.current_stream_ptr(device)))
+    return o, lse
+
+
+def decode_workspace_bytes(b: int, lq: int, lk: int, h: int, dv: int, num_splits: int = 0) -> int:
+    return int(_d.load_library().tpa_decode_workspace_bytes(b, lq, lk, h, dv, num_splits))
+
+
+class _TpaFunction(torch.autograd.Function):
+    """Forward-only operator: the reference registers a vjp (tpa/tpa.py:217); this build raises."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, num_heads, qseg, kvseg, sm_scale, causal, kernel):
+        qa, qb = q[..., :num_heads], q[..., num_heads:]
+        ka, kb = k[..., :num_heads], k[..., num_heads:]
+        va, vb = v[..., :num_heads], v[..., num_heads:]
+        o, lse = tpa_factors(qa, qb, ka, kb, va, vb, qseg, kvseg, sm_scale, causal, kernel)
+        ctx.mark_non_differentiable(lse)
+        return o, lse
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise NotImplementedError("the TPA backward pass is not implemented in this build (forward only)")
+
+
+def _tpa_fwd(
+    q, k, v, num_heads, q_segment_ids, kv_segment_ids, sm_scale, causal, block_sizes, nomat, debug, interpret
+):
+    """tpa/tpa.py:124-165: returns (o, residuals) with residuals (q, k, v, qseg, kvseg, o, l),
+    l[b, lq, h] being the logsumexp in the reference's layout (a transposed view, fp32)."""
+    del block_sizes, nomat, debug
+    device = _pick_device(q, k, v)
+    q, k, v = (_as_device_tensor(x, device) for x in (q, k, v))
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("q, k, v must be [b, l, r, h + d]")
+    b, lq, rq, h_dk = q.shape
+    _, lk, rk, _ = v.shape  # rank and length of the keys are read from v (tpa/tpa.py:474)
+    assert tuple(k.shape) == (b, lk, rk, h_dk), k.shape  # tpa/tpa.py:475
+    assert 0 < num_heads < h_dk and num_heads < v.shape[-1], (num_heads, q.shape, v.shape)
+    kernel = _d.KERNEL_GENERIC if interpret else _d.KERNEL_AUTO
+    o, lse = _TpaFunction.apply(q, k, v, int(num_heads), q_segment_ids, kv_segment_ids, float(sm_scale), bool(causal), kernel)
+    l = lse.permute(0, 2, 1)
+    return o, (q, k, v, q_segment_ids, kv_segment_ids, o, l)
+
+
+def tpa(
+    q, k, v,
+    num_heads: int,
+    q_segment_ids=None,
+    kv_segment_ids=None,
+    sm_scale: float = 1.0,
+    causal: bool = False,
+    block_sizes: BlockSizes | None = None,
+    nomat: bool = False,
+    debug: bool = False,
+    interpret: bool = False,
+):
+    """Tensor Product Attention (tpa/tpa.py:73-121).
+
+    q[b,lq,rq,h+dk], k[b,lk,rk,h+dk], v[b,lk,rk,h+dv]: rank factors concatenated along the
+    last dimension, head factor first.  Returns o[b,lq,h,dv] in q's dtype.  numpy inputs give a
+    numpy result.
+    """
+    was_numpy = not isinstance(q, torch.Tensor)
+    o, _ = _tpa_fwd(
+        q, k, v, num_heads, q_segment_ids, kv_segment_ids, sm_scale, causal, block_sizes, nomat, debug, interpret
+    )
+    return o.cpu().numpy() if was_numpy and o.dtype != torch.bfloat16 else o
+
+
+def _fwd(
+    q, k, v, q_segment_ids, kv_segment_ids, num_heads, sm_scale, causal, block_sizes, nomat, debug, interpret
+):
+    """Per-batch-element forward (tpa/tpa.py:446-543): q[lq,rq,h+dk] ... -> (o[lq,h,dv], l[lq,h])."""
+    qs = None if q_segment_ids is None else torch.as_tensor(q_segment_ids)[None]
+    ks = None if kv_segment_ids is None else torch.as_tensor(kv_segment_ids)[None]
+    device = _pick_device(q, k, v)
+    q, k, v = (_as_device_tensor(x, device)[None] for x in (q, k, v))
+    o, res = _tpa_fwd(q, k, v, num_heads, qs, ks, sm_scale, causal, block_sizes, nomat, debug, interpret)
+    return o[0], res[-1][0]

@@ -1,0 +1,381 @@
+"""Parity of the HIP kernels (through the Python API -> C ABI) against the CPU oracle.
+
+Tolerances: fp32 outputs max-abs <= 1e-4, bf16 outputs <= 2e-2, logsumexp <= 1e-3.  The
+reference's own forward grid (tpa/tpa_test.py:60-125) uses rtol = atol = 1e-3 on fp32; it is
+run here at the tighter 1e-4.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import make_factors, segment_ids
+from oracle import tpa_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = 1e-4
+BF16_TOL = 2e-2
+LSE_TOL = 1e-3
+
+
+def to_gpu(x, dtype, device):
+    return torch.from_numpy(x).to(dtype).to(device)
+
+
+def as_f64(t):
+    return t.detach().float().cpu().numpy().astype(np.float64)
+
+
+def check(o, lse_bhl, o_ref, lse_ref_blh, tol, lse_tol=LSE_TOL):
+    o = as_f64(o)
+    lse = as_f64(lse_bhl).transpose(0, 2, 1)
+    np.testing.assert_array_equal(np.isnan(o), np.isnan(o_ref))
+    np.testing.assert_array_equal(np.isneginf(lse), np.isneginf(lse_ref_blh))
+    ok = ~np.isnan(o_ref)
+    # bf16 outputs carry 8 mantissa bits: the absolute bound is stated for outputs of order one
+    # and scales with the largest output when a test's values are larger than that
+    if tol == BF16_TOL:
+        tol = tol * max(1.0, float(np.max(np.abs(o_ref[ok]), initial=0.0)))
+    assert np.max(np.abs(o[ok] - o_ref[ok]), initial=0.0) <= tol
+    okl = ~np.isneginf(lse_ref_blh)
+    assert np.max(np.abs(lse[okl] - lse_ref_blh[okl]), initial=0.0) <= lse_tol
+
+
+# ---------------------------------------------------------------- the reference's forward grid
+@pytest.mark.parametrize("rank_q", [1, 6])
+@pytest.mark.parametrize("rank_k", [1, 4])
+@pytest.mark.parametrize("nomat", [False, True])
+@pytest.mark.parametrize(
+    "batch_size,lq,lk,h,dk,dv,segment_size",
+    [
+        (1, 8, 8, 1, 4, 6, 8),
+        (2, 1024, 128, 2, 3, 5, 42),
+        (2, 1024, 128, 2, 3, 5, None),
+        (2, 128, 1024, 2, 3, 5, 42),
+        (2, 128, 1024, 2, 3, 5, None),
+        (1, 1024, 1024, 2, 3, 5, 321),
+    ],
+)
+def test_reference_forward_grid(gpu, batch_size, rank_q, rank_k, nomat, lq, lk, h, dk, dv, segment_size):
+    """Shapes, ranks, segment sizes and uniform inputs of tpa/tpa_test.py:60-125."""
+    from tpa import tpa
+
+    q, k, v = make_factors(0, batch_size, lq, lk, h, dk, dv, rank_q, rank_k, dist="uniform")
+    qseg = segment_ids(lq, segment_size, batch_size) if segment_size else None
+    kvseg = segment_ids(lk, segment_size, batch_size) if segment_size else None
+    o_ref, l_ref = orc.tpa_reference(q, k, v, qseg, kvseg, h)
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    o, res = tpa._tpa_fwd(tq, tk, tv, h, qseg, kvseg, 1.0, False, None, nomat, False, False)
+    assert tuple(o.shape) == (batch_size, lq, h, dv)
+    check(o, res[-1].permute(0, 2, 1), o_ref, l_ref, F32_TOL)
+    # the public entry point returns the same array
+    o2 = tpa.tpa(tq, tk, tv, num_heads=h, q_segment_ids=qseg, kv_segment_ids=kvseg, nomat=nomat, interpret=True)
+    assert torch.equal(torch.nan_to_num(o2, nan=7.0), torch.nan_to_num(o, nan=7.0))
+
+
+# ---------------------------------------------------------------- fp32: config 1 and masks
+def test_config1_fp32_causal(gpu):
+    """B=1, T=512, H=8, D=64, Rq=6, Rk=Rv=2, N(0,1) factors, sm_scale = 1/sqrt(D), causal."""
+    from tpa import tpa
+
+    b, t, h, d = 1, 512, 8, 64
+    q, k, v = make_factors(0, b, t, t, h, d, d, 6, 2)
+    o_ref, l_ref = orc.tpa_reference(q, k, v, None, None, h, sm_scale=d**-0.5, causal=True)
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    o, res = tpa._tpa_fwd(tq, tk, tv, h, None, None, d**-0.5, True, None, False, False, False)
+    check(o, res[-1].permute(0, 2, 1), o_ref, l_ref, F32_TOL)
+
+
+@pytest.mark.parametrize("lq,lk", [(64, 64), (200, 77), (77, 200), (1, 300)])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("seg", [None, 19])
+def test_fp32_masks_and_ragged(gpu, lq, lk, causal, seg):
+    from tpa import tpa
+
+    b, h, dk, dv, rq, rk = 2, 3, 20, 12, 3, 2
+    q, k, v = make_factors(1, b, lq, lk, h, dk, dv, rq, rk)
+    qseg = segment_ids(lq, seg, b) if seg else None
+    kvseg = segment_ids(lk, seg, b) if seg else None
+    o_ref, l_ref = orc.tpa_reference(q, k, v, qseg, kvseg, h, sm_scale=0.25, causal=causal)
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    o, res = tpa._tpa_fwd(tq, tk, tv, h, qseg, kvseg, 0.25, causal, None, False, False, False)
+    check(o, res[-1].permute(0, 2, 1), o_ref, l_ref, F32_TOL)
+
+
+# ---------------------------------------------------------------- bf16 MFMA prefill
+def split(tq, tk, tv, h):
+    """The six split, contiguous factor arrays (the kernel-level operands, tpa/tpa.py:477-479)."""
+    return tuple(t.contiguous() for x in (tq, tk, tv) for t in (x[..., :h], x[..., h:]))
+
+
+def run_bf16(gpu, q, k, v, h, sm_scale, causal, kernel=2):
+    from tpa import tpa
+
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=sm_scale, causal=causal, kernel=kernel)
+    return (tq, tk, tv), o, lse
+
+
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize(
+    "b,lq,lk,h,rq,rk",
+    [
+        (2, 512, 512, 4, 6, 2),   # the benchmark ranks
+        (1, 300, 300, 2, 6, 2),   # ragged tails in both directions
+        (1, 257, 130, 2, 1, 1),   # lq > lk, rank 1
+        (1, 100, 700, 3, 3, 4),   # lk > lq, generic-rank loader
+        (1, 256, 256, 2, 16, 8),  # the high-rank configuration's ranks
+    ],
+)
+def test_prefill_bf16_mfma(gpu, d, causal, b, lq, lk, h, rq, rk):
+    # rank 1 has no 1/sqrt(R) damping: N(0,1) factors would give logits of order ten, where the
+    # bf16 rounding of Q and K alone moves the logsumexp by more than 1e-3; use the reference
+    # test's uniform [0,1) inputs there (tpa/tpa_test.py:89-91)
+    dist = "uniform" if rk == 1 else "normal"
+    q, k, v = make_factors(2, b, lq, lk, h, d, d, rq, rk, dist=dist, scale_by_rank=True)
+    scale = d**-0.5
+    (tq, tk, tv), o, lse = run_bf16(gpu, q, k, v, h, scale, causal)
+    o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h, sm_scale=scale, causal=causal)
+    check(o, lse, o_ref, l_ref, BF16_TOL)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_prefill_bf16_sharp_softmax(gpu, causal):
+    """Unscaled N(0,1) factors: logits of order one, so the softmax is far from flat and the
+    absolute tolerance actually bites (with the benchmark's 1/sqrt(R) scaling it hardly does)."""
+    b, t, h, d = 1, 512, 4, 64
+    q, k, v = make_factors(4, b, t, t, h, d, d, 6, 2)
+    (tq, tk, tv), o, lse = run_bf16(gpu, q, k, v, h, d**-0.5, causal)
+    o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h, sm_scale=d**-0.5, causal=causal)
+    check(o, lse, o_ref, l_ref, BF16_TOL, lse_tol=2e-3)
+    rel = np.abs(as_f64(o) - o_ref).max() / np.abs(o_ref).max()
+    assert rel < 2e-2
+
+
+def test_prefill_concatenated_layout_in_place(gpu):
+    """tpa() reads the A and B factors in place from the concatenated tensors (strided views)."""
+    from tpa import tpa
+
+    b, t, h, d = 1, 384, 8, 128
+    q, k, v = make_factors(5, b, t, t, h, d, d, 6, 2, scale_by_rank=True)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    o = tpa.tpa(tq, tk, tv, num_heads=h, sm_scale=d**-0.5, causal=True)
+    o_ref, _ = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h, sm_scale=d**-0.5, causal=True)
+    assert np.abs(as_f64(o) - o_ref).max() <= BF16_TOL
+    # and the generic kernel agrees on the same bf16 inputs
+    o_gen = tpa.tpa(tq, tk, tv, num_heads=h, sm_scale=d**-0.5, causal=True, interpret=True)
+    assert np.abs(as_f64(o_gen) - o_ref).max() <= BF16_TOL
+
+
+def sampled_rows_check(gpu, b, t, h, d, rq, rk, causal, rows, batches, seed=0):
+    q, k, v = make_factors(seed, b, t, t, h, d, d, rq, rk, scale_by_rank=True)
+    scale = d**-0.5
+    (tq, tk, tv), o, lse = run_bf16(gpu, q, k, v, h, scale, causal)
+    for bi in batches:
+        sl = slice(bi, bi + 1)
+        o_ref, l_ref = orc.tpa_reference_rows(
+            as_f64(tq[sl]), as_f64(tk[sl]), as_f64(tv[sl]), None, None, h, rows, sm_scale=scale, causal=causal, dtype=np.float32
+        )
+        got = as_f64(o[sl][:, rows])
+        got_l = as_f64(lse[sl][:, :, rows]).transpose(0, 2, 1)
+        assert np.abs(got - o_ref).max() <= BF16_TOL
+        assert np.abs(got_l - l_ref).max() <= LSE_TOL
+    return (tq, tk, tv), o, lse
+
+
+def test_config2_full_size_sampled_rows_and_prefix(gpu):
+    """B=4, T=4096, H=16, D=128, Rq=6, Rk=Rv=2, causal: sampled rows against the oracle, plus the
+    causal prefix property on the GPU result itself (rows < n of the full run equal a run on the
+    first n tokens, bit for bit up to tile-order effects -> compared at the bf16 tolerance)."""
+    from tpa import tpa
+
+    rows = np.array([0, 1, 63, 64, 255, 256, 1000, 2047, 2048, 4095])
+    (tq, tk, tv), o, lse = sampled_rows_check(gpu, 4, 4096, 16, 128, 6, 2, True, rows, batches=[0, 3])
+    n = 1024
+    h = 16
+    o_p, lse_p = tpa.tpa_factors(
+        tq[:, :n, :, :h], tq[:, :n, :, h:], tk[:, :n, :, :h], tk[:, :n, :, h:], tv[:, :n, :, :h], tv[:, :n, :, h:],
+        sm_scale=128**-0.5, causal=True,
+    )
+    assert torch.equal(o_p, o[:, :n])
+    assert torch.equal(lse_p, lse[:, :, :n])
+    # same inputs twice -> identical bits
+    o2, lse2 = tpa.tpa_factors(
+        tq[..., :h], tq[..., h:], tk[..., :h], tk[..., h:], tv[..., :h], tv[..., h:], sm_scale=128**-0.5, causal=True
+    )
+    assert torch.equal(o2, o) and torch.equal(lse2, lse)
+
+
+def test_config3_long_context_sampled_rows(gpu):
+    """B=1, T=32768, H=32, D=128, causal: sampled rows."""
+    rows = np.array([0, 255, 256, 4097, 16383, 32767])
+    sampled_rows_check(gpu, 1, 32768, 32, 128, 6, 2, True, rows, batches=[0])
+
+
+def test_config5_high_rank_noncausal_sampled_rows(gpu):
+    """B=8, T=2048, H=64, D=64, Rq=16, Rk=Rv=8, non-causal."""
+    rows = np.array([0, 100, 1023, 2047])
+    sampled_rows_check(gpu, 8, 2048, 64, 64, 16, 8, False, rows, batches=[0, 7])
+
+
+# ---------------------------------------------------------------- decode over the factored cache
+def run_decode(gpu, q, k, v, h, sm_scale, num_splits=0, kernel=2):
+    from tpa import tpa
+
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    o, lse = tpa.tpa_decode(*split(tq, tk, tv, h), sm_scale=sm_scale, num_splits=num_splits, kernel=kernel)
+    return (tq, tk, tv), o, lse
+
+
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize(
+    "b,lq,lk,h,rq,rk",
+    [
+        (3, 1, 1024, 32, 6, 2),
+        (2, 1, 1000, 32, 6, 2),  # cache length not a multiple of the block
+        (2, 1, 37, 32, 6, 2),    # shorter than one block per wave
+        (1, 2, 777, 16, 3, 1),   # two query tokens, 16 heads, rank 1
+        (1, 1, 515, 64, 2, 4),   # two head blocks, rank 4
+        (2, 1, 640, 8, 6, 2),
+    ],
+)
+def test_decode_bf16_mfma(gpu, d, b, lq, lk, h, rq, rk):
+    q, k, v = make_factors(6, b, lq, lk, h, d, d, rq, rk, scale_by_rank=True)
+    scale = d**-0.5
+    (tq, tk, tv), o, lse = run_decode(gpu, q, k, v, h, scale)
+    o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h, sm_scale=scale)
+    check(o, lse, o_ref, l_ref, BF16_TOL)
+
+
+def test_decode_sharp_softmax_and_split_invariance(gpu):
+    b, lk, h, d = 2, 2048, 32, 128
+    q, k, v = make_factors(8, b, 1, lk, h, d, d, 6, 2)
+    scale = d**-0.5
+    results = []
+    for s in (1, 2, 3, 8):
+        (tq, tk, tv), o, lse = run_decode(gpu, q, k, v, h, scale, num_splits=s)
+        results.append((as_f64(o), as_f64(lse)))
+    o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h, sm_scale=scale)
+    for o, lse in results:
+        assert np.abs(o - o_ref).max() <= BF16_TOL
+        assert np.abs(lse.transpose(0, 2, 1) - l_ref).max() <= 2e-3
+    # any number of key ranges gives the same answer up to fp32 re-association
+    for o, lse in results[1:]:
+        assert np.abs(o - results[0][0]).max() <= 2**-7 * np.abs(results[0][0]).max()
+        assert np.abs(lse - results[0][1]).max() <= 1e-4
+
+
+def test_decode_equals_last_causal_prefill_row(gpu):
+    """A single query over the whole cache == the last row of the causal prefill (lq == lk)."""
+    b, t, h, d = 2, 768, 32, 128
+    q, k, v = make_factors(9, b, t, t, h, d, d, 6, 2, scale_by_rank=True)
+    scale = d**-0.5
+    (tq, tk, tv), o, lse = run_bf16(gpu, q, k, v, h, scale, True)
+    _, od, lsed = run_decode(gpu, q[:, -1:], k, v, h, scale)
+    assert np.abs(as_f64(od[:, 0]) - as_f64(o[:, -1])).max() <= BF16_TOL
+    assert np.abs(as_f64(lsed[:, :, 0]) - as_f64(lse[:, :, -1])).max() <= LSE_TOL
+
+
+def test_config4_full_size_decode(gpu):
+    """B=64, lk=8192, H=32, D=128, Rq=6, Rk=Rv=2: batch entries 0 and 63 against the oracle."""
+    b, lk, h, d = 64, 8192, 32, 128
+    q, k, v = make_factors(0, b, 1, lk, h, d, d, 6, 2, scale_by_rank=True)
+    scale = d**-0.5
+    (tq, tk, tv), o, lse = run_decode(gpu, q, k, v, h, scale)
+    for bi in (0, 63):
+        sl = slice(bi, bi + 1)
+        o_ref, l_ref = orc.tpa_reference(as_f64(tq[sl]), as_f64(tk[sl]), as_f64(tv[sl]), None, None, h, sm_scale=scale, dtype=np.float32)
+        assert np.abs(as_f64(o[sl]) - o_ref).max() <= BF16_TOL
+        assert np.abs(as_f64(lse[sl]).transpose(0, 2, 1) - l_ref).max() <= LSE_TOL
+    # the generic kernel on the same inputs (no MFMA, no split) agrees
+    from tpa import tpa
+
+    og, lg = tpa.tpa_factors(
+        tq[:2, ..., :h], tq[:2, ..., h:], tk[:2, ..., :h], tk[:2, ..., h:], tv[:2, ..., :h], tv[:2, ..., h:], sm_scale=scale, kernel=1
+    )
+    assert np.abs(as_f64(og) - as_f64(o[:2])).max() <= BF16_TOL
+    assert np.abs(as_f64(lg) - as_f64(lse[:2])).max() <= LSE_TOL
+
+
+# ---------------------------------------------------------------- dense MHA baseline
+def test_mha_known_answer(gpu):
+    """tpa/mha_test.py:44-118: o = [[1,1],[1,1],[nan,nan]]."""
+    from tpa.mha import mha
+
+    q = torch.tensor([[2.0, 1.0], [1.0, 1.0], [1.0, 1.0]], device=gpu)[None, :, None, :]
+    k = torch.ones((1, 3, 1, 2), device=gpu)
+    v = torch.ones((1, 3, 1, 2), device=gpu)
+    ninf = float("-inf")
+    bias = torch.tensor([[0.0, ninf, 0.0], [0.0, ninf, 0.0], [ninf, ninf, ninf]], device=gpu)[None]
+    o = mha(q, k, v, bias).cpu().numpy()
+    np.testing.assert_allclose(o[0, :2, 0], [[1.0, 1.0], [1.0, 1.0]], rtol=1e-6)
+    assert np.isnan(o[0, 2, 0]).all()
+
+
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_mha_fp32_vs_oracle(gpu, with_bias):
+    from tpa.mha import _mha_fwd
+
+    rng = np.random.Generator(np.random.Philox(3))
+    b, lq, lk, h, dk, dv = 2, 70, 90, 3, 8, 5
+    q = rng.standard_normal((b, lq, h, dk), dtype=np.float32)
+    k = rng.standard_normal((b, lk, h, dk), dtype=np.float32)
+    v = rng.standard_normal((b, lk, h, dv), dtype=np.float32)
+    bias = None
+    if with_bias:
+        bias = rng.standard_normal((b, lq, lk), dtype=np.float32)
+        bias[rng.random((b, lq, lk)) < 0.3] = -np.inf
+        bias[:, 5] = -np.inf  # one empty row
+    o_ref, l_ref = orc.mha_forward(q.astype(np.float64), k.astype(np.float64), v.astype(np.float64), None if bias is None else bias.astype(np.float64), 0.5)
+    o, (lse,) = _mha_fwd(torch.from_numpy(q).to(gpu), torch.from_numpy(k).to(gpu), torch.from_numpy(v).to(gpu), bias, 0.5)
+    check(o, lse, o_ref, l_ref, F32_TOL)
+
+
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("causal", [False, True])
+def test_mha_bf16_flash_vs_oracle(gpu, d, causal):
+    from tpa.mha import _mha_fwd
+
+    rng = np.random.Generator(np.random.Philox(4))
+    b, lq, lk, h = 2, 333, 333, 4
+    q, k, v = (torch.from_numpy(rng.standard_normal((b, l, h, d), dtype=np.float32)).to(torch.bfloat16).to(gpu) for l in (lq, lk, lk))
+    bias = None
+    if causal:
+        bias = np.where(np.tril(np.ones((lq, lk), bool)), 0.0, -np.inf)[None].repeat(b, 0)
+    o_ref, l_ref = orc.mha_forward(as_f64(q), as_f64(k), as_f64(v), bias, d**-0.5)
+    o, (lse,) = _mha_fwd(q, k, v, None, d**-0.5, causal=causal, kernel=2)
+    check(o, lse, o_ref, l_ref, BF16_TOL, lse_tol=2e-3)
+
+
+def test_mha_equals_tpa_on_reconstructed_kv(gpu):
+    """Dense attention on the reconstructed Q, K, V agrees with TPA on the factors (what the
+    reference's oracle does, tpa/tpa_test.py:42-57)."""
+    from tpa.mha import mha
+
+    b, t, h, d = 1, 512, 4, 128
+    q, k, v = make_factors(10, b, t, t, h, d, d, 6, 2, scale_by_rank=True)
+    (tq, tk, tv), o, _ = run_bf16(gpu, q, k, v, h, d**-0.5, True)
+    rec = lambda x, r: (torch.einsum("blrh,blrd->blhd", x[..., :h].float(), x[..., h:].float()) / r).to(torch.bfloat16)
+    od = mha(rec(tq, 6), rec(tk, 2), rec(tv, 2), None, d**-0.5, causal=True)
+    assert np.abs(as_f64(od) - as_f64(o)).max() <= BF16_TOL
+
+
+# ---------------------------------------------------------------- error behaviour through the ABI
+def test_abi_error_codes(gpu):
+    from tpa import _dispatch as d
+    from tpa import tpa
+
+    x = torch.zeros((1, 8, 1, 4 + 3), device=gpu)
+    with pytest.raises(AssertionError):  # k does not match v's length (tpa/tpa.py:475)
+        tpa.tpa(x, x[:, :4], x, num_heads=4)
+    with pytest.raises(TypeError):
+        tpa.tpa(x.half(), x.half(), x.half(), num_heads=4)
+    with pytest.raises(NotImplementedError):
+        xr = x.clone().requires_grad_(True)
+        tpa.tpa(xr, x, x, num_heads=4).nansum().backward()
+    # MFMA kernel requested for a problem it cannot run -> TPA_ERR_UNSUPPORTED, nothing launched
+    with pytest.raises(d.TpaError) as e:
+        tpa.tpa_factors(x[..., :4], x[..., 4:], x[..., :4], x[..., 4:], x[..., :4], x[..., 4:], kernel=d.KERNEL_MFMA)
+    assert e.value.code == -6

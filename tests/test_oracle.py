@@ -1,0 +1,217 @@
+"""Pins the CPU oracle (oracle/tpa_oracle.py) without importing the reference: brute force,
+independent library routines, closed forms, invariances and the one literal known-answer the
+reference holds."""
+
+import numpy as np
+import pytest
+import scipy.special
+import torch
+
+from conftest import make_factors, segment_ids
+from oracle import tpa_oracle as orc
+
+
+def brute_force(q, k, v, qseg, kvseg, h, sm_scale, causal):
+    """Float64 scalar loops straight from the definition (tpa/tpa_test.py:22-57, tpa/mha.py:23-37)."""
+    b, lq, rq, _ = q.shape
+    _, lk, rk, _ = k.shape
+    dk = q.shape[-1] - h
+    dv = v.shape[-1] - h
+    o = np.zeros((b, lq, h, dv))
+    lse = np.zeros((b, lq, h))
+    for bi in range(b):
+        for hi in range(h):
+            for i in range(lq):
+                qv = np.zeros(dk)
+                for r in range(rq):
+                    qv += q[bi, i, r, hi] * q[bi, i, r, h:]
+                qv /= rq
+                logits = []
+                vals = []
+                for t in range(lk):
+                    kvec = np.zeros(dk)
+                    vvec = np.zeros(dv)
+                    for r in range(rk):
+                        kvec += k[bi, t, r, hi] * k[bi, t, r, h:]
+                        vvec += v[bi, t, r, hi] * v[bi, t, r, h:]
+                    kvec /= rk
+                    vvec /= rk
+                    x = sm_scale * float(qv @ kvec)
+                    if qseg is not None and qseg[bi, i] != kvseg[bi, t]:
+                        x = -np.inf
+                    if causal and t > i:
+                        x = -np.inf
+                    logits.append(x)
+                    vals.append(vvec)
+                logits = np.array(logits)
+                if np.all(np.isneginf(logits)):
+                    o[bi, i, hi] = np.nan
+                    lse[bi, i, hi] = -np.inf
+                    continue
+                mx = logits.max()
+                w = np.exp(logits - mx)
+                o[bi, i, hi] = (w[:, None] * np.array(vals)).sum(0) / w.sum()
+                lse[bi, i, hi] = mx + np.log(w.sum())
+    return o, lse
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("seg", [None, 3])
+@pytest.mark.parametrize("rq,rk", [(1, 1), (6, 4), (3, 2)])
+def test_brute_force_tiny(causal, seg, rq, rk):
+    # the reference's smallest shape (1, 8, 8, 1, 4, 6) and a ragged one
+    for (b, lq, lk, h, dk, dv) in [(1, 8, 8, 1, 4, 6), (2, 5, 7, 3, 2, 3)]:
+        q, k, v = make_factors(7, b, lq, lk, h, dk, dv, rq, rk)
+        qseg = segment_ids(lq, seg, b) if seg else None
+        kvseg = segment_ids(lk, seg, b) if seg else None
+        o, l = orc.tpa_reference(q, k, v, qseg, kvseg, h, sm_scale=0.7, causal=causal)
+        o_bf, l_bf = brute_force(q.astype(np.float64), k.astype(np.float64), v.astype(np.float64), qseg, kvseg, h, 0.7, causal)
+        np.testing.assert_allclose(o, o_bf, rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(l, l_bf, rtol=1e-12, atol=1e-12)
+
+
+def test_known_answer_from_reference_mha_test():
+    """tpa/mha_test.py:44-118 (commented out upstream): the only literal expected output."""
+    q = np.array([[2, 1], [1, 1], [1, 1]], dtype=float)[None, :, None, :]
+    k = np.ones((3, 2))[None, :, None, :]
+    v = np.ones((3, 2))[None, :, None, :]
+    ninf = -np.inf
+    bias = np.array([[0, ninf, 0], [0, ninf, 0], [ninf, ninf, ninf]])[None]
+    o, l = orc.mha_forward(q, k, v, bias)
+    expect = np.array([[1.0, 1.0], [1.0, 1.0], [np.nan, np.nan]])[None, :, None, :]
+    np.testing.assert_array_equal(o, expect)
+    assert np.isneginf(l[0, 2, 0])
+    # rows 0 and 1: logits (3, -inf, 3) and (2, -inf, 2)
+    np.testing.assert_allclose(l[0, :2, 0], [3 + np.log(2), 2 + np.log(2)], rtol=1e-14)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_against_torch_sdpa_and_scipy(causal):
+    b, l, h, dk, dv, rq, rk = 2, 33, 4, 16, 16, 6, 2
+    q, k, v = make_factors(3, b, l, l, h, dk, dv, rq, rk)
+    scale = 0.31
+    o, lse = orc.tpa_reference(q, k, v, None, None, h, sm_scale=scale, causal=causal)
+    # independent reconstruction with torch, attention with the library routine
+    tq, tk, tv = (torch.from_numpy(x).double() for x in (q, k, v))
+    Q = torch.einsum("blrh,blrd->bhld", tq[..., :h], tq[..., h:]) / rq
+    K = torch.einsum("blrh,blrd->bhld", tk[..., :h], tk[..., h:]) / rk
+    V = torch.einsum("blrh,blrd->bhld", tv[..., :h], tv[..., h:]) / rk
+    ref = torch.nn.functional.scaled_dot_product_attention(Q, K, V, is_causal=causal, scale=scale)
+    np.testing.assert_allclose(o, ref.permute(0, 2, 1, 3).numpy(), rtol=1e-9, atol=1e-11)
+    logits = scale * torch.einsum("bhqd,bhkd->bhqk", Q, K).numpy()
+    if causal:
+        logits = np.where(np.tril(np.ones((l, l), bool)), logits, -np.inf)
+    np.testing.assert_allclose(lse, scipy.special.logsumexp(logits, axis=-1).transpose(0, 2, 1), rtol=1e-12)
+    p = scipy.special.softmax(logits, axis=-1)
+    np.testing.assert_allclose(o, np.einsum("bhqk,bhkd->bqhd", p, V.numpy()), rtol=1e-9, atol=1e-12)
+
+
+def test_segments_against_sdpa_mask():
+    b, lq, lk, h, dk, dv, rq, rk = 2, 40, 24, 2, 8, 8, 2, 4
+    q, k, v = make_factors(5, b, lq, lk, h, dk, dv, rq, rk, dist="uniform")
+    qseg, kvseg = segment_ids(lq, 7, b), segment_ids(lk, 7, b)
+    o, lse = orc.tpa_reference(q, k, v, qseg, kvseg, h)
+    tq, tk, tv = (torch.from_numpy(x).double() for x in (q, k, v))
+    Q = torch.einsum("blrh,blrd->bhld", tq[..., :h], tq[..., h:]) / rq
+    K = torch.einsum("blrh,blrd->bhld", tk[..., :h], tk[..., h:]) / rk
+    V = torch.einsum("blrh,blrd->bhld", tv[..., :h], tv[..., h:]) / rk
+    mask = torch.from_numpy(qseg[:, :, None] == kvseg[:, None, :])[:, None]
+    ref = torch.nn.functional.scaled_dot_product_attention(Q, K, V, attn_mask=mask, scale=1.0).permute(0, 2, 1, 3).numpy()
+    has_key = mask[:, 0].any(-1).numpy()  # rows with at least one visible key
+    assert not has_key.all() and has_key.any()  # q ids run past the kv ids: some rows are empty
+    np.testing.assert_allclose(o[has_key], ref[has_key], rtol=1e-9, atol=1e-12)
+    # empty rows: NaN output, -inf logsumexp (tpa/tpa.py:437-439)
+    assert np.isnan(o[~has_key]).all()
+    assert np.isneginf(lse[~has_key]).all()
+
+
+def test_reference_shape_with_empty_rows():
+    """(2, 1024, 128, 2, 3, 5, 42) of tpa/tpa_test.py:67: q ids reach 24, kv ids stop at 3,
+    so rows >= 168 see no key."""
+    q, k, v = make_factors(0, 2, 1024, 128, 2, 3, 5, 1, 1, dist="uniform")
+    o, lse = orc.tpa_reference(q, k, v, segment_ids(1024, 42, 2), segment_ids(128, 42, 2), 2)
+    assert np.isfinite(o[:, :168]).all() and np.isnan(o[:, 168:]).all()
+    assert np.isfinite(lse[:, :168]).all() and np.isneginf(lse[:, 168:]).all()
+
+
+def test_closed_forms():
+    b, l, h, dk, dv, rq, rk = 1, 17, 3, 4, 5, 2, 3
+    q, k, v = make_factors(11, b, l, l, h, dk, dv, rq, rk)
+    q0 = q.copy()
+    q0[..., h:] = 0.0  # zero queries: uniform attention
+    V = orc.reconstruct(v[..., :h].astype(np.float64), v[..., h:].astype(np.float64))
+    o, lse = orc.tpa_reference(q0, k, v, None, None, h, causal=True)
+    running_mean = np.cumsum(V, axis=1) / np.arange(1, l + 1)[None, :, None, None]
+    np.testing.assert_allclose(o, running_mean, rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(lse, np.broadcast_to(np.log(np.arange(1, l + 1))[None, :, None], lse.shape), rtol=1e-12, atol=1e-14)
+    o, lse = orc.tpa_reference(q0, k, v, None, None, h, causal=False)
+    np.testing.assert_allclose(o, np.broadcast_to(V.mean(1, keepdims=True), o.shape), rtol=1e-12)
+    np.testing.assert_allclose(lse, np.log(l), rtol=1e-12)
+    # a single key: o = V[0], lse = the logit
+    o, lse = orc.tpa_reference(q, k[:, :1], v[:, :1], None, None, h, sm_scale=0.5)
+    np.testing.assert_allclose(o, np.broadcast_to(V[:, :1], o.shape), rtol=1e-12)
+    Q = orc.reconstruct(q[..., :h].astype(np.float64), q[..., h:].astype(np.float64))
+    K = orc.reconstruct(k[..., :h].astype(np.float64), k[..., h:].astype(np.float64))
+    np.testing.assert_allclose(lse, 0.5 * np.einsum("bqhd,bhd->bqh", Q, K[:, 0]), rtol=1e-12)
+
+
+def test_rank_invariances():
+    b, lq, lk, h, dk, dv, rq, rk = 2, 9, 11, 2, 4, 3, 3, 2
+    q, k, v = make_factors(13, b, lq, lk, h, dk, dv, rq, rk)
+    base, base_l = orc.tpa_reference(q, k, v, None, None, h, sm_scale=0.9)
+    # duplicating every rank leaves (1/R) sum unchanged
+    o, l = orc.tpa_reference(np.concatenate([q, q], 2), np.concatenate([k, k], 2), np.concatenate([v, v], 2), None, None, h, sm_scale=0.9)
+    np.testing.assert_allclose(o, base, rtol=1e-12)
+    np.testing.assert_allclose(l, base_l, rtol=1e-12)
+    # permuting ranks
+    o, _ = orc.tpa_reference(q[:, :, ::-1], k[:, :, ::-1], v[:, :, ::-1], None, None, h, sm_scale=0.9)
+    np.testing.assert_allclose(o, base, rtol=1e-12)
+    # a * c with b / c
+    k2 = k.astype(np.float64).copy()
+    k2[..., :h] *= 4.0
+    k2[..., h:] /= 4.0
+    o, _ = orc.tpa_reference(q, k2, v, None, None, h, sm_scale=0.9)
+    np.testing.assert_allclose(o, base, rtol=1e-12)
+    # rank 1 with a == 1: every head shares b (multi-query attention)
+    k1 = k[:, :, :1].copy()
+    k1[..., :h] = 1.0
+    K = orc.reconstruct(k1[..., :h].astype(np.float64), k1[..., h:].astype(np.float64))
+    np.testing.assert_allclose(K[:, :, 0], K[:, :, 1], rtol=0)
+
+
+def test_causal_prefix_and_decode_row():
+    b, l, h, dk, dv, rq, rk = 1, 24, 2, 8, 8, 6, 2
+    q, k, v = make_factors(17, b, l, l, h, dk, dv, rq, rk)
+    full, full_l = orc.tpa_reference(q, k, v, None, None, h, sm_scale=0.4, causal=True)
+    part, part_l = orc.tpa_reference(q[:, :10], k[:, :10], v[:, :10], None, None, h, sm_scale=0.4, causal=True)
+    np.testing.assert_allclose(full[:, :10], part, rtol=1e-12)
+    np.testing.assert_allclose(full_l[:, :10], part_l, rtol=1e-12)
+    # the last causal row equals an unmasked single-query call over the whole cache
+    dec, dec_l = orc.tpa_reference(q[:, -1:], k, v, None, None, h, sm_scale=0.4, causal=False)
+    np.testing.assert_allclose(full[:, -1:], dec, rtol=1e-12)
+    np.testing.assert_allclose(full_l[:, -1:], dec_l, rtol=1e-12)
+
+
+def test_rows_variant_matches_full():
+    b, lq, lk, h, dk, dv, rq, rk = 2, 37, 29, 3, 4, 6, 2, 2
+    q, k, v = make_factors(19, b, lq, lk, h, dk, dv, rq, rk)
+    qseg, kvseg = segment_ids(lq, 9, b), segment_ids(lk, 9, b)
+    rows = np.array([0, 5, 28, 36])
+    for causal in (False, True):
+        full, full_l = orc.tpa_reference(q, k, v, qseg, kvseg, h, sm_scale=0.3, causal=causal)
+        sub, sub_l = orc.tpa_reference_rows(q, k, v, qseg, kvseg, h, rows, sm_scale=0.3, causal=causal)
+        np.testing.assert_array_equal(np.isnan(sub), np.isnan(full[:, rows]))
+        np.testing.assert_allclose(sub, full[:, rows], rtol=1e-12)
+        np.testing.assert_allclose(sub_l, full_l[:, rows], rtol=1e-12)
+
+
+def test_lse_helpers():
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((4, 9))
+    np.testing.assert_allclose(orc.lse(x), scipy.special.logsumexp(x, axis=-1), rtol=1e-13)
+    # split-and-merge gives the logsumexp of the whole (tpa/tpa.py:228-242)
+    np.testing.assert_allclose(orc.lse_accum(orc.lse(x[:, :4]), orc.lse(x[:, 4:])), orc.lse(x), rtol=1e-13)
+    ninf = np.full((4,), -np.inf)
+    assert np.isneginf(orc.lse(np.full((4, 3), -np.inf))).all()
+    assert np.isneginf(orc.lse_accum(ninf, ninf)).all()
+    np.testing.assert_allclose(orc.lse_accum(ninf, x[:, 0]), x[:, 0])
