@@ -1,0 +1,228 @@
+#!/usr/bin/env python3
+"""Benchmark of the TPA forward hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5] [--no-cpu]
+
+A step is one forward pass over one batch of synthetic, seeded inputs that are resident in HBM
+before the timed region starts.  The default workload is the prefill configuration the headline
+metric is quoted on (c2: B=4, T=4096, H=16, D=128, Rq=6, Rk=Rv=2, bf16, causal); the same run
+also times the decode configuration (c4: B=64, cache 8192, H=32, D=128) and reports it in the
+"decode" object, and times the CPU oracle on a bounded sample of c2 ("cpu_baseline").
+One JSON line is printed on stdout; progress goes to stderr.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "tensor-product-attention-jax_amd"))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2516.6  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+WORKLOADS = {
+    # name: (kind, B, lq, lk, H, D, rq, rk, causal)
+    "c2": ("prefill", 4, 4096, 4096, 16, 128, 6, 2, True),
+    "c3": ("prefill", 1, 32768, 32768, 32, 128, 6, 2, True),
+    "c5": ("prefill", 8, 2048, 2048, 64, 64, 16, 8, False),
+    "c4": ("decode", 64, 1, 8192, 32, 128, 6, 2, False),
+}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed):
+    """Split factor arrays, i.i.d. N(0,1) / sqrt(R), bf16, generated on the device."""
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+
+    def draw(shape, r):
+        return (torch.randn(shape, generator=g, device=device, dtype=torch.float32) / r**0.5).to(torch.bfloat16)
+
+    return (
+        draw((B, lq, rq, H), rq), draw((B, lq, rq, D), rq),
+        draw((B, lk, rk, H), rk), draw((B, lk, rk, D), rk),
+        draw((B, lk, rk, H), rk), draw((B, lk, rk, D), rk),
+    )
+
+
+def prefill_flops(B, lq, lk, H, D, causal):
+    pairs = lq * lk / 2 if causal else lq * lk
+    return 2.0 * B * H * (D + D) * pairs
+
+
+def decode_bytes(B, lq, lk, H, D, rq, rk):
+    cache = B * lk * (rk + rk) * (H + D) * 2
+    qf = B * lq * rq * (H + D) * 2
+    out = B * lq * H * D * 2 + B * H * lq * 4
+    return cache + qf + out
+
+
+def time_steps(torch, fn, steps, warmup):
+    """Returns (wall ms per step over the whole timed region, mean ms per launch from events)."""
+    for _ in range(warmup):
+        fn(0)
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        fn(i)
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev = [s.elapsed_time(e) for s, e in zip(starts, ends)]
+    return wall_ms, sum(ev) / len(ev), min(ev)
+
+
+def run_prefill(torch, tpa, device, name, steps, warmup):
+    _, B, lq, lk, H, D, rq, rk, causal = WORKLOADS[name]
+    x = make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed=0)
+    scale = D**-0.5
+    out = {}
+
+    def step(i):
+        out["o"], out["lse"] = tpa.tpa_factors(*x, sm_scale=scale, causal=causal, kernel=2)
+
+    wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
+    fl = prefill_flops(B, lq, lk, H, D, causal)
+    return dict(
+        wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, flops=fl,
+        tflops_wall=fl / wall_ms / 1e9, tflops_kernel=fl / ev_ms / 1e9,
+        shape=dict(B=B, lq=lq, lk=lk, H=H, D=D, rank_q=rq, rank_k=rk, causal=causal), inputs=x, out=out,
+    )
+
+
+def run_decode(torch, tpa, device, name, steps, warmup):
+    _, B, lq, lk, H, D, rq, rk, _ = WORKLOADS[name]
+    # two distinct caches, alternated, so that no launch finds its cache in the 256 MB last-level cache
+    xs = [make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed=s) for s in (0, 1)]
+    scale = D**-0.5
+    ws = torch.empty(max(tpa.decode_workspace_bytes(B, lq, lk, H, D), 16), dtype=torch.uint8, device=device)
+    out = {}
+
+    def step(i):
+        out["o"], out["lse"] = tpa.tpa_decode(*xs[i & 1], sm_scale=scale, workspace=ws, kernel=2)
+
+    wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
+    nbytes = decode_bytes(B, lq, lk, H, D, rq, rk)
+    return dict(
+        wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, bytes=nbytes,
+        gbs_wall=nbytes / wall_ms / 1e6, gbs_kernel=nbytes / ev_ms / 1e6,
+        shape=dict(B=B, lq=lq, lk=lk, H=H, D=D, rank_q=rq, rank_k=rk), inputs=xs[0], out=out,
+    )
+
+
+def cpu_baseline_prefill(torch, inputs, shape, heads=8):
+    """The numpy oracle on batch 0 and the first `heads` heads of the prefill workload."""
+    import numpy as np
+
+    from oracle import tpa_oracle as orc
+
+    qa, qb, ka, kb, va, vb = (t[:1].float().cpu().numpy() for t in inputs)
+    cat = lambda a, b: np.concatenate([a[..., :heads], b], axis=-1)
+    q, k, v = cat(qa, qb), cat(ka, kb), cat(va, vb)
+    D = shape["D"]
+    t0 = time.perf_counter()
+    o, lse = orc.tpa_reference(q, k, v, None, None, heads, sm_scale=D**-0.5, causal=shape["causal"], dtype=np.float32)
+    dt = time.perf_counter() - t0
+    fl = prefill_flops(1, shape["lq"], shape["lk"], heads, D, shape["causal"])
+    try:
+        from threadpoolctl import threadpool_info
+
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] + [1])
+    except Exception:
+        threads = os.cpu_count() or 1
+    return dict(
+        value=fl / dt / 1e12, unit="TFLOP/s", cores=threads, kind="port",
+        sample=f"numpy fp32 oracle, batch 0, heads 0..{heads - 1} of the workload ({dt:.1f} s); "
+        f"matmuls on {threads} BLAS threads of {os.cpu_count()} host cores, the rest single-threaded",
+    ), o, lse
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-decode", action="store_true", help="skip the secondary decode measurement")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (no collectives are built); use --gpus 1")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no HIP device visible")
+    from tpa import tpa
+
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    kind = WORKLOADS[args.workload][0]
+    result = {}
+    if kind == "prefill":
+        log(f"[bench] prefill {args.workload}: warmup {args.warmup}, steps {args.steps}")
+        r = run_prefill(torch, tpa, device, args.workload, args.steps, args.warmup)
+        log(f"[bench] {r['kernel_ms']:.4f} ms/launch (min {r['kernel_ms_min']:.4f}), {r['tflops_kernel']:.1f} TFLOP/s")
+        result.update(
+            metric="TPA causal prefill forward throughput" if r["shape"]["causal"] else "TPA prefill forward throughput",
+            value=r["tflops_wall"], unit="TFLOP/s", ms_per_step=r["wall_ms"],
+            roofline=dict(bound="mfma", achieved=r["tflops_kernel"], peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
+                          frac=r["tflops_kernel"] / PEAK_BF16_TFLOPS, traffic=None,
+                          kernel="prefill_kernel", ms_per_launch=r["kernel_ms"], ms_per_launch_min=r["kernel_ms_min"],
+                          algorithmic_flops_per_launch=r["flops"]),
+            config=dict(workload=f"{args.workload}: TPA prefill", **r["shape"]),
+        )
+        if not args.no_decode:
+            log("[bench] decode c4")
+            d = run_decode(torch, tpa, device, "c4", args.steps, args.warmup)
+            log(f"[bench] {d['kernel_ms']*1e3:.1f} us/launch (min {d['kernel_ms_min']*1e3:.1f}), {d['gbs_kernel']:.0f} GB/s")
+            result["decode"] = dict(
+                metric="TPA decode effective HBM bandwidth", value=d["gbs_wall"], unit="GB/s", ms_per_step=d["wall_ms"],
+                roofline=dict(bound="hbm", achieved=d["gbs_kernel"], peak=PEAK_HBM_GBS, unit="GB/s",
+                              frac=d["gbs_kernel"] / PEAK_HBM_GBS, traffic=None, kernel="decode_kernel + decode_merge_kernel",
+                              ms_per_launch=d["kernel_ms"], ms_per_launch_min=d["kernel_ms_min"],
+                              algorithmic_bytes_per_launch=d["bytes"]),
+                config=dict(workload="c4: TPA decode over the factored KV cache", **d["shape"]),
+            )
+        if not args.no_cpu and args.workload == "c2":
+            log("[bench] cpu baseline (numpy oracle on a sample)")
+            base, o_ref, _ = cpu_baseline_prefill(torch, r["inputs"], r["shape"])
+            result["cpu_baseline"] = base
+            # the sample doubles as a parity check of the timed kernel's output
+            heads = o_ref.shape[2]
+            err = float(abs(r["out"]["o"][:1, :, :heads].float().cpu().numpy() - o_ref).max())
+            result["max_abs_err_vs_oracle_sample"] = err
+            log(f"[bench] cpu {base['value']*1e3:.2f} GFLOP/s; max abs err vs oracle on the sample {err:.2e}")
+    else:
+        log(f"[bench] decode {args.workload}: warmup {args.warmup}, steps {args.steps}")
+        d = run_decode(torch, tpa, device, args.workload, args.steps, args.warmup)
+        log(f"[bench] {d['kernel_ms']*1e3:.1f} us/launch (min {d['kernel_ms_min']*1e3:.1f}), {d['gbs_kernel']:.0f} GB/s")
+        result.update(
+            metric="TPA decode effective HBM bandwidth", value=d["gbs_wall"], unit="GB/s", ms_per_step=d["wall_ms"],
+            roofline=dict(bound="hbm", achieved=d["gbs_kernel"], peak=PEAK_HBM_GBS, unit="GB/s",
+                          frac=d["gbs_kernel"] / PEAK_HBM_GBS, traffic=None, kernel="decode_kernel + decode_merge_kernel",
+                          ms_per_launch=d["kernel_ms"], ms_per_launch_min=d["kernel_ms_min"],
+                          algorithmic_bytes_per_launch=d["bytes"]),
+            config=dict(workload=f"{args.workload}: TPA decode over the factored KV cache", **d["shape"]),
+        )
+    result.update(
+        n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True, scaling="weak",
+        vs_baseline=None, dtype="bf16", data="synthetic",
+    )
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -50,7 +50,8 @@ def split_factors(x: np.ndarray, num_heads: int):
 def reconstruct(a: np.ndarray, b: np.ndarray) -> np.ndarray:
     """(1/R) * sum_r a[b,l,r,h] * b[b,l,r,d] -> [b, l, h, d].  tpa/tpa_test.py:42-44."""
     rank = a.shape[2]
-    return np.einsum("blrh,blrd->blhd", a, b) / rank
+    # per token an [h, r] x [r, d] product
+    return np.matmul(np.swapaxes(a, 2, 3), b) / rank
 
 
 def attention_bias(batch, lq, lk, q_segment_ids, kv_segment_ids, causal, dtype=np.float64):
@@ -90,7 +91,8 @@ def mha_forward(q, k, v, bias=None, sm_scale=1.0):
     q[b,lq,h,dk] k[b,lk,h,dk] v[b,lk,h,dv] bias[b,lq,lk] -> (o[b,lq,h,dv], lse[b,lq,h]).
     A row whose logits are all -inf gives o = NaN and lse = -inf.
     """
-    x = np.einsum("bqhd,bkhd->bhqk", q, k)
+    # the two contractions go through matmul (BLAS) rather than einsum's scalar loops
+    x = np.matmul(np.transpose(q, (0, 2, 1, 3)), np.transpose(k, (0, 2, 3, 1)))  # b h lq lk
     x = sm_scale * x
     if bias is not None:
         x = x + bias[:, None, :, :]
@@ -100,7 +102,7 @@ def mha_forward(q, k, v, bias=None, sm_scale=1.0):
         s = np.sum(e, axis=-1, keepdims=True)
         p = e / s
         l_ = np.where(np.isneginf(m[..., 0]), -np.inf, m[..., 0] + np.log(s[..., 0]))
-    o = np.einsum("bhqk,bkhd->bqhd", p, v)
+    o = np.transpose(np.matmul(p, np.transpose(v, (0, 2, 1, 3))), (0, 2, 1, 3))  # b lq h dv
     return o, np.transpose(l_, (0, 2, 1))
 
 

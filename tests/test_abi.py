@@ -1,0 +1,98 @@
+"""CPU-side checks of the C ABI: the library loads, exports every function include/tpa_abi.h
+declares, and the ctypes structures have the layout the C compiler gives the header's."""
+
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+from conftest import ROOT
+
+HEADER = os.path.join(ROOT, "include", "tpa_abi.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    body = text[text.index('extern "C" {'):]
+    names = re.findall(r"^\s*(?:const\s+)?[A-Za-z_][\w\s\*]*?\b(\w+)\s*\([^;{]*\)\s*;", body, flags=re.M)
+    return sorted(set(names))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_functions()
+    for f in ("tpa_fwd", "tpa_decode", "mha_fwd", "tpa_decode_workspace_bytes", "tpa_strerror", "tpa_abi_version"):
+        assert f in names, names
+
+
+def test_library_exports_every_declared_symbol():
+    from tpa import _dispatch
+
+    lib = _dispatch.load_library()
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} is declared in tpa_abi.h but not exported"
+    assert lib.tpa_abi_version() == _dispatch.ABI_VERSION
+    assert lib.tpa_strerror(0) == b"ok"
+    assert b"workspace" in lib.tpa_strerror(-5)
+
+
+def test_struct_layout_matches_the_c_compiler(tmp_path):
+    from tpa import _dispatch as d
+
+    fields = {"TpaFactor": d.TpaFactor, "TpaFwdArgs": d.TpaFwdArgs, "MhaFwdArgs": d.MhaFwdArgs}
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "tpa_abi.h"', "int main(void) {"]
+    for sname, cls in fields.items():
+        lines.append(f'printf("{sname} %zu\\n", sizeof({sname}));')
+        for fname, _ in cls._fields_:
+            lines.append(f'printf("{sname}.{fname} %zu\\n", offsetof({sname}, {fname}));')
+    lines.append("return 0; }")
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout
+    got = dict(line.split() for line in out.strip().splitlines())
+    for sname, cls in fields.items():
+        assert int(got[sname]) == ctypes.sizeof(cls), sname
+        for fname, _ in cls._fields_:
+            assert int(got[f"{sname}.{fname}"]) == getattr(cls, fname).offset, f"{sname}.{fname}"
+
+
+def test_size_queries_need_no_gpu():
+    from tpa import _dispatch
+
+    lib = _dispatch.load_library()
+    # config 4: 64 sequences, one query token, 32 heads -> 4 key ranges fill the 256 CUs
+    assert lib.tpa_decode_default_splits(64, 1, 8192, 32) == 4
+    assert lib.tpa_decode_workspace_bytes(64, 1, 8192, 32, 128, 0) == 64 * 4 * 32 * (128 + 2) * 4
+    assert lib.tpa_decode_workspace_bytes(64, 1, 8192, 32, 128, 7) == 64 * 7 * 32 * (128 + 2) * 4
+    assert lib.tpa_decode_default_splits(0, 1, 8192, 32) == 0
+
+
+def test_null_and_shape_errors_are_reported_before_any_launch():
+    """Validation happens on the host: these calls return error codes without touching a GPU."""
+    from tpa import _dispatch as d
+
+    lib = d.load_library()
+    assert lib.tpa_fwd(None, None) == -1
+    args = d.TpaFwdArgs()
+    args.dtype = 5
+    assert lib.tpa_fwd(ctypes.byref(args), None) == -3
+    args.dtype = d.TPA_DTYPE_BF16
+    assert lib.tpa_fwd(ctypes.byref(args), None) == -2  # all dimensions are zero
+    args.B = args.lq = args.lk = args.H = args.dk = args.dv = args.rq = args.rk = 1
+    assert lib.tpa_fwd(ctypes.byref(args), None) == -1  # factor pointers are NULL
+    args.dk = 1000
+    assert lib.tpa_decode(ctypes.byref(args), None) == -2
+    margs = d.MhaFwdArgs()
+    assert lib.mha_fwd(ctypes.byref(margs), None) == -2
+    assert lib.mha_fwd(None, None) == -1
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    from tpa import _dispatch
+
+    with pytest.raises(RuntimeError, match="not built"):
+        _dispatch.load_library(str(tmp_path / "nope.so"))

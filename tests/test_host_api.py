@@ -1,0 +1,71 @@
+"""Host-side behaviour of the Python operator API that needs no GPU."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import tpa_oracle as orc
+
+
+def test_module_layout_mirrors_the_reference():
+    from tpa import mha, tpa
+
+    # names other code reaches for (tpa/ring_tpa.py:82,241,244; tpa/mha_test.py:6)
+    for name in ("tpa", "BlockSizes", "_fwd", "_tpa_fwd", "_lse", "_lse_accum"):
+        assert hasattr(tpa, name), name
+    for name in ("mha", "_mha_fwd"):
+        assert hasattr(mha, name), name
+    bs = tpa.BlockSizes()
+    assert (bs.block_q, bs.block_kv, bs.block_h) == (128, 128, 4)  # tpa/tpa.py:39-70
+
+
+def test_signature_matches_the_reference():
+    import inspect
+
+    from tpa import mha, tpa
+
+    params = list(inspect.signature(tpa.tpa).parameters)
+    assert params == [
+        "q", "k", "v", "num_heads", "q_segment_ids", "kv_segment_ids", "sm_scale", "causal",
+        "block_sizes", "nomat", "debug", "interpret",
+    ]  # tpa/tpa.py:74-87
+    sig = inspect.signature(tpa.tpa)
+    assert sig.parameters["sm_scale"].default == 1.0 and sig.parameters["causal"].default is False
+    assert list(inspect.signature(mha.mha).parameters)[:5] == ["q", "k", "v", "bias", "sm_scale"]  # tpa/mha.py:11-17
+
+
+def test_lse_helpers_match_the_oracle():
+    from tpa import tpa
+
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((5, 7)).astype(np.float32)
+    x[2] = -np.inf
+    got = tpa._lse(torch.from_numpy(x)).numpy()
+    np.testing.assert_allclose(got, orc.lse(x.astype(np.float64)), rtol=1e-6)
+    a = torch.tensor([0.3, -np.inf, -np.inf, 2.0])
+    b = torch.tensor([1.1, -np.inf, 0.5, -np.inf])
+    np.testing.assert_allclose(tpa._lse_accum(a, b).numpy(), orc.lse_accum(a.numpy().astype(np.float64), b.numpy().astype(np.float64)), rtol=1e-6)
+
+
+def test_no_gpu_means_an_error_not_a_fallback():
+    from tpa import tpa
+
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is visible")
+    x = np.zeros((1, 4, 1, 6), dtype=np.float32)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        tpa.tpa(x, x, x, num_heads=2)
+
+
+def test_product_package_never_imports_the_oracle():
+    import os
+    import re
+
+    from conftest import PKG_PARENT
+
+    pat = re.compile(r"^\s*(from|import)\s+\.*oracle\b|tpa_oracle|oracle/", re.M)
+    for dirpath, _, files in os.walk(PKG_PARENT):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cc", "Makefile")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert not pat.search(text), os.path.join(dirpath, f)
