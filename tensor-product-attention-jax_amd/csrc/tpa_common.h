@@ -70,6 +70,47 @@ __device__ __forceinline__ float halves_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// Q fragments from rank factors: qf[ks] = bf16( scale * sum_r a[r] * b[r][16 ks + 0..7] ), where
+// `ap` points at this lane's a[0] (rank stride a_stride) and `bp` at b[0][this lane's first
+// element] (rank stride b_stride).  Ranks are taken G at a time with all 16-byte loads of the
+// group in flight together, so the exposed memory latency is ceil(rq / G) round trips.
+template <int NKS, int G>
+__device__ __forceinline__ void build_q_fragments(const uint16_t* ap, int64_t a_stride, const uint16_t* bp, int64_t b_stride,
+                                                  int rq, float scale, bf16x8 (&qf)[NKS]) {
+  float acc[NKS][8];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[ks][j] = 0.f;
+  for (int r0 = 0; r0 < rq; r0 += G) {
+    float a[G];
+    u32x4 bv[G][NKS];
+#pragma unroll
+    for (int q = 0; q < G; ++q) {
+      const int r = min(r0 + q, rq - 1);  // clamped reads past the last rank get weight 0
+      a[q] = r0 + q < rq ? bf16bits_to_f32(ap[r * a_stride]) : 0.f;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) bv[q][ks] = *reinterpret_cast<const u32x4*>(bp + r * b_stride + 16 * ks);
+    }
+#pragma unroll
+    for (int q = 0; q < G; ++q)
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[ks][2 * j] += a[q] * bf16lo_to_f32(bv[q][ks][j]);
+          acc[ks][2 * j + 1] += a[q] * bf16hi_to_f32(bv[q][ks][j]);
+        }
+  }
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) {
+    u32x4 packed;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) packed[j] = pack_bf16(acc[ks][2 * j] * scale, acc[ks][2 * j + 1] * scale);
+    qf[ks] = __builtin_bit_cast(bf16x8, packed);
+  }
+}
+
 }  // namespace tpa
 
 // host-side entry points of the individual kernel files (launchers return TPA_* codes)

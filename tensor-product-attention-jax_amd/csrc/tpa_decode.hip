@@ -9,12 +9,14 @@
 // heads as the N dimension.  Every cache byte is read from HBM exactly once for all heads.
 //
 // A workgroup has 4 independent waves; each streams its own range of 32-row blocks
-// (32 / Rk tokens) with fully coalesced 16-byte loads that stay in flight in registers one
-// block ahead, stages the block in its private LDS region (XOR-swizzled so that both the
+// (32 / Rk tokens) with fully coalesced 16-byte loads that stay in flight in registers two
+// blocks ahead, stages the block in its private LDS region (XOR-swizzled so that both the
 // 16-byte operand reads and the transposed reads are bank-conflict free), and keeps a private
 // online softmax (tpa/tpa.py:389-424).  The waves are merged through LDS, the key ranges
 // through a workspace and a small second kernel, both with the rule of _lse_accum
 // (tpa/tpa.py:228-242).
+#include <type_traits>
+
 #include "tpa_common.h"
 
 namespace tpa {
@@ -22,6 +24,7 @@ namespace {
 
 constexpr int kWaves = 4;
 constexpr int kRowsPerBlock = 32;
+
 
 struct DecodeParams {
   TpaFactor qa, qb, ka, kb, va, vb;
@@ -70,38 +73,22 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   uint16_t* lds_ak = lds + 2 * DecodeLds<D>::kB;
   uint16_t* lds_av = lds_ak + DecodeLds<D>::kA;
 
-  // ---- Qm^T fragments (B operand of S'^T = B_k Qm^T): lane (h, g) holds Qm[h][16ks + 8g + 0..7]
+  // ---- Qm^T fragments (B operand of S'^T = B_k Qm^T): lane (h, g) holds Qm[h][16ks + 8g + 0..7].
+  // Called after the first cache loads are in flight so that their latency is not exposed.
   bf16x8 qf[NKS];
-  {
+  auto build_q = [&]() {
     const uint16_t* ap = static_cast<const uint16_t*>(p.qa.ptr) + b * p.qa.stride_b + (int64_t)qi * p.qa.stride_l + hl;
     const uint16_t* bp = static_cast<const uint16_t*>(p.qb.ptr) + b * p.qb.stride_b + (int64_t)qi * p.qb.stride_l + 8 * g;
-#pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) {
-      float acc[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) acc[j] = 0.f;
-      for (int r = 0; r < p.rq; ++r) {
-        const float a = bf16bits_to_f32(ap[r * p.qa.stride_r]);
-        const u32x4 bv = *reinterpret_cast<const u32x4*>(bp + r * p.qb.stride_r + 16 * ks);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          acc[2 * j] += a * bf16lo_to_f32(bv[j]);
-          acc[2 * j + 1] += a * bf16hi_to_f32(bv[j]);
-        }
-      }
-      u32x4 packed;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) packed[j] = pack_bf16(acc[2 * j] * p.qscale, acc[2 * j + 1] * p.qscale);
-      qf[ks] = __builtin_bit_cast(bf16x8, packed);
-    }
-  }
+    build_q_fragments<NKS, 6>(ap, p.qa.stride_r, bp, p.qb.stride_r, p.rq, p.qscale, qf);
+  };
 
-  // ---- this wave's block range
+  // ---- this wave's blocks: part, part + nparts, part + 2 nparts, ... (dealt round robin, so the
+  // waves of the grid, which advance in step, read neighbouring addresses at any one time)
   const int nparts = S * kWaves;
   const int part = split * kWaves + w;
-  const int per = (p.nblocks + nparts - 1) / nparts;
-  const int blk_begin = min(part * per, p.nblocks);
-  const int blk_end = min(blk_begin + per, p.nblocks);
+  const int blk_begin = part;
+  const int blk_end = p.nblocks;
+  const int blk_step = nparts;
   const int last_row = p.lk * RK - 1;
 
   // rows of the cache matrices: row = token * RK + rank, row stride = stride_r
@@ -115,35 +102,38 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   const int lb_row = l / CPR, lb_c = l % CPR;             // B tiles: row within the instruction, chunk
   const int la_row = l >> 2, la_c = min(l & 3, a_chunks - 1);  // A tiles: 16 rows per instruction
 
-  u32x4 rbk[NLB], rbv[NLB], rak[2], rav[2];
-  auto issue = [&](int blk) {
+  // two register sets: while one block is staged and consumed, two more are in flight
+  u32x4 rbk[2][NLB], rbv[2][NLB], rak[2][2], rav[2][2];
+  auto issue = [&](auto set_c, int blk) {
+    constexpr int set = decltype(set_c)::value;
     const int row0 = blk * kRowsPerBlock;
 #pragma unroll
     for (int n = 0; n < NLB; ++n) {
       const int row = min(row0 + n * RPI + lb_row, last_row);
-      rbk[n] = *reinterpret_cast<const u32x4*>(kb_base + (int64_t)row * p.kb.stride_r + 8 * lb_c);
-      rbv[n] = *reinterpret_cast<const u32x4*>(vb_base + (int64_t)row * p.vb.stride_r + 8 * lb_c);
+      rbk[set][n] = *reinterpret_cast<const u32x4*>(kb_base + (int64_t)row * p.kb.stride_r + 8 * lb_c);
+      rbv[set][n] = *reinterpret_cast<const u32x4*>(vb_base + (int64_t)row * p.vb.stride_r + 8 * lb_c);
     }
 #pragma unroll
     for (int n = 0; n < 2; ++n) {
       const int row = min(row0 + 16 * n + la_row, last_row);
-      rak[n] = *reinterpret_cast<const u32x4*>(ka_base + (int64_t)row * p.ka.stride_r + 8 * la_c);
-      rav[n] = *reinterpret_cast<const u32x4*>(va_base + (int64_t)row * p.va.stride_r + 8 * la_c);
+      rak[set][n] = *reinterpret_cast<const u32x4*>(ka_base + (int64_t)row * p.ka.stride_r + 8 * la_c);
+      rav[set][n] = *reinterpret_cast<const u32x4*>(va_base + (int64_t)row * p.va.stride_r + 8 * la_c);
     }
   };
-  auto stage = [&]() {
+  auto stage = [&](auto set_c) {
+    constexpr int set = decltype(set_c)::value;
 #pragma unroll
     for (int n = 0; n < NLB; ++n) {
       const int row = n * RPI + lb_row;
       const int pos = lb_c ^ (row & (CPR - 1));
-      *reinterpret_cast<u32x4*>(lds_bk + row * D + 8 * pos) = rbk[n];
-      *reinterpret_cast<u32x4*>(lds_bv + row * D + 8 * pos) = rbv[n];
+      *reinterpret_cast<u32x4*>(lds_bk + row * D + 8 * pos) = rbk[set][n];
+      *reinterpret_cast<u32x4*>(lds_bv + row * D + 8 * pos) = rbv[set][n];
     }
 #pragma unroll
     for (int n = 0; n < 2; ++n) {
       const int row = 16 * n + la_row;
-      *reinterpret_cast<u32x4*>(lds_ak + row * 32 + 8 * (l & 3)) = rak[n];
-      *reinterpret_cast<u32x4*>(lds_av + row * 32 + 8 * (l & 3)) = rav[n];
+      *reinterpret_cast<u32x4*>(lds_ak + row * 32 + 8 * (l & 3)) = rak[set][n];
+      *reinterpret_cast<u32x4*>(lds_av + row * 32 + 8 * (l & 3)) = rav[set][n];
     }
   };
 
@@ -156,11 +146,13 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
 
   const int lp = l & 15, dhalf = (l >> 4) & 1;
 
-  if (blk_begin < blk_end) issue(blk_begin);
-  for (int blk = blk_begin; blk < blk_end; ++blk) {
-    stage();  // waits for this block's loads, then the registers are free again
-    if (blk + 1 < blk_end) issue(blk + 1);
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+  if (blk_begin < blk_end) issue(Set0{}, blk_begin);
+  if (blk_begin + blk_step < blk_end) issue(Set1{}, blk_begin + blk_step);
+  build_q();
 
+  auto compute = [&](int blk) {
     // ---- S'^T[row, h] = sum_d B_k[row, d] Qm[h, d]
     f32x16 sp;
 #pragma unroll
@@ -252,6 +244,17 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
         const bf16x8 vf = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
         o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kk], o[db], 0, 0, 0);
       }
+    }
+  };
+
+  for (int blk = blk_begin; blk < blk_end; blk += 2 * blk_step) {
+    stage(Set0{});  // waits for this block's loads only; its registers are then free again
+    if (blk + 2 * blk_step < blk_end) issue(Set0{}, blk + 2 * blk_step);
+    compute(blk);
+    if (blk + blk_step < blk_end) {
+      stage(Set1{});
+      if (blk + 3 * blk_step < blk_end) issue(Set1{}, blk + 3 * blk_step);
+      compute(blk + blk_step);
     }
   }
 

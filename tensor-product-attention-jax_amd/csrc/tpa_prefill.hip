@@ -72,36 +72,20 @@ __global__ __launch_bounds__(NW * 64) void prefill_kernel(PrefillParams p) {
   const int qrow_ld = min(qrow, p.lq - 1);
   const float c = p.sm_scale * kLog2e;
 
-  // ---- Q fragments (B operand of S^T = K Q^T): lane (i, g) holds Q[qrow][16ks + 8g + 0..7]
+  // ---- Q fragments (B operand of S^T = K Q^T): lane (i, g) holds Q[qrow][16ks + 8g + 0..7].
+  // Built after the first K/V factor loads are in flight; per rank all loads are issued together.
   bf16x8 qf[NKS];
-  if constexpr (LOADER == LOAD_DENSE) {
-    const uint16_t* qp = static_cast<const uint16_t*>(p.qb.ptr) + b * p.qb.stride_b + (int64_t)qrow_ld * p.qb.stride_l + (int64_t)h * D;
+  auto build_q = [&]() {
+    if constexpr (LOADER == LOAD_DENSE) {
+      const uint16_t* qp = static_cast<const uint16_t*>(p.qb.ptr) + b * p.qb.stride_b + (int64_t)qrow_ld * p.qb.stride_l + (int64_t)h * D;
 #pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks + 8 * g);
-  } else {
-    const uint16_t* ap = static_cast<const uint16_t*>(p.qa.ptr) + b * p.qa.stride_b + (int64_t)qrow_ld * p.qa.stride_l + h;
-    const uint16_t* bp = static_cast<const uint16_t*>(p.qb.ptr) + b * p.qb.stride_b + (int64_t)qrow_ld * p.qb.stride_l + 8 * g;
-    const float inv_rq = 1.f / (float)p.rq;
-#pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) {
-      float acc[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) acc[j] = 0.f;
-      for (int r = 0; r < p.rq; ++r) {
-        const float a = bf16bits_to_f32(ap[r * p.qa.stride_r]);
-        const u32x4 bv = *reinterpret_cast<const u32x4*>(bp + r * p.qb.stride_r + 16 * ks);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          acc[2 * j] += a * bf16lo_to_f32(bv[j]);
-          acc[2 * j + 1] += a * bf16hi_to_f32(bv[j]);
-        }
-      }
-      u32x4 packed;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) packed[j] = pack_bf16(acc[2 * j] * inv_rq, acc[2 * j + 1] * inv_rq);
-      qf[ks] = __builtin_bit_cast(bf16x8, packed);
+      for (int ks = 0; ks < NKS; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks + 8 * g);
+    } else {
+      const uint16_t* ap = static_cast<const uint16_t*>(p.qa.ptr) + b * p.qa.stride_b + (int64_t)qrow_ld * p.qa.stride_l + h;
+      const uint16_t* bp = static_cast<const uint16_t*>(p.qb.ptr) + b * p.qb.stride_b + (int64_t)qrow_ld * p.qb.stride_l + 8 * g;
+      build_q_fragments<NKS, 3>(ap, p.qa.stride_r, bp, p.qb.stride_r, p.rq, 1.f / (float)p.rq, qf);
     }
-  }
+  };
 
   // ---- tile range
   int ntiles = (p.lk + kTK - 1) / kTK;
@@ -214,6 +198,7 @@ __global__ __launch_bounds__(NW * 64) void prefill_kernel(PrefillParams p) {
   float lsum = 0.f;     // this lane's share of sum exp2(c*(s - m))
 
   issue(0);
+  build_q();
   commit(0, 0);
   __syncthreads();
 
