@@ -1,23 +1,38 @@
 // Flash-style prefill for gfx950: bf16 MFMA contractions, fp32 online softmax.
 //
-// One workgroup = one (batch, head, block of kBQ query rows); each of its waves owns 32 query
-// rows.  Per tile of 64 keys the workgroup rebuilds the head's K and V tile from the rank
-// factors (K = (1/R) sum_r a_r (x) b_r, tpa/tpa.py:364,417) straight out of coalesced 16-byte
-// factor loads and stores it once, as bf16, in LDS.  The waves then compute
-//     S^T = K Q^T        (v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = Q kept in registers)
+// One workgroup = one (batch, head, block of 256 query rows) and has eight waves, two per SIMD,
+// each owning 32 query rows.  Per tile of 64 keys the workgroup rebuilds the head's K and V
+// tile from the rank factors (K = (1/R) sum_r a_r (x) b_r, tpa/tpa.py:364,417) straight out of
+// coalesced 16-byte factor loads and stores it once, as bf16, in LDS.  Each wave then computes
+//     S^T = K Q^T        (v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = Q kept in registers,
+//                         Q pre-scaled by sm_scale*log2(e) and the accumulator started at minus
+//                         the running reference, so the result is the exponent itself)
 //     online softmax     (each lane holds 32 logits of ONE query row, so the row max and sum
 //                         are in-lane apart from one exchange with lane ^ 32)
 //     O^T += V^T P^T     (A = V^T read with ds_read_b64_tr_b16 from row-major V, B = P^T, which
 //                         is the S^T accumulator converted in place: no LDS round trip for P)
-// and keep the deferred normalisation of flash attention (m, l per row), which is the
-// normalise-every-step recurrence of tpa/tpa.py:389-424 in another order of operations.
+// with the deferred normalisation of flash attention (a reference m and a sum l per row), which
+// is the normalise-every-step recurrence of tpa/tpa.py:389-424 in another order of operations.
+// Waves 0-3 and waves 4-7 (w and w + 4 share a SIMD) run half a tile apart: between two
+// workgroup barriers one group issues its MFMA work while the other does its vector-ALU work
+// (softmax, rebuilding the next K/V tile), then they swap, so the matrix pipe and the vector
+// ALU of a SIMD are fed by different waves at the same time.
 // The dense flash baseline (tpa/mha.py:23-37) is the same kernel with a plain K/V loader.
+#include <type_traits>
+#include <utility>
+
 #include "tpa_common.h"
 
 namespace tpa {
 namespace {
 
-constexpr int kTK = 64;  // keys per tile
+constexpr int kTK = 64;   // keys per tile
+constexpr int kNW = 8;    // waves per workgroup
+constexpr int kBQ = 256;  // query rows per workgroup (32 per wave)
+#ifdef EXP_TIME
+__device__ unsigned long long g_dbg[8192 * 8];
+#define TS() __builtin_amdgcn_s_memtime()
+#endif
 
 enum { LOAD_TPA_R2 = 0, LOAD_TPA_ANY = 1, LOAD_DENSE = 2 };
 
@@ -36,14 +51,26 @@ template <int D>
 struct Lds {
   static constexpr int KS = D + 8;   // K row stride (elements): 16-byte reads of 16 rows hit distinct banks
   static constexpr int VS = D + 32;  // V row stride: 4 consecutive rows of a transposed read hit distinct banks
-  static constexpr int kStage = kTK * KS + kTK * VS;  // elements per stage
-  static constexpr size_t kBytes = 2 * kStage * sizeof(uint16_t);
+  static constexpr int kK = kTK * KS;  // elements of one K buffer
+  static constexpr int kV = kTK * VS;  // elements of one V buffer
+  static constexpr int kA = 2 * kTK * 2;  // one slot of head factors: [K|V][token][rank 0|1]
+  static constexpr size_t kBytes = (2 * (kK + kV) + 2 * kA) * sizeof(uint16_t);
 };
 
-template <int D, int NW, int LOADER>
-__global__ __launch_bounds__(NW * 64) void prefill_kernel(PrefillParams p) {
-  constexpr int NT = NW * 64;
-  constexpr int BQ = NW * 32;
+// a0*b0 + a1*b1 on packed bf16 pairs, fp32 result.  Through the builtin on purpose: the dot
+// instructions need software wait states before a dependent VALU instruction, which the compiler
+// only inserts for instructions it selected itself (not for inline assembly).
+__device__ __forceinline__ float dot2_bf16(uint32_t pair, uint32_t aa) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pair), __builtin_bit_cast(bf16x2, aa), 0.f, false);
+}
+
+// Workgroup barrier that waits for this wave's LDS traffic only.  __syncthreads() would also
+// wait for the global loads of the next tile's factors, which are meant to stay in flight.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <int D, int LOADER>
+__global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
+  constexpr int NT = kNW * 64;
   constexpr int KS = Lds<D>::KS, VS = Lds<D>::VS;
   constexpr int CPR = D / 8;             // 16-byte chunks per row
   constexpr int TPP = NT / CPR;          // tokens per loader pass
@@ -51,8 +78,19 @@ __global__ __launch_bounds__(NW * 64) void prefill_kernel(PrefillParams p) {
   static_assert(kTK % TPP == 0 && NPASS >= 1, "loader shape");
   constexpr int NKS = D / 16;            // k-steps of the QK^T contraction
   constexpr int NDB = D / 32;            // 32-row blocks of O^T
+  constexpr float kSlack = 8.f;          // the reference only moves when a tile max exceeds it by 2^8
+
+  // scalars out of the argument block (never take the address of the block itself)
+  struct Fac { const uint16_t* ptr; int64_t stride_b; int stride_l, stride_r; };
+  auto fac = [](const TpaFactor& f) { return Fac{static_cast<const uint16_t*>(f.ptr), f.stride_b, (int)f.stride_l, (int)f.stride_r}; };
+  struct { Fac qa, qb, ka, kb, va, vb; uint16_t* o; float* lse; int B, lq, lk, H, rq, rk; float sm_scale; int causal, nqb, npairs; } const p = {
+      fac(pp.qa), fac(pp.qb), fac(pp.ka), fac(pp.kb), fac(pp.va), fac(pp.vb), pp.o, pp.lse, pp.B, pp.lq, pp.lk, pp.H, pp.rq, pp.rk,
+      pp.sm_scale, pp.causal, pp.nqb, pp.npairs};
 
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  uint16_t* const lds_k = smem;                                  // [2][kTK][KS]
+  uint16_t* const lds_v = smem + 2 * Lds<D>::kK;                 // [2][kTK][VS]
+  uint16_t* const lds_a = smem + 2 * (Lds<D>::kK + Lds<D>::kV);  // [2][K|V][kTK][2]
 
   // ---- which (query block, batch, head): heads of one (block, batch) pair sit on one XCD
   // (workgroup ids are dealt round-robin to the 8 XCDs) so they share the B-factor tiles in
@@ -65,87 +103,138 @@ __global__ __launch_bounds__(NW * 64) void prefill_kernel(PrefillParams p) {
   const int qblk = p.nqb - 1 - pair / p.B;
   const int b = pair % p.B;
 
+#ifdef EXP_TIME
+  const unsigned long long t_start = TS();
+#endif
   const int tid = threadIdx.x;
   const int w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
-  const int q0 = qblk * BQ;
-  const int qrow = q0 + 32 * w + i;
+  const int q0 = qblk * kBQ;
+  const int wrow0 = q0 + 32 * w;  // first query row of this wave
+  const int qrow = wrow0 + i;
   const int qrow_ld = min(qrow, p.lq - 1);
   const float c = p.sm_scale * kLog2e;
 
-  // ---- Q fragments (B operand of S^T = K Q^T): lane (i, g) holds Q[qrow][16ks + 8g + 0..7].
-  // Built after the first K/V factor loads are in flight; per rank all loads are issued together.
+  // ---- Q fragments (B operand of S^T = K Q^T), scaled by c: lane (i, g) holds
+  // c * Q[qrow][16ks + 8g + 0..7]
   bf16x8 qf[NKS];
-  auto build_q = [&]() {
+  auto build_q = [&]() __attribute__((always_inline)) {
     if constexpr (LOADER == LOAD_DENSE) {
-      const uint16_t* qp = static_cast<const uint16_t*>(p.qb.ptr) + b * p.qb.stride_b + (int64_t)qrow_ld * p.qb.stride_l + (int64_t)h * D;
+      const uint16_t* qp = p.qb.ptr + b * p.qb.stride_b + (int64_t)qrow_ld * p.qb.stride_l + (int64_t)h * D;
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks + 8 * g);
+      for (int ks = 0; ks < NKS; ++ks) {
+        const u32x4 raw = *reinterpret_cast<const u32x4*>(qp + 16 * ks + 8 * g);
+        u32x4 sc;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sc[j] = pack_bf16(bf16lo_to_f32(raw[j]) * c, bf16hi_to_f32(raw[j]) * c);
+        qf[ks] = __builtin_bit_cast(bf16x8, sc);
+      }
     } else {
-      const uint16_t* ap = static_cast<const uint16_t*>(p.qa.ptr) + b * p.qa.stride_b + (int64_t)qrow_ld * p.qa.stride_l + h;
-      const uint16_t* bp = static_cast<const uint16_t*>(p.qb.ptr) + b * p.qb.stride_b + (int64_t)qrow_ld * p.qb.stride_l + 8 * g;
-      build_q_fragments<NKS, 3>(ap, p.qa.stride_r, bp, p.qb.stride_r, p.rq, 1.f / (float)p.rq, qf);
+      const uint16_t* ap = p.qa.ptr + b * p.qa.stride_b + (int64_t)qrow_ld * p.qa.stride_l + h;
+      const uint16_t* bp = p.qb.ptr + b * p.qb.stride_b + (int64_t)qrow_ld * p.qb.stride_l + 8 * g;
+      build_q_fragments<NKS, 3>(ap, p.qa.stride_r, bp, p.qb.stride_r, p.rq, c / (float)p.rq, qf);
     }
   };
 
   // ---- tile range
   int ntiles = (p.lk + kTK - 1) / kTK;
-  if (p.causal) ntiles = min(ntiles, (min(q0 + BQ, p.lq) + kTK - 1) / kTK);
-  // last tile this wave needs under the causal mask (rows of the wave: q0+32w .. +31)
-  const int wave_last_tile = p.causal ? min(ntiles - 1, (q0 + 32 * w + 31) / kTK) : ntiles - 1;
+  if (p.causal) ntiles = min(ntiles, (min(q0 + kBQ, p.lq) + kTK - 1) / kTK);
+  const int last = ntiles - 1;
+  // last tile this wave needs under the causal mask (its rows: wrow0 .. wrow0 + 31)
+  const int wave_last_tile = p.causal ? min(last, (wrow0 + 31) / kTK) : last;
 
-  // ---- loader state: this thread rebuilds chunk lc (8 elements) of token lt (+ TPP per pass)
+  // ---- loader: this thread rebuilds chunk lc (8 elements) of token lt (+ TPP per pass).
+  // Addresses are a uniform (scalar) tile base plus a per-thread 32-bit element offset.
   const int lt = tid / CPR, lc = tid % CPR;
   u32x4 kreg[NPASS][2], vreg[NPASS][2];  // LOAD_TPA_R2: two ranks; LOAD_DENSE: [0] only
-  uint32_t kaa[NPASS], vaa[NPASS];       // LOAD_TPA_R2: packed (a0/2, a1/2) bf16 pair
 
-  const uint16_t* kbp = static_cast<const uint16_t*>(p.kb.ptr) + b * p.kb.stride_b + 8 * lc;
-  const uint16_t* vbp = static_cast<const uint16_t*>(p.vb.ptr) + b * p.vb.stride_b + 8 * lc;
-  const uint16_t* kap = static_cast<const uint16_t*>(p.ka.ptr) + b * p.ka.stride_b + h;
-  const uint16_t* vap = static_cast<const uint16_t*>(p.va.ptr) + b * p.va.stride_b + h;
-  if constexpr (LOADER == LOAD_DENSE) {
-    kbp += (int64_t)h * D;
-    vbp += (int64_t)h * D;
-  }
+  const uint16_t* const kb_b = p.kb.ptr + b * p.kb.stride_b + (LOADER == LOAD_DENSE ? (int64_t)h * D : 0);
+  const uint16_t* const vb_b = p.vb.ptr + b * p.vb.stride_b + (LOADER == LOAD_DENSE ? (int64_t)h * D : 0);
+  const uint16_t* const ka_b = p.ka.ptr + b * p.ka.stride_b + h;
+  const uint16_t* const va_b = p.va.ptr + b * p.va.stride_b + h;
 
-  auto issue = [&](int tile) {
+  // B-factor loads of one matrix (K or V) for one tile into registers
+  auto issue = [&](auto is_v_c, int tile) __attribute__((always_inline)) {
+    constexpr bool is_v = decltype(is_v_c)::value;
     if constexpr (LOADER == LOAD_TPA_ANY) return;
+    const uint16_t* b_base = is_v ? vb_b : kb_b;
+    const int sl = is_v ? p.vb.stride_l : p.kb.stride_l, sr = is_v ? p.vb.stride_r : p.kb.stride_r;
 #pragma unroll
     for (int ps = 0; ps < NPASS; ++ps) {
-      const int tok = min(tile * kTK + ps * TPP + lt, p.lk - 1);
-      if constexpr (LOADER == LOAD_TPA_R2) {
-        kreg[ps][0] = *reinterpret_cast<const u32x4*>(kbp + (int64_t)tok * p.kb.stride_l);
-        kreg[ps][1] = *reinterpret_cast<const u32x4*>(kbp + (int64_t)tok * p.kb.stride_l + p.kb.stride_r);
-        vreg[ps][0] = *reinterpret_cast<const u32x4*>(vbp + (int64_t)tok * p.vb.stride_l);
-        vreg[ps][1] = *reinterpret_cast<const u32x4*>(vbp + (int64_t)tok * p.vb.stride_l + p.vb.stride_r);
-        const uint32_t ka0 = kap[(int64_t)tok * p.ka.stride_l], ka1 = kap[(int64_t)tok * p.ka.stride_l + p.ka.stride_r];
-        const uint32_t va0 = vap[(int64_t)tok * p.va.stride_l], va1 = vap[(int64_t)tok * p.va.stride_l + p.va.stride_r];
-        kaa[ps] = ka0 | (ka1 << 16);
-        vaa[ps] = va0 | (va1 << 16);
+      const uint16_t* bt = b_base + (int64_t)(tile * kTK + ps * TPP) * sl;                   // uniform
+      const int tl = min(tile * kTK + ps * TPP + lt, p.lk - 1) - (tile * kTK + ps * TPP);   // clamp a ragged tail
+      const int boff = tl * sl + 8 * lc;
+      if constexpr (is_v) {
+        vreg[ps][0] = *reinterpret_cast<const u32x4*>(bt + boff);
+        if constexpr (LOADER == LOAD_TPA_R2) vreg[ps][1] = *reinterpret_cast<const u32x4*>(bt + sr + boff);
       } else {
-        kreg[ps][0] = *reinterpret_cast<const u32x4*>(kbp + (int64_t)tok * p.kb.stride_l);
-        vreg[ps][0] = *reinterpret_cast<const u32x4*>(vbp + (int64_t)tok * p.vb.stride_l);
+        kreg[ps][0] = *reinterpret_cast<const u32x4*>(bt + boff);
+        if constexpr (LOADER == LOAD_TPA_R2) kreg[ps][1] = *reinterpret_cast<const u32x4*>(bt + sr + boff);
       }
     }
   };
+  using IsK = std::integral_constant<bool, false>;
+  using IsV = std::integral_constant<bool, true>;
 
-  // a0*b0[d] + a1*b1[d] for the two elements of a dword pair, as two bf16 dot products
-  auto rebuild_r2 = [&](const u32x4& b0, const u32x4& b1, uint32_t aa_bits) -> u32x4 {
+  // Head factors (LOAD_TPA_R2): threads 0..255 (waves 0-3) fetch one value a[matrix][token][rank]
+  // each, matrix = tid / 128 (0: K of tile kt, 1: V of tile vt), token = (tid / 2) % 64, rank = tid % 2,
+  // and park it in a register until it is stored into an LDS slot one iteration later.
+  uint32_t a_pending = 0;
+  auto issue_a = [&](int kt, int vt) __attribute__((always_inline)) {
+    if constexpr (LOADER != LOAD_TPA_R2) return;
+    if (tid >= 4 * kTK) return;
+    const int mat = tid / (2 * kTK), tok_in = (tid >> 1) % kTK, rank = tid & 1;
+    const int tok = min((mat ? vt : kt) * kTK + tok_in, p.lk - 1);
+    const uint16_t* ap = mat ? va_b + (int64_t)tok * p.va.stride_l + rank * p.va.stride_r
+                             : ka_b + (int64_t)tok * p.ka.stride_l + rank * p.ka.stride_r;
+    a_pending = *ap;
+  };
+  auto store_a = [&](int slot_idx) __attribute__((always_inline)) {
+    if constexpr (LOADER != LOAD_TPA_R2) return;
+    if (tid < 4 * kTK) lds_a[slot_idx * Lds<D>::kA + tid] = (uint16_t)a_pending;
+  };
+
+  // (a0/2)*b0[d] + (a1/2)*b1[d] for 8 consecutive d; aa = packed (a0, a1).
+  // One assembly block of 8 v_perm_b32 (pair b0[d] with b1[d]), 8 v_dot2_f32_bf16 (the VOP3P form
+  // with a zero addend, so no accumulator has to be cleared first) and 4 v_cvt_pk_bf16_f32.  A dot
+  // result may only be read by another vector-ALU instruction three wait states later and the
+  // hardware does not interlock; the order below keeps at least three instructions (or an s_nop)
+  // between every dot and its conversion.
+  auto rebuild_r2 = [&](const u32x4& b0, const u32x4& b1, uint32_t aa_bits) __attribute__((always_inline)) -> u32x4 {
     // halve the a pair (exact in bf16): 1/R with R = 2
-    const float a0 = bf16lo_to_f32(aa_bits) * 0.5f, a1 = bf16hi_to_f32(aa_bits) * 0.5f;
-    const bf16x2 aa = __builtin_bit_cast(bf16x2, pack_bf16(a0, a1));
-    u32x4 out;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint32_t lo = __builtin_amdgcn_perm(b1[j], b0[j], 0x05040100u);  // (b0[d],   b1[d])
-      const uint32_t hi = __builtin_amdgcn_perm(b1[j], b0[j], 0x07060302u);  // (b0[d+1], b1[d+1])
-      const float x0 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, lo), aa, 0.f, false);
-      const float x1 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, hi), aa, 0.f, false);
-      out[j] = pack_bf16(x0, x1);
-    }
+    const uint32_t aa = pack_bf16(bf16lo_to_f32(aa_bits) * 0.5f, bf16hi_to_f32(aa_bits) * 0.5f);
+    const uint32_t sel_lo = 0x05040100u, sel_hi = 0x07060302u;
+    uint32_t t0, t1, t2, t3, t4, t5, t6, t7;
+    asm volatile(
+        "v_perm_b32 %0, %9, %8, %17\n\t"   // (b0[0], b1[0])
+        "v_perm_b32 %1, %9, %8, %18\n\t"   // (b0[1], b1[1])
+        "v_perm_b32 %2, %11, %10, %17\n\t"
+        "v_perm_b32 %3, %11, %10, %18\n\t"
+        "v_perm_b32 %4, %13, %12, %17\n\t"
+        "v_perm_b32 %5, %13, %12, %18\n\t"
+        "v_perm_b32 %6, %15, %14, %17\n\t"
+        "v_perm_b32 %7, %15, %14, %18\n\t"
+        "v_dot2_f32_bf16 %0, %0, %16, 0\n\t"
+        "v_dot2_f32_bf16 %1, %1, %16, 0\n\t"
+        "v_dot2_f32_bf16 %2, %2, %16, 0\n\t"
+        "v_dot2_f32_bf16 %3, %3, %16, 0\n\t"
+        "v_dot2_f32_bf16 %4, %4, %16, 0\n\t"
+        "v_dot2_f32_bf16 %5, %5, %16, 0\n\t"
+        "v_dot2_f32_bf16 %6, %6, %16, 0\n\t"
+        "v_dot2_f32_bf16 %7, %7, %16, 0\n\t"
+        "s_nop 0\n\t"
+        "v_cvt_pk_bf16_f32 %0, %0, %1\n\t"
+        "v_cvt_pk_bf16_f32 %2, %2, %3\n\t"
+        "v_cvt_pk_bf16_f32 %4, %4, %5\n\t"
+        "s_nop 0\n\t"
+        "v_cvt_pk_bf16_f32 %6, %6, %7"
+        : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3), "=&v"(t4), "=&v"(t5), "=&v"(t6), "=&v"(t7)
+        : "v"(b0[0]), "v"(b1[0]), "v"(b0[1]), "v"(b1[1]), "v"(b0[2]), "v"(b1[2]), "v"(b0[3]), "v"(b1[3]),
+          "v"(aa), "s"(sel_lo), "s"(sel_hi));
+    u32x4 out = {t0, t2, t4, t6};
     return out;
   };
 
-  auto rebuild_any = [&](const uint16_t* bptr, const uint16_t* aptr, int64_t b_stride_r, int64_t a_stride_r) -> u32x4 {
+  auto rebuild_any = [&](const uint16_t* bptr, const uint16_t* aptr, int b_stride_r, int a_stride_r) __attribute__((always_inline)) -> u32x4 {
     float acc[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = 0.f;
@@ -165,134 +254,235 @@ __global__ __launch_bounds__(NW * 64) void prefill_kernel(PrefillParams p) {
     return out;
   };
 
-  auto commit = [&](int tile, int stage) {
-    uint16_t* ks = smem + stage * Lds<D>::kStage;
-    uint16_t* vs = ks + kTK * KS;
+  // Rebuild one matrix of tile `tile` from the registers `issue` filled and store it in LDS.
+  // a_slot = head factors in LDS ([K|V][token][rank]) or nullptr to fetch them from global memory.
+  auto commit = [&](auto is_v_c, int tile, const uint16_t* a_slot) __attribute__((always_inline)) {
+    constexpr bool is_v = decltype(is_v_c)::value;
+    const uint16_t* bb = is_v ? vb_b : kb_b;
+    const uint16_t* ab = is_v ? va_b : ka_b;
+    const int b_sl = is_v ? p.vb.stride_l : p.kb.stride_l, b_sr = is_v ? p.vb.stride_r : p.kb.stride_r;
+    const int a_sl = is_v ? p.va.stride_l : p.ka.stride_l, a_sr = is_v ? p.va.stride_r : p.ka.stride_r;
+    uint16_t* dst = is_v ? lds_v + (tile & 1) * Lds<D>::kV : lds_k + (tile & 1) * Lds<D>::kK;
+    constexpr int row_stride = is_v ? VS : KS;
 #pragma unroll
     for (int ps = 0; ps < NPASS; ++ps) {
       const int t = ps * TPP + lt;
-      u32x4 kv, vv;
+      u32x4 val;
       if constexpr (LOADER == LOAD_TPA_R2) {
-        kv = rebuild_r2(kreg[ps][0], kreg[ps][1], kaa[ps]);
-        vv = rebuild_r2(vreg[ps][0], vreg[ps][1], vaa[ps]);
+        uint32_t aa;
+        if (a_slot) {
+          aa = *reinterpret_cast<const uint32_t*>(a_slot + (is_v ? 2 * kTK : 0) + 2 * t);
+        } else {
+          const int tok = min(tile * kTK + t, p.lk - 1);
+          const uint32_t a0 = ab[(int64_t)tok * a_sl], a1 = ab[(int64_t)tok * a_sl + a_sr];
+          aa = a0 | (a1 << 16);
+        }
+        if constexpr (is_v) val = rebuild_r2(vreg[ps][0], vreg[ps][1], aa);
+        else val = rebuild_r2(kreg[ps][0], kreg[ps][1], aa);
       } else if constexpr (LOADER == LOAD_TPA_ANY) {
         const int tok = min(tile * kTK + t, p.lk - 1);
-        kv = rebuild_any(kbp + (int64_t)tok * p.kb.stride_l, kap + (int64_t)tok * p.ka.stride_l, p.kb.stride_r, p.ka.stride_r);
-        vv = rebuild_any(vbp + (int64_t)tok * p.vb.stride_l, vap + (int64_t)tok * p.va.stride_l, p.vb.stride_r, p.va.stride_r);
+        val = rebuild_any(bb + (int64_t)tok * b_sl + 8 * lc, ab + (int64_t)tok * a_sl, b_sr, a_sr);
       } else {
-        kv = kreg[ps][0];
-        vv = vreg[ps][0];
+        if constexpr (is_v) val = vreg[ps][0]; else val = kreg[ps][0];
       }
-      *reinterpret_cast<u32x4*>(ks + t * KS + 8 * lc) = kv;
-      *reinterpret_cast<u32x4*>(vs + t * VS + 8 * lc) = vv;
+      *reinterpret_cast<u32x4*>(dst + t * row_stride + 8 * lc) = val;
     }
   };
 
-  // ---- accumulators
+  // ---- per-wave state
   f32x16 o[NDB];
 #pragma unroll
   for (int db = 0; db < NDB; ++db)
 #pragma unroll
     for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
-  float m = -INFINITY;  // running max of the raw (unscaled) logits of row qrow
-  float lsum = 0.f;     // this lane's share of sum exp2(c*(s - m))
+  f32x16 s[2];          // exponents x*c - mref of the tile in flight: two 32-key blocks
+  bf16x8 pf[4];         // P^T of the last softmaxed tile, as B operands of the four 16-key steps
+  float mref = 0.f;     // reference (log2 domain, includes c) of row qrow
+  float lsum = 0.f;     // this lane's share of sum exp2(x*c - mref)
+  const int lp = l & 15, dhalf = (l >> 4) & 1;
 
-  issue(0);
-  build_q();
-  commit(0, 0);
-  __syncthreads();
-
-  for (int tile = 0; tile < ntiles; ++tile) {
-    const int stage = tile & 1;
-    if (tile + 1 < ntiles) issue(tile + 1);
-
-    if (tile <= wave_last_tile) {
-      const uint16_t* ks = smem + stage * Lds<D>::kStage;
-      const uint16_t* vs = ks + kTK * KS;
-      const int k0 = tile * kTK;
-
-      // ---- S^T = K Q^T : two 32-key blocks
-      f32x16 s[2];
+  // S^T = K Q^T - mref for tile `tile`
+  auto do_qk = [&](int tile) __attribute__((always_inline)) {
+    const uint16_t* ks = lds_k + (tile & 1) * Lds<D>::kK;
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) {
+    for (int mb = 0; mb < 2; ++mb) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) s[mb][v] = 0.f;
+      for (int v = 0; v < 16; ++v) s[mb][v] = -mref;
 #pragma unroll
-        for (int kk = 0; kk < NKS; ++kk) {
-          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(ks + (32 * mb + i) * KS + 16 * kk + 8 * g);
-          s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s[mb], 0, 0, 0);
-        }
+      for (int kk = 0; kk < NKS; ++kk) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(ks + (32 * mb + i) * KS + 16 * kk + 8 * g);
+        s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s[mb], 0, 0, 0);
       }
+    }
+  };
 
-      // ---- masks: keys beyond lk, and keys after the query under the causal mask
-      const bool need_mask = (k0 + kTK > p.lk) || (p.causal && (k0 + kTK - 1 > q0 + 32 * w));
-      if (need_mask) {
-        const int limit = p.causal ? min(qrow, p.lk - 1) : p.lk - 1;  // largest visible key index
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const int t = k0 + 32 * mb + 8 * (v >> 2) + 4 * g + (v & 3);
-            if (t > limit) s[mb][v] = -INFINITY;
-          }
-      }
-
-      // ---- online softmax for row qrow (32 of its 64 logits live in this lane)
-      float tmax = s[0][0];
+  // masks + online softmax of tile `tile` (32 of the 64 logits of row qrow live in this lane)
+  auto do_softmax = [&](int tile) __attribute__((always_inline)) {
+    const int k0 = tile * kTK;
+    // keys beyond lk, and keys after the query under the causal mask
+    const bool need_mask = (k0 + kTK > p.lk) || (p.causal && (k0 + kTK - 1 > wrow0));
+    if (need_mask) {
+      const int limit = p.causal ? min(qrow, p.lk - 1) : p.lk - 1;  // largest visible key index
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) tmax = fmaxf(tmax, s[mb][v]);
-      tmax = halves_max(tmax);
-      const float m_new = fmaxf(m, tmax);
-      const float alpha = __builtin_amdgcn_exp2f((m - m_new) * c);
-      const float mc = m_new * c;
-      m = m_new;
-      float psum = 0.f;
-      bf16x8 pf[4];
-#pragma unroll
-      for (int mb = 0; mb < 2; ++mb) {
-        float pv[16];
-#pragma unroll
         for (int v = 0; v < 16; ++v) {
-          pv[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mb][v], c, -mc));
-          psum += pv[v];
+          const int t = k0 + 32 * mb + 8 * (v >> 2) + 4 * g + (v & 3);
+          if (t > limit) s[mb][v] = -INFINITY;
         }
+    }
+    float tmax = s[0][0];
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          u32x4 pk;
+    for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) pk[j] = pack_bf16(pv[8 * half + 2 * j], pv[8 * half + 2 * j + 1]);
-          pf[2 * mb + half] = __builtin_bit_cast(bf16x8, pk);
-        }
-      }
-      lsum = lsum * alpha + psum;
+      for (int v = 0; v < 16; ++v) tmax = fmaxf(tmax, s[mb][v]);
+    tmax = halves_max(tmax);
+    if (tile == 0) {
+      // first tile: take its max as the reference (the accumulators started at 0)
+      mref = tmax;
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[mb][v] -= tmax;
+    } else if (__any(tmax > kSlack)) {
+      // rare: some row's max left the slack; move the references up and rescale
+      const float delta = fmaxf(tmax, 0.f);
+      const float alpha = __builtin_amdgcn_exp2f(-delta);
+      mref += delta;
+      lsum *= alpha;
 #pragma unroll
       for (int db = 0; db < NDB; ++db)
 #pragma unroll
         for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
-
-      // ---- O^T += V^T P^T : k-step kk covers keys 16kk .. 16kk+15 of the tile, in the slot
-      // order the S^T accumulator already has: slot (g, j) = key 16kk + 8(j/4) + 4g + j%4
-      const int lp = l & 15, dhalf = (l >> 4) & 1;
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        const uint16_t* vrow = vs + (16 * kk + 4 * g + (lp >> 2)) * VS + 16 * dhalf + 4 * (lp & 3);
+      for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-        for (int db = 0; db < NDB; ++db) {
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (s16x4 __attribute__((address_space(3)))*)(vrow + 32 * db));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (s16x4 __attribute__((address_space(3)))*)(vrow + 8 * VS + 32 * db));
-          const bf16x8 vf = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kk], o[db], 0, 0, 0);
+        for (int v = 0; v < 16; ++v) s[mb][v] -= delta;
+    }
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        u32x4 pk;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float p0 = __builtin_amdgcn_exp2f(s[mb][8 * half + 2 * j]);
+          const float p1 = __builtin_amdgcn_exp2f(s[mb][8 * half + 2 * j + 1]);
+          lsum += p0 + p1;
+          pk[j] = pack_bf16(p0, p1);
         }
+        pf[2 * mb + half] = __builtin_bit_cast(bf16x8, pk);
       }
     }
+  };
 
-    if (tile + 1 < ntiles) commit(tile + 1, stage ^ 1);
-    __syncthreads();
+  // O^T += V^T P^T for tile `tile`: k-step kk covers keys 16kk .. 16kk+15 of the tile, in the slot
+  // order the S^T accumulator already has: slot (g, j) = key 16kk + 8(j/4) + 4g + j%4
+  auto do_pv = [&](int tile) __attribute__((always_inline)) {
+    const uint16_t* vs = lds_v + (tile & 1) * Lds<D>::kV;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const uint16_t* vrow = vs + (16 * kk + 4 * g + (lp >> 2)) * VS + 16 * dhalf + 4 * (lp & 3);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) {
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vrow + 32 * db));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vrow + 8 * VS + 32 * db));
+        const bf16x8 vf = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kk], o[db], 0, 0, 0);
+      }
+    }
+  };
+
+  // Invariant at entry of iteration j (tile indices clamped to the last tile): kreg = B factors of
+  // K tile j+1, vreg = B factors of V tile j, LDS head-factor slot j&1 = (K of tile j+1, V of tile
+  // j), a_pending (waves 0-3) = head factors of iteration j+1, K tile j in K buffer j&1, V tile
+  // j-1 in V buffer (j-1)&1.
+  // vector-ALU half of iteration j: softmax of tile `sm_tile` (if this wave needs it), rebuild K of
+  // tile j+1 and V of tile j into LDS, start the loads for the next iteration
+  auto valu_phase = [&](int j, int sm_tile) __attribute__((always_inline)) {
+    if (sm_tile >= 0 && sm_tile < ntiles && sm_tile <= wave_last_tile) do_softmax(sm_tile);
+    const uint16_t* a_slot = LOADER == LOAD_TPA_R2 ? lds_a + (j & 1) * Lds<D>::kA : nullptr;
+    if (j + 1 < ntiles) commit(IsK{}, j + 1, a_slot);
+    if (j < ntiles) commit(IsV{}, j, a_slot);
+    issue(IsK{}, min(j + 2, last));
+    issue(IsV{}, min(j + 1, last));
+    if (w < 4) {
+      // waves 0-3 run their vector half in the second half of the iteration, after waves 4-7
+      // have read slot j&1 ^ 1 for the last time: publish the next slot, fetch the one after
+      store_a((j + 1) & 1);
+      issue_a(min(j + 3, last), min(j + 2, last));
+    }
+  };
+  // matrix half of iteration j: PV of tile j-1, QK of tile j
+  auto mfma_phase = [&](int j) __attribute__((always_inline)) {
+    if (j >= 1 && j - 1 <= wave_last_tile) do_pv(j - 1);
+    if (j < ntiles && j <= wave_last_tile) do_qk(j);
+  };
+
+  // ---- prologue: K of tile 0 into LDS (head factors straight from global memory), the head
+  // factors of iteration 0 in their LDS slot, those of iteration 1 pending, and the B-factor
+  // loads of iteration 0 in flight
+  issue(IsK{}, 0);
+  issue_a(min(1, last), 0);
+  build_q();
+  commit(IsK{}, 0, nullptr);
+  issue(IsK{}, min(1, last));
+  issue(IsV{}, 0);
+  store_a(0);
+  issue_a(min(2, last), min(1, last));
+  lds_barrier();
+
+#ifdef EXP_TIME
+  unsigned long long tacc[6] = {0, 0, 0, 0, 0, 0};
+  const unsigned long long t_pro = TS();
+  if (w < 4) {
+    for (int j = 0; j <= ntiles; ++j) {
+      unsigned long long t0 = TS();
+      mfma_phase(j);
+      unsigned long long t1 = TS();
+      lds_barrier();
+      unsigned long long t2 = TS();
+      valu_phase(j, j);
+      unsigned long long t3 = TS();
+      lds_barrier();
+      unsigned long long t4 = TS();
+      tacc[0] += t1 - t0; tacc[1] += t2 - t1; tacc[2] += t3 - t2; tacc[3] += t4 - t3;
+    }
+  } else {
+    for (int j = 0; j <= ntiles; ++j) {
+      unsigned long long t0 = TS();
+      valu_phase(j, j - 1);
+      unsigned long long t1 = TS();
+      lds_barrier();
+      unsigned long long t2 = TS();
+      mfma_phase(j);
+      unsigned long long t3 = TS();
+      lds_barrier();
+      unsigned long long t4 = TS();
+      tacc[2] += t1 - t0; tacc[1] += t2 - t1; tacc[0] += t3 - t2; tacc[3] += t4 - t3;
+    }
   }
+  if (l == 0) {
+    unsigned long long* d = g_dbg + ((size_t)(blockIdx.x % 1024) * 8 + w) * 8;
+    d[0] = tacc[0]; d[1] = tacc[1]; d[2] = tacc[2]; d[3] = tacc[3]; d[4] = ntiles + 1; d[5] = t_pro - t_start; d[6] = TS() - t_pro; d[7] = 1;
+  }
+#else
+  if (w < 4) {
+    for (int j = 0; j <= ntiles; ++j) {
+      mfma_phase(j);
+      lds_barrier();
+      valu_phase(j, j);
+      lds_barrier();
+    }
+  } else {
+    for (int j = 0; j <= ntiles; ++j) {
+      valu_phase(j, j - 1);
+      lds_barrier();
+      mfma_phase(j);
+      lds_barrier();
+    }
+  }
+#endif
 
   // ---- epilogue: normalise, store O[b, qrow, h, :] and LSE[b, h, qrow]
   const float ltot = halves_sum(lsum);
@@ -308,13 +498,13 @@ __global__ __launch_bounds__(NW * 64) void prefill_kernel(PrefillParams p) {
         pk[1] = pack_bf16(o[db][4 * vq + 2] * inv, o[db][4 * vq + 3] * inv);
         *reinterpret_cast<u32x2*>(op + 32 * db + 8 * vq + 4 * g) = pk;
       }
-    if (p.lse && g == 0) p.lse[((int64_t)b * p.H + h) * p.lq + qrow] = (m * c + __builtin_amdgcn_logf(ltot)) * kLn2;
+    if (p.lse && g == 0) p.lse[((int64_t)b * p.H + h) * p.lq + qrow] = (mref + __builtin_amdgcn_logf(ltot)) * kLn2;
   }
 }
 
-template <int D, int NW, int LOADER>
+template <int D, int LOADER>
 int launch_prefill(const PrefillParams& p, hipStream_t stream) {
-  auto kern = prefill_kernel<D, NW, LOADER>;
+  auto kern = prefill_kernel<D, LOADER>;
   static bool configured = false;  // idempotent attribute; a race only repeats the same call
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)Lds<D>::kBytes) != hipSuccess)
@@ -323,7 +513,7 @@ int launch_prefill(const PrefillParams& p, hipStream_t stream) {
   }
   const int groups = (p.npairs + 7) / 8;
   dim3 grid(groups * 8 * p.H);
-  hipLaunchKernelGGL(kern, grid, dim3(NW * 64), Lds<D>::kBytes, stream, p);
+  hipLaunchKernelGGL(kern, grid, dim3(kNW * 64), Lds<D>::kBytes, stream, p);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
 }
 
@@ -332,10 +522,12 @@ bool factor_ok(const TpaFactor& f) {
   return aligned16(f.ptr) && f.stride_b % 8 == 0 && f.stride_l % 8 == 0 && f.stride_r % 8 == 0;
 }
 
-constexpr int kNW = 8;
-
 }  // namespace
 }  // namespace tpa
+
+#ifdef EXP_TIME
+extern "C" void tpa_debug_dump(unsigned long long* host) { (void)hipMemcpyFromSymbol(host, HIP_SYMBOL(tpa::g_dbg), sizeof(tpa::g_dbg)); }
+#endif
 
 int tpa_prefill_mfma_supported(const TpaFwdArgs* a) {
   if (a->dtype != TPA_DTYPE_BF16) return 0;
@@ -354,14 +546,14 @@ int tpa_prefill_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
   p.o = static_cast<uint16_t*>(a->o); p.lse = a->lse;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.rk = a->rk;
   p.sm_scale = a->sm_scale; p.causal = a->causal;
-  p.nqb = (a->lq + kNW * 32 - 1) / (kNW * 32);
+  p.nqb = (a->lq + kBQ - 1) / kBQ;
   p.npairs = p.nqb * a->B;
   if (a->dk == 128) {
-    if (a->rk == 2) return launch_prefill<128, kNW, LOAD_TPA_R2>(p, stream);
-    return launch_prefill<128, kNW, LOAD_TPA_ANY>(p, stream);
+    if (a->rk == 2) return launch_prefill<128, LOAD_TPA_R2>(p, stream);
+    return launch_prefill<128, LOAD_TPA_ANY>(p, stream);
   }
-  if (a->rk == 2) return launch_prefill<64, kNW, LOAD_TPA_R2>(p, stream);
-  return launch_prefill<64, kNW, LOAD_TPA_ANY>(p, stream);
+  if (a->rk == 2) return launch_prefill<64, LOAD_TPA_R2>(p, stream);
+  return launch_prefill<64, LOAD_TPA_ANY>(p, stream);
 }
 
 int mha_prefill_mfma_supported(const MhaFwdArgs* a) {
@@ -384,8 +576,8 @@ int mha_prefill_mfma_launch(const MhaFwdArgs* a, hipStream_t stream) {
   p.o = static_cast<uint16_t*>(a->o); p.lse = a->lse;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = 1; p.rk = 1;
   p.sm_scale = a->sm_scale; p.causal = a->causal;
-  p.nqb = (a->lq + kNW * 32 - 1) / (kNW * 32);
+  p.nqb = (a->lq + kBQ - 1) / kBQ;
   p.npairs = p.nqb * a->B;
-  if (a->dk == 128) return launch_prefill<128, kNW, LOAD_DENSE>(p, stream);
-  return launch_prefill<64, kNW, LOAD_DENSE>(p, stream);
+  if (a->dk == 128) return launch_prefill<128, LOAD_DENSE>(p, stream);
+  return launch_prefill<64, LOAD_DENSE>(p, stream);
 }

@@ -13,7 +13,7 @@ import threading
 import torch
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(_PKG_DIR), "lib", "libtpa_gfx950.so")
+LIB_PATH = os.environ.get("TPA_GFX950_LIB") or os.path.join(os.path.dirname(_PKG_DIR), "lib", "libtpa_gfx950.so")
 
 TPA_DTYPE_F32 = 0
 TPA_DTYPE_BF16 = 1
