@@ -13,10 +13,10 @@
 //                         is the S^T accumulator converted in place: no LDS round trip for P)
 // with the deferred normalisation of flash attention (a reference m and a sum l per row), which
 // is the normalise-every-step recurrence of tpa/tpa.py:389-424 in another order of operations.
-// Waves 0-3 and waves 4-7 (w and w + 4 share a SIMD) run half a tile apart: between two
-// workgroup barriers one group issues its MFMA work while the other does its vector-ALU work
-// (softmax, rebuilding the next K/V tile), then they swap, so the matrix pipe and the vector
-// ALU of a SIMD are fed by different waves at the same time.
+// There is one workgroup barrier per tile (K, V and the head factors are double buffered in
+// LDS); between barriers the two waves of a SIMD drift apart, so one wave's vector-ALU work
+// (softmax) overlaps the other's MFMAs.  The rebuild of the next K/V tile is cut into short
+// pieces that sit between a wave's own MFMAs.
 // The dense flash baseline (tpa/mha.py:23-37) is the same kernel with a plain K/V loader.
 #include <type_traits>
 #include <utility>
@@ -67,6 +67,16 @@ __device__ __forceinline__ float dot2_bf16(uint32_t pair, uint32_t aa) {
 // Workgroup barrier that waits for this wave's LDS traffic only.  __syncthreads() would also
 // wait for the global loads of the next tile's factors, which are meant to stay in flight.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N-1>{})
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 template <int D, int LOADER>
 __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
@@ -129,9 +139,62 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
         qf[ks] = __builtin_bit_cast(bf16x8, sc);
       }
     } else {
-      const uint16_t* ap = p.qa.ptr + b * p.qa.stride_b + (int64_t)qrow_ld * p.qa.stride_l + h;
-      const uint16_t* bp = p.qb.ptr + b * p.qb.stride_b + (int64_t)qrow_ld * p.qb.stride_l + 8 * g;
-      build_q_fragments<NKS, 3>(ap, p.qa.stride_r, bp, p.qb.stride_r, p.rq, c / (float)p.rq, qf);
+      // One rank at a time through LDS: the workgroup copies the 256 x D slab qb[q0.., r, :] with
+      // coalesced 16-byte loads (each row is read once, not once per lane pair), then every lane
+      // picks up its own row's fragments.  The next rank's loads are in flight meanwhile.
+      constexpr int QS = D + 8;                  // row stride in LDS (elements)
+      constexpr int CH = kBQ * CPR / NT;         // 16-byte chunks per thread and rank
+      uint16_t* const qs = smem;                 // [kBQ][QS]
+      uint16_t* const qas = smem + kBQ * QS;     // [kBQ] head factors of this rank
+      static_assert((kBQ * QS + kBQ) * sizeof(uint16_t) <= Lds<D>::kBytes, "Q staging fits the K/V buffers");
+      const uint16_t* qb_b = p.qb.ptr + b * p.qb.stride_b;
+      const uint16_t* qa_b = p.qa.ptr + b * p.qa.stride_b + h;
+      u32x4 nxt[CH];
+      uint32_t a_nxt = 0;
+      auto load_rank = [&](int r) __attribute__((always_inline)) {
+#pragma unroll
+        for (int q = 0; q < CH; ++q) {
+          const int chunk = q * NT + tid, row = chunk / CPR, cc = chunk % CPR;
+          const int grow = min(q0 + row, p.lq - 1);
+          nxt[q] = *reinterpret_cast<const u32x4*>(qb_b + (int64_t)grow * p.qb.stride_l + r * p.qb.stride_r + 8 * cc);
+        }
+        if (tid < kBQ) a_nxt = qa_b[(int64_t)min(q0 + tid, p.lq - 1) * p.qa.stride_l + r * p.qa.stride_r];
+      };
+      float acc[NKS][8];
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[ks][j] = 0.f;
+      load_rank(0);
+      for (int r = 0; r < p.rq; ++r) {
+#pragma unroll
+        for (int q = 0; q < CH; ++q) {
+          const int chunk = q * NT + tid, row = chunk / CPR, cc = chunk % CPR;
+          *reinterpret_cast<u32x4*>(qs + row * QS + 8 * cc) = nxt[q];
+        }
+        if (tid < kBQ) qas[tid] = (uint16_t)a_nxt;
+        if (r + 1 < p.rq) load_rank(r + 1);
+        lds_barrier();
+        const float a = bf16bits_to_f32(qas[32 * w + i]);
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+          const u32x4 bv = *reinterpret_cast<const u32x4*>(qs + (32 * w + i) * QS + 16 * ks + 8 * g);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            acc[ks][2 * j] += a * bf16lo_to_f32(bv[j]);
+            acc[ks][2 * j + 1] += a * bf16hi_to_f32(bv[j]);
+          }
+        }
+        lds_barrier();  // everyone has read this rank before the next one overwrites it
+      }
+      const float scale = c / (float)p.rq;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        u32x4 packed;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) packed[j] = pack_bf16(acc[ks][2 * j] * scale, acc[ks][2 * j + 1] * scale);
+        qf[ks] = __builtin_bit_cast(bf16x8, packed);
+      }
     }
   };
 
@@ -193,45 +256,59 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     if (tid < 4 * kTK) lds_a[slot_idx * Lds<D>::kA + tid] = (uint16_t)a_pending;
   };
 
-  // (a0/2)*b0[d] + (a1/2)*b1[d] for 8 consecutive d; aa = packed (a0, a1).
-  // One assembly block of 8 v_perm_b32 (pair b0[d] with b1[d]), 8 v_dot2_f32_bf16 (the VOP3P form
-  // with a zero addend, so no accumulator has to be cleared first) and 4 v_cvt_pk_bf16_f32.  A dot
-  // result may only be read by another vector-ALU instruction three wait states later and the
-  // hardware does not interlock; the order below keeps at least three instructions (or an s_nop)
-  // between every dot and its conversion.
-  auto rebuild_r2 = [&](const u32x4& b0, const u32x4& b1, uint32_t aa_bits) __attribute__((always_inline)) -> u32x4 {
-    // halve the a pair (exact in bf16): 1/R with R = 2
-    const uint32_t aa = pack_bf16(bf16lo_to_f32(aa_bits) * 0.5f, bf16hi_to_f32(aa_bits) * 0.5f);
+  // (a0/2)*b0[d] + (a1/2)*b1[d] for 8 consecutive d; aa = packed (a0, a1), already halved.
+  // Three short assembly pieces, so that they can sit between MFMAs: 8 v_perm_b32 (pair b0[d]
+  // with b1[d]), 8 v_dot2_f32_bf16 (the VOP3P form with a zero addend, so no accumulator has to
+  // be cleared first) and 4 v_cvt_pk_bf16_f32.  A dot result may only be read by another
+  // vector-ALU instruction three wait states later and the hardware does not interlock; the
+  // s_nop at the head of the last piece guarantees them whatever was scheduled in between.
+  struct Chunk { uint32_t t0, t1, t2, t3, t4, t5, t6, t7; };
+  auto rebuild_perm = [&](Chunk& c_, const u32x4& b0, const u32x4& b1) __attribute__((always_inline)) {
     const uint32_t sel_lo = 0x05040100u, sel_hi = 0x07060302u;
-    uint32_t t0, t1, t2, t3, t4, t5, t6, t7;
     asm volatile(
-        "v_perm_b32 %0, %9, %8, %17\n\t"   // (b0[0], b1[0])
-        "v_perm_b32 %1, %9, %8, %18\n\t"   // (b0[1], b1[1])
-        "v_perm_b32 %2, %11, %10, %17\n\t"
-        "v_perm_b32 %3, %11, %10, %18\n\t"
-        "v_perm_b32 %4, %13, %12, %17\n\t"
-        "v_perm_b32 %5, %13, %12, %18\n\t"
-        "v_perm_b32 %6, %15, %14, %17\n\t"
-        "v_perm_b32 %7, %15, %14, %18\n\t"
-        "v_dot2_f32_bf16 %0, %0, %16, 0\n\t"
-        "v_dot2_f32_bf16 %1, %1, %16, 0\n\t"
-        "v_dot2_f32_bf16 %2, %2, %16, 0\n\t"
-        "v_dot2_f32_bf16 %3, %3, %16, 0\n\t"
-        "v_dot2_f32_bf16 %4, %4, %16, 0\n\t"
-        "v_dot2_f32_bf16 %5, %5, %16, 0\n\t"
-        "v_dot2_f32_bf16 %6, %6, %16, 0\n\t"
-        "v_dot2_f32_bf16 %7, %7, %16, 0\n\t"
-        "s_nop 0\n\t"
+        "v_perm_b32 %0, %9, %8, %16\n\t"   // (b0[0], b1[0])
+        "v_perm_b32 %1, %9, %8, %17\n\t"   // (b0[1], b1[1])
+        "v_perm_b32 %2, %11, %10, %16\n\t"
+        "v_perm_b32 %3, %11, %10, %17\n\t"
+        "v_perm_b32 %4, %13, %12, %16\n\t"
+        "v_perm_b32 %5, %13, %12, %17\n\t"
+        "v_perm_b32 %6, %15, %14, %16\n\t"
+        "v_perm_b32 %7, %15, %14, %17"
+        : "=&v"(c_.t0), "=&v"(c_.t1), "=&v"(c_.t2), "=&v"(c_.t3), "=&v"(c_.t4), "=&v"(c_.t5), "=&v"(c_.t6), "=&v"(c_.t7)
+        : "v"(b0[0]), "v"(b1[0]), "v"(b0[1]), "v"(b1[1]), "v"(b0[2]), "v"(b1[2]), "v"(b0[3]), "v"(b1[3]), "s"(sel_lo), "s"(sel_hi));
+  };
+  auto rebuild_dot = [&](Chunk& c_, uint32_t aa) __attribute__((always_inline)) {
+    asm volatile(
+        "v_dot2_f32_bf16 %0, %0, %8, 0\n\t"
+        "v_dot2_f32_bf16 %1, %1, %8, 0\n\t"
+        "v_dot2_f32_bf16 %2, %2, %8, 0\n\t"
+        "v_dot2_f32_bf16 %3, %3, %8, 0\n\t"
+        "v_dot2_f32_bf16 %4, %4, %8, 0\n\t"
+        "v_dot2_f32_bf16 %5, %5, %8, 0\n\t"
+        "v_dot2_f32_bf16 %6, %6, %8, 0\n\t"
+        "v_dot2_f32_bf16 %7, %7, %8, 0"
+        : "+v"(c_.t0), "+v"(c_.t1), "+v"(c_.t2), "+v"(c_.t3), "+v"(c_.t4), "+v"(c_.t5), "+v"(c_.t6), "+v"(c_.t7)
+        : "v"(aa));
+  };
+  auto rebuild_cvt = [&](Chunk& c_) __attribute__((always_inline)) -> u32x4 {
+    asm volatile(
+        "s_nop 2\n\t"
         "v_cvt_pk_bf16_f32 %0, %0, %1\n\t"
         "v_cvt_pk_bf16_f32 %2, %2, %3\n\t"
         "v_cvt_pk_bf16_f32 %4, %4, %5\n\t"
-        "s_nop 0\n\t"
         "v_cvt_pk_bf16_f32 %6, %6, %7"
-        : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3), "=&v"(t4), "=&v"(t5), "=&v"(t6), "=&v"(t7)
-        : "v"(b0[0]), "v"(b1[0]), "v"(b0[1]), "v"(b1[1]), "v"(b0[2]), "v"(b1[2]), "v"(b0[3]), "v"(b1[3]),
-          "v"(aa), "s"(sel_lo), "s"(sel_hi));
-    u32x4 out = {t0, t2, t4, t6};
-    return out;
+        : "+v"(c_.t0), "+v"(c_.t1), "+v"(c_.t2), "+v"(c_.t3), "+v"(c_.t4), "+v"(c_.t5), "+v"(c_.t6), "+v"(c_.t7));
+    return u32x4{c_.t0, c_.t2, c_.t4, c_.t6};
+  };
+  // halve a packed (a0, a1) pair (exact in bf16): 1/R with R = 2
+  auto halve_pair = [&](uint32_t aa_bits) __attribute__((always_inline)) -> uint32_t {
+    return pack_bf16(bf16lo_to_f32(aa_bits) * 0.5f, bf16hi_to_f32(aa_bits) * 0.5f);
+  };
+  auto rebuild_r2 = [&](const u32x4& b0, const u32x4& b1, uint32_t aa_bits) __attribute__((always_inline)) -> u32x4 {
+    Chunk c_;
+    rebuild_perm(c_, b0, b1);
+    rebuild_dot(c_, halve_pair(aa_bits));
+    return rebuild_cvt(c_);
   };
 
   auto rebuild_any = [&](const uint16_t* bptr, const uint16_t* aptr, int b_stride_r, int a_stride_r) __attribute__((always_inline)) -> u32x4 {
@@ -254,9 +331,28 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     return out;
   };
 
+  // Head factors of this thread's tokens for one matrix of tile `tile`, as packed (a0, a1) pairs:
+  // from the LDS slot ([K|V][token][rank]) or, with a_slot == nullptr, from global memory.
+  auto fetch_aa = [&](auto is_v_c, int tile, const uint16_t* a_slot, uint32_t (&aa)[NPASS]) __attribute__((always_inline)) {
+    constexpr bool is_v = decltype(is_v_c)::value;
+    if constexpr (LOADER != LOAD_TPA_R2) return;
+    const uint16_t* ab = is_v ? va_b : ka_b;
+    const int a_sl = is_v ? p.va.stride_l : p.ka.stride_l, a_sr = is_v ? p.va.stride_r : p.ka.stride_r;
+#pragma unroll
+    for (int ps = 0; ps < NPASS; ++ps) {
+      const int t = ps * TPP + lt;
+      if (a_slot) {
+        aa[ps] = *reinterpret_cast<const uint32_t*>(a_slot + (is_v ? 2 * kTK : 0) + 2 * t);
+      } else {
+        const int tok = min(tile * kTK + t, p.lk - 1);
+        const uint32_t a0 = ab[(int64_t)tok * a_sl], a1 = ab[(int64_t)tok * a_sl + a_sr];
+        aa[ps] = a0 | (a1 << 16);
+      }
+    }
+  };
+
   // Rebuild one matrix of tile `tile` from the registers `issue` filled and store it in LDS.
-  // a_slot = head factors in LDS ([K|V][token][rank]) or nullptr to fetch them from global memory.
-  auto commit = [&](auto is_v_c, int tile, const uint16_t* a_slot) __attribute__((always_inline)) {
+  auto commit = [&](auto is_v_c, int tile, const uint32_t (&aa)[NPASS]) __attribute__((always_inline)) {
     constexpr bool is_v = decltype(is_v_c)::value;
     const uint16_t* bb = is_v ? vb_b : kb_b;
     const uint16_t* ab = is_v ? va_b : ka_b;
@@ -269,16 +365,8 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
       const int t = ps * TPP + lt;
       u32x4 val;
       if constexpr (LOADER == LOAD_TPA_R2) {
-        uint32_t aa;
-        if (a_slot) {
-          aa = *reinterpret_cast<const uint32_t*>(a_slot + (is_v ? 2 * kTK : 0) + 2 * t);
-        } else {
-          const int tok = min(tile * kTK + t, p.lk - 1);
-          const uint32_t a0 = ab[(int64_t)tok * a_sl], a1 = ab[(int64_t)tok * a_sl + a_sr];
-          aa = a0 | (a1 << 16);
-        }
-        if constexpr (is_v) val = rebuild_r2(vreg[ps][0], vreg[ps][1], aa);
-        else val = rebuild_r2(kreg[ps][0], kreg[ps][1], aa);
+        if constexpr (is_v) val = rebuild_r2(vreg[ps][0], vreg[ps][1], aa[ps]);
+        else val = rebuild_r2(kreg[ps][0], kreg[ps][1], aa[ps]);
       } else if constexpr (LOADER == LOAD_TPA_ANY) {
         const int tok = min(tile * kTK + t, p.lk - 1);
         val = rebuild_any(bb + (int64_t)tok * b_sl + 8 * lc, ab + (int64_t)tok * a_sl, b_sr, a_sr);
@@ -300,21 +388,6 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   float mref = 0.f;     // reference (log2 domain, includes c) of row qrow
   float lsum = 0.f;     // this lane's share of sum exp2(x*c - mref)
   const int lp = l & 15, dhalf = (l >> 4) & 1;
-
-  // S^T = K Q^T - mref for tile `tile`
-  auto do_qk = [&](int tile) __attribute__((always_inline)) {
-    const uint16_t* ks = lds_k + (tile & 1) * Lds<D>::kK;
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
-#pragma unroll
-      for (int v = 0; v < 16; ++v) s[mb][v] = -mref;
-#pragma unroll
-      for (int kk = 0; kk < NKS; ++kk) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(ks + (32 * mb + i) * KS + 16 * kk + 8 * g);
-        s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s[mb], 0, 0, 0);
-      }
-    }
-  };
 
   // masks + online softmax of tile `tile` (32 of the 64 logits of row qrow live in this lane)
   auto do_softmax = [&](int tile) __attribute__((always_inline)) {
@@ -376,47 +449,93 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     }
   };
 
-  // O^T += V^T P^T for tile `tile`: k-step kk covers keys 16kk .. 16kk+15 of the tile, in the slot
-  // order the S^T accumulator already has: slot (g, j) = key 16kk + 8(j/4) + 4g + j%4
-  auto do_pv = [&](int tile) __attribute__((always_inline)) {
-    const uint16_t* vs = lds_v + (tile & 1) * Lds<D>::kV;
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      const uint16_t* vrow = vs + (16 * kk + 4 * g + (lp >> 2)) * VS + 16 * dhalf + 4 * (lp & 3);
-#pragma unroll
-      for (int db = 0; db < NDB; ++db) {
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vrow + 32 * db));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vrow + 8 * VS + 32 * db));
-        const bf16x8 vf = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kk], o[db], 0, 0, 0);
-      }
-    }
-  };
-
   // Invariant at entry of iteration j (tile indices clamped to the last tile): kreg = B factors of
   // K tile j+1, vreg = B factors of V tile j, LDS head-factor slot j&1 = (K of tile j+1, V of tile
   // j), a_pending (waves 0-3) = head factors of iteration j+1, K tile j in K buffer j&1, V tile
   // j-1 in V buffer (j-1)&1.
-  // vector-ALU half of iteration j: softmax of tile `sm_tile` (if this wave needs it), rebuild K of
-  // tile j+1 and V of tile j into LDS, start the loads for the next iteration
-  auto valu_phase = [&](int j, int sm_tile) __attribute__((always_inline)) {
-    if (sm_tile >= 0 && sm_tile < ntiles && sm_tile <= wave_last_tile) do_softmax(sm_tile);
+  //
+  // Matrix half of iteration j: O^T += V^T P^T of tile j-1, then S^T = K Q^T - mref of tile j.
+  // The rebuild of K tile j+1 and V tile j (vector-ALU work that only this thread's registers
+  // and the LDS buffers nobody reads during iteration j are involved in) is cut into short pieces
+  // placed between the MFMAs, where their issue slots are free; afterwards the registers are
+  // refilled with the loads of the next iteration.
+  constexpr int N_PV = 4 * NDB, N_QK = 2 * NKS, N_MFMA = N_PV + N_QK;
+  constexpr int N_PIECES = LOADER == LOAD_TPA_R2 ? 2 * NPASS * 3 : 0;  // (perm, dot, cvt+store) per chunk
+  constexpr int PIECE_STRIDE = N_PIECES ? N_MFMA / N_PIECES : 1;
+  auto mfma_phase = [&](int j) __attribute__((always_inline)) {
+    const bool do_pv = j >= 1 && j - 1 <= wave_last_tile;
+    const bool do_qk = j < ntiles && j <= wave_last_tile;
+    const bool do_k = j + 1 < ntiles, do_v = j < ntiles;
     const uint16_t* a_slot = LOADER == LOAD_TPA_R2 ? lds_a + (j & 1) * Lds<D>::kA : nullptr;
-    if (j + 1 < ntiles) commit(IsK{}, j + 1, a_slot);
-    if (j < ntiles) commit(IsV{}, j, a_slot);
+    uint32_t aa_k[NPASS], aa_v[NPASS];
+    fetch_aa(IsK{}, j + 1, a_slot, aa_k);
+    fetch_aa(IsV{}, j, a_slot, aa_v);
+    const uint16_t* vs = lds_v + ((j - 1) & 1) * Lds<D>::kV;
+    const uint16_t* ks = lds_k + (j & 1) * Lds<D>::kK;
+    // one MFMA step: steps 0 .. N_PV-1 are O^T += V^T P^T (k-step kk covers keys 16kk .. 16kk+15 of
+    // the tile, in the slot order the S^T accumulator already has: slot (g, j) = key 16kk + 8(j/4)
+    // + 4g + j%4), the rest are S^T = K Q^T
+    auto mfma_step = [&](auto n_c) __attribute__((always_inline)) {
+      constexpr int n = decltype(n_c)::value;
+      if constexpr (n < N_PV) {
+        constexpr int kk = n / NDB, db = n % NDB;
+        const uint16_t* vrow = vs + (16 * kk + 4 * g + (lp >> 2)) * VS + 16 * dhalf + 4 * (lp & 3);
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vrow + 32 * db));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vrow + 8 * VS + 32 * db));
+        const bf16x8 vf = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kk], o[db], 0, 0, 0);
+      } else {
+        constexpr int m = n - N_PV, mb = m / NKS, kk = m % NKS;
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(ks + (32 * mb + i) * KS + 16 * kk + 8 * g);
+        s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s[mb], 0, 0, 0);
+      }
+    };
+    if (do_qk) {
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[mb][v] = -mref;
+    }
+    if (LOADER == LOAD_TPA_R2 && do_pv && do_qk && do_k && do_v) {
+      // hot path: straight-line code, one rebuild piece after every PIECE_STRIDE MFMAs
+      Chunk ch;
+      static_for<N_MFMA>([&](auto n_c) __attribute__((always_inline)) {
+        constexpr int n = decltype(n_c)::value;
+        mfma_step(n_c);
+        if constexpr (N_PIECES > 0 && (n % PIECE_STRIDE) == PIECE_STRIDE - 1 && n / PIECE_STRIDE < N_PIECES) {
+          constexpr int q = n / PIECE_STRIDE;          // piece index
+          constexpr int chunk = q / 3, part = q % 3;   // chunks: K passes, then V passes
+          constexpr bool is_v = chunk >= NPASS;
+          constexpr int ps = is_v ? chunk - NPASS : chunk;
+          if constexpr (part == 0) {
+            if constexpr (is_v) rebuild_perm(ch, vreg[ps][0], vreg[ps][1]); else rebuild_perm(ch, kreg[ps][0], kreg[ps][1]);
+          } else if constexpr (part == 1) {
+            rebuild_dot(ch, halve_pair(is_v ? aa_v[ps] : aa_k[ps]));
+          } else {
+            const u32x4 val = rebuild_cvt(ch);
+            const int t = ps * TPP + lt;
+            uint16_t* dst = is_v ? lds_v + (j & 1) * Lds<D>::kV + t * VS : lds_k + ((j + 1) & 1) * Lds<D>::kK + t * KS;
+            *reinterpret_cast<u32x4*>(dst + 8 * lc) = val;
+          }
+        }
+      });
+    } else {
+      if (do_k) commit(IsK{}, j + 1, aa_k);
+      if (do_v) commit(IsV{}, j, aa_v);
+      if (do_pv) static_for<N_PV>([&](auto n_c) __attribute__((always_inline)) { mfma_step(n_c); });
+      if (do_qk) static_for<N_QK>([&](auto n_c) __attribute__((always_inline)) { mfma_step(std::integral_constant<int, N_PV + decltype(n_c)::value>{}); });
+    }
     issue(IsK{}, min(j + 2, last));
     issue(IsV{}, min(j + 1, last));
+  };
+  // vector half of iteration j: softmax of tile j (if this wave needs it); waves 0-3 also move
+  // the head factors along: publish the slot of iteration j+1, fetch those of iteration j+2
+  auto valu_phase = [&](int j) __attribute__((always_inline)) {
+    if (j < ntiles && j <= wave_last_tile) do_softmax(j);
     if (w < 4) {
-      // waves 0-3 run their vector half in the second half of the iteration, after waves 4-7
-      // have read slot j&1 ^ 1 for the last time: publish the next slot, fetch the one after
       store_a((j + 1) & 1);
       issue_a(min(j + 3, last), min(j + 2, last));
     }
-  };
-  // matrix half of iteration j: PV of tile j-1, QK of tile j
-  auto mfma_phase = [&](int j) __attribute__((always_inline)) {
-    if (j >= 1 && j - 1 <= wave_last_tile) do_pv(j - 1);
-    if (j < ntiles && j <= wave_last_tile) do_qk(j);
   };
 
   // ---- prologue: K of tile 0 into LDS (head factors straight from global memory), the head
@@ -425,7 +544,11 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   issue(IsK{}, 0);
   issue_a(min(1, last), 0);
   build_q();
-  commit(IsK{}, 0, nullptr);
+  {
+    uint32_t aa0[NPASS];
+    fetch_aa(IsK{}, 0, nullptr, aa0);
+    commit(IsK{}, 0, aa0);
+  }
   issue(IsK{}, min(1, last));
   issue(IsV{}, 0);
   store_a(0);
@@ -433,55 +556,15 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   lds_barrier();
 
 #ifdef EXP_TIME
-  unsigned long long tacc[6] = {0, 0, 0, 0, 0, 0};
   const unsigned long long t_pro = TS();
-  if (w < 4) {
-    for (int j = 0; j <= ntiles; ++j) {
-      unsigned long long t0 = TS();
-      mfma_phase(j);
-      unsigned long long t1 = TS();
-      lds_barrier();
-      unsigned long long t2 = TS();
-      valu_phase(j, j);
-      unsigned long long t3 = TS();
-      lds_barrier();
-      unsigned long long t4 = TS();
-      tacc[0] += t1 - t0; tacc[1] += t2 - t1; tacc[2] += t3 - t2; tacc[3] += t4 - t3;
-    }
-  } else {
-    for (int j = 0; j <= ntiles; ++j) {
-      unsigned long long t0 = TS();
-      valu_phase(j, j - 1);
-      unsigned long long t1 = TS();
-      lds_barrier();
-      unsigned long long t2 = TS();
-      mfma_phase(j);
-      unsigned long long t3 = TS();
-      lds_barrier();
-      unsigned long long t4 = TS();
-      tacc[2] += t1 - t0; tacc[1] += t2 - t1; tacc[0] += t3 - t2; tacc[3] += t4 - t3;
-    }
+#endif
+  for (int j = 0; j <= ntiles; ++j) {
+    mfma_phase(j);
+    valu_phase(j);
+    lds_barrier();
   }
-  if (l == 0) {
-    unsigned long long* d = g_dbg + ((size_t)(blockIdx.x % 1024) * 8 + w) * 8;
-    d[0] = tacc[0]; d[1] = tacc[1]; d[2] = tacc[2]; d[3] = tacc[3]; d[4] = ntiles + 1; d[5] = t_pro - t_start; d[6] = TS() - t_pro; d[7] = 1;
-  }
-#else
-  if (w < 4) {
-    for (int j = 0; j <= ntiles; ++j) {
-      mfma_phase(j);
-      lds_barrier();
-      valu_phase(j, j);
-      lds_barrier();
-    }
-  } else {
-    for (int j = 0; j <= ntiles; ++j) {
-      valu_phase(j, j - 1);
-      lds_barrier();
-      mfma_phase(j);
-      lds_barrier();
-    }
-  }
+#ifdef EXP_TIME
+  const unsigned long long t_loop = TS();
 #endif
 
   // ---- epilogue: normalise, store O[b, qrow, h, :] and LSE[b, h, qrow]
@@ -500,6 +583,13 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
       }
     if (p.lse && g == 0) p.lse[((int64_t)b * p.H + h) * p.lq + qrow] = (mref + __builtin_amdgcn_logf(ltot)) * kLn2;
   }
+#ifdef EXP_TIME
+  if (l == 0) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    unsigned long long* d = g_dbg + ((size_t)(blockIdx.x % 1024) * 8 + w) * 8;
+    d[0] = t_pro - t_start; d[1] = t_loop - t_pro; d[2] = TS() - t_loop; d[3] = ntiles + 1; d[7] = 1;
+  }
+#endif
 }
 
 template <int D, int LOADER>
