@@ -1,0 +1,146 @@
+// XLA FFI handlers over the C ABI of libtpa_gfx950.so, for use from jax on ROCm:
+//   jax.ffi.register_ffi_target("tpa_gfx950_TpaFwd", jax.ffi.pycapsule(lib.TpaFwd), platform="ROCM")
+// These replace the pl.pallas_call of _fwd (tpa/tpa.py:492-543) and the jax.vmap around it
+// (tpa/tpa.py:144-163): the operands are the reference's concatenated q[b,lq,rq,h+dk],
+// k[b,lk,rk,h+dk], v[b,lk,rk,h+dv], read in place through strides.
+//
+// Not part of `make`: it needs the XLA FFI headers (python -c "import jax; print(jax.ffi.include_dir())").
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <string>
+
+#include "tpa_abi.h"
+#include "xla/ffi/api/ffi.h"
+
+namespace ffi = xla::ffi;
+
+namespace {
+
+int dtype_code(ffi::DataType t) {
+  switch (t) {
+    case ffi::DataType::F32: return TPA_DTYPE_F32;
+    case ffi::DataType::BF16: return TPA_DTYPE_BF16;
+    default: return -1;
+  }
+}
+
+size_t elem_bytes(int code) { return code == TPA_DTYPE_F32 ? 4 : 2; }
+
+// A / B factor views of a concatenated [b, l, r, h + d] buffer
+void split(const ffi::AnyBuffer& x, int h, int code, TpaFactor* a, TpaFactor* b) {
+  const auto d = x.dimensions();
+  const int64_t sr = d[3], sl = d[2] * sr, sb = d[1] * sl;
+  const char* base = static_cast<const char*>(x.untyped_data());
+  *a = TpaFactor{base, sb, sl, sr};
+  *b = TpaFactor{base + (size_t)h * elem_bytes(code), sb, sl, sr};
+}
+
+ffi::Error fail(int rc) { return ffi::Error::InvalidArgument(std::string("libtpa_gfx950: ") + tpa_strerror(rc)); }
+
+ffi::Error fill(TpaFwdArgs* a, const ffi::AnyBuffer& q, const ffi::AnyBuffer& k, const ffi::AnyBuffer& v,
+                ffi::Result<ffi::AnyBuffer>& o, ffi::Result<ffi::AnyBuffer>& lse, int32_t num_heads, float sm_scale,
+                bool causal) {
+  const auto qd = q.dimensions(), kd = k.dimensions(), vd = v.dimensions();
+  if (qd.size() != 4 || kd.size() != 4 || vd.size() != 4) return ffi::Error::InvalidArgument("q, k, v must be [b, l, r, h+d]");
+  const int code = dtype_code(q.element_type());
+  if (code < 0 || k.element_type() != q.element_type() || v.element_type() != q.element_type())
+    return ffi::Error::InvalidArgument("q, k, v must share one of f32 / bf16");
+  // shape rules of tpa/tpa.py:475
+  if (kd[0] != qd[0] || vd[0] != qd[0] || kd[1] != vd[1] || kd[2] != vd[2] || kd[3] != qd[3] || num_heads <= 0 ||
+      qd[3] <= num_heads || vd[3] <= num_heads)
+    return ffi::Error::InvalidArgument("inconsistent q / k / v shapes");
+  *a = TpaFwdArgs{};
+  split(q, num_heads, code, &a->qa, &a->qb);
+  split(k, num_heads, code, &a->ka, &a->kb);
+  split(v, num_heads, code, &a->va, &a->vb);
+  a->o = o->untyped_data();
+  a->lse = static_cast<float*>(lse->untyped_data());
+  a->B = (int32_t)qd[0]; a->lq = (int32_t)qd[1]; a->lk = (int32_t)kd[1]; a->H = num_heads;
+  a->dk = (int32_t)qd[3] - num_heads; a->dv = (int32_t)vd[3] - num_heads;
+  a->rq = (int32_t)qd[2]; a->rk = (int32_t)kd[2];
+  a->dtype = code; a->sm_scale = sm_scale; a->causal = causal ? 1 : 0; a->kernel = TPA_KERNEL_AUTO;
+  return ffi::Error::Success();
+}
+
+ffi::Error TpaFwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v,
+                      ffi::Result<ffi::AnyBuffer> o, ffi::Result<ffi::AnyBuffer> lse, int32_t num_heads,
+                      float sm_scale, bool causal) {
+  TpaFwdArgs a;
+  if (ffi::Error e = fill(&a, q, k, v, o, lse, num_heads, sm_scale, causal); e.failure()) return e;
+  const int rc = tpa_fwd(&a, stream);
+  return rc == TPA_OK ? ffi::Error::Success() : fail(rc);
+}
+
+ffi::Error TpaFwdSegImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v,
+                         ffi::Buffer<ffi::DataType::S32> q_segment_ids, ffi::Buffer<ffi::DataType::S32> kv_segment_ids,
+                         ffi::Result<ffi::AnyBuffer> o, ffi::Result<ffi::AnyBuffer> lse, int32_t num_heads,
+                         float sm_scale, bool causal) {
+  TpaFwdArgs a;
+  if (ffi::Error e = fill(&a, q, k, v, o, lse, num_heads, sm_scale, causal); e.failure()) return e;
+  a.q_segment_ids = q_segment_ids.typed_data();
+  a.kv_segment_ids = kv_segment_ids.typed_data();
+  const int rc = tpa_fwd(&a, stream);
+  return rc == TPA_OK ? ffi::Error::Success() : fail(rc);
+}
+
+// workspace: an extra u8 result of tpa_decode_workspace_bytes(...) bytes, allocated by XLA
+ffi::Error TpaDecodeImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v,
+                         ffi::Result<ffi::AnyBuffer> o, ffi::Result<ffi::AnyBuffer> lse,
+                         ffi::Result<ffi::AnyBuffer> workspace, int32_t num_heads, float sm_scale) {
+  TpaFwdArgs a;
+  if (ffi::Error e = fill(&a, q, k, v, o, lse, num_heads, sm_scale, false); e.failure()) return e;
+  a.workspace = workspace->untyped_data();
+  a.workspace_bytes = workspace->size_bytes();
+  const int rc = tpa_decode(&a, stream);
+  return rc == TPA_OK ? ffi::Error::Success() : fail(rc);
+}
+
+// dense q[b,lq,h,dk] k[b,lk,h,dk] v[b,lk,h,dv] (tpa/mha.py:11-17); causal instead of a dense bias
+ffi::Error MhaFwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v,
+                      ffi::Result<ffi::AnyBuffer> o, ffi::Result<ffi::AnyBuffer> lse,
+                      ffi::Result<ffi::AnyBuffer> workspace, float sm_scale, bool causal) {
+  const auto qd = q.dimensions(), kd = k.dimensions(), vd = v.dimensions();
+  if (qd.size() != 4 || kd.size() != 4 || vd.size() != 4) return ffi::Error::InvalidArgument("q, k, v must be [b, l, h, d]");
+  MhaFwdArgs a{};
+  a.q = q.untyped_data(); a.k = k.untyped_data(); a.v = v.untyped_data();
+  a.o = o->untyped_data(); a.lse = static_cast<float*>(lse->untyped_data());
+  a.B = (int32_t)qd[0]; a.lq = (int32_t)qd[1]; a.lk = (int32_t)kd[1]; a.H = (int32_t)qd[2];
+  a.dk = (int32_t)qd[3]; a.dv = (int32_t)vd[3];
+  a.dtype = dtype_code(q.element_type());
+  a.sm_scale = sm_scale; a.causal = causal ? 1 : 0; a.kernel = TPA_KERNEL_AUTO;
+  a.workspace = workspace->untyped_data(); a.workspace_bytes = workspace->size_bytes();
+  const int rc = mha_fwd(&a, stream);
+  return rc == TPA_OK ? ffi::Error::Success() : fail(rc);
+}
+
+}  // namespace
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(TpaFwd, TpaFwdImpl,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
+                                  .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
+                                  .Attr<int32_t>("num_heads").Attr<float>("sm_scale").Attr<bool>("causal"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(TpaFwdSeg, TpaFwdSegImpl,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
+                                  .Arg<ffi::Buffer<ffi::DataType::S32>>().Arg<ffi::Buffer<ffi::DataType::S32>>()
+                                  .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
+                                  .Attr<int32_t>("num_heads").Attr<float>("sm_scale").Attr<bool>("causal"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(TpaDecode, TpaDecodeImpl,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
+                                  .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
+                                  .Attr<int32_t>("num_heads").Attr<float>("sm_scale"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(MhaFwd, MhaFwdImpl,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
+                                  .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
+                                  .Attr<float>("sm_scale").Attr<bool>("causal"));
