@@ -131,6 +131,28 @@ def run_decode(torch, tpa, device, name, steps, warmup):
     )
 
 
+def run_dense_decode(torch, mha, device, name, steps, warmup):
+    """Dense attention (tpa/mha.py) at the decode configuration: the baseline the factored cache is
+    compared with.  K and V hold H*D values per token instead of R*(H+D)."""
+    _, B, lq, lk, H, D, _, _, _ = WORKLOADS[name]
+    g = torch.Generator(device=device)
+    g.manual_seed(3)
+    draw = lambda *shape: torch.randn(shape, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    q = draw(B, lq, H, D)
+    kvs = []
+    for _ in range(2):  # two caches, alternated (each is far larger than the last-level cache anyway)
+        kvs.append((torch.cat([draw(B // 4, lk, H, D) for _ in range(4)]), torch.cat([draw(B // 4, lk, H, D) for _ in range(4)])))
+    scale = D**-0.5
+
+    def step(i):
+        k, v = kvs[i & 1]
+        mha._mha_fwd(q, k, v, None, scale, kernel=2)
+
+    wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
+    nbytes = 2 * B * lk * H * D * 2 + B * lq * H * D * 2 * 2 + B * H * lq * 4
+    return dict(wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, bytes=nbytes, gbs_kernel=nbytes / ev_ms / 1e6)
+
+
 def cpu_baseline_prefill(torch, inputs, shape, budget_s=12.0):
     """The numpy oracle on the prefill workload, one batch element (all heads) at a time, until the
     workload is done or `budget_s` seconds of CPU work have been spent.  Returns the figures and
@@ -226,6 +248,14 @@ def main():
                               algorithmic_bytes_per_launch=d["bytes"]),
                 config=dict(workload="c4: TPA decode over the factored KV cache", **d["shape"]),
             )
+            log("[bench] dense decode at the c4 shape")
+            from tpa import mha
+
+            dd = run_dense_decode(torch, mha, device, "c4", max(10, args.steps // 5), 3)
+            log(f"[bench] {dd['kernel_ms']*1e3:.1f} us/launch, {dd['gbs_kernel']:.0f} GB/s")
+            result["decode"]["dense_mha_same_shape"] = dict(
+                ms_per_launch=dd["kernel_ms"], achieved=dd["gbs_kernel"], unit="GB/s", frac=dd["gbs_kernel"] / PEAK_HBM_GBS,
+                algorithmic_bytes_per_launch=dd["bytes"], speedup_of_factored_cache=dd["kernel_ms"] / d["kernel_ms"])
         if not args.no_cpu and args.workload == "c2":
             log("[bench] cpu baseline (numpy oracle on a sample)")
             base, o_ref, _ = cpu_baseline_prefill(torch, r["inputs"], r["shape"])

@@ -77,7 +77,8 @@ int mha_fwd(const MhaFwdArgs* a, void* stream) {
   if (rc != TPA_OK) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (a->kernel != TPA_KERNEL_GENERIC) {
-    if (mha_decode_supported(a)) return mha_decode_launch(a, s);
+    // few query tokens over a long cache: split over keys, if the caller brought the workspace
+    if (mha_decode_supported(a) && a->workspace) return mha_decode_launch(a, s);
     if (mha_prefill_mfma_supported(a)) return mha_prefill_mfma_launch(a, s);
   }
   if (a->kernel == TPA_KERNEL_MFMA) return TPA_ERR_UNSUPPORTED;

@@ -384,3 +384,70 @@ def test_abi_error_codes(gpu):
     with pytest.raises(d.TpaError) as e:
         tpa.tpa_factors(x[..., :4], x[..., 4:], x[..., :4], x[..., 4:], x[..., :4], x[..., 4:], kernel=d.KERNEL_MFMA)
     assert e.value.code == -6
+
+
+# ---------------------------------------------------------------- dense decode (split over keys)
+@pytest.mark.parametrize("b,lq,lk,h,d", [(2, 1, 1000, 32, 128), (3, 2, 4096, 16, 128), (2, 1, 777, 40, 64), (1, 3, 300, 8, 64)])
+def test_mha_decode_bf16_vs_oracle(gpu, b, lq, lk, h, d):
+    from tpa.mha import _mha_fwd
+
+    rng = np.random.Generator(np.random.Philox(21))
+    q, k, v = (torch.from_numpy(rng.standard_normal(s, dtype=np.float32)).to(torch.bfloat16).to(gpu)
+               for s in ((b, lq, h, d), (b, lk, h, d), (b, lk, h, d)))
+    o_ref, l_ref = orc.mha_forward(as_f64(q), as_f64(k), as_f64(v), None, d**-0.5)
+    o, (lse,) = _mha_fwd(q, k, v, None, d**-0.5, kernel=2)
+    check(o, lse, o_ref, l_ref, BF16_TOL)
+
+
+def test_mha_decode_split_invariance_and_config4_sample(gpu):
+    """Dense decode at B=4 of the decode configuration (lk = 8192, H = 32, D = 128) on the K/V the
+    factored cache stands for: equals the factored decode, for several split counts."""
+    from tpa import _dispatch as d_
+    from tpa import tpa
+
+    b, lk, h, d = 4, 8192, 32, 128
+    q, k, v = make_factors(4, b, 1, lk, h, d, d, 6, 2, scale_by_rank=True)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    rec = lambda x, r: torch.einsum("blrh,blrd->blhd", x[..., :h].float(), x[..., h:].float()) / r
+    Q, K, V = (rec(tq, 6).to(torch.bfloat16), rec(tk, 2).to(torch.bfloat16), rec(tv, 2).to(torch.bfloat16))
+    o_ref, l_ref = orc.mha_forward(as_f64(Q), as_f64(K), as_f64(V), None, d**-0.5)
+    lib = d_.load_library()
+    outs = []
+    for splits in (0, 1, 3, 16):
+        o = torch.empty((b, 1, h, d), dtype=torch.bfloat16, device=gpu)
+        lse = torch.empty((b, h, 1), dtype=torch.float32, device=gpu)
+        ws = torch.empty(lib.mha_fwd_workspace_bytes(b, 1, lk, h, d, splits), dtype=torch.uint8, device=gpu)
+        args = d_.MhaFwdArgs(q=Q.data_ptr(), k=K.data_ptr(), v=V.data_ptr(), bias=None, o=o.data_ptr(), lse=lse.data_ptr(),
+                             B=b, lq=1, lk=lk, H=h, dk=d, dv=d, dtype=1, sm_scale=d**-0.5, causal=0, kernel=2,
+                             workspace=ws.data_ptr(), workspace_bytes=ws.numel(), num_splits=splits)
+        d_.check("mha_fwd", lib.mha_fwd(args, d_.current_stream_ptr(gpu)))
+        torch.cuda.synchronize()
+        check(o, lse, o_ref, l_ref, BF16_TOL)
+        outs.append(o.float())
+    for o in outs[1:]:
+        assert (o - outs[0]).abs().max().item() <= 2e-3
+    # and the factored decode gives the same attention (its K, V are not rounded to bf16)
+    of, lf = tpa.tpa_decode(*tpa_split(tq, tk, tv, h), sm_scale=d**-0.5)
+    assert (of.float() - outs[0]).abs().max().item() <= BF16_TOL
+
+
+def tpa_split(tq, tk, tv, h):
+    return tuple(x.contiguous() for t in (tq, tk, tv) for x in (t[..., :h], t[..., h:]))
+
+
+def test_mha_decode_without_workspace_uses_other_kernels(gpu):
+    from tpa import _dispatch as d_
+
+    b, lk, h, d = 1, 512, 8, 64
+    rng = np.random.Generator(np.random.Philox(22))
+    q, k, v = (torch.from_numpy(rng.standard_normal(s, dtype=np.float32)).to(torch.bfloat16).to(gpu)
+               for s in ((b, 1, h, d), (b, lk, h, d), (b, lk, h, d)))
+    o_ref, l_ref = orc.mha_forward(as_f64(q), as_f64(k), as_f64(v), None, d**-0.5)
+    lib = d_.load_library()
+    o = torch.empty((b, 1, h, d), dtype=torch.bfloat16, device=gpu)
+    lse = torch.empty((b, h, 1), dtype=torch.float32, device=gpu)
+    args = d_.MhaFwdArgs(q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), bias=None, o=o.data_ptr(), lse=lse.data_ptr(),
+                         B=b, lq=1, lk=lk, H=h, dk=d, dv=d, dtype=1, sm_scale=d**-0.5, causal=0, kernel=0,
+                         workspace=None, workspace_bytes=0, num_splits=0)
+    d_.check("mha_fwd", lib.mha_fwd(args, d_.current_stream_ptr(gpu)))
+    check(o, lse, o_ref, l_ref, BF16_TOL)
