@@ -384,7 +384,16 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
   f32x16 s[2];          // exponents x*c - mref of the tile in flight: two 32-key blocks
-  bf16x8 pf[4];         // P^T of the last softmaxed tile, as B operands of the four 16-key steps
+  // P^T of the tile (packed bf16 pairs, the B operands of the four 16-key steps of O^T) is kept
+  // in the registers of the logits it was made from: fragment k = s[k / 2][4 (k % 2) .. + 3]
+  auto pf_set = [&](auto mb_c, auto idx_c, uint32_t bits) __attribute__((always_inline)) {
+    s[decltype(mb_c)::value][decltype(idx_c)::value] = __uint_as_float(bits);
+  };
+  auto pf_get = [&](auto kk_c) __attribute__((always_inline)) -> bf16x8 {
+    constexpr int kk = decltype(kk_c)::value, mb = kk / 2, h4 = 4 * (kk % 2);
+    const u32x4 w4 = {__float_as_uint(s[mb][h4]), __float_as_uint(s[mb][h4 + 1]), __float_as_uint(s[mb][h4 + 2]), __float_as_uint(s[mb][h4 + 3])};
+    return __builtin_bit_cast(bf16x8, w4);
+  };
   float mref = 0.f;     // reference (log2 domain, includes c) of row qrow
   float lsum = 0.f;     // this lane's share of sum exp2(x*c - mref)
   const int lp = l & 15, dhalf = (l >> 4) & 1;
@@ -432,137 +441,268 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) s[mb][v] -= delta;
     }
+    static_for<4>([&](auto k_c) __attribute__((always_inline)) {
+      constexpr int k = decltype(k_c)::value, mb = k / 2, half = k % 2;
+      u32x4 pk;
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        u32x4 pk;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float p0 = __builtin_amdgcn_exp2f(s[mb][8 * half + 2 * j]);
-          const float p1 = __builtin_amdgcn_exp2f(s[mb][8 * half + 2 * j + 1]);
-          lsum += p0 + p1;
-          pk[j] = pack_bf16(p0, p1);
-        }
-        pf[2 * mb + half] = __builtin_bit_cast(bf16x8, pk);
+      for (int j = 0; j < 4; ++j) {
+        const float p0 = __builtin_amdgcn_exp2f(s[mb][8 * half + 2 * j]);
+        const float p1 = __builtin_amdgcn_exp2f(s[mb][8 * half + 2 * j + 1]);
+        lsum += p0 + p1;
+        pk[j] = pack_bf16(p0, p1);
       }
-    }
+      static_for<4>([&](auto j_c) __attribute__((always_inline)) {
+        pf_set(std::integral_constant<int, mb>{}, std::integral_constant<int, 4 * half + decltype(j_c)::value>{}, pk[decltype(j_c)::value]);
+      });
+    });
   };
 
-  // Invariant at entry of iteration j (tile indices clamped to the last tile): kreg = B factors of
-  // K tile j+1, vreg = B factors of V tile j, LDS head-factor slot j&1 = (K of tile j+1, V of tile
-  // j), a_pending (waves 0-3) = head factors of iteration j+1, K tile j in K buffer j&1, V tile
-  // j-1 in V buffer (j-1)&1.
-  //
-  // Matrix half of iteration j: O^T += V^T P^T of tile j-1, then S^T = K Q^T - mref of tile j.
-  // The rebuild of K tile j+1 and V tile j (vector-ALU work that only this thread's registers
-  // and the LDS buffers nobody reads during iteration j are involved in) is cut into short pieces
-  // placed between the MFMAs, where their issue slots are free; afterwards the registers are
-  // refilled with the loads of the next iteration.
-  constexpr int N_PV = 4 * NDB, N_QK = 2 * NKS, N_MFMA = N_PV + N_QK;
-  constexpr int N_PIECES = LOADER == LOAD_TPA_R2 ? 2 * NPASS * 3 : 0;  // (perm, dot, cvt+store) per chunk
-  constexpr int PIECE_STRIDE = N_PIECES ? N_MFMA / N_PIECES : 1;
-  auto mfma_phase = [&](int j) __attribute__((always_inline)) {
-    const bool do_pv = j >= 1 && j - 1 <= wave_last_tile;
-    const bool do_qk = j < ntiles && j <= wave_last_tile;
-    const bool do_k = j + 1 < ntiles, do_v = j < ntiles;
-    const uint16_t* a_slot = LOADER == LOAD_TPA_R2 ? lds_a + (j & 1) * Lds<D>::kA : nullptr;
+  // ---------------------------------------------------------------------------------------
+  // Main loop.  Invariant at entry of iteration j: K tile j and V tile j are in LDS buffers j&1;
+  // kreg / vreg hold the B factors of tile j+1; head-factor slot j&1 holds those of tile j+1 and
+  // a_pending (waves 0-3) those of tile j+2 (tile indices clamped to the last tile); s[] = -mref.
+  // An iteration computes S^T = K Q^T, the softmax and O^T += V^T P^T of tile j, rebuilds tile
+  // j+1 into the other buffers and refills the registers with tile j+2; one barrier ends it.
+  constexpr int N_QK = 2 * NKS, N_PV = 4 * NDB, N_MFMA = N_QK + N_PV;
+  // operand fragment of MFMA step n from LDS: steps 0..N_QK-1 are S^T (32-key block mb = n / NKS),
+  // the rest O^T (k-step kk covers keys 16kk .. 16kk+15 of the tile in the slot order the S^T
+  // accumulator already has: slot (g, j) = key 16kk + 8(j/4) + 4g + j%4)
+  auto load_frag = [&](auto n_c, const uint16_t* ks, const uint16_t* vs) __attribute__((always_inline)) -> bf16x8 {
+    constexpr int n = decltype(n_c)::value;
+    if constexpr (n < N_QK) {
+      constexpr int mb = n / NKS, kk = n % NKS;
+      return *reinterpret_cast<const bf16x8*>(ks + (32 * mb + i) * KS + 16 * kk + 8 * g);
+    } else {
+      constexpr int m = n - N_QK, kk = m / NDB, db = m % NDB;
+      const uint16_t* vrow = vs + (16 * kk + 4 * g + (lp >> 2)) * VS + 16 * dhalf + 4 * (lp & 3);
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vrow + 32 * db));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vrow + 8 * VS + 32 * db));
+      return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    }
+  };
+  auto mfma_with = [&](auto n_c, const bf16x8& f) __attribute__((always_inline)) {
+    constexpr int n = decltype(n_c)::value;
+    if constexpr (n < N_QK) {
+      constexpr int mb = n / NKS, kk = n % NKS;
+      s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, qf[kk], s[mb], 0, 0, 0);
+    } else {
+      constexpr int m = n - N_QK, kk = m / NDB, db = m % NDB;
+      o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, pf_get(std::integral_constant<int, kk>{}), o[db], 0, 0, 0);
+    }
+  };
+  auto splat = [&](auto mb_c) __attribute__((always_inline)) {
+    constexpr int mb = decltype(mb_c)::value;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[mb][v] = -mref;
+  };
+
+  // ---- pieces of the softmax of one 32-key block, for the interleaved (unmasked) path
+  // Move the reference up where this block's row max left the slack (rare).  delta is a whole
+  // number, so the scale factors are exact powers of two.  `pf_done` = number of already packed
+  // P fragments of this tile, which are rescaled too; s[1] is adjusted with s[0] because its
+  // accumulation (still running when block 0 is inspected) started from the old reference.
+  auto move_reference = [&](float tmax, int pf_done) __attribute__((always_inline)) {
+    const float delta = tmax > 0.f ? __builtin_ceilf(tmax) : 0.f;
+    const float alpha = __builtin_amdgcn_exp2f(-delta);
+    mref += delta;
+    lsum *= alpha;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+    // pf_done = 0: block 0 is being inspected, nothing of this tile is packed yet, both blocks move;
+    // pf_done = 2: block 0 has become fragments 0 and 1 (s[0][0..7]), block 1 moves
+    if (pf_done == 0) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s[0][v] -= delta;
+    } else {
+#pragma unroll
+      for (int v = 0; v < 8; ++v) {
+        const uint32_t w1 = __float_as_uint(s[0][v]);
+        s[0][v] = __uint_as_float(pack_bf16(bf16lo_to_f32(w1) * alpha, bf16hi_to_f32(w1) * alpha));
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[1][v] -= delta;
+  };
+  auto sm_max = [&](auto mb_c) __attribute__((always_inline)) {
+    constexpr int mb = decltype(mb_c)::value;
+    float t = s[mb][0];
+#pragma unroll
+    for (int v = 1; v < 16; ++v) t = fmaxf(t, s[mb][v]);
+    t = halves_max(t);
+    if (__any(t > kSlack)) move_reference(t, 2 * mb);
+  };
+  auto sm_exp = [&](auto mb_c, auto q_c) __attribute__((always_inline)) {  // 4 of the block's 16 logits
+    constexpr int mb = decltype(mb_c)::value, q = decltype(q_c)::value;
+    const float p0 = __builtin_amdgcn_exp2f(s[mb][4 * q]);
+    const float p1 = __builtin_amdgcn_exp2f(s[mb][4 * q + 1]);
+    const float p2 = __builtin_amdgcn_exp2f(s[mb][4 * q + 2]);
+    const float p3 = __builtin_amdgcn_exp2f(s[mb][4 * q + 3]);
+    lsum += (p0 + p1) + (p2 + p3);
+    pf_set(mb_c, std::integral_constant<int, 2 * q>{}, pack_bf16(p0, p1));
+    pf_set(mb_c, std::integral_constant<int, 2 * q + 1>{}, pack_bf16(p2, p3));
+  };
+
+  // ---- interleaved iteration (tiles that need no mask, with a next tile to rebuild): every
+  // MFMA is followed by a short slice of independent vector work of the same wave, so that the
+  // vector ALU runs in the shadow of the matrix pipe:
+  //   S^T block 0   | rebuild K tile j+1, refill kreg
+  //   S^T block 1   | softmax of block 0
+  //   O^T, keys 0-31  | softmax of block 1 (its max is taken before these MFMAs start)
+  //   O^T, keys 32-63 | rebuild V tile j+1, refill vreg, s[] = -mref for the next tile
+  // LDS operands are read LA steps ahead of the MFMA that consumes them.
+  auto hot_iteration = [&](int j) __attribute__((always_inline)) {
+    constexpr int LA = 2;
+    const uint16_t* ks = lds_k + (j & 1) * Lds<D>::kK;
+    const uint16_t* vs = lds_v + (j & 1) * Lds<D>::kV;
+    const uint16_t* a_slot = lds_a + (j & 1) * Lds<D>::kA;
+    uint16_t* k_dst = lds_k + ((j + 1) & 1) * Lds<D>::kK;
+    uint16_t* v_dst = lds_v + ((j + 1) & 1) * Lds<D>::kV;
     uint32_t aa_k[NPASS], aa_v[NPASS];
     fetch_aa(IsK{}, j + 1, a_slot, aa_k);
-    fetch_aa(IsV{}, j, a_slot, aa_v);
-    const uint16_t* vs = lds_v + ((j - 1) & 1) * Lds<D>::kV;
-    const uint16_t* ks = lds_k + (j & 1) * Lds<D>::kK;
-    // one MFMA step: steps 0 .. N_PV-1 are O^T += V^T P^T (k-step kk covers keys 16kk .. 16kk+15 of
-    // the tile, in the slot order the S^T accumulator already has: slot (g, j) = key 16kk + 8(j/4)
-    // + 4g + j%4), the rest are S^T = K Q^T
-    auto mfma_step = [&](auto n_c) __attribute__((always_inline)) {
-      constexpr int n = decltype(n_c)::value;
-      if constexpr (n < N_PV) {
-        constexpr int kk = n / NDB, db = n % NDB;
-        const uint16_t* vrow = vs + (16 * kk + 4 * g + (lp >> 2)) * VS + 16 * dhalf + 4 * (lp & 3);
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vrow + 32 * db));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(vrow + 8 * VS + 32 * db));
-        const bf16x8 vf = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kk], o[db], 0, 0, 0);
+    fetch_aa(IsV{}, j + 1, a_slot, aa_v);
+    Chunk ch;
+    // one rebuild piece: 3 per loader pass (pair up the ranks, dot with the head factors, pack + store)
+    auto piece = [&](auto is_v_c, auto q_c) __attribute__((always_inline)) {
+      constexpr bool is_v = decltype(is_v_c)::value;
+      constexpr int q = decltype(q_c)::value, ps = q / 3, part = q % 3;
+      if constexpr (part == 0) {
+        if constexpr (is_v) rebuild_perm(ch, vreg[ps][0], vreg[ps][1]); else rebuild_perm(ch, kreg[ps][0], kreg[ps][1]);
+      } else if constexpr (part == 1) {
+        rebuild_dot(ch, halve_pair(is_v ? aa_v[ps] : aa_k[ps]));
       } else {
-        constexpr int m = n - N_PV, mb = m / NKS, kk = m % NKS;
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(ks + (32 * mb + i) * KS + 16 * kk + 8 * g);
-        s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s[mb], 0, 0, 0);
+        const u32x4 val = rebuild_cvt(ch);
+        const int t = ps * TPP + lt;
+        uint16_t* dst = is_v ? v_dst + t * VS : k_dst + t * KS;
+        *reinterpret_cast<u32x4*>(dst + 8 * lc) = val;
       }
     };
-    if (do_qk) {
-#pragma unroll
-      for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) s[mb][v] = -mref;
-    }
-    if (LOADER == LOAD_TPA_R2 && do_pv && do_qk && do_k && do_v) {
-      // hot path: straight-line code, one rebuild piece after every PIECE_STRIDE MFMAs
-      Chunk ch;
-      static_for<N_MFMA>([&](auto n_c) __attribute__((always_inline)) {
-        constexpr int n = decltype(n_c)::value;
-        mfma_step(n_c);
-        if constexpr (N_PIECES > 0 && (n % PIECE_STRIDE) == PIECE_STRIDE - 1 && n / PIECE_STRIDE < N_PIECES) {
-          constexpr int q = n / PIECE_STRIDE;          // piece index
-          constexpr int chunk = q / 3, part = q % 3;   // chunks: K passes, then V passes
-          constexpr bool is_v = chunk >= NPASS;
-          constexpr int ps = is_v ? chunk - NPASS : chunk;
-          if constexpr (part == 0) {
-            if constexpr (is_v) rebuild_perm(ch, vreg[ps][0], vreg[ps][1]); else rebuild_perm(ch, kreg[ps][0], kreg[ps][1]);
-          } else if constexpr (part == 1) {
-            rebuild_dot(ch, halve_pair(is_v ? aa_v[ps] : aa_k[ps]));
-          } else {
-            const u32x4 val = rebuild_cvt(ch);
-            const int t = ps * TPP + lt;
-            uint16_t* dst = is_v ? lds_v + (j & 1) * Lds<D>::kV + t * VS : lds_k + ((j + 1) & 1) * Lds<D>::kK + t * KS;
-            *reinterpret_cast<u32x4*>(dst + 8 * lc) = val;
+    constexpr int NP = 3 * NPASS;       // rebuild pieces per matrix
+    constexpr int G1 = NKS, G2 = NKS, G3 = 2 * NDB, G4 = 2 * NDB;  // MFMAs per group
+    static_assert(G1 > NP && G4 >= 1, "slices fit their groups");
+    auto slice = [&](auto n_c) __attribute__((always_inline)) {
+      constexpr int n = decltype(n_c)::value;
+      if constexpr (n < G1) {
+        if constexpr (n < NP) piece(IsK{}, n_c);
+        if constexpr (n == NP) issue(IsK{}, min(j + 2, last));
+      } else if constexpr (n < G1 + G2) {
+        constexpr int q = n - G1;  // items 0..4 = max, exp 0..3; item k sits in slot k*G2/5
+        static_for<5>([&](auto k_c) __attribute__((always_inline)) {
+          constexpr int k = decltype(k_c)::value;
+          if constexpr (k * G2 / 5 == q) {
+            if constexpr (k == 0) sm_max(std::integral_constant<int, 0>{});
+            else sm_exp(std::integral_constant<int, 0>{}, std::integral_constant<int, k - 1>{});
           }
-        }
-      });
-    } else {
-      if (do_k) commit(IsK{}, j + 1, aa_k);
-      if (do_v) commit(IsV{}, j, aa_v);
-      if (do_pv) static_for<N_PV>([&](auto n_c) __attribute__((always_inline)) { mfma_step(n_c); });
-      if (do_qk) static_for<N_QK>([&](auto n_c) __attribute__((always_inline)) { mfma_step(std::integral_constant<int, N_PV + decltype(n_c)::value>{}); });
-    }
-    issue(IsK{}, min(j + 2, last));
-    issue(IsV{}, min(j + 1, last));
+        });
+      } else if constexpr (n < G1 + G2 + G3) {
+        constexpr int q = n - G1 - G2;  // exp 0..3 of block 1; item k sits in slot k*G3/4
+        static_for<4>([&](auto k_c) __attribute__((always_inline)) {
+          constexpr int k = decltype(k_c)::value;
+          if constexpr (k * G3 / 4 == q) sm_exp(std::integral_constant<int, 1>{}, k_c);
+        });
+      } else {
+        constexpr int q = n - G1 - G2 - G3;  // items: NP rebuild pieces of V, refill vreg, two splats
+        constexpr int NI = NP + 3;
+        static_for<NI>([&](auto k_c) __attribute__((always_inline)) {
+          constexpr int k = decltype(k_c)::value;
+          if constexpr (k * G4 / NI == q) {
+            if constexpr (k < NP) piece(IsV{}, k_c);
+            else if constexpr (k == NP) issue(IsV{}, min(j + 2, last));
+            else splat(std::integral_constant<int, k - NP - 1>{});
+          }
+        });
+      }
+    };
+    bf16x8 fr[N_MFMA];
+    static_for<LA>([&](auto n_c) __attribute__((always_inline)) { fr[decltype(n_c)::value] = load_frag(n_c, ks, vs); });
+    static_for<N_MFMA>([&](auto n_c) __attribute__((always_inline)) {
+      constexpr int n = decltype(n_c)::value;
+      if constexpr (n == G1 + G2) {
+        sm_max(std::integral_constant<int, 1>{});  // before any O^T MFMA of this tile is issued
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (n + LA < N_MFMA) fr[n + LA] = load_frag(std::integral_constant<int, n + LA>{}, ks, vs);
+      mfma_with(n_c, fr[n]);
+      slice(n_c);
+#ifdef EXP_PIN
+      __builtin_amdgcn_sched_barrier(0);
+#endif
+    });
   };
-  // vector half of iteration j: softmax of tile j (if this wave needs it); waves 0-3 also move
-  // the head factors along: publish the slot of iteration j+1, fetch those of iteration j+2
-  auto valu_phase = [&](int j) __attribute__((always_inline)) {
-    if (j < ntiles && j <= wave_last_tile) do_softmax(j);
-    if (w < 4) {
-      store_a((j + 1) & 1);
-      issue_a(min(j + 3, last), min(j + 2, last));
+
+  // ---- plain iteration: first tile, masked tiles, tiles a wave skips, last tile
+  auto cold_iteration = [&](int j) __attribute__((always_inline)) {
+    if (j <= wave_last_tile) {
+      const uint16_t* ks = lds_k + (j & 1) * Lds<D>::kK;
+      const uint16_t* vs = lds_v + (j & 1) * Lds<D>::kV;
+      static_for<N_QK>([&](auto n_c) __attribute__((always_inline)) { mfma_with(n_c, load_frag(n_c, ks, vs)); });
+      do_softmax(j);
+      static_for<N_PV>([&](auto n_c) __attribute__((always_inline)) {
+        constexpr auto m_c = std::integral_constant<int, N_QK + decltype(n_c)::value>{};
+        mfma_with(m_c, load_frag(m_c, ks, vs));
+      });
+      splat(std::integral_constant<int, 0>{});
+      splat(std::integral_constant<int, 1>{});
+    }
+    if (j + 1 < ntiles) {
+      const uint16_t* a_slot = LOADER == LOAD_TPA_R2 ? lds_a + (j & 1) * Lds<D>::kA : nullptr;
+      uint32_t aa_k[NPASS], aa_v[NPASS];
+      fetch_aa(IsK{}, j + 1, a_slot, aa_k);
+      fetch_aa(IsV{}, j + 1, a_slot, aa_v);
+      commit(IsK{}, j + 1, aa_k);
+      commit(IsV{}, j + 1, aa_v);
+      issue(IsK{}, min(j + 2, last));
+      issue(IsV{}, min(j + 2, last));
     }
   };
 
-  // ---- prologue: K of tile 0 into LDS (head factors straight from global memory), the head
-  // factors of iteration 0 in their LDS slot, those of iteration 1 pending, and the B-factor
-  // loads of iteration 0 in flight
+  // ---- prologue: tile 0 into LDS (head factors straight from global memory), the head factors
+  // of tile 1 in slot 0, those of tile 2 pending, the B factors of tile 1 in registers
   issue(IsK{}, 0);
-  issue_a(min(1, last), 0);
+  issue(IsV{}, 0);
+  issue_a(min(1, last), min(1, last));
   build_q();
   {
-    uint32_t aa0[NPASS];
+    uint32_t aa0[NPASS], aa1[NPASS];
     fetch_aa(IsK{}, 0, nullptr, aa0);
+    fetch_aa(IsV{}, 0, nullptr, aa1);
     commit(IsK{}, 0, aa0);
+    commit(IsV{}, 0, aa1);
   }
   issue(IsK{}, min(1, last));
-  issue(IsV{}, 0);
+  issue(IsV{}, min(1, last));
   store_a(0);
-  issue_a(min(2, last), min(1, last));
+  issue_a(min(2, last), min(2, last));
+  splat(std::integral_constant<int, 0>{});
+  splat(std::integral_constant<int, 1>{});
   lds_barrier();
 
 #ifdef EXP_TIME
   const unsigned long long t_pro = TS();
 #endif
-  for (int j = 0; j <= ntiles; ++j) {
-    mfma_phase(j);
-    valu_phase(j);
+  // Per wave: tile 0 plain, then the run of unmasked tiles interleaved, then plain again (masked
+  // tiles, tiles past this wave's causal range, the last tile).  Three separate loops rather than
+  // a branch inside one: every wave passes the same number of barriers either way.
+  auto tail = [&](int j) __attribute__((always_inline)) {
+    if (w < 4) {  // head factors: publish those of tile j+2, fetch those of tile j+3
+      store_a((j + 1) & 1);
+      issue_a(min(j + 3, last), min(j + 3, last));
+    }
     lds_barrier();
+  };
+  int hot_end = 1;
+  if constexpr (LOADER == LOAD_TPA_R2) {
+    int first_masked = p.lk / kTK;                                   // ragged last tile
+    if (p.causal) first_masked = min(first_masked, (wrow0 + 1) / kTK);  // first tile with a key past row wrow0
+    hot_end = max(1, min(min(ntiles - 1, first_masked), wave_last_tile + 1));
   }
+  int j = 0;
+  for (; j < 1; ++j) { cold_iteration(j); tail(j); }
+  if constexpr (LOADER == LOAD_TPA_R2) {
+    for (; j < hot_end; ++j) { hot_iteration(j); tail(j); }
+  }
+  for (; j < ntiles; ++j) { cold_iteration(j); tail(j); }
 #ifdef EXP_TIME
   const unsigned long long t_loop = TS();
 #endif
@@ -587,7 +727,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   if (l == 0) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     unsigned long long* d = g_dbg + ((size_t)(blockIdx.x % 1024) * 8 + w) * 8;
-    d[0] = t_pro - t_start; d[1] = t_loop - t_pro; d[2] = TS() - t_loop; d[3] = ntiles + 1; d[7] = 1;
+    d[0] = t_pro - t_start; d[1] = t_loop - t_pro; d[2] = TS() - t_loop; d[3] = ntiles; d[7] = 1;
   }
 #endif
 }
