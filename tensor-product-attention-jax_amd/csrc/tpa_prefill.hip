@@ -14,9 +14,13 @@
 // with the deferred normalisation of flash attention (a reference m and a sum l per row), which
 // is the normalise-every-step recurrence of tpa/tpa.py:389-424 in another order of operations.
 // There is one workgroup barrier per tile (K, V and the head factors are double buffered in
-// LDS); between barriers the two waves of a SIMD drift apart, so one wave's vector-ALU work
-// (softmax) overlaps the other's MFMAs.  The rebuild of the next K/V tile is cut into short
-// pieces that sit between a wave's own MFMAs.
+// LDS).  On tiles that need no mask a wave runs everything as ONE instruction stream in which
+// each MFMA is followed by a short slice of independent vector work: the softmax of a 32-key
+// block runs in the shadow of the MFMAs of the next block, the rebuild of the next K/V tile in
+// the shadow of the first S^T and the last O^T MFMAs.  (A vector instruction issued while a
+// matrix instruction of the same wave executes is nearly free on this hardware, whereas two
+// waves of a SIMD that are both in a vector-only or both in a matrix-only phase just queue up;
+// the dot instruction is the exception: it occupies the matrix pipe.)
 // The dense flash baseline (tpa/mha.py:23-37) is the same kernel with a plain K/V loader.
 #include <type_traits>
 #include <utility>
@@ -29,10 +33,6 @@ namespace {
 constexpr int kTK = 64;   // keys per tile
 constexpr int kNW = 8;    // waves per workgroup
 constexpr int kBQ = 256;  // query rows per workgroup (32 per wave)
-#ifdef EXP_TIME
-__device__ unsigned long long g_dbg[8192 * 8];
-#define TS() __builtin_amdgcn_s_memtime()
-#endif
 
 enum { LOAD_TPA_R2 = 0, LOAD_TPA_ANY = 1, LOAD_DENSE = 2 };
 
@@ -113,9 +113,6 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   const int qblk = p.nqb - 1 - pair / p.B;
   const int b = pair % p.B;
 
-#ifdef EXP_TIME
-  const unsigned long long t_start = TS();
-#endif
   const int tid = threadIdx.x;
   const int w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
   const int q0 = qblk * kBQ;
@@ -253,10 +250,12 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   };
   auto store_a = [&](int slot_idx) __attribute__((always_inline)) {
     if constexpr (LOADER != LOAD_TPA_R2) return;
-    if (tid < 4 * kTK) lds_a[slot_idx * Lds<D>::kA + tid] = (uint16_t)a_pending;
+    // stored halved (exact in bf16): the 1/R of the reconstruction with R = 2
+    if (tid < 4 * kTK) lds_a[slot_idx * Lds<D>::kA + tid] = (uint16_t)(pack_bf16(bf16lo_to_f32(a_pending) * 0.5f, 0.f));
   };
 
-  // (a0/2)*b0[d] + (a1/2)*b1[d] for 8 consecutive d; aa = packed (a0, a1), already halved.
+  // (a0/2)*b0[d] + (a1/2)*b1[d] for 8 consecutive d; aa = packed (a0/2, a1/2): fetch_aa hands out
+  // halved head factors.
   // Three short assembly pieces, so that they can sit between MFMAs: 8 v_perm_b32 (pair b0[d]
   // with b1[d]), 8 v_dot2_f32_bf16 (the VOP3P form with a zero addend, so no accumulator has to
   // be cleared first) and 4 v_cvt_pk_bf16_f32.  A dot result may only be read by another
@@ -307,7 +306,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   auto rebuild_r2 = [&](const u32x4& b0, const u32x4& b1, uint32_t aa_bits) __attribute__((always_inline)) -> u32x4 {
     Chunk c_;
     rebuild_perm(c_, b0, b1);
-    rebuild_dot(c_, halve_pair(aa_bits));
+    rebuild_dot(c_, aa_bits);
     return rebuild_cvt(c_);
   };
 
@@ -346,7 +345,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
       } else {
         const int tok = min(tile * kTK + t, p.lk - 1);
         const uint32_t a0 = ab[(int64_t)tok * a_sl], a1 = ab[(int64_t)tok * a_sl + a_sr];
-        aa[ps] = a0 | (a1 << 16);
+        aa[ps] = halve_pair(a0 | (a1 << 16));
       }
     }
   };
@@ -570,7 +569,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
       if constexpr (part == 0) {
         if constexpr (is_v) rebuild_perm(ch, vreg[ps][0], vreg[ps][1]); else rebuild_perm(ch, kreg[ps][0], kreg[ps][1]);
       } else if constexpr (part == 1) {
-        rebuild_dot(ch, halve_pair(is_v ? aa_v[ps] : aa_k[ps]));
+        rebuild_dot(ch, is_v ? aa_v[ps] : aa_k[ps]);
       } else {
         const u32x4 val = rebuild_cvt(ch);
         const int t = ps * TPP + lt;
@@ -625,9 +624,6 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
       if constexpr (n + LA < N_MFMA) fr[n + LA] = load_frag(std::integral_constant<int, n + LA>{}, ks, vs);
       mfma_with(n_c, fr[n]);
       slice(n_c);
-#ifdef EXP_PIN
-      __builtin_amdgcn_sched_barrier(0);
-#endif
     });
   };
 
@@ -678,9 +674,6 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   splat(std::integral_constant<int, 1>{});
   lds_barrier();
 
-#ifdef EXP_TIME
-  const unsigned long long t_pro = TS();
-#endif
   // Per wave: tile 0 plain, then the run of unmasked tiles interleaved, then plain again (masked
   // tiles, tiles past this wave's causal range, the last tile).  Three separate loops rather than
   // a branch inside one: every wave passes the same number of barriers either way.
@@ -703,9 +696,6 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     for (; j < hot_end; ++j) { hot_iteration(j); tail(j); }
   }
   for (; j < ntiles; ++j) { cold_iteration(j); tail(j); }
-#ifdef EXP_TIME
-  const unsigned long long t_loop = TS();
-#endif
 
   // ---- epilogue: normalise, store O[b, qrow, h, :] and LSE[b, h, qrow]
   const float ltot = halves_sum(lsum);
@@ -723,13 +713,6 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
       }
     if (p.lse && g == 0) p.lse[((int64_t)b * p.H + h) * p.lq + qrow] = (mref + __builtin_amdgcn_logf(ltot)) * kLn2;
   }
-#ifdef EXP_TIME
-  if (l == 0) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    unsigned long long* d = g_dbg + ((size_t)(blockIdx.x % 1024) * 8 + w) * 8;
-    d[0] = t_pro - t_start; d[1] = t_loop - t_pro; d[2] = TS() - t_loop; d[3] = ntiles; d[7] = 1;
-  }
-#endif
 }
 
 template <int D, int LOADER>
@@ -755,9 +738,6 @@ bool factor_ok(const TpaFactor& f) {
 }  // namespace
 }  // namespace tpa
 
-#ifdef EXP_TIME
-extern "C" void tpa_debug_dump(unsigned long long* host) { (void)hipMemcpyFromSymbol(host, HIP_SYMBOL(tpa::g_dbg), sizeof(tpa::g_dbg)); }
-#endif
 
 int tpa_prefill_mfma_supported(const TpaFwdArgs* a) {
   if (a->dtype != TPA_DTYPE_BF16) return 0;
