@@ -42,7 +42,8 @@ struct DecodeLds {
   static constexpr int kB = kRowsPerBlock * D;       // elements of one B tile
   static constexpr int kA = kRowsPerBlock * 32;      // elements of one A tile (32 heads)
   static constexpr int kWave = 2 * kB + 2 * kA;      // elements per wave
-  static constexpr int kReduce = 32 * D * 2 + 128;   // fp32 O^T + m + l, in uint16 units
+  static constexpr int kRedStride = D + 4;           // fp32 row stride of the wave-merge staging (spreads the banks)
+  static constexpr int kReduce = 32 * kRedStride * 2 + 128;  // fp32 O^T + m + l, in uint16 units
   static constexpr int kPerWave = kWave > kReduce ? kWave : kReduce;
   static constexpr size_t kBytes = (size_t)kWaves * kPerWave * sizeof(uint16_t);
 };
@@ -259,14 +260,17 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   }
 
   // ---- merge the 4 waves through LDS (each wave reuses its own staging region)
+  constexpr int RS = DecodeLds<D>::kRedStride;
   const float ltot = halves_sum(lsum);
-  float* red_o = reinterpret_cast<float*>(lds);  // [32 heads][D]
-  float* red_m = red_o + 32 * D;
+  float* red_o = reinterpret_cast<float*>(lds);  // [32 heads][RS]
+  float* red_m = red_o + 32 * RS;
   float* red_l = red_m + 32;
 #pragma unroll
   for (int db = 0; db < NDB; ++db)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) red_o[i * D + 32 * db + 8 * (v >> 2) + 4 * g + (v & 3)] = o[db][v];
+    for (int vq = 0; vq < 4; ++vq)
+      *reinterpret_cast<f32x4*>(red_o + i * RS + 32 * db + 8 * vq + 4 * g) =
+          f32x4{o[db][4 * vq], o[db][4 * vq + 1], o[db][4 * vq + 2], o[db][4 * vq + 3]};
   if (g == 0) {
     red_m[i] = m;
     red_l[i] = ltot;
@@ -280,7 +284,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
     float mw[kWaves], mmax = -INFINITY;
 #pragma unroll
     for (int ww = 0; ww < kWaves; ++ww) {
-      mw[ww] = reinterpret_cast<const float*>(smem + ww * DecodeLds<D>::kPerWave)[32 * D + hh];
+      mw[ww] = reinterpret_cast<const float*>(smem + ww * DecodeLds<D>::kPerWave)[32 * RS + hh];
       mmax = fmaxf(mmax, mw[ww]);
     }
     float acc = 0.f, lacc = 0.f;
@@ -288,8 +292,8 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
     for (int ww = 0; ww < kWaves; ++ww) {
       const float* ro = reinterpret_cast<const float*>(smem + ww * DecodeLds<D>::kPerWave);
       const float f = mw[ww] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw[ww] - mmax);
-      acc += f * ro[hh * D + d];
-      lacc += f * ro[32 * D + 32 + hh];
+      acc += f * ro[hh * RS + d];
+      lacc += f * ro[32 * RS + 32 + hh];
     }
     p.part_o[(pbase + hh) * D + d] = acc;
     if (d == 0) {
