@@ -566,7 +566,13 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     auto piece = [&](auto is_v_c, auto q_c) __attribute__((always_inline)) {
       constexpr bool is_v = decltype(is_v_c)::value;
       constexpr int q = decltype(q_c)::value, ps = q / 3, part = q % 3;
-      if constexpr (part == 0) {
+      if constexpr (LOADER == LOAD_DENSE) {  // nothing to rebuild: the loaded rows are the tile
+        if constexpr (part == 2) {
+          const int t = ps * TPP + lt;
+          uint16_t* dst = is_v ? v_dst + t * VS : k_dst + t * KS;
+          *reinterpret_cast<u32x4*>(dst + 8 * lc) = is_v ? vreg[ps][0] : kreg[ps][0];
+        }
+      } else if constexpr (part == 0) {
         if constexpr (is_v) rebuild_perm(ch, vreg[ps][0], vreg[ps][1]); else rebuild_perm(ch, kreg[ps][0], kreg[ps][1]);
       } else if constexpr (part == 1) {
         rebuild_dot(ch, is_v ? aa_v[ps] : aa_k[ps]);
@@ -685,14 +691,14 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     lds_barrier();
   };
   int hot_end = 1;
-  if constexpr (LOADER == LOAD_TPA_R2) {
+  if constexpr (LOADER != LOAD_TPA_ANY) {
     int first_masked = p.lk / kTK;                                   // ragged last tile
     if (p.causal) first_masked = min(first_masked, (wrow0 + 1) / kTK);  // first tile with a key past row wrow0
     hot_end = max(1, min(min(ntiles - 1, first_masked), wave_last_tile + 1));
   }
   int j = 0;
   for (; j < 1; ++j) { cold_iteration(j); tail(j); }
-  if constexpr (LOADER == LOAD_TPA_R2) {
+  if constexpr (LOADER != LOAD_TPA_ANY) {
     for (; j < hot_end; ++j) { hot_iteration(j); tail(j); }
   }
   for (; j < ntiles; ++j) { cold_iteration(j); tail(j); }
