@@ -638,11 +638,21 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     if (j <= wave_last_tile) {
       const uint16_t* ks = lds_k + (j & 1) * Lds<D>::kK;
       const uint16_t* vs = lds_v + (j & 1) * Lds<D>::kV;
-      static_for<N_QK>([&](auto n_c) __attribute__((always_inline)) { mfma_with(n_c, load_frag(n_c, ks, vs)); });
+      // operands are read three MFMAs ahead here too (the V fragments of the first O^T steps
+      // while the softmax runs)
+      constexpr int LA = 3;
+      bf16x8 fr[N_MFMA];
+      static_for<LA>([&](auto n_c) __attribute__((always_inline)) { fr[decltype(n_c)::value] = load_frag(n_c, ks, vs); });
+      static_for<N_QK>([&](auto n_c) __attribute__((always_inline)) {
+        constexpr int n = decltype(n_c)::value;
+        if constexpr (n + LA < N_MFMA) fr[n + LA] = load_frag(std::integral_constant<int, n + LA>{}, ks, vs);
+        mfma_with(n_c, fr[n]);
+      });
       do_softmax(j);
       static_for<N_PV>([&](auto n_c) __attribute__((always_inline)) {
-        constexpr auto m_c = std::integral_constant<int, N_QK + decltype(n_c)::value>{};
-        mfma_with(m_c, load_frag(m_c, ks, vs));
+        constexpr int n = N_QK + decltype(n_c)::value;
+        if constexpr (n + LA < N_MFMA) fr[n + LA] = load_frag(std::integral_constant<int, n + LA>{}, ks, vs);
+        mfma_with(std::integral_constant<int, n>{}, fr[n]);
       });
       splat(std::integral_constant<int, 0>{});
       splat(std::integral_constant<int, 1>{});

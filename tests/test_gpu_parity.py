@@ -451,3 +451,33 @@ def test_mha_decode_without_workspace_uses_other_kernels(gpu):
                          workspace=None, workspace_bytes=0, num_splits=0)
     d_.check("mha_fwd", lib.mha_fwd(args, d_.current_stream_ptr(gpu)))
     check(o, lse, o_ref, l_ref, BF16_TOL)
+
+
+# ---------------------------------------------------------------- reference moves inside the interleaved loop
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("where", ["first_block", "second_block", "both"])
+def test_prefill_reference_moves_on_unmasked_tiles(gpu, d, causal, where):
+    """Logits that grow along the keys, with jumps of more than 2^8 placed in the first or the
+    second 32-key block of tiles far from the diagonal: the running reference has to move (and
+    O, the row sums and the already packed P fragments have to be rescaled) in the middle of the
+    tiles that take the interleaved path.  Checked per row against the oracle."""
+    b, t, h = 1, 1024, 2
+    q, k, v = make_factors(41, b, t, t, h, d, d, 6, 2, scale_by_rank=True)
+    # one strong direction shared by all queries; keys pick it up with a gain that steps up
+    hq = q[..., h:]
+    hq[..., 0] = 3.0
+    gain = np.zeros(t, dtype=np.float32)
+    steps = {"first_block": [64 * 3 + 5, 64 * 9 + 17], "second_block": [64 * 2 + 40, 64 * 11 + 60],
+             "both": [64 * 2 + 3, 64 * 2 + 50, 64 * 7 + 31, 64 * 7 + 33]}[where]
+    for pos in steps:
+        gain[pos:] += 3.5  # 10.5 in the log2 domain per step (sm_scale = ln 2 below)
+    k[..., h:][..., 0] = gain[None, :, None]
+    q[..., :h] = 1.0
+    k[..., :h] = 1.0
+    # sm_scale * log2(e) = 1: the kernel's pre-scaled bf16 Q then equals Q, so the one strong
+    # coordinate carries no rounding of its own into every logit
+    scale = float(np.log(2.0))
+    (tq, tk, tv), o, lse = run_bf16(gpu, q, k, v, h, scale, causal)
+    o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h, sm_scale=scale, causal=causal)
+    check(o, lse, o_ref, l_ref, BF16_TOL, lse_tol=2e-3)
