@@ -1,7 +1,7 @@
 // Any-shape forward kernel: fp32 arithmetic on the vector ALUs, no MFMA.
 //
-// It serves the problems the MFMA kernels do not take: fp32 inputs, head dimensions that are
-// not multiples of 32, segment-id masks and dense biases.  One thread owns one query row of one
+// It serves the problems the MFMA kernels do not take: fp32 inputs, head dimensions other than
+// 64 and 128, unaligned operands and dense biases.  One thread owns one query row of one
 // head and keeps q and the output accumulator in registers; the workgroup rebuilds the head's
 // K and V tile from the rank factors in LDS (tpa/tpa.py:364,417) and every thread walks the
 // tile with an online softmax (tpa/tpa.py:389-424, in the deferred-normalisation form).

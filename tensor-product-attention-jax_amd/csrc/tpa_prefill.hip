@@ -38,6 +38,8 @@ enum { LOAD_TPA_R2 = 0, LOAD_TPA_ANY = 1, LOAD_DENSE = 2 };
 
 struct PrefillParams {
   TpaFactor qa, qb, ka, kb, va, vb;  // dense: qb/kb/vb hold q/k/v with stride_l = H*D, ptr at head 0
+  const int32_t* qseg;   // [B, lq] or null
+  const int32_t* kvseg;  // [B, lk] or null (both or neither)
   uint16_t* o;
   float* lse;
   int B, lq, lk, H, rq, rk;
@@ -54,7 +56,8 @@ struct Lds {
   static constexpr int kK = kTK * KS;  // elements of one K buffer
   static constexpr int kV = kTK * VS;  // elements of one V buffer
   static constexpr int kA = 2 * kTK * 2;  // one slot of head factors: [K|V][token][rank 0|1]
-  static constexpr size_t kBytes = (2 * (kK + kV) + 2 * kA) * sizeof(uint16_t);
+  static constexpr int kSeg = 2 * kTK;    // one slot of key segment ids (int32), in uint16 units
+  static constexpr size_t kBytes = (2 * (kK + kV) + 2 * kA + 2 * kSeg) * sizeof(uint16_t);
 };
 
 // a0*b0 + a1*b1 on packed bf16 pairs, fp32 result.  Through the builtin on purpose: the dot
@@ -93,14 +96,15 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   // scalars out of the argument block (never take the address of the block itself)
   struct Fac { const uint16_t* ptr; int64_t stride_b; int stride_l, stride_r; };
   auto fac = [](const TpaFactor& f) { return Fac{static_cast<const uint16_t*>(f.ptr), f.stride_b, (int)f.stride_l, (int)f.stride_r}; };
-  struct { Fac qa, qb, ka, kb, va, vb; uint16_t* o; float* lse; int B, lq, lk, H, rq, rk; float sm_scale; int causal, nqb, npairs; } const p = {
-      fac(pp.qa), fac(pp.qb), fac(pp.ka), fac(pp.kb), fac(pp.va), fac(pp.vb), pp.o, pp.lse, pp.B, pp.lq, pp.lk, pp.H, pp.rq, pp.rk,
+  struct { Fac qa, qb, ka, kb, va, vb; const int32_t* qseg; const int32_t* kvseg; uint16_t* o; float* lse; int B, lq, lk, H, rq, rk; float sm_scale; int causal, nqb, npairs; } const p = {
+      fac(pp.qa), fac(pp.qb), fac(pp.ka), fac(pp.kb), fac(pp.va), fac(pp.vb), pp.qseg, pp.kvseg, pp.o, pp.lse, pp.B, pp.lq, pp.lk, pp.H, pp.rq, pp.rk,
       pp.sm_scale, pp.causal, pp.nqb, pp.npairs};
 
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   uint16_t* const lds_k = smem;                                  // [2][kTK][KS]
   uint16_t* const lds_v = smem + 2 * Lds<D>::kK;                 // [2][kTK][VS]
   uint16_t* const lds_a = smem + 2 * (Lds<D>::kK + Lds<D>::kV);  // [2][K|V][kTK][2]
+  int32_t* const lds_seg = reinterpret_cast<int32_t*>(lds_a + 2 * Lds<D>::kA);  // [2][kTK] key segment ids
 
   // ---- which (query block, batch, head): heads of one (block, batch) pair sit on one XCD
   // (workgroup ids are dealt round-robin to the 8 XCDs) so they share the B-factor tiles in
@@ -254,6 +258,20 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     if (tid < 4 * kTK) lds_a[slot_idx * Lds<D>::kA + tid] = (uint16_t)(pack_bf16(bf16lo_to_f32(a_pending) * 0.5f, 0.f));
   };
 
+  // Key segment ids (packed sequences, tpa/tpa.py:369-375): threads 256..319 fetch one id of a tile
+  // each, park it in a register and store it into an LDS slot one iteration later, like the head
+  // factors; slot j&1 holds the ids of tile j during iteration j.
+  const bool has_seg = p.kvseg != nullptr;
+  int32_t seg_pending = 0;
+  auto issue_seg = [&](int tile) __attribute__((always_inline)) {
+    if (has_seg && tid >= 4 * kTK && tid < 5 * kTK)
+      seg_pending = p.kvseg[(int64_t)b * p.lk + min(tile * kTK + tid - 4 * kTK, p.lk - 1)];
+  };
+  auto store_seg = [&](int slot_idx) __attribute__((always_inline)) {
+    if (has_seg && tid >= 4 * kTK && tid < 5 * kTK) lds_seg[slot_idx * kTK + tid - 4 * kTK] = seg_pending;
+  };
+  const int32_t qseg = has_seg ? p.qseg[(int64_t)b * p.lq + qrow_ld] : 0;
+
   // (a0/2)*b0[d] + (a1/2)*b1[d] for 8 consecutive d; aa = packed (a0/2, a1/2): fetch_aa hands out
   // halved head factors.
   // Three short assembly pieces, so that they can sit between MFMAs: 8 v_perm_b32 (pair b0[d]
@@ -398,6 +416,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   const int lp = l & 15, dhalf = (l >> 4) & 1;
 
   // masks + online softmax of tile `tile` (32 of the 64 logits of row qrow live in this lane)
+  bool seen = false;  // this row has met a visible key (its reference is set)
   auto do_softmax = [&](int tile) __attribute__((always_inline)) {
     const int k0 = tile * kTK;
     // keys beyond lk, and keys after the query under the causal mask
@@ -412,33 +431,45 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
           if (t > limit) s[mb][v] = -INFINITY;
         }
     }
+    if (has_seg) {  // keys of another segment (tpa/tpa.py:369-375)
+      const int32_t* slot = lds_seg + (tile & 1) * kTK;
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) {
+          const int4 ids = *reinterpret_cast<const int4*>(slot + 32 * mb + 8 * vq + 4 * g);
+          if (ids.x != qseg) s[mb][4 * vq] = -INFINITY;
+          if (ids.y != qseg) s[mb][4 * vq + 1] = -INFINITY;
+          if (ids.z != qseg) s[mb][4 * vq + 2] = -INFINITY;
+          if (ids.w != qseg) s[mb][4 * vq + 3] = -INFINITY;
+        }
+    }
     float tmax = s[0][0];
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) tmax = fmaxf(tmax, s[mb][v]);
     tmax = halves_max(tmax);
-    if (tile == 0) {
-      // first tile: take its max as the reference (the accumulators started at 0)
-      mref = tmax;
-#pragma unroll
-      for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) s[mb][v] -= tmax;
-    } else if (__any(tmax > kSlack)) {
-      // rare: some row's max left the slack; move the references up and rescale
-      const float delta = fmaxf(tmax, 0.f);
-      const float alpha = __builtin_amdgcn_exp2f(-delta);
+    const bool first = !seen && tmax > -INFINITY;  // first tile with a visible key for this row
+    const bool up = seen && tmax > kSlack;         // rare: the row's max left the slack
+    if (__any(first || up)) {
+      // a first tile sets the reference (nothing accumulated yet, so nothing to rescale); later
+      // the references move up and O and the row sums are rescaled
+      const float delta = first ? tmax : (up ? tmax : 0.f);
+      const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);
       mref += delta;
       lsum *= alpha;
+      if (__any(up)) {
 #pragma unroll
-      for (int db = 0; db < NDB; ++db)
+        for (int db = 0; db < NDB; ++db)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+          for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+      }
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
         for (int v = 0; v < 16; ++v) s[mb][v] -= delta;
+      seen = seen || first;
     }
     static_for<4>([&](auto k_c) __attribute__((always_inline)) {
       constexpr int k = decltype(k_c)::value, mb = k / 2, half = k % 2;
@@ -686,6 +717,9 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   issue(IsV{}, min(1, last));
   store_a(0);
   issue_a(min(2, last), min(2, last));
+  issue_seg(0);
+  store_seg(0);
+  issue_seg(min(1, last));
   splat(std::integral_constant<int, 0>{});
   splat(std::integral_constant<int, 1>{});
   lds_barrier();
@@ -697,6 +731,9 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     if (w < 4) {  // head factors: publish those of tile j+2, fetch those of tile j+3
       store_a((j + 1) & 1);
       issue_a(min(j + 3, last), min(j + 3, last));
+    } else {      // key segment ids: publish those of tile j+1, fetch those of tile j+2
+      store_seg((j + 1) & 1);
+      issue_seg(min(j + 2, last));
     }
     lds_barrier();
   };
@@ -705,6 +742,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     int first_masked = p.lk / kTK;                                   // ragged last tile
     if (p.causal) first_masked = min(first_masked, (wrow0 + 1) / kTK);  // first tile with a key past row wrow0
     hot_end = max(1, min(min(ntiles - 1, first_masked), wave_last_tile + 1));
+    if (has_seg) hot_end = 1;  // segment masks are applied by the plain iteration only
   }
   int j = 0;
   for (; j < 1; ++j) { cold_iteration(j); tail(j); }
@@ -758,7 +796,6 @@ bool factor_ok(const TpaFactor& f) {
 int tpa_prefill_mfma_supported(const TpaFwdArgs* a) {
   if (a->dtype != TPA_DTYPE_BF16) return 0;
   if (a->dk != a->dv || (a->dk != 64 && a->dk != 128)) return 0;
-  if (a->q_segment_ids || a->kv_segment_ids) return 0;
   if (!(a->sm_scale > 0.f)) return 0;
   if (!tpa::factor_ok(a->qb) || !tpa::factor_ok(a->kb) || !tpa::factor_ok(a->vb)) return 0;
   if (!tpa::aligned16(a->o)) return 0;
@@ -769,6 +806,7 @@ int tpa_prefill_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
   using namespace tpa;
   PrefillParams p{};
   p.qa = a->qa; p.qb = a->qb; p.ka = a->ka; p.kb = a->kb; p.va = a->va; p.vb = a->vb;
+  p.qseg = a->q_segment_ids; p.kvseg = a->kv_segment_ids;
   p.o = static_cast<uint16_t*>(a->o); p.lse = a->lse;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.rk = a->rk;
   p.sm_scale = a->sm_scale; p.causal = a->causal;

@@ -481,3 +481,29 @@ def test_prefill_reference_moves_on_unmasked_tiles(gpu, d, causal, where):
     (tq, tk, tv), o, lse = run_bf16(gpu, q, k, v, h, scale, causal)
     o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h, sm_scale=scale, causal=causal)
     check(o, lse, o_ref, l_ref, BF16_TOL, lse_tol=2e-3)
+
+
+# ---------------------------------------------------------------- packed sequences through the MFMA prefill kernel
+@pytest.mark.parametrize(
+    "b,lq,lk,h,d,rk,seg,causal",
+    [
+        (2, 512, 512, 4, 128, 2, 100, True),
+        (2, 640, 384, 2, 64, 2, 77, False),    # query rows whose segment has no key at all: NaN / -inf
+        (1, 1024, 1024, 2, 128, 2, 321, True),  # the segment size of tpa/tpa_test.py:72
+        (2, 300, 300, 8, 64, 4, 64, False),     # any-rank loader, segment = tile size
+        (1, 256, 1024, 2, 128, 2, 42, False),   # tpa/tpa_test.py:69-70 style: lq != lk
+    ],
+)
+def test_prefill_bf16_segment_ids(gpu, b, lq, lk, h, d, rk, seg, causal):
+    """Segment-id masks (tpa/tpa.py:369-375) in the bf16 MFMA kernel, requested explicitly (kernel=2)."""
+    from tpa import tpa
+
+    q, k, v = make_factors(51, b, lq, lk, h, d, d, 6, rk, scale_by_rank=True)
+    qseg, kvseg = segment_ids(lq, seg, b), segment_ids(lk, seg, b)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    tqs, tks = torch.from_numpy(qseg).to(gpu), torch.from_numpy(kvseg).to(gpu)
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), tqs, tks, d**-0.5, causal, 2)
+    o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), qseg, kvseg, h, sm_scale=d**-0.5, causal=causal)
+    check(o, lse, o_ref, l_ref, BF16_TOL)
+    if lq > lk:
+        assert np.isnan(o_ref).any()  # the case really has empty rows
