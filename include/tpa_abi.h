@@ -91,7 +91,7 @@ typedef struct TpaFwdArgs {
   float sm_scale; /* multiplies the logits after the dot product (tpa/tpa.py:367) */
   int32_t causal; /* non-zero: key index <= query index, top-left aligned (tpa/tpa.py:377-379) */
   int32_t kernel; /* TPA_KERNEL_* */
-  void* workspace;        /* tpa_decode only: scratch for split partials, else ignored */
+  void* workspace;        /* scratch for split partials: required by tpa_decode, optional for tpa_fwd */
   size_t workspace_bytes; /* size of workspace */
   int32_t num_splits;     /* tpa_decode only: 0 = choose; otherwise the number of key ranges */
 } TpaFwdArgs;
@@ -129,6 +129,9 @@ const char* tpa_strerror(int code);
 /*
  * Forward pass for any lq (prefill).  Replaces pl.pallas_call(..., name="tpa_fwd") at
  * tpa/tpa.py:492-543 for all batch entries at once (the reference vmaps it, tpa/tpa.py:144-163).
+ * If `workspace` holds at least tpa_decode_workspace_bytes(...) bytes and the problem is a
+ * decode (lq <= 16, lk >= 1024, no mask) that tpa_decode's kernel takes, the call is served by
+ * it; without a workspace the same problem runs on the prefill kernel.
  */
 int tpa_fwd(const TpaFwdArgs* args, void* stream);
 

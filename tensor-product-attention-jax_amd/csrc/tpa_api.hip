@@ -57,6 +57,12 @@ int tpa_fwd(const TpaFwdArgs* a, void* stream) {
   const int rc = validate_tpa(a);
   if (rc != TPA_OK) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  // few query tokens over a long cache (the reference's decode is this same call with lq = 1,
+  // tpa/tpa.py:485): split over keys, if the caller brought the workspace for it
+  if (a->kernel != TPA_KERNEL_GENERIC && a->workspace && a->lq <= 16 && a->lk >= 1024 && !a->causal &&
+      !a->q_segment_ids && tpa_decode_mfma_supported(a) &&
+      a->workspace_bytes >= tpa_decode_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dv, a->num_splits))
+    return tpa_decode_mfma_launch(a, s);
   if (a->kernel != TPA_KERNEL_GENERIC && tpa_prefill_mfma_supported(a)) return tpa_prefill_mfma_launch(a, s);
   if (a->kernel == TPA_KERNEL_MFMA) return TPA_ERR_UNSUPPORTED;
   return tpa_generic_launch(a, s);

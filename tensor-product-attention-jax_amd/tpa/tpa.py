@@ -123,6 +123,12 @@ def tpa_factors(
 
     o = torch.empty((b, lq, h, dv), dtype=dtype, device=device)
     lse = torch.empty((b, h, lq), dtype=torch.float32, device=device) if return_lse else None
+    lib = _d.load_library()
+    # decode through the reference's own entry point (lq = 1 over a long cache): hand the library
+    # the workspace its split-key kernel needs; it decides whether the problem qualifies
+    ws = None
+    if lq <= 16 and lk >= 1024 and not causal and qseg is None and dtype == torch.bfloat16 and kernel != _d.KERNEL_GENERIC:
+        ws = torch.empty(max(lib.tpa_decode_workspace_bytes(b, lq, lk, h, dv, 0), 16), dtype=torch.uint8, device=device)
     args = _d.TpaFwdArgs(
         qa=_d.factor(qa), qb=_d.factor(qb), ka=_d.factor(ka), kb=_d.factor(kb), va=_d.factor(va), vb=_d.factor(vb),
         q_segment_ids=qseg.data_ptr() if qseg is not None else None,
@@ -130,9 +136,8 @@ def tpa_factors(
         o=o.data_ptr(), lse=lse.data_ptr() if lse is not None else None,
         B=b, lq=lq, lk=lk, H=h, dk=dk, dv=dv, rq=rq, rk=rk,
         dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=int(bool(causal)), kernel=int(kernel),
-        workspace=None, workspace_bytes=0, num_splits=0,
+        workspace=ws.data_ptr() if ws is not None else None, workspace_bytes=ws.numel() if ws is not None else 0, num_splits=0,
     )
-    lib = _d.load_library()
     with torch.cuda.device(device):
         _d.check("tpa_fwd", lib.tpa_fwd(args, _d.current_stream_ptr(device)))
     return o, lse

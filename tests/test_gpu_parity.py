@@ -507,3 +507,19 @@ def test_prefill_bf16_segment_ids(gpu, b, lq, lk, h, d, rk, seg, causal):
     check(o, lse, o_ref, l_ref, BF16_TOL)
     if lq > lk:
         assert np.isnan(o_ref).any()  # the case really has empty rows
+
+
+def test_tpa_entry_point_serves_decode_with_the_split_key_kernel(gpu):
+    """tpa(q[b, 1, ...], k, v) - how the reference itself expresses decode - gives the result of
+    tpa_decode (bit for bit: it is the same kernel) and matches the oracle, reading the
+    concatenated cache in place."""
+    from tpa import tpa
+
+    b, lk, h, d = 3, 4096, 32, 128
+    q, k, v = make_factors(61, b, 1, lk, h, d, d, 6, 2, scale_by_rank=True)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    o = tpa.tpa(tq, tk, tv, num_heads=h, sm_scale=d**-0.5)
+    od, _ = tpa.tpa_decode(*tpa_split(tq, tk, tv, h), sm_scale=d**-0.5)
+    assert torch.equal(o, od)
+    o_ref, _ = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h, sm_scale=d**-0.5)
+    assert np.abs(as_f64(o) - o_ref).max() <= BF16_TOL
