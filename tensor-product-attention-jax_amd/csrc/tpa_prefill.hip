@@ -81,7 +81,7 @@ __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-template <int D, int LOADER>
+template <int D, int LOADER, bool SEG>
 __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   constexpr int NT = kNW * 64;
   constexpr int KS = Lds<D>::KS, VS = Lds<D>::VS;
@@ -261,16 +261,19 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   // Key segment ids (packed sequences, tpa/tpa.py:369-375): threads 256..319 fetch one id of a tile
   // each, park it in a register and store it into an LDS slot one iteration later, like the head
   // factors; slot j&1 holds the ids of tile j during iteration j.
-  const bool has_seg = p.kvseg != nullptr;
+  constexpr bool has_seg = SEG;  // a kernel of its own: the mask code slows the others down even when skipped
   int32_t seg_pending = 0;
   auto issue_seg = [&](int tile) __attribute__((always_inline)) {
-    if (has_seg && tid >= 4 * kTK && tid < 5 * kTK)
-      seg_pending = p.kvseg[(int64_t)b * p.lk + min(tile * kTK + tid - 4 * kTK, p.lk - 1)];
+    if constexpr (has_seg)
+      if (tid >= 4 * kTK && tid < 5 * kTK)
+        seg_pending = p.kvseg[(int64_t)b * p.lk + min(tile * kTK + tid - 4 * kTK, p.lk - 1)];
   };
   auto store_seg = [&](int slot_idx) __attribute__((always_inline)) {
-    if (has_seg && tid >= 4 * kTK && tid < 5 * kTK) lds_seg[slot_idx * kTK + tid - 4 * kTK] = seg_pending;
+    if constexpr (has_seg)
+      if (tid >= 4 * kTK && tid < 5 * kTK) lds_seg[slot_idx * kTK + tid - 4 * kTK] = seg_pending;
   };
-  const int32_t qseg = has_seg ? p.qseg[(int64_t)b * p.lq + qrow_ld] : 0;
+  int32_t qseg = 0;
+  if constexpr (has_seg) qseg = p.qseg[(int64_t)b * p.lq + qrow_ld];
 
   // (a0/2)*b0[d] + (a1/2)*b1[d] for 8 consecutive d; aa = packed (a0/2, a1/2): fetch_aa hands out
   // halved head factors.
@@ -431,7 +434,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
           if (t > limit) s[mb][v] = -INFINITY;
         }
     }
-    if (has_seg) {  // keys of another segment (tpa/tpa.py:369-375)
+    if constexpr (has_seg) {  // keys of another segment (tpa/tpa.py:369-375)
       const int32_t* slot = lds_seg + (tile & 1) * kTK;
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
@@ -670,8 +673,8 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
       const uint16_t* ks = lds_k + (j & 1) * Lds<D>::kK;
       const uint16_t* vs = lds_v + (j & 1) * Lds<D>::kV;
       // operands are read three MFMAs ahead here too (the V fragments of the first O^T steps
-      // while the softmax runs)
-      constexpr int LA = 3;
+      // while the softmax runs); not with the any-rank loader, whose kernel got slower with it
+      constexpr int LA = LOADER == LOAD_TPA_ANY ? 0 : 3;
       bf16x8 fr[N_MFMA];
       static_for<LA>([&](auto n_c) __attribute__((always_inline)) { fr[decltype(n_c)::value] = load_frag(n_c, ks, vs); });
       static_for<N_QK>([&](auto n_c) __attribute__((always_inline)) {
@@ -742,7 +745,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     int first_masked = p.lk / kTK;                                   // ragged last tile
     if (p.causal) first_masked = min(first_masked, (wrow0 + 1) / kTK);  // first tile with a key past row wrow0
     hot_end = max(1, min(min(ntiles - 1, first_masked), wave_last_tile + 1));
-    if (has_seg) hot_end = 1;  // segment masks are applied by the plain iteration only
+    if constexpr (has_seg) hot_end = 1;  // segment masks are applied by the plain iteration only
   }
   int j = 0;
   for (; j < 1; ++j) { cold_iteration(j); tail(j); }
@@ -769,9 +772,9 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   }
 }
 
-template <int D, int LOADER>
+template <int D, int LOADER, bool SEG = false>
 int launch_prefill(const PrefillParams& p, hipStream_t stream) {
-  auto kern = prefill_kernel<D, LOADER>;
+  auto kern = prefill_kernel<D, LOADER, SEG>;
   static bool configured = false;  // idempotent attribute; a race only repeats the same call
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)Lds<D>::kBytes) != hipSuccess)
@@ -812,6 +815,14 @@ int tpa_prefill_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
   p.sm_scale = a->sm_scale; p.causal = a->causal;
   p.nqb = (a->lq + kBQ - 1) / kBQ;
   p.npairs = p.nqb * a->B;
+  if (p.kvseg) {
+    if (a->dk == 128) {
+      if (a->rk == 2) return launch_prefill<128, LOAD_TPA_R2, true>(p, stream);
+      return launch_prefill<128, LOAD_TPA_ANY, true>(p, stream);
+    }
+    if (a->rk == 2) return launch_prefill<64, LOAD_TPA_R2, true>(p, stream);
+    return launch_prefill<64, LOAD_TPA_ANY, true>(p, stream);
+  }
   if (a->dk == 128) {
     if (a->rk == 2) return launch_prefill<128, LOAD_TPA_R2>(p, stream);
     return launch_prefill<128, LOAD_TPA_ANY>(p, stream);
