@@ -216,23 +216,30 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   const uint16_t* const ka_b = p.ka.ptr + b * p.ka.stride_b + h;
   const uint16_t* const va_b = p.va.ptr + b * p.va.stride_b + h;
 
-  // B-factor loads of one matrix (K or V) for one tile into registers
+  // B-factor loads of one matrix (K or V) for one tile into registers.  They are raw buffer
+  // loads: resource = this batch entry's matrix (in scalar registers), scalar offset = (tile,
+  // pass, rank), vector offset = this thread's fixed place inside a pass - no vector instruction
+  // is spent on addresses, and rows past the end of the sequence read as zero (the range check
+  // of the resource), so a ragged last tile needs no clamping.
+  constexpr int kRsrcFlags = 0x00020000;  // raw 32-bit data format
+  const int k_rows_bytes = ((p.lk - 1) * p.kb.stride_l + (LOADER == LOAD_TPA_R2 ? p.kb.stride_r : 0) + D) * 2;
+  const int v_rows_bytes = ((p.lk - 1) * p.vb.stride_l + (LOADER == LOAD_TPA_R2 ? p.vb.stride_r : 0) + D) * 2;
+  const __amdgpu_buffer_rsrc_t kb_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(kb_b), 0, k_rows_bytes, kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t vb_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(vb_b), 0, v_rows_bytes, kRsrcFlags);
+  const int kvoff = (lt * p.kb.stride_l + 8 * lc) * 2, vvoff = (lt * p.vb.stride_l + 8 * lc) * 2;
   auto issue = [&](auto is_v_c, int tile) __attribute__((always_inline)) {
     constexpr bool is_v = decltype(is_v_c)::value;
     if constexpr (LOADER == LOAD_TPA_ANY) return;
-    const uint16_t* b_base = is_v ? vb_b : kb_b;
     const int sl = is_v ? p.vb.stride_l : p.kb.stride_l, sr = is_v ? p.vb.stride_r : p.kb.stride_r;
 #pragma unroll
     for (int ps = 0; ps < NPASS; ++ps) {
-      const uint16_t* bt = b_base + (int64_t)(tile * kTK + ps * TPP) * sl;                   // uniform
-      const int tl = min(tile * kTK + ps * TPP + lt, p.lk - 1) - (tile * kTK + ps * TPP);   // clamp a ragged tail
-      const int boff = tl * sl + 8 * lc;
+      const int soff = (tile * kTK + ps * TPP) * sl * 2;  // uniform
       if constexpr (is_v) {
-        vreg[ps][0] = *reinterpret_cast<const u32x4*>(bt + boff);
-        if constexpr (LOADER == LOAD_TPA_R2) vreg[ps][1] = *reinterpret_cast<const u32x4*>(bt + sr + boff);
+        vreg[ps][0] = __builtin_amdgcn_raw_buffer_load_b128(vb_rs, vvoff, soff, 0);
+        if constexpr (LOADER == LOAD_TPA_R2) vreg[ps][1] = __builtin_amdgcn_raw_buffer_load_b128(vb_rs, vvoff, soff + 2 * sr, 0);
       } else {
-        kreg[ps][0] = *reinterpret_cast<const u32x4*>(bt + boff);
-        if constexpr (LOADER == LOAD_TPA_R2) kreg[ps][1] = *reinterpret_cast<const u32x4*>(bt + sr + boff);
+        kreg[ps][0] = __builtin_amdgcn_raw_buffer_load_b128(kb_rs, kvoff, soff, 0);
+        if constexpr (LOADER == LOAD_TPA_R2) kreg[ps][1] = __builtin_amdgcn_raw_buffer_load_b128(kb_rs, kvoff, soff + 2 * sr, 0);
       }
     }
   };
@@ -243,14 +250,17 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   // each, matrix = tid / 128 (0: K of tile kt, 1: V of tile vt), token = (tid / 2) % 64, rank = tid % 2,
   // and park it in a register until it is stored into an LDS slot one iteration later.
   uint32_t a_pending = 0;
+  const int a_mat = tid / (2 * kTK), a_tok = (tid >> 1) % kTK, a_rank = tid & 1;
+  const int ka_bytes = ((p.lk - 1) * p.ka.stride_l + p.ka.stride_r + 1) * 2, va_bytes = ((p.lk - 1) * p.va.stride_l + p.va.stride_r + 1) * 2;
+  const __amdgpu_buffer_rsrc_t ka_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(ka_b), 0, ka_bytes, kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t va_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(va_b), 0, va_bytes, kRsrcFlags);
+  const int ka_voff = (a_tok * p.ka.stride_l + a_rank * p.ka.stride_r) * 2, va_voff = (a_tok * p.va.stride_l + a_rank * p.va.stride_r) * 2;
   auto issue_a = [&](int kt, int vt) __attribute__((always_inline)) {
     if constexpr (LOADER != LOAD_TPA_R2) return;
     if (tid >= 4 * kTK) return;
-    const int mat = tid / (2 * kTK), tok_in = (tid >> 1) % kTK, rank = tid & 1;
-    const int tok = min((mat ? vt : kt) * kTK + tok_in, p.lk - 1);
-    const uint16_t* ap = mat ? va_b + (int64_t)tok * p.va.stride_l + rank * p.va.stride_r
-                             : ka_b + (int64_t)tok * p.ka.stride_l + rank * p.ka.stride_r;
-    a_pending = *ap;
+    // waves 0, 1 fetch K's head factors, waves 2, 3 V's (uniform per wave); tokens past the end read as 0
+    if (a_mat == 0) a_pending = __builtin_amdgcn_raw_buffer_load_b16(ka_rs, ka_voff, kt * kTK * p.ka.stride_l * 2, 0);
+    else a_pending = __builtin_amdgcn_raw_buffer_load_b16(va_rs, va_voff, vt * kTK * p.va.stride_l * 2, 0);
   };
   auto store_a = [&](int slot_idx) __attribute__((always_inline)) {
     if constexpr (LOADER != LOAD_TPA_R2) return;
