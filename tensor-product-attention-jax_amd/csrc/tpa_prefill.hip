@@ -425,6 +425,15 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     return __builtin_bit_cast(bf16x8, w4);
   };
   float mref = 0.f;     // reference (log2 domain, includes c) of row qrow
+  // -mref in all 16 registers of an accumulator tuple: the addend of the first S^T MFMA of a
+  // block, so the contraction lands on x*c - mref.  Rewritten only when the reference moves.
+  f32x16 nmref;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) nmref[v] = 0.f;
+  auto refresh_nmref = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) nmref[v] = -mref;
+  };
   float lsum = 0.f;     // this lane's share of sum exp2(x*c - mref)
   const int lp = l & 15, dhalf = (l >> 4) & 1;
 
@@ -471,6 +480,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
       const float delta = first ? tmax : (up ? tmax : 0.f);
       const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);
       mref += delta;
+      refresh_nmref();
       lsum *= alpha;
       if (__any(up)) {
 #pragma unroll
@@ -503,7 +513,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   // ---------------------------------------------------------------------------------------
   // Main loop.  Invariant at entry of iteration j: K tile j and V tile j are in LDS buffers j&1;
   // kreg / vreg hold the B factors of tile j+1; head-factor slot j&1 holds those of tile j+1 and
-  // a_pending (waves 0-3) those of tile j+2 (tile indices clamped to the last tile); s[] = -mref.
+  // a_pending (waves 0-3) those of tile j+2 (tile indices clamped to the last tile).
   // An iteration computes S^T = K Q^T, the softmax and O^T += V^T P^T of tile j, rebuilds tile
   // j+1 into the other buffers and refills the registers with tile j+2; one barrier ends it.
   constexpr int N_QK = 2 * NKS, N_PV = 4 * NDB, N_MFMA = N_QK + N_PV;
@@ -527,18 +537,13 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     constexpr int n = decltype(n_c)::value;
     if constexpr (n < N_QK) {
       constexpr int mb = n / NKS, kk = n % NKS;
-      s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, qf[kk], s[mb], 0, 0, 0);
+      if constexpr (kk == 0) s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, qf[kk], nmref, 0, 0, 0);
+      else s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, qf[kk], s[mb], 0, 0, 0);
     } else {
       constexpr int m = n - N_QK, kk = m / NDB, db = m % NDB;
       o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, pf_get(std::integral_constant<int, kk>{}), o[db], 0, 0, 0);
     }
   };
-  auto splat = [&](auto mb_c) __attribute__((always_inline)) {
-    constexpr int mb = decltype(mb_c)::value;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) s[mb][v] = -mref;
-  };
-
   // ---- pieces of the softmax of one 32-key block, for the interleaved (unmasked) path
   // Move the reference up where this block's row max left the slack (rare).  delta is a whole
   // number, so the scale factors are exact powers of two.  `pf_done` = number of already packed
@@ -548,6 +553,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     const float delta = tmax > 0.f ? __builtin_ceilf(tmax) : 0.f;
     const float alpha = __builtin_amdgcn_exp2f(-delta);
     mref += delta;
+    refresh_nmref();
     lsum *= alpha;
 #pragma unroll
     for (int db = 0; db < NDB; ++db)
@@ -593,7 +599,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   //   S^T block 0   | rebuild K tile j+1, refill kreg
   //   S^T block 1   | softmax of block 0
   //   O^T, keys 0-31  | softmax of block 1 (its max is taken before these MFMAs start)
-  //   O^T, keys 32-63 | rebuild V tile j+1, refill vreg, s[] = -mref for the next tile
+  //   O^T, keys 32-63 | rebuild V tile j+1, refill vreg
   // LDS operands are read LA steps ahead of the MFMA that consumes them.
   auto hot_iteration = [&](int j) __attribute__((always_inline)) {
     constexpr int LA = 2;
@@ -651,14 +657,13 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
           if constexpr (k * G3 / 4 == q) sm_exp(std::integral_constant<int, 1>{}, k_c);
         });
       } else {
-        constexpr int q = n - G1 - G2 - G3;  // items: NP rebuild pieces of V, refill vreg, two splats
-        constexpr int NI = NP + 3;
+        constexpr int q = n - G1 - G2 - G3;  // items: NP rebuild pieces of V, refill vreg
+        constexpr int NI = NP + 1;
         static_for<NI>([&](auto k_c) __attribute__((always_inline)) {
           constexpr int k = decltype(k_c)::value;
           if constexpr (k * G4 / NI == q) {
             if constexpr (k < NP) piece(IsV{}, k_c);
             else if constexpr (k == NP) issue(IsV{}, min(j + 2, last));
-            else splat(std::integral_constant<int, k - NP - 1>{});
           }
         });
       }
@@ -698,8 +703,6 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
         if constexpr (n + LA < N_MFMA) fr[n + LA] = load_frag(std::integral_constant<int, n + LA>{}, ks, vs);
         mfma_with(std::integral_constant<int, n>{}, fr[n]);
       });
-      splat(std::integral_constant<int, 0>{});
-      splat(std::integral_constant<int, 1>{});
     }
     if (j + 1 < ntiles) {
       const uint16_t* a_slot = LOADER == LOAD_TPA_R2 ? lds_a + (j & 1) * Lds<D>::kA : nullptr;
@@ -733,8 +736,6 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   issue_seg(0);
   store_seg(0);
   issue_seg(min(1, last));
-  splat(std::integral_constant<int, 0>{});
-  splat(std::integral_constant<int, 1>{});
   lds_barrier();
 
   // Per wave: tile 0 plain, then the run of unmasked tiles interleaved, then plain again (masked
@@ -801,6 +802,12 @@ bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15)
 bool factor_ok(const TpaFactor& f) {
   return aligned16(f.ptr) && f.stride_b % 8 == 0 && f.stride_l % 8 == 0 && f.stride_r % 8 == 0;
 }
+// one batch entry of a K/V-side array is addressed through a buffer resource with 32-bit byte
+// offsets: its extent must stay below 2 GiB and its strides must not be negative
+bool range_ok(const TpaFactor& f, int64_t tokens, int64_t ranks, int64_t width) {
+  if (f.stride_l < 0 || f.stride_r < 0) return false;
+  return ((tokens - 1) * f.stride_l + (ranks - 1) * f.stride_r + width) * 2 < (int64_t(1) << 31);
+}
 
 }  // namespace
 }  // namespace tpa
@@ -811,6 +818,9 @@ int tpa_prefill_mfma_supported(const TpaFwdArgs* a) {
   if (a->dk != a->dv || (a->dk != 64 && a->dk != 128)) return 0;
   if (!(a->sm_scale > 0.f)) return 0;
   if (!tpa::factor_ok(a->qb) || !tpa::factor_ok(a->kb) || !tpa::factor_ok(a->vb)) return 0;
+  if (!tpa::range_ok(a->kb, a->lk, a->rk, a->dk) || !tpa::range_ok(a->vb, a->lk, a->rk, a->dv) ||
+      !tpa::range_ok(a->ka, a->lk, a->rk, 1) || !tpa::range_ok(a->va, a->lk, a->rk, 1))
+    return 0;
   if (!tpa::aligned16(a->o)) return 0;
   return 1;
 }
@@ -847,6 +857,7 @@ int mha_prefill_mfma_supported(const MhaFwdArgs* a) {
   if (a->bias) return 0;
   if (!(a->sm_scale > 0.f)) return 0;
   if (!tpa::aligned16(a->q) || !tpa::aligned16(a->k) || !tpa::aligned16(a->v) || !tpa::aligned16(a->o)) return 0;
+  if ((int64_t)a->lk * a->H * (a->dk > a->dv ? a->dk : a->dv) * 2 >= (int64_t(1) << 31)) return 0;  // 32-bit buffer offsets per batch entry
   return 1;
 }
 
