@@ -310,15 +310,32 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(const float* part_o, co
   const int bq = blockIdx.x;  // b * lq + qi
   const int h = blockIdx.y;
   const int d = threadIdx.x;
-  float mmax = -INFINITY;
-  for (int s = 0; s < S; ++s) mmax = fmaxf(mmax, part_m[((int64_t)bq * S + s) * H + h]);
-  float acc = 0.f, lacc = 0.f;
-  for (int s = 0; s < S; ++s) {
-    const int64_t idx = ((int64_t)bq * S + s) * H + h;
-    const float ms = part_m[idx];
-    const float f = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - mmax);
-    acc += f * part_o[idx * D + d];
-    lacc += f * part_l[idx];
+  // ranges are taken eight at a time with all their loads in flight together (one round trip
+  // to memory for the usual S <= 8); a running (max, sum, acc) triple carries across groups
+  float mmax = -INFINITY, acc = 0.f, lacc = 0.f;
+  for (int s0 = 0; s0 < S; s0 += 8) {
+    float ms[8], ls[8], os[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int s = min(s0 + q, S - 1);
+      const int64_t idx = ((int64_t)bq * S + s) * H + h;
+      ms[q] = s0 + q < S ? part_m[idx] : -INFINITY;
+      ls[q] = part_l[idx];
+      os[q] = part_o[idx * D + d];
+    }
+    float gmax = mmax;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) gmax = fmaxf(gmax, ms[q]);
+    const float carry = mmax == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mmax - gmax);
+    acc *= carry;
+    lacc *= carry;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const float f = ms[q] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms[q] - gmax);
+      acc += f * os[q];
+      lacc += f * ls[q];
+    }
+    mmax = gmax;
   }
   store_from_f32(o + ((int64_t)bq * H + h) * D + d, acc * inv_rk / lacc);
   if (lse && d == 0) {
