@@ -523,3 +523,47 @@ def test_tpa_entry_point_serves_decode_with_the_split_key_kernel(gpu):
     assert torch.equal(o, od)
     o_ref, _ = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h, sm_scale=d**-0.5)
     assert np.abs(as_f64(o) - o_ref).max() <= BF16_TOL
+
+
+# ---------------------------------------------------------------- seeded random shapes
+@pytest.mark.parametrize("seed", range(16))
+def test_random_shapes_fp32_generic(gpu, seed):
+    """Small random problems (any head size, ragged lengths, masks on or off) on the fp32 path."""
+    from tpa import tpa
+
+    rng = np.random.default_rng(1000 + seed)
+    b, lq, lk = int(rng.integers(1, 4)), int(rng.integers(1, 260)), int(rng.integers(1, 260))
+    h, dk, dv = int(rng.integers(1, 6)), int(rng.integers(1, 41)), int(rng.integers(1, 41))
+    rq, rk = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+    causal = bool(rng.integers(0, 2))
+    seg = int(rng.integers(3, 60)) if rng.integers(0, 2) else None
+    scale = float(rng.uniform(0.1, 1.0))
+    q, k, v = make_factors(2000 + seed, b, lq, lk, h, dk, dv, rq, rk)
+    qseg = segment_ids(lq, seg, b) if seg else None
+    kvseg = segment_ids(lk, seg, b) if seg else None
+    o_ref, l_ref = orc.tpa_reference(q, k, v, qseg, kvseg, h, sm_scale=scale, causal=causal)
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    o, res = tpa._tpa_fwd(tq, tk, tv, h, qseg, kvseg, scale, causal, None, False, False, False)
+    check(o, res[-1].permute(0, 2, 1), o_ref, l_ref, F32_TOL)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_shapes_bf16_mfma(gpu, seed):
+    """Random problems the MFMA prefill kernel takes (kernel=2 makes a silent fallback an error)."""
+    from tpa import tpa
+
+    rng = np.random.default_rng(3000 + seed)
+    b, lq, lk = int(rng.integers(1, 4)), int(rng.integers(1, 900)), int(rng.integers(1, 900))
+    h, d = int(rng.integers(1, 5)) * 8, int(rng.choice([64, 128]))
+    rq, rk = int(rng.integers(1, 7)), int(rng.choice([1, 2, 2, 2, 3, 4]))
+    causal = bool(rng.integers(0, 2))
+    seg = int(rng.integers(20, 400)) if rng.integers(0, 3) == 0 else None
+    q, k, v = make_factors(4000 + seed, b, lq, lk, h, d, d, rq, rk, scale_by_rank=True)
+    qseg = segment_ids(lq, seg, b) if seg else None
+    kvseg = segment_ids(lk, seg, b) if seg else None
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    tqs = torch.from_numpy(qseg).to(gpu) if seg else None
+    tks = torch.from_numpy(kvseg).to(gpu) if seg else None
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), tqs, tks, d**-0.5, causal, 2)
+    o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), qseg, kvseg, h, sm_scale=d**-0.5, causal=causal)
+    check(o, lse, o_ref, l_ref, BF16_TOL)
