@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|copy] [--no-cpu] [--no-decode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|c2p|c3p|copy] [--no-cpu] [--no-decode]
 
 A step is one forward pass over one batch of synthetic, seeded inputs that are resident in HBM
 before the timed region starts.  The default workload is the prefill configuration the headline
@@ -32,6 +32,9 @@ WORKLOADS = {
     "c3": ("prefill", 1, 32768, 32768, 32, 128, 6, 2, True),
     "c5": ("prefill", 8, 2048, 2048, 64, 64, 16, 8, False),
     "c4": ("decode", 64, 1, 8192, 32, 128, 6, 2, False),
+    # packed sequences (segment ids, tpa/tpa.py:369-375): the c2 / c3 shapes holding documents of DOC_LEN tokens
+    "c2p": ("prefill", 4, 4096, 4096, 16, 128, 6, 2, True),
+    "c3p": ("prefill", 1, 32768, 32768, 32, 128, 6, 2, True),
 }
 COPY_BYTES = 1 << 30  # --workload copy: bytes read (and bytes written) by each plain copy launch
 
@@ -61,6 +64,9 @@ def make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed):
         draw((B, lk, rk, H), rk), draw((B, lk, rk, D), rk),
         draw((B, lk, rk, H), rk), draw((B, lk, rk, D), rk),
     )
+
+
+DOC_LEN = {"c2p": 1024, "c3p": 4096}
 
 
 def prefill_flops(B, lq, lk, H, D, causal):
@@ -98,16 +104,22 @@ def run_prefill(torch, tpa, device, name, steps, warmup):
     x = make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed=0)
     scale = D**-0.5
     out = {}
+    doc = DOC_LEN.get(name)
+    seg = None
+    if doc:
+        seg = (torch.arange(lq, device=device, dtype=torch.int32) // doc).repeat(B, 1).contiguous()
 
     def step(i):
-        out["o"], out["lse"] = tpa.tpa_factors(*x, sm_scale=scale, causal=causal, kernel=2)
+        out["o"], out["lse"] = tpa.tpa_factors(*x, seg, seg, sm_scale=scale, causal=causal, kernel=2)
 
     wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
-    fl = prefill_flops(B, lq, lk, H, D, causal)
+    # packed: only pairs inside a document count
+    fl = prefill_flops(B * (lq // doc), doc, doc, H, D, causal) if doc else prefill_flops(B, lq, lk, H, D, causal)
     return dict(
         wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, flops=fl,
         tflops_wall=fl / wall_ms / 1e9, tflops_kernel=fl / ev_ms / 1e9,
-        shape=dict(B=B, lq=lq, lk=lk, H=H, D=D, rank_q=rq, rank_k=rk, causal=causal), inputs=x, out=out,
+        shape=dict(B=B, lq=lq, lk=lk, H=H, D=D, rank_q=rq, rank_k=rk, causal=causal, **({"document_len": doc} if doc else {})),
+        inputs=x, out=out,
     )
 
 

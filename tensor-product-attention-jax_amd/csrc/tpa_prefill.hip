@@ -199,22 +199,83 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     }
   };
 
-  // ---- tile range
-  int ntiles = (p.lk + kTK - 1) / kTK;
-  if (p.causal) ntiles = min(ntiles, (min(q0 + kBQ, p.lq) + kTK - 1) / kTK);
+  // ---- key range [kpos0, kend) this workgroup visits; tiles are counted from kpos0
+  int kpos0 = 0;
+  int kend = p.causal ? min(p.lk, min(q0 + kBQ, p.lq)) : p.lk;
+  bool seg_pure = false;  // every visited key from the second tile on carries the rows' one segment id
+  if constexpr (SEG) {
+    // Packed sequences: a key can only be visible to this block if its id lies within the
+    // [min, max] of the block's query ids.  The workgroup scans the key ids once, keeps the first
+    // and the last such key, and visits only the tiles between them (exact for ids that do not
+    // decrease along the sequence; any other id pattern just visits more tiles, the mask itself
+    // is applied per key as before).  If the rows share one id and the keys with that id form one
+    // contiguous run, the tiles inside the run need no segment mask at all.
+    int32_t* const red = reinterpret_cast<int32_t*>(smem);
+    if (tid == 0) { red[0] = INT32_MAX; red[1] = INT32_MIN; red[2] = INT32_MAX; red[3] = -1; red[4] = 0; }
+    __syncthreads();
+    if (tid < kBQ && q0 + tid < p.lq) {
+      const int32_t sid = p.qseg[(int64_t)b * p.lq + q0 + tid];
+      __hip_atomic_fetch_min(&red[0], sid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_fetch_max(&red[1], sid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    __syncthreads();
+    const int32_t qmin = red[0], qmax = red[1];
+    int lo = INT32_MAX, hi = -1, cnt = 0;
+    auto visit = [&](int t, int32_t sid) __attribute__((always_inline)) {
+      if (sid >= qmin && sid <= qmax) { lo = min(lo, t); hi = max(hi, t); ++cnt; }
+    };
+    const int32_t* const kid = p.kvseg + (int64_t)b * p.lk;
+    // four ids per load and four loads in flight per thread where the row of ids is 16-byte aligned
+    const int kv4 = (reinterpret_cast<uintptr_t>(kid) & 15) == 0 ? (kend & ~3) : 0;
+    constexpr int U = 4;
+    for (int base = 4 * tid; base < kv4; base += 4 * NT * U) {
+      int4 ids[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int t = base + 4 * NT * u;
+        ids[u] = *reinterpret_cast<const int4*>(kid + (t < kv4 ? t : 0));
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int t = base + 4 * NT * u;
+        if (t < kv4) { visit(t, ids[u].x); visit(t + 1, ids[u].y); visit(t + 2, ids[u].z); visit(t + 3, ids[u].w); }
+      }
+    }
+    for (int t = kv4 + tid; t < kend; t += NT) visit(t, kid[t]);
+    if (cnt) {
+      __hip_atomic_fetch_min(&red[2], lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_fetch_max(&red[3], hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_fetch_add(&red[4], cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    __syncthreads();
+    lo = red[2]; hi = red[3]; cnt = red[4];
+    __syncthreads();  // the staging below reuses this memory
+    if (hi >= 0) {
+      kpos0 = lo / kTK * kTK;
+      kend = hi + 1;
+      seg_pure = qmin == qmax && cnt == hi - lo + 1;
+    } else {
+      kend = min(kend, kTK);  // nothing visible: one (fully masked) tile, the rows end as NaN / -inf
+    }
+  }
+  const int lk_r = kend - kpos0;          // keys counted from kpos0
+  const int wrow_r = wrow0 - kpos0;       // this wave's first row, and this lane's row, on that scale
+  const int qrow_r = qrow - kpos0;
+  const int ntiles = (lk_r + kTK - 1) / kTK;
   const int last = ntiles - 1;
   // last tile this wave needs under the causal mask (its rows: wrow0 .. wrow0 + 31)
-  const int wave_last_tile = p.causal ? min(last, (wrow0 + 31) / kTK) : last;
+  const int wave_last_tile = p.causal ? min(last, max(wrow_r + 31, 0) / kTK) : last;
 
   // ---- loader: this thread rebuilds chunk lc (8 elements) of token lt (+ TPP per pass).
   // Addresses are a uniform (scalar) tile base plus a per-thread 32-bit element offset.
   const int lt = tid / CPR, lc = tid % CPR;
   u32x4 kreg[NPASS][2], vreg[NPASS][2];  // LOAD_TPA_R2: two ranks; LOAD_DENSE: [0] only
 
-  const uint16_t* const kb_b = p.kb.ptr + b * p.kb.stride_b + (LOADER == LOAD_DENSE ? (int64_t)h * D : 0);
-  const uint16_t* const vb_b = p.vb.ptr + b * p.vb.stride_b + (LOADER == LOAD_DENSE ? (int64_t)h * D : 0);
-  const uint16_t* const ka_b = p.ka.ptr + b * p.ka.stride_b + h;
-  const uint16_t* const va_b = p.va.ptr + b * p.va.stride_b + h;
+  // all key-side bases point at key kpos0
+  const uint16_t* const kb_b = p.kb.ptr + b * p.kb.stride_b + (int64_t)kpos0 * p.kb.stride_l + (LOADER == LOAD_DENSE ? (int64_t)h * D : 0);
+  const uint16_t* const vb_b = p.vb.ptr + b * p.vb.stride_b + (int64_t)kpos0 * p.vb.stride_l + (LOADER == LOAD_DENSE ? (int64_t)h * D : 0);
+  const uint16_t* const ka_b = p.ka.ptr + b * p.ka.stride_b + (int64_t)kpos0 * p.ka.stride_l + h;
+  const uint16_t* const va_b = p.va.ptr + b * p.va.stride_b + (int64_t)kpos0 * p.va.stride_l + h;
 
   // B-factor loads of one matrix (K or V) for one tile into registers.  They are raw buffer
   // loads: resource = this batch entry's matrix (in scalar registers), scalar offset = (tile,
@@ -222,8 +283,8 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   // is spent on addresses, and rows past the end of the sequence read as zero (the range check
   // of the resource), so a ragged last tile needs no clamping.
   constexpr int kRsrcFlags = 0x00020000;  // raw 32-bit data format
-  const int k_rows_bytes = ((p.lk - 1) * p.kb.stride_l + (LOADER == LOAD_TPA_R2 ? p.kb.stride_r : 0) + D) * 2;
-  const int v_rows_bytes = ((p.lk - 1) * p.vb.stride_l + (LOADER == LOAD_TPA_R2 ? p.vb.stride_r : 0) + D) * 2;
+  const int k_rows_bytes = ((lk_r - 1) * p.kb.stride_l + (LOADER == LOAD_TPA_R2 ? p.kb.stride_r : 0) + D) * 2;
+  const int v_rows_bytes = ((lk_r - 1) * p.vb.stride_l + (LOADER == LOAD_TPA_R2 ? p.vb.stride_r : 0) + D) * 2;
   const __amdgpu_buffer_rsrc_t kb_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(kb_b), 0, k_rows_bytes, kRsrcFlags);
   const __amdgpu_buffer_rsrc_t vb_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(vb_b), 0, v_rows_bytes, kRsrcFlags);
   const int kvoff = (lt * p.kb.stride_l + 8 * lc) * 2, vvoff = (lt * p.vb.stride_l + 8 * lc) * 2;
@@ -251,7 +312,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   // and park it in a register until it is stored into an LDS slot one iteration later.
   uint32_t a_pending = 0;
   const int a_mat = tid / (2 * kTK), a_tok = (tid >> 1) % kTK, a_rank = tid & 1;
-  const int ka_bytes = ((p.lk - 1) * p.ka.stride_l + p.ka.stride_r + 1) * 2, va_bytes = ((p.lk - 1) * p.va.stride_l + p.va.stride_r + 1) * 2;
+  const int ka_bytes = ((lk_r - 1) * p.ka.stride_l + p.ka.stride_r + 1) * 2, va_bytes = ((lk_r - 1) * p.va.stride_l + p.va.stride_r + 1) * 2;
   const __amdgpu_buffer_rsrc_t ka_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(ka_b), 0, ka_bytes, kRsrcFlags);
   const __amdgpu_buffer_rsrc_t va_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(va_b), 0, va_bytes, kRsrcFlags);
   const int ka_voff = (a_tok * p.ka.stride_l + a_rank * p.ka.stride_r) * 2, va_voff = (a_tok * p.va.stride_l + a_rank * p.va.stride_r) * 2;
@@ -276,7 +337,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   auto issue_seg = [&](int tile) __attribute__((always_inline)) {
     if constexpr (has_seg)
       if (tid >= 4 * kTK && tid < 5 * kTK)
-        seg_pending = p.kvseg[(int64_t)b * p.lk + min(tile * kTK + tid - 4 * kTK, p.lk - 1)];
+        seg_pending = p.kvseg[(int64_t)b * p.lk + kpos0 + min(tile * kTK + tid - 4 * kTK, lk_r - 1)];
   };
   auto store_seg = [&](int slot_idx) __attribute__((always_inline)) {
     if constexpr (has_seg)
@@ -374,7 +435,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
       if (a_slot) {
         aa[ps] = *reinterpret_cast<const uint32_t*>(a_slot + (is_v ? 2 * kTK : 0) + 2 * t);
       } else {
-        const int tok = min(tile * kTK + t, p.lk - 1);
+        const int tok = min(tile * kTK + t, lk_r - 1);
         const uint32_t a0 = ab[(int64_t)tok * a_sl], a1 = ab[(int64_t)tok * a_sl + a_sr];
         aa[ps] = halve_pair(a0 | (a1 << 16));
       }
@@ -398,7 +459,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
         if constexpr (is_v) val = rebuild_r2(vreg[ps][0], vreg[ps][1], aa[ps]);
         else val = rebuild_r2(kreg[ps][0], kreg[ps][1], aa[ps]);
       } else if constexpr (LOADER == LOAD_TPA_ANY) {
-        const int tok = min(tile * kTK + t, p.lk - 1);
+        const int tok = min(tile * kTK + t, lk_r - 1);
         val = rebuild_any(bb + (int64_t)tok * b_sl + 8 * lc, ab + (int64_t)tok * a_sl, b_sr, a_sr);
       } else {
         if constexpr (is_v) val = vreg[ps][0]; else val = kreg[ps][0];
@@ -442,9 +503,9 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   auto do_softmax = [&](int tile) __attribute__((always_inline)) {
     const int k0 = tile * kTK;
     // keys beyond lk, and keys after the query under the causal mask
-    const bool need_mask = (k0 + kTK > p.lk) || (p.causal && (k0 + kTK - 1 > wrow0));
+    const bool need_mask = (k0 + kTK > lk_r) || (p.causal && (k0 + kTK - 1 > wrow_r));
     if (need_mask) {
-      const int limit = p.causal ? min(qrow, p.lk - 1) : p.lk - 1;  // largest visible key index
+      const int limit = p.causal ? min(qrow_r, lk_r - 1) : lk_r - 1;  // largest visible key index
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
@@ -753,10 +814,12 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   };
   int hot_end = 1;
   if constexpr (LOADER != LOAD_TPA_ANY) {
-    int first_masked = p.lk / kTK;                                   // ragged last tile
-    if (p.causal) first_masked = min(first_masked, (wrow0 + 1) / kTK);  // first tile with a key past row wrow0
+    int first_masked = lk_r / kTK;                                   // ragged last tile
+    if (p.causal) first_masked = min(first_masked, max(wrow_r + 1, 0) / kTK);  // first tile with a key past row wrow0
     hot_end = max(1, min(min(ntiles - 1, first_masked), wave_last_tile + 1));
-    if constexpr (has_seg) hot_end = 1;  // segment masks are applied by the plain iteration only
+    // segment masks are applied by the plain iteration only: the interleaved one runs where no
+    // key of another segment can turn up (tile 0, which may start before the run, is plain anyway)
+    if constexpr (has_seg) if (!seg_pure) hot_end = 1;
   }
   int j = 0;
   for (; j < 1; ++j) { cold_iteration(j); tail(j); }

@@ -567,3 +567,71 @@ def test_random_shapes_bf16_mfma(gpu, seed):
     o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), tqs, tks, d**-0.5, causal, 2)
     o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), qseg, kvseg, h, sm_scale=d**-0.5, causal=causal)
     check(o, lse, o_ref, l_ref, BF16_TOL)
+
+
+def _id_pattern(name, b, lq, lk):
+    """Query and key segment ids [b, l] for the named layout (int32)."""
+    rng = np.random.default_rng(77)
+    qs, ks = np.zeros((b, lq), np.int32), np.zeros((b, lk), np.int32)
+    for i in range(b):
+        if name == "long_runs":  # packed documents, boundaries differ per batch entry
+            cuts = [0, 700 + 37 * i, 1500 - 11 * i, max(lq, lk)]
+            for s, (lo, hi) in enumerate(zip(cuts[:-1], cuts[1:])):
+                qs[i, lo:hi] = s
+                ks[i, lo:hi] = s
+        elif name == "shuffled":  # ids in no order at all
+            qs[i] = rng.integers(0, 3, lq)
+            ks[i] = rng.integers(0, 3, lk)
+        elif name == "island":  # all rows see one contiguous run of keys in the middle
+            qs[i] = 7
+            ks[i] = 3
+            ks[i, 300 + 5 * i : 1100] = 7
+        elif name == "island_with_hole":
+            qs[i] = 7
+            ks[i] = 3
+            ks[i, 300:1100] = 7
+            ks[i, 600:611] = 9
+        elif name == "absent":  # no key carries the rows' id
+            qs[i] = 5
+            ks[i] = 1
+        elif name == "descending":
+            qs[i] = (lq - 1 - np.arange(lq)) // 400
+            ks[i] = (lk - 1 - np.arange(lk)) // 400
+        else:
+            raise ValueError(name)
+    return qs, ks
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("pattern", ["long_runs", "shuffled", "island", "island_with_hole", "absent", "descending"])
+def test_prefill_bf16_segment_id_patterns(gpu, pattern, causal):
+    """The MFMA kernel visits only the key tiles between the first and the last key whose id lies in
+    the range of a block's query ids, and drops the per-key mask inside a run of one id: the result
+    must not depend on how the ids are laid out (tpa/tpa.py:369-375 compares ids pairwise)."""
+    from tpa import tpa
+
+    b, lq, lk, h, d = 2, 1536, 1536, 8, 128
+    q, k, v = make_factors(71, b, lq, lk, h, d, d, 6, 2, scale_by_rank=True)
+    qseg, kvseg = _id_pattern(pattern, b, lq, lk)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    tqs, tks = torch.from_numpy(qseg).to(gpu), torch.from_numpy(kvseg).to(gpu)
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), tqs, tks, d**-0.5, causal, 2)
+    o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), qseg, kvseg, h, sm_scale=d**-0.5, causal=causal)
+    check(o, lse, o_ref, l_ref, BF16_TOL)
+    if pattern == "absent":
+        assert np.isnan(o_ref).all()
+
+
+@pytest.mark.parametrize("d,rk", [(64, 2), (128, 3)])
+def test_prefill_bf16_segment_runs_other_instances(gpu, d, rk):
+    """Packed documents through the D = 64 kernel and through the any-rank loader, lq != lk."""
+    from tpa import tpa
+
+    b, lq, lk, h = 2, 900, 1301, 8
+    q, k, v = make_factors(72, b, lq, lk, h, d, d, 4, rk, scale_by_rank=True)
+    qseg, kvseg = _id_pattern("long_runs", b, lq, lk)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    tqs, tks = torch.from_numpy(qseg).to(gpu), torch.from_numpy(kvseg).to(gpu)
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), tqs, tks, d**-0.5, True, 2)
+    o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), qseg, kvseg, h, sm_scale=d**-0.5, causal=True)
+    check(o, lse, o_ref, l_ref, BF16_TOL)
