@@ -17,6 +17,18 @@ What follows what (reference file:line):
 The reference returns LSE as l[b, lq, h] (tpa/tpa.py:255,443); this oracle returns it in that
 layout too (`lse_blh`); callers transpose when they compare with the kernels' [b, h, lq].
 
+Backward (the gradients of the same functions):
+  * `mha_backward`       - tpa/mha.py:40-65       (p with NaN -> 0, dv = p^T do, dp = do v^T,
+                                                   dx = scale * p * (dp - sum(dp * p)), dq = dx k, dk = dx^T q)
+  * `project_to_factors` - tpa/tpa.py:781-783,793-799 (da = dX . b / R, db = dX . a / R, the chain rule
+                                                   through X = (1/R) sum_r a_r (x) b_r)
+  * `tpa_backward`       - tpa/tpa.py:168-214,546-962 (what `_tpa_bwd` returns: dq, dk, dv in the
+                                                   concatenated factor layout; rows without a visible key
+                                                   contribute nothing, tpa/tpa.py:675-676,979)
+  pinned by tests/test_oracle.py against torch autograd (float64, CPU) of an independently written
+  dense attention, central finite differences on a tiny case, and the literal gradients the
+  reference holds (tpa/mha_test.py:87-118: dq = dk = 0, dv = [[1,1],[0,0],[1,1]]).
+
 How this oracle is pinned (tests/test_oracle.py): brute-force float64 loops on tiny shapes,
 torch's scaled_dot_product_attention and scipy's softmax/logsumexp as independent library
 routines, closed forms (zero queries -> running mean of V and LSE = ln(count); lk = 1), rank
@@ -39,6 +51,9 @@ __all__ = [
     "tpa_reference_rows",
     "lse",
     "lse_accum",
+    "mha_backward",
+    "project_to_factors",
+    "tpa_backward",
 ]
 
 
@@ -158,3 +173,64 @@ def tpa_reference_rows(
         keep = rows[:, None] >= np.arange(lk)[None, :]
         bias = bias + np.where(keep, 0.0, -np.inf)[None]
     return mha_forward(q_, k_, v_, bias=bias, sm_scale=sm_scale)
+
+
+def mha_backward(q, k, v, bias, sm_scale, do):
+    """Gradients of dense attention, tpa/mha.py:40-65.
+
+    q[b,lq,h,dk] k[b,lk,h,dk] v[b,lk,h,dv] bias[b,lq,lk]|None do[b,lq,h,dv] -> (dq, dk, dv), same
+    shapes as q, k, v.  The softmax is recomputed; rows whose logits are all -inf have p = 0
+    (tpa/mha.py:55) and so contribute nothing.
+    """
+    qt = np.transpose(q, (0, 2, 1, 3))   # b h lq dk
+    kt = np.transpose(k, (0, 2, 1, 3))   # b h lk dk
+    vt = np.transpose(v, (0, 2, 1, 3))   # b h lk dv
+    dot = np.transpose(do, (0, 2, 1, 3))  # b h lq dv
+    x = sm_scale * np.matmul(qt, np.swapaxes(kt, 2, 3))
+    if bias is not None:
+        x = x + bias[:, None, :, :]
+    m = np.max(x, axis=-1, keepdims=True)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        e = np.exp(x - m)
+        p = e / np.sum(e, axis=-1, keepdims=True)
+    p = np.where(np.isnan(p), 0.0, p)
+    dot = np.where(np.isnan(dot), 0.0, dot)
+    dv = np.matmul(np.swapaxes(p, 2, 3), dot)                # b h lk dv
+    dp = np.matmul(dot, np.swapaxes(vt, 2, 3))               # b h lq lk
+    dx = sm_scale * p * (dp - np.sum(dp * p, axis=-1, keepdims=True))
+    dq = np.matmul(dx, kt)                                   # b h lq dk
+    dk = np.matmul(np.swapaxes(dx, 2, 3), qt)                # b h lk dk
+    back = lambda t: np.transpose(t, (0, 2, 1, 3))
+    return back(dq), back(dk), back(dv)
+
+
+def project_to_factors(dx, a, b):
+    """Chain rule through X = (1/R) sum_r a[b,l,r,h] b[b,l,r,d]: dX[b,l,h,d] -> (da, db).
+
+    da[b,l,r,h] = (1/R) sum_d dX[b,l,h,d] b[b,l,r,d];  db[b,l,r,d] = (1/R) sum_h dX[b,l,h,d] a[b,l,r,h]
+    (tpa/tpa.py:781-783 for q, 793-799 for k).
+    """
+    rank = a.shape[2]
+    da = np.matmul(b, np.swapaxes(dx, 2, 3)) / rank   # [r, d] x [d, h] per token
+    db = np.matmul(a, dx) / rank                       # [r, h] x [h, d] per token
+    return da, db
+
+
+def tpa_backward(q, k, v, q_segment_ids, kv_segment_ids, num_heads, do, sm_scale=1.0, causal=False, dtype=np.float64):
+    """What the reference's `_tpa_bwd` returns (tpa/tpa.py:168-214): (dq, dk, dv) in the layout of q, k, v.
+
+    q[b,lq,rq,h+dk] k[b,lk,rk,h+dk] v[b,lk,rk,h+dv] do[b,lq,h,dv].
+    """
+    q = np.asarray(q, dtype=dtype)
+    k = np.asarray(k, dtype=dtype)
+    v = np.asarray(v, dtype=dtype)
+    do = np.asarray(do, dtype=dtype)
+    qa, qb = split_factors(q, num_heads)
+    ka, kb = split_factors(k, num_heads)
+    va, vb = split_factors(v, num_heads)
+    b, lq = qa.shape[:2]
+    lk = ka.shape[1]
+    bias = attention_bias(b, lq, lk, q_segment_ids, kv_segment_ids, causal, dtype=dtype)
+    dq_, dk_, dv_ = mha_backward(reconstruct(qa, qb), reconstruct(ka, kb), reconstruct(va, vb), bias, sm_scale, do)
+    cat = lambda pair: np.concatenate(pair, axis=-1)
+    return cat(project_to_factors(dq_, qa, qb)), cat(project_to_factors(dk_, ka, kb)), cat(project_to_factors(dv_, va, vb))

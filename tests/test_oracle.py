@@ -215,3 +215,91 @@ def test_lse_helpers():
     assert np.isneginf(orc.lse(np.full((4, 3), -np.inf))).all()
     assert np.isneginf(orc.lse_accum(ninf, ninf)).all()
     np.testing.assert_allclose(orc.lse_accum(ninf, x[:, 0]), x[:, 0])
+
+
+# ---------------------------------------------------------------- backward
+def torch_tpa_loss(q, k, v, qseg, kvseg, h, sm_scale, causal, do):
+    """An independently written dense attention in torch (float64), differentiated by autograd:
+    sum(nan_to_zero(o) * do), the scalar whose gradient `_tpa_bwd` returns (tpa/tpa_test.py:170-197
+    uses nansum(o), i.e. do = 1)."""
+    tq, tk, tv = (torch.tensor(x, dtype=torch.float64, requires_grad=True) for x in (q, k, v))
+    rec = lambda t: torch.einsum("blrh,blrd->blhd", t[..., :h], t[..., h:]) / t.shape[2]
+    Q, K, V = rec(tq), rec(tk), rec(tv)
+    x = sm_scale * torch.einsum("bqhd,bkhd->bhqk", Q, K)
+    lq, lk = q.shape[1], k.shape[1]
+    keep = torch.ones((q.shape[0], lq, lk), dtype=torch.bool)
+    if qseg is not None:
+        keep &= torch.tensor(qseg)[:, :, None] == torch.tensor(kvseg)[:, None, :]
+    if causal:
+        keep &= torch.arange(lq)[:, None] >= torch.arange(lk)[None, :]
+    live = keep.any(-1)  # rows with at least one visible key
+    x = x.masked_fill(~keep[:, None], -1e300)  # finite, so autograd never meets inf - inf
+    p = torch.softmax(x, dim=-1) * keep[:, None]
+    o = torch.einsum("bhqk,bkhd->bqhd", p, V) * live[:, :, None, None]
+    loss = (o * torch.tensor(do, dtype=torch.float64)).sum()
+    loss.backward()
+    return tq.grad.numpy(), tk.grad.numpy(), tv.grad.numpy()
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("seg", [None, 5])
+@pytest.mark.parametrize("lq,lk", [(24, 24), (30, 12)])  # (30, 12) with seg = 5: rows whose segment has no key
+def test_backward_against_torch_autograd(causal, seg, lq, lk):
+    b, h, dk, dv, rq, rk = 2, 3, 7, 5, 4, 2
+    q, k, v = make_factors(11, b, lq, lk, h, dk, dv, rq, rk)
+    rng = np.random.default_rng(5)
+    do = rng.standard_normal((b, lq, h, dv))
+    qseg = segment_ids(lq, seg, b) if seg else None
+    kvseg = segment_ids(lk, seg, b) if seg else None
+    got = orc.tpa_backward(q, k, v, qseg, kvseg, h, do, sm_scale=0.4, causal=causal)
+    want = torch_tpa_loss(q, k, v, qseg, kvseg, h, 0.4, causal, do)
+    for g, w in zip(got, want):
+        np.testing.assert_allclose(g, w, rtol=1e-9, atol=1e-11)
+
+
+def test_backward_against_finite_differences():
+    """Central differences of sum(o * do) on the forward oracle, every input element of a tiny case."""
+    b, lq, lk, h, dk, dv, rq, rk = 1, 4, 5, 2, 3, 2, 2, 3
+    q, k, v = (x.astype(np.float64) for x in make_factors(12, b, lq, lk, h, dk, dv, rq, rk))
+    do = np.random.default_rng(6).standard_normal((b, lq, h, dv))
+    f = lambda q_, k_, v_: float(np.sum(orc.tpa_reference(q_, k_, v_, None, None, h, sm_scale=0.7, causal=True)[0] * do))
+    grads = orc.tpa_backward(q, k, v, None, None, h, do, sm_scale=0.7, causal=True)
+    eps = 1e-6
+    for which, (x, g) in enumerate(zip((q, k, v), grads)):
+        num = np.zeros_like(x)
+        for idx in np.ndindex(*x.shape):
+            args = [q.copy(), k.copy(), v.copy()]
+            args[which][idx] += eps
+            up = f(*args)
+            args[which][idx] -= 2 * eps
+            num[idx] = (up - f(*args)) / (2 * eps)
+        np.testing.assert_allclose(g, num, rtol=1e-6, atol=1e-8)
+
+
+def test_backward_known_answer_from_reference_mha_test():
+    """tpa/mha_test.py:87-118 (commented out upstream): gradients of nansum(o) on the literal case."""
+    q = np.array([[2, 1], [1, 1], [1, 1]], dtype=float)[None, :, None, :]
+    k = np.ones((3, 2))[None, :, None, :]
+    v = np.ones((3, 2))[None, :, None, :]
+    ninf = -np.inf
+    bias = np.array([[0, ninf, 0], [0, ninf, 0], [ninf, ninf, ninf]])[None]
+    dq, dk, dv = orc.mha_backward(q, k, v, bias, 1.0, np.ones((1, 3, 1, 2)))
+    np.testing.assert_allclose(dq, np.zeros_like(q), atol=1e-15)
+    np.testing.assert_allclose(dk, np.zeros_like(k), atol=1e-15)
+    np.testing.assert_allclose(dv[0, :, 0], [[1, 1], [0, 0], [1, 1]], atol=1e-15)
+
+
+def test_mha_backward_with_finite_bias_against_autograd():
+    """tpa/mha_test.py:9-41: dense attention with a random additive bias."""
+    b, lq, lk, h, dk, dv = 2, 4, 6, 3, 8, 8
+    rng = np.random.default_rng(7)
+    q, k, v = rng.standard_normal((b, lq, h, dk)), rng.standard_normal((b, lk, h, dk)), rng.standard_normal((b, lk, h, dv))
+    bias, do = rng.standard_normal((b, lq, lk)), rng.standard_normal((b, lq, h, dv))
+    for scale in (0.5, 1.0, 2.0):
+        tq, tk, tv = (torch.tensor(x, requires_grad=True) for x in (q, k, v))
+        x = scale * torch.einsum("bqhd,bkhd->bhqk", tq, tk) + torch.tensor(bias)[:, None]
+        o = torch.einsum("bhqk,bkhd->bqhd", torch.softmax(x, -1), tv)
+        (o * torch.tensor(do)).sum().backward()
+        got = orc.mha_backward(q, k, v, bias, scale, do)
+        for g, w in zip(got, (tq.grad, tk.grad, tv.grad)):
+            np.testing.assert_allclose(g, w.numpy(), rtol=1e-10, atol=1e-12)
