@@ -1,6 +1,7 @@
 /*
- * C ABI of libtpa_gfx950.so: Tensor Product Attention forward (prefill + decode) and a
- * same-shape dense multi-head flash attention, as hand-written HIP kernels for gfx950.
+ * C ABI of libtpa_gfx950.so: Tensor Product Attention forward (prefill + decode), a
+ * same-shape dense multi-head flash attention, and the backward pass of both, as hand-written
+ * HIP kernels for gfx950.
  *
  * The reference has no native ABI.  Its operator boundary for this path is the Pallas call
  *   pl.pallas_call(_fwd_kernel, ...)(qa, qb, ka, kb, va, vb, q_segment_ids, kv_segment_ids) -> [o, l]
@@ -27,7 +28,7 @@
 extern "C" {
 #endif
 
-#define TPA_ABI_VERSION 1
+#define TPA_ABI_VERSION 2
 
 /* element types of the factor / output arrays */
 enum { TPA_DTYPE_F32 = 0, TPA_DTYPE_BF16 = 1 };
@@ -120,6 +121,72 @@ typedef struct MhaFwdArgs {
   int32_t num_splits;
 } MhaFwdArgs;
 
+/*
+ * One gradient array, fp32 whatever the element type of the inputs is: same indexing as the
+ * TpaFactor it is the gradient of (innermost dimension contiguous, ELEMENT strides), so the
+ * concatenated dq[b, lq, rq, h+dk] that _tpa_bwd returns (tpa/tpa.py:960-962) is written in place
+ * (A part = base, B part = base + h, rank stride h+dk).
+ */
+typedef struct TpaGrad {
+  float* ptr;
+  int64_t stride_b;
+  int64_t stride_l;
+  int64_t stride_r;
+} TpaGrad;
+
+/*
+ * tpa_bwd arguments.  Replaces the operand list of pl.pallas_call(_bwd_kernel, ..., name="tpa_bwd")
+ * at tpa/tpa.py:872-958 together with _precompute_delta (tpa/tpa.py:965-995), for all batch
+ * entries at once (the reference vmaps _bwd, tpa/tpa.py:191-213).  With x, p as in the forward pass:
+ *   delta = sum_d o * do (NaN products skipped)                        (tpa/tpa.py:979)
+ *   p = exp(x - lse), 0 where masked or where the row has no visible key  (tpa/tpa.py:675-676)
+ *   dV = p^T do ; dp = do V^T ; ds = sm_scale * p * (dp - delta)       (tpa/tpa.py:765-773)
+ *   dK = ds^T Q ; dQ = ds K                                            (tpa/tpa.py:775-781)
+ *   da_r = (1/R) dX . b_r ; db_r = (1/R) a_r . dX  for X in {Q, K, V}  (tpa/tpa.py:767-768,776-777,782-783)
+ * Every element of the six gradient arrays is written (no accumulation into their old contents).
+ */
+typedef struct TpaBwdArgs {
+  TpaFactor qa, qb, ka, kb, va, vb;  /* the forward inputs, as in TpaFwdArgs */
+  const int32_t* q_segment_ids;      /* [B, lq] or NULL */
+  const int32_t* kv_segment_ids;     /* [B, lk] or NULL */
+  const void* o;     /* [B, lq, H, dv] forward output, element type = dtype */
+  const float* lse;  /* [B, H, lq] forward logsumexp (fp32) */
+  const void* d_o;   /* [B, lq, H, dv] gradient of the loss with respect to o, element type = dtype */
+  TpaGrad dqa, dqb, dka, dkb, dva, dvb; /* outputs, fp32 */
+  int32_t B, lq, lk, H, dk, dv, rq, rk;
+  int32_t dtype;
+  float sm_scale;
+  int32_t causal;
+  int32_t kernel;         /* TPA_KERNEL_AUTO or TPA_KERNEL_GENERIC (no MFMA backward kernel yet) */
+  void* workspace;        /* required: at least tpa_bwd_workspace_bytes(...) bytes, 256-byte aligned */
+  size_t workspace_bytes;
+} TpaBwdArgs;
+
+/*
+ * mha_bwd arguments: gradients of dense attention, _mha_bwd at tpa/mha.py:40-65, recomputing p
+ * from (q, k, lse) instead of keeping the [b, h, lq, lk] matrix the reference saves
+ * (tpa/mha.py:37).  dq, dk_out, dv_out are fp32, contiguous, with the shapes of q, k, v.
+ */
+typedef struct MhaBwdArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  const float* bias; /* [B, lq, lk] fp32 additive or NULL; no gradient is produced for it (tpa/mha.py:64) */
+  const void* o;
+  const float* lse;
+  const void* d_o;
+  float* dq;
+  float* dk_out;
+  float* dv_out;
+  int32_t B, lq, lk, H, dk, dv;
+  int32_t dtype;
+  float sm_scale;
+  int32_t causal;
+  int32_t kernel;
+  void* workspace;        /* required: at least mha_bwd_workspace_bytes(...) bytes, 256-byte aligned */
+  size_t workspace_bytes;
+} MhaBwdArgs;
+
 /* ABI version of the loaded library (TPA_ABI_VERSION it was built with). */
 int tpa_abi_version(void);
 
@@ -155,6 +222,21 @@ int mha_fwd(const MhaFwdArgs* args, void* stream);
 
 /* Bytes of workspace mha_fwd needs (0 unless lq is small enough for the split-key kernel). */
 size_t mha_fwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dv, int32_t num_splits);
+
+/*
+ * Backward pass of tpa_fwd: gradients with respect to the six factor arrays.  Replaces _bwd /
+ * _tpa_bwd (tpa/tpa.py:168-214,823-962).  Needs the forward's o and lse.
+ */
+int tpa_bwd(const TpaBwdArgs* args, void* stream);
+
+/* Bytes of workspace tpa_bwd needs (dense Q, K, V, their gradients and delta, all fp32). */
+size_t tpa_bwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dk, int32_t dv);
+
+/* Backward pass of mha_fwd (tpa/mha.py:40-65). */
+int mha_bwd(const MhaBwdArgs* args, void* stream);
+
+/* Bytes of workspace mha_bwd needs (delta; plus fp32 copies of q, k, v when dtype is not fp32). */
+size_t mha_bwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dk, int32_t dv, int32_t dtype);
 
 #ifdef __cplusplus
 }

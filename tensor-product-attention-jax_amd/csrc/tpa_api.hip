@@ -91,4 +91,50 @@ int mha_fwd(const MhaFwdArgs* a, void* stream) {
   return mha_generic_launch(a, s);
 }
 
+int tpa_bwd(const TpaBwdArgs* a, void* stream) {
+  if (!a) return TPA_ERR_NULL;
+  if (a->dtype != TPA_DTYPE_F32 && a->dtype != TPA_DTYPE_BF16) return TPA_ERR_DTYPE;
+  if (a->B <= 0 || a->lq <= 0 || a->lk <= 0 || a->H <= 0 || a->dk <= 0 || a->dv <= 0 || a->rq <= 0 || a->rk <= 0)
+    return TPA_ERR_SHAPE;
+  if (a->dk > 256 || a->dv > 256) return TPA_ERR_SHAPE;
+  const TpaFactor* fs[6] = {&a->qa, &a->qb, &a->ka, &a->kb, &a->va, &a->vb};
+  for (const TpaFactor* f : fs)
+    if (check_factor(*f) != TPA_OK) return TPA_ERR_NULL;
+  const TpaGrad* gs[6] = {&a->dqa, &a->dqb, &a->dka, &a->dkb, &a->dva, &a->dvb};
+  for (const TpaGrad* g : gs)
+    if (!g->ptr) return TPA_ERR_NULL;
+  if (!a->o || !a->lse || !a->d_o) return TPA_ERR_NULL;
+  if ((a->q_segment_ids == nullptr) != (a->kv_segment_ids == nullptr)) return TPA_ERR_NULL;
+  if (a->kernel == TPA_KERNEL_MFMA) return TPA_ERR_UNSUPPORTED;  // there is no MFMA backward kernel
+  if (a->kernel != TPA_KERNEL_AUTO && a->kernel != TPA_KERNEL_GENERIC) return TPA_ERR_UNSUPPORTED;
+  if (!a->workspace || a->workspace_bytes < tpa_bwd_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dk, a->dv))
+    return TPA_ERR_WORKSPACE;
+  if (reinterpret_cast<uintptr_t>(a->workspace) & 255) return TPA_ERR_ALIGN;
+  return tpa_bwd_generic_launch(a, static_cast<hipStream_t>(stream));
+}
+
+size_t tpa_bwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dk, int32_t dv) {
+  if (B <= 0 || lq <= 0 || lk <= 0 || H <= 0 || dk <= 0 || dv <= 0) return 0;
+  return tpa_bwd_workspace_size(B, lq, lk, H, dk, dv);
+}
+
+int mha_bwd(const MhaBwdArgs* a, void* stream) {
+  if (!a) return TPA_ERR_NULL;
+  if (a->dtype != TPA_DTYPE_F32 && a->dtype != TPA_DTYPE_BF16) return TPA_ERR_DTYPE;
+  if (a->B <= 0 || a->lq <= 0 || a->lk <= 0 || a->H <= 0 || a->dk <= 0 || a->dv <= 0) return TPA_ERR_SHAPE;
+  if (a->dk > 256 || a->dv > 256) return TPA_ERR_SHAPE;
+  if (!a->q || !a->k || !a->v || !a->o || !a->lse || !a->d_o || !a->dq || !a->dk_out || !a->dv_out) return TPA_ERR_NULL;
+  if (a->kernel == TPA_KERNEL_MFMA) return TPA_ERR_UNSUPPORTED;
+  if (a->kernel != TPA_KERNEL_AUTO && a->kernel != TPA_KERNEL_GENERIC) return TPA_ERR_UNSUPPORTED;
+  if (!a->workspace || a->workspace_bytes < mha_bwd_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dk, a->dv, a->dtype))
+    return TPA_ERR_WORKSPACE;
+  if (reinterpret_cast<uintptr_t>(a->workspace) & 255) return TPA_ERR_ALIGN;
+  return mha_bwd_generic_launch(a, static_cast<hipStream_t>(stream));
+}
+
+size_t mha_bwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dk, int32_t dv, int32_t dtype) {
+  if (B <= 0 || lq <= 0 || lk <= 0 || H <= 0 || dk <= 0 || dv <= 0) return 0;
+  return mha_bwd_workspace_size(B, lq, lk, H, dk, dv, dtype);
+}
+
 }  // extern "C"

@@ -1,0 +1,392 @@
+// Backward pass: gradients of the attention output with respect to the rank factors
+// (tpa/tpa.py:168-214,546-995) and, for the dense baseline, with respect to q, k, v
+// (tpa/mha.py:40-65).  Any-shape fp32 arithmetic on the vector ALUs.
+//
+// The factored problem is taken through dense intermediates that live in the caller's
+// workspace, so that every stage is a plain, separately checkable kernel:
+//   1. recon:    Q, K, V [B, l, H, d] = (1/R) sum_r a_r (x) b_r               (tpa/tpa.py:605-606,623)
+//   2. delta:    delta[b, h, i] = sum_d o * do, NaN products skipped          (tpa/tpa.py:965-995)
+//   3. dq:       one thread per query row walks the keys:  p = exp(x - lse),
+//                dp = do . v, ds = scale * p * (dp - delta), dQ += ds * k      (tpa/tpa.py:779-781)
+//   4. dkv:      one thread per key walks the query rows: dV += p * do,
+//                dK += ds * q                                                  (tpa/tpa.py:765-777)
+//   5. project:  da[r, h] = (1/R) sum_d dX[h, d] b[r, d],  db[r, d] = (1/R) sum_h dX[h, d] a[r, h]
+//                for X in {Q, K, V}                                            (tpa/tpa.py:767-768,776-777,782-783)
+// Rows without a visible key (lse = -inf) contribute nothing (tpa/tpa.py:675-676).
+// Gradients are written as fp32 whatever the input type is.
+#include "tpa_common.h"
+
+namespace tpa {
+namespace {
+
+constexpr int kThreads = 128;  // rows (dq) or keys (dkv) per workgroup
+// keys (dq) or rows (dkv) per LDS tile: the tiles of the widest heads stay below 64 KB
+constexpr int tile_of(int dmax) { return dmax > 128 ? 16 : 32; }
+
+// ------------------------------------------------------------------------------------ stage 1
+template <typename T>
+__global__ void recon_kernel(TpaFactor fa, TpaFactor fb, float* out, int L, int H, int D, int R) {
+  const int t = blockIdx.x, b = blockIdx.y;
+  const T* ap = static_cast<const T*>(fa.ptr) + b * fa.stride_b + t * fa.stride_l;
+  const T* bp = static_cast<const T*>(fb.ptr) + b * fb.stride_b + t * fb.stride_l;
+  float* op = out + ((int64_t)b * L + t) * H * D;
+  const float inv = 1.f / (float)R;
+  for (int idx = threadIdx.x; idx < H * D; idx += blockDim.x) {
+    const int h = idx / D, d = idx - h * D;
+    float acc = 0.f;
+    for (int r = 0; r < R; ++r) acc += load_as_f32(ap + r * fa.stride_r + h) * load_as_f32(bp + r * fb.stride_r + d);
+    op[idx] = acc * inv;
+  }
+}
+
+template <typename T>
+__global__ void to_f32_kernel(const T* in, float* out, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    out[i] = load_as_f32(in + i);
+}
+
+// ------------------------------------------------------------------------------------ stage 2
+// delta[b, h, i] = sum_d o[b, i, h, d] * do[b, i, h, d], skipping NaN products (an empty row's o)
+template <typename T>
+__global__ void delta_kernel(const T* o, const T* d_o, float* delta, int B, int lq, int H, int dv) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // over (b, i, h)
+  if (idx >= (int64_t)B * lq * H) return;
+  const int h = idx % H;
+  const int64_t bi = idx / H;
+  const int i = bi % lq, b = bi / lq;
+  const T* op = o + idx * dv;
+  const T* gp = d_o + idx * dv;
+  float acc = 0.f;
+  for (int d = 0; d < dv; ++d) {
+    const float x = load_as_f32(op + d) * load_as_f32(gp + d);
+    if (x == x) acc += x;
+  }
+  delta[((int64_t)b * H + h) * lq + i] = acc;
+}
+
+struct DenseParams {
+  const float* q;  // [B, lq, H, dk]
+  const float* k;  // [B, lk, H, dk]
+  const float* v;  // [B, lk, H, dv]
+  const void* d_o;  // [B, lq, H, dv], element type T
+  const float* lse;    // [B, H, lq]
+  const float* delta;  // [B, H, lq]
+  const int32_t* qseg;
+  const int32_t* kvseg;
+  const float* bias;  // [B, lq, lk] or null
+  float* dq;          // [B, lq, H, dk]
+  float* dk_out;      // [B, lk, H, dk]
+  float* dv_out;      // [B, lk, H, dv]
+  int B, lq, lk, H, dk, dv;
+  float sm_scale;
+  int causal;
+};
+
+// ------------------------------------------------------------------------------------ stage 3
+template <typename T, int DMAX>
+__global__ __launch_bounds__(kThreads) void bwd_dq_kernel(DenseParams p) {
+  constexpr int kTile = tile_of(DMAX);
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int row = blockIdx.x * kThreads + threadIdx.x;
+  const int dk = p.dk, dv = p.dv;
+  extern __shared__ float smem[];
+  float* ks = smem;               // [kTile][dk]
+  float* vs = smem + kTile * dk;  // [kTile][dv]
+  int* segs = reinterpret_cast<int*>(vs + kTile * dv);
+
+  float lse = -INFINITY, delta = 0.f;
+  float q[DMAX], g[DMAX], acc[DMAX];
+#pragma unroll
+  for (int d = 0; d < DMAX; ++d) { q[d] = 0.f; g[d] = 0.f; acc[d] = 0.f; }
+  const bool row_ok = row < p.lq;
+  if (row_ok) {
+    lse = p.lse[((int64_t)b * p.H + h) * p.lq + row];
+    delta = p.delta[((int64_t)b * p.H + h) * p.lq + row];
+    const float* qp = p.q + (((int64_t)b * p.lq + row) * p.H + h) * dk;
+    const T* gp = static_cast<const T*>(p.d_o) + (((int64_t)b * p.lq + row) * p.H + h) * dv;
+#pragma unroll
+    for (int d = 0; d < DMAX; ++d) {
+      if (d < dk) q[d] = qp[d];
+      if (d < dv) {
+        const float x = load_as_f32(gp + d);
+        g[d] = x == x ? x : 0.f;
+      }
+    }
+  }
+  const bool live = row_ok && lse > -INFINITY;  // a row without a visible key has no gradient
+  const int qseg = (row_ok && p.qseg) ? p.qseg[(int64_t)b * p.lq + row] : 0;
+
+  int k_end = p.lk;
+  if (p.causal) k_end = min(p.lk, min(p.lq, (int)(blockIdx.x + 1) * kThreads));
+  for (int k0 = 0; k0 < k_end; k0 += kTile) {
+    const int nk = min(kTile, k_end - k0);
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < nk * dk; idx += kThreads) {
+      const int t = idx / dk, d = idx - t * dk;
+      ks[idx] = p.k[(((int64_t)b * p.lk + k0 + t) * p.H + h) * dk + d];
+    }
+    for (int idx = threadIdx.x; idx < nk * dv; idx += kThreads) {
+      const int t = idx / dv, d = idx - t * dv;
+      vs[idx] = p.v[(((int64_t)b * p.lk + k0 + t) * p.H + h) * dv + d];
+    }
+    if (p.kvseg)
+      for (int t = threadIdx.x; t < nk; t += kThreads) segs[t] = p.kvseg[(int64_t)b * p.lk + k0 + t];
+    __syncthreads();
+    if (!live) continue;
+    for (int t = 0; t < nk; ++t) {
+      bool keep = true;
+      if (p.kvseg) keep = segs[t] == qseg;
+      if (p.causal) keep = keep && (k0 + t <= row);
+      if (!keep) continue;
+      float dot = 0.f;
+#pragma unroll
+      for (int d = 0; d < DMAX; ++d)
+        if (d < dk) dot += q[d] * ks[t * dk + d];
+      float x = dot * p.sm_scale;
+      if (p.bias) x += p.bias[((int64_t)b * p.lq + row) * p.lk + k0 + t];
+      const float pt = expf(x - lse);
+      float dp = 0.f;
+#pragma unroll
+      for (int d = 0; d < DMAX; ++d)
+        if (d < dv) dp += g[d] * vs[t * dv + d];
+      const float ds = p.sm_scale * pt * (dp - delta);
+#pragma unroll
+      for (int d = 0; d < DMAX; ++d)
+        if (d < dk) acc[d] += ds * ks[t * dk + d];
+    }
+  }
+  if (!row_ok) return;
+  float* op = p.dq + (((int64_t)b * p.lq + row) * p.H + h) * dk;
+#pragma unroll
+  for (int d = 0; d < DMAX; ++d)
+    if (d < dk) op[d] = acc[d];
+}
+
+// ------------------------------------------------------------------------------------ stage 4
+template <typename T, int DMAX>
+__global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(DenseParams p) {
+  constexpr int kTile = tile_of(DMAX);
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int key = blockIdx.x * kThreads + threadIdx.x;
+  const int dk = p.dk, dv = p.dv;
+  extern __shared__ float smem[];
+  float* qs = smem;                   // [kTile][dk]
+  float* gs = smem + kTile * dk;      // [kTile][dv]  upstream gradient rows
+  float* ls = gs + kTile * dv;        // [kTile] lse
+  float* des = ls + kTile;            // [kTile] delta
+  int* segs = reinterpret_cast<int*>(des + kTile);
+
+  float kr[DMAX], vr[DMAX], dkr[DMAX], dvr[DMAX];
+#pragma unroll
+  for (int d = 0; d < DMAX; ++d) { kr[d] = 0.f; vr[d] = 0.f; dkr[d] = 0.f; dvr[d] = 0.f; }
+  const bool key_ok = key < p.lk;
+  if (key_ok) {
+    const float* kp = p.k + (((int64_t)b * p.lk + key) * p.H + h) * dk;
+    const float* vp = p.v + (((int64_t)b * p.lk + key) * p.H + h) * dv;
+#pragma unroll
+    for (int d = 0; d < DMAX; ++d) {
+      if (d < dk) kr[d] = kp[d];
+      if (d < dv) vr[d] = vp[d];
+    }
+  }
+  const int kseg = (key_ok && p.kvseg) ? p.kvseg[(int64_t)b * p.lk + key] : 0;
+
+  // under the causal mask only rows at or after this workgroup's first key can see its keys
+  const int q_begin = p.causal ? min(p.lq, (int)blockIdx.x * kThreads) / kTile * kTile : 0;
+  for (int q0 = q_begin; q0 < p.lq; q0 += kTile) {
+    const int nq = min(kTile, p.lq - q0);
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < nq * dk; idx += kThreads) {
+      const int i = idx / dk, d = idx - i * dk;
+      qs[idx] = p.q[(((int64_t)b * p.lq + q0 + i) * p.H + h) * dk + d];
+    }
+    for (int idx = threadIdx.x; idx < nq * dv; idx += kThreads) {
+      const int i = idx / dv, d = idx - i * dv;
+      const float x = load_as_f32(static_cast<const T*>(p.d_o) + (((int64_t)b * p.lq + q0 + i) * p.H + h) * dv + d);
+      gs[idx] = x == x ? x : 0.f;
+    }
+    for (int i = threadIdx.x; i < nq; i += kThreads) {
+      ls[i] = p.lse[((int64_t)b * p.H + h) * p.lq + q0 + i];
+      des[i] = p.delta[((int64_t)b * p.H + h) * p.lq + q0 + i];
+      if (p.qseg) segs[i] = p.qseg[(int64_t)b * p.lq + q0 + i];
+    }
+    __syncthreads();
+    if (!key_ok) continue;
+    for (int i = 0; i < nq; ++i) {
+      const float lse = ls[i];
+      bool keep = lse > -INFINITY;
+      if (p.qseg) keep = keep && segs[i] == kseg;
+      if (p.causal) keep = keep && (key <= q0 + i);
+      if (!keep) continue;
+      float dot = 0.f;
+#pragma unroll
+      for (int d = 0; d < DMAX; ++d)
+        if (d < dk) dot += kr[d] * qs[i * dk + d];
+      float x = dot * p.sm_scale;
+      if (p.bias) x += p.bias[((int64_t)b * p.lq + q0 + i) * p.lk + key];
+      const float pt = expf(x - lse);
+      float dp = 0.f;
+#pragma unroll
+      for (int d = 0; d < DMAX; ++d)
+        if (d < dv) {
+          const float gd = gs[i * dv + d];
+          dp += gd * vr[d];
+          dvr[d] += pt * gd;
+        }
+      const float ds = p.sm_scale * pt * (dp - des[i]);
+#pragma unroll
+      for (int d = 0; d < DMAX; ++d)
+        if (d < dk) dkr[d] += ds * qs[i * dk + d];
+    }
+  }
+  if (!key_ok) return;
+  float* okp = p.dk_out + (((int64_t)b * p.lk + key) * p.H + h) * dk;
+  float* ovp = p.dv_out + (((int64_t)b * p.lk + key) * p.H + h) * dv;
+#pragma unroll
+  for (int d = 0; d < DMAX; ++d) {
+    if (d < dk) okp[d] = dkr[d];
+    if (d < dv) ovp[d] = dvr[d];
+  }
+}
+
+// ------------------------------------------------------------------------------------ stage 5
+// One workgroup per token: da[r, h] and db[r, d] from the token's dense gradient dX[h, d].
+template <typename T>
+__global__ void project_kernel(const float* dx, TpaFactor fa, TpaFactor fb, TpaGrad ga, TpaGrad gb, int L, int H, int D, int R) {
+  const int t = blockIdx.x, b = blockIdx.y;
+  const float* xp = dx + ((int64_t)b * L + t) * H * D;
+  const T* ap = static_cast<const T*>(fa.ptr) + b * fa.stride_b + t * fa.stride_l;
+  const T* bp = static_cast<const T*>(fb.ptr) + b * fb.stride_b + t * fb.stride_l;
+  float* oa = ga.ptr + b * ga.stride_b + t * ga.stride_l;
+  float* ob = gb.ptr + b * gb.stride_b + t * gb.stride_l;
+  const float inv = 1.f / (float)R;
+  for (int idx = threadIdx.x; idx < R * H; idx += blockDim.x) {
+    const int r = idx / H, h = idx - r * H;
+    float acc = 0.f;
+    for (int d = 0; d < D; ++d) acc += xp[h * D + d] * load_as_f32(bp + r * fb.stride_r + d);
+    oa[r * ga.stride_r + h] = acc * inv;
+  }
+  for (int idx = threadIdx.x; idx < R * D; idx += blockDim.x) {
+    const int r = idx / D, d = idx - r * D;
+    float acc = 0.f;
+    for (int h = 0; h < H; ++h) acc += xp[h * D + d] * load_as_f32(ap + r * fa.stride_r + h);
+    ob[r * gb.stride_r + d] = acc * inv;
+  }
+}
+
+template <typename T, int DMAX>
+int launch_dense_t(const DenseParams& p, hipStream_t stream) {
+  constexpr int kTile = tile_of(DMAX);
+  const size_t smem_q = (size_t)kTile * (p.dk + p.dv) * sizeof(float) + kTile * sizeof(int);
+  const size_t smem_kv = (size_t)kTile * (p.dk + p.dv + 2) * sizeof(float) + kTile * sizeof(int);
+  hipLaunchKernelGGL((bwd_dq_kernel<T, DMAX>), dim3((p.lq + kThreads - 1) / kThreads, p.H, p.B), dim3(kThreads), smem_q, stream, p);
+  if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
+  hipLaunchKernelGGL((bwd_dkv_kernel<T, DMAX>), dim3((p.lk + kThreads - 1) / kThreads, p.H, p.B), dim3(kThreads), smem_kv, stream, p);
+  return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
+}
+
+template <typename T>
+int launch_dense(const DenseParams& p, hipStream_t stream) {
+  const int dmax = p.dk > p.dv ? p.dk : p.dv;
+  if (dmax <= 8) return launch_dense_t<T, 8>(p, stream);
+  if (dmax <= 32) return launch_dense_t<T, 32>(p, stream);
+  if (dmax <= 64) return launch_dense_t<T, 64>(p, stream);
+  if (dmax <= 128) return launch_dense_t<T, 128>(p, stream);
+  if (dmax <= 256) return launch_dense_t<T, 256>(p, stream);
+  return TPA_ERR_SHAPE;
+}
+
+inline size_t align256(size_t n) { return (n + 255) & ~size_t(255); }
+
+template <typename T>
+int tpa_bwd_t(const TpaBwdArgs* a, hipStream_t stream) {
+  const size_t nq = (size_t)a->B * a->lq * a->H * a->dk, nk = (size_t)a->B * a->lk * a->H * a->dk,
+               nv = (size_t)a->B * a->lk * a->H * a->dv, nd = (size_t)a->B * a->H * a->lq;
+  char* w = static_cast<char*>(a->workspace);
+  auto take = [&](size_t floats) { float* ptr = reinterpret_cast<float*>(w); w += align256(floats * sizeof(float)); return ptr; };
+  float *qd = take(nq), *kd = take(nk), *vd = take(nv), *dqd = take(nq), *dkd = take(nk), *dvd = take(nv), *delta = take(nd);
+
+  const int threads = 256;
+  hipLaunchKernelGGL((recon_kernel<T>), dim3(a->lq, a->B), dim3(threads), 0, stream, a->qa, a->qb, qd, a->lq, a->H, a->dk, a->rq);
+  hipLaunchKernelGGL((recon_kernel<T>), dim3(a->lk, a->B), dim3(threads), 0, stream, a->ka, a->kb, kd, a->lk, a->H, a->dk, a->rk);
+  hipLaunchKernelGGL((recon_kernel<T>), dim3(a->lk, a->B), dim3(threads), 0, stream, a->va, a->vb, vd, a->lk, a->H, a->dv, a->rk);
+  hipLaunchKernelGGL((delta_kernel<T>), dim3((unsigned)((nd + threads - 1) / threads)), dim3(threads), 0, stream,
+                     static_cast<const T*>(a->o), static_cast<const T*>(a->d_o), delta, a->B, a->lq, a->H, a->dv);
+  if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
+
+  DenseParams p{};
+  p.q = qd; p.k = kd; p.v = vd; p.d_o = a->d_o; p.lse = a->lse; p.delta = delta;
+  p.qseg = a->q_segment_ids; p.kvseg = a->kv_segment_ids; p.bias = nullptr;
+  p.dq = dqd; p.dk_out = dkd; p.dv_out = dvd;
+  p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.dk = a->dk; p.dv = a->dv;
+  p.sm_scale = a->sm_scale; p.causal = a->causal;
+  const int rc = launch_dense<T>(p, stream);
+  if (rc != TPA_OK) return rc;
+
+  hipLaunchKernelGGL((project_kernel<T>), dim3(a->lq, a->B), dim3(threads), 0, stream, dqd, a->qa, a->qb, a->dqa, a->dqb, a->lq, a->H, a->dk, a->rq);
+  hipLaunchKernelGGL((project_kernel<T>), dim3(a->lk, a->B), dim3(threads), 0, stream, dkd, a->ka, a->kb, a->dka, a->dkb, a->lk, a->H, a->dk, a->rk);
+  hipLaunchKernelGGL((project_kernel<T>), dim3(a->lk, a->B), dim3(threads), 0, stream, dvd, a->va, a->vb, a->dva, a->dvb, a->lk, a->H, a->dv, a->rk);
+  return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
+}
+
+template <typename T>
+int mha_bwd_t(const MhaBwdArgs* a, hipStream_t stream) {
+  const size_t nq = (size_t)a->B * a->lq * a->H * a->dk, nk = (size_t)a->B * a->lk * a->H * a->dk,
+               nv = (size_t)a->B * a->lk * a->H * a->dv, nd = (size_t)a->B * a->H * a->lq;
+  char* w = static_cast<char*>(a->workspace);
+  auto take = [&](size_t floats) { float* ptr = reinterpret_cast<float*>(w); w += align256(floats * sizeof(float)); return ptr; };
+  float* delta = take(nd);
+  const float *qd, *kd, *vd;
+  const int threads = 256;
+  if constexpr (sizeof(T) == sizeof(float)) {
+    qd = static_cast<const float*>(a->q); kd = static_cast<const float*>(a->k); vd = static_cast<const float*>(a->v);
+  } else {
+    float *q32 = take(nq), *k32 = take(nk), *v32 = take(nv);
+    auto blocks = [&](size_t n) { return dim3((unsigned)((n + threads - 1) / threads < 65535 * 16 ? (n + threads - 1) / threads : 65535 * 16)); };
+    hipLaunchKernelGGL((to_f32_kernel<T>), blocks(nq), dim3(threads), 0, stream, static_cast<const T*>(a->q), q32, (int64_t)nq);
+    hipLaunchKernelGGL((to_f32_kernel<T>), blocks(nk), dim3(threads), 0, stream, static_cast<const T*>(a->k), k32, (int64_t)nk);
+    hipLaunchKernelGGL((to_f32_kernel<T>), blocks(nv), dim3(threads), 0, stream, static_cast<const T*>(a->v), v32, (int64_t)nv);
+    qd = q32; kd = k32; vd = v32;
+  }
+  hipLaunchKernelGGL((delta_kernel<T>), dim3((unsigned)((nd + threads - 1) / threads)), dim3(threads), 0, stream,
+                     static_cast<const T*>(a->o), static_cast<const T*>(a->d_o), delta, a->B, a->lq, a->H, a->dv);
+  if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
+  DenseParams p{};
+  p.q = qd; p.k = kd; p.v = vd; p.d_o = a->d_o; p.lse = a->lse; p.delta = delta;
+  p.qseg = nullptr; p.kvseg = nullptr; p.bias = a->bias;
+  p.dq = a->dq; p.dk_out = a->dk_out; p.dv_out = a->dv_out;
+  p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.dk = a->dk; p.dv = a->dv;
+  p.sm_scale = a->sm_scale; p.causal = a->causal;
+  return launch_dense<T>(p, stream);
+}
+
+}  // namespace
+}  // namespace tpa
+
+size_t tpa_bwd_workspace_size(int64_t B, int64_t lq, int64_t lk, int64_t H, int64_t dk, int64_t dv) {
+  using tpa::align256;
+  const size_t nq = (size_t)(B * lq * H * dk), nk = (size_t)(B * lk * H * dk), nv = (size_t)(B * lk * H * dv), nd = (size_t)(B * H * lq);
+  return 2 * (align256(nq * 4) + align256(nk * 4) + align256(nv * 4)) + align256(nd * 4);
+}
+
+size_t mha_bwd_workspace_size(int64_t B, int64_t lq, int64_t lk, int64_t H, int64_t dk, int64_t dv, int dtype) {
+  using tpa::align256;
+  const size_t nq = (size_t)(B * lq * H * dk), nk = (size_t)(B * lk * H * dk), nv = (size_t)(B * lk * H * dv), nd = (size_t)(B * H * lq);
+  size_t bytes = align256(nd * 4);
+  if (dtype != TPA_DTYPE_F32) bytes += align256(nq * 4) + align256(nk * 4) + align256(nv * 4);
+  return bytes;
+}
+
+int tpa_bwd_generic_launch(const TpaBwdArgs* a, hipStream_t stream) {
+  if (a->B > 65535 || a->H > 65535) return TPA_ERR_SHAPE;
+  if (a->dtype == TPA_DTYPE_F32) return tpa::tpa_bwd_t<float>(a, stream);
+  if (a->dtype == TPA_DTYPE_BF16) return tpa::tpa_bwd_t<uint16_t>(a, stream);
+  return TPA_ERR_DTYPE;
+}
+
+int mha_bwd_generic_launch(const MhaBwdArgs* a, hipStream_t stream) {
+  if (a->B > 65535 || a->H > 65535) return TPA_ERR_SHAPE;
+  if (a->dtype == TPA_DTYPE_F32) return tpa::mha_bwd_t<float>(a, stream);
+  if (a->dtype == TPA_DTYPE_BF16) return tpa::mha_bwd_t<uint16_t>(a, stream);
+  return TPA_ERR_DTYPE;
+}

@@ -124,3 +124,7 @@ int tpa_decode_mfma_supported(const TpaFwdArgs* a);
 int tpa_decode_mfma_launch(const TpaFwdArgs* a, hipStream_t stream);
 int mha_decode_supported(const MhaFwdArgs* a);
 int mha_decode_launch(const MhaFwdArgs* a, hipStream_t stream);
+int tpa_bwd_generic_launch(const TpaBwdArgs* a, hipStream_t stream);
+int mha_bwd_generic_launch(const MhaBwdArgs* a, hipStream_t stream);
+size_t tpa_bwd_workspace_size(int64_t B, int64_t lq, int64_t lk, int64_t H, int64_t dk, int64_t dv);
+size_t mha_bwd_workspace_size(int64_t B, int64_t lq, int64_t lk, int64_t H, int64_t dk, int64_t dv, int dtype);

@@ -22,7 +22,7 @@ KERNEL_AUTO = 0
 KERNEL_GENERIC = 1
 KERNEL_MFMA = 2
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 
 class TpaFactor(ctypes.Structure):
@@ -88,6 +88,73 @@ class MhaFwdArgs(ctypes.Structure):
     ]
 
 
+class TpaGrad(ctypes.Structure):
+    _fields_ = TpaFactor._fields_
+
+
+class TpaBwdArgs(ctypes.Structure):
+    _fields_ = [
+        ("qa", TpaFactor),
+        ("qb", TpaFactor),
+        ("ka", TpaFactor),
+        ("kb", TpaFactor),
+        ("va", TpaFactor),
+        ("vb", TpaFactor),
+        ("q_segment_ids", ctypes.c_void_p),
+        ("kv_segment_ids", ctypes.c_void_p),
+        ("o", ctypes.c_void_p),
+        ("lse", ctypes.c_void_p),
+        ("d_o", ctypes.c_void_p),
+        ("dqa", TpaGrad),
+        ("dqb", TpaGrad),
+        ("dka", TpaGrad),
+        ("dkb", TpaGrad),
+        ("dva", TpaGrad),
+        ("dvb", TpaGrad),
+        ("B", ctypes.c_int32),
+        ("lq", ctypes.c_int32),
+        ("lk", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("dk", ctypes.c_int32),
+        ("dv", ctypes.c_int32),
+        ("rq", ctypes.c_int32),
+        ("rk", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("sm_scale", ctypes.c_float),
+        ("causal", ctypes.c_int32),
+        ("kernel", ctypes.c_int32),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_size_t),
+    ]
+
+
+class MhaBwdArgs(ctypes.Structure):
+    _fields_ = [
+        ("q", ctypes.c_void_p),
+        ("k", ctypes.c_void_p),
+        ("v", ctypes.c_void_p),
+        ("bias", ctypes.c_void_p),
+        ("o", ctypes.c_void_p),
+        ("lse", ctypes.c_void_p),
+        ("d_o", ctypes.c_void_p),
+        ("dq", ctypes.c_void_p),
+        ("dk_out", ctypes.c_void_p),
+        ("dv_out", ctypes.c_void_p),
+        ("B", ctypes.c_int32),
+        ("lq", ctypes.c_int32),
+        ("lk", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("dk", ctypes.c_int32),
+        ("dv", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("sm_scale", ctypes.c_float),
+        ("causal", ctypes.c_int32),
+        ("kernel", ctypes.c_int32),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_size_t),
+    ]
+
+
 class TpaError(RuntimeError):
     """A non-zero return code of the C ABI."""
 
@@ -129,6 +196,14 @@ def load_library(path: str | None = None) -> ctypes.CDLL:
         lib.tpa_decode_default_splits.argtypes = [ctypes.c_int32] * 4
         lib.mha_fwd_workspace_bytes.restype = ctypes.c_size_t
         lib.mha_fwd_workspace_bytes.argtypes = [ctypes.c_int32] * 6
+        lib.tpa_bwd.restype = ctypes.c_int
+        lib.tpa_bwd.argtypes = [ctypes.POINTER(TpaBwdArgs), ctypes.c_void_p]
+        lib.mha_bwd.restype = ctypes.c_int
+        lib.mha_bwd.argtypes = [ctypes.POINTER(MhaBwdArgs), ctypes.c_void_p]
+        lib.tpa_bwd_workspace_bytes.restype = ctypes.c_size_t
+        lib.tpa_bwd_workspace_bytes.argtypes = [ctypes.c_int32] * 6
+        lib.mha_bwd_workspace_bytes.restype = ctypes.c_size_t
+        lib.mha_bwd_workspace_bytes.argtypes = [ctypes.c_int32] * 7
         if lib.tpa_abi_version() != ABI_VERSION:
             raise RuntimeError(f"{p}: ABI version {lib.tpa_abi_version()} != {ABI_VERSION}")
         if path is None:
@@ -156,6 +231,14 @@ def factor(t: torch.Tensor) -> TpaFactor:
     if t.shape[-1] > 1 and t.stride(-1) != 1:
         raise ValueError("the last dimension of a factor array must be contiguous")
     return TpaFactor(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+
+
+def grad(t: torch.Tensor) -> TpaGrad:
+    """A float32 [b, l, r, x] tensor (or a view of one) that a gradient is written into."""
+    if t.dtype != torch.float32:
+        raise TypeError("gradient arrays are float32")
+    f = factor(t)
+    return TpaGrad(f.ptr, f.stride_b, f.stride_l, f.stride_r)
 
 
 def current_stream_ptr(device: torch.device) -> int:

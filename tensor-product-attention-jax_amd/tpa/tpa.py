@@ -14,8 +14,9 @@ reference, all on purpose:
     non-materialising form;
   * `interpret=True` (the Pallas CPU interpreter upstream) selects the plain fp32-arithmetic
     kernel instead of the MFMA kernels; `debug` is ignored;
-  * the backward pass is not implemented: differentiating raises NotImplementedError (the
-    reference's own backward test skips on exactly that, tpa/tpa_test.py:198-201).
+  * the backward pass (tpa/tpa.py:168-214,546-995) runs as fp32 vector-ALU kernels through dense
+    intermediates (there is no MFMA backward kernel); gradients are computed in fp32 and cast to
+    the input dtype; torch.autograd reaches it through `tpa()`.
 """
 
 from __future__ import annotations
@@ -27,7 +28,10 @@ import torch
 
 from . import _dispatch as _d
 
-__all__ = ["BlockSizes", "tpa", "tpa_factors", "tpa_decode", "_tpa_fwd", "_fwd", "_lse", "_lse_accum"]
+__all__ = [
+    "BlockSizes", "tpa", "tpa_factors", "tpa_decode", "tpa_factors_bwd", "_tpa_fwd", "_tpa_bwd", "_fwd", "_bwd",
+    "_precompute_delta", "_lse", "_lse_accum",
+]
 
 
 @dataclasses.dataclass
@@ -188,8 +192,73 @@ def decode_workspace_bytes(b: int, lq: int, lk: int, h: int, dv: int, num_splits
     return int(_d.load_library().tpa_decode_workspace_bytes(b, lq, lk, h, dv, num_splits))
 
 
+def tpa_factors_bwd(
+    qa, qb, ka, kb, va, vb,
+    q_segment_ids, kv_segment_ids,
+    o, lse, do,
+    sm_scale: float = 1.0,
+    causal: bool = False,
+    grads=None,
+    workspace: torch.Tensor | None = None,
+):
+    """Backward pass on the split factor arrays: the operands of the reference's backward kernel
+    launch (tpa/tpa.py:872-958) with a leading batch dimension, `lse` as [b, h, lq] fp32.
+
+    Returns the six fp32 gradients (dqa, dqb, dka, dkb, dva, dvb), each shaped like its factor.
+    `grads` may hold six fp32 tensors (or views, e.g. the two parts of a concatenated
+    dq[b, lq, rq, h+dk]) to be written in place.
+    """
+    device = _pick_device(qa, qb, ka, kb, va, vb)
+    qa, qb, ka, kb, va, vb, o, lse, do = (_as_device_tensor(x, device) for x in (qa, qb, ka, kb, va, vb, o, lse, do))
+    dtype = qa.dtype
+    b, lq, rq, h = qa.shape
+    _, lk, rk, dv = vb.shape
+    dk = qb.shape[-1]
+    assert tuple(kb.shape) == (b, lk, rk, dk), kb.shape
+    assert tuple(o.shape) == (b, lq, h, dv) and tuple(do.shape) == (b, lq, h, dv), (o.shape, do.shape)
+    assert tuple(lse.shape) == (b, h, lq), lse.shape
+    qseg = _segment_ids(q_segment_ids, b, lq, device)
+    kvseg = _segment_ids(kv_segment_ids, b, lk, device)
+    o = o.to(dtype).contiguous()
+    do = do.to(dtype).contiguous()
+    lse = lse.to(torch.float32).contiguous()
+    if grads is None:
+        grads = tuple(torch.empty(t.shape, dtype=torch.float32, device=device) for t in (qa, qb, ka, kb, va, vb))
+    lib = _d.load_library()
+    need = lib.tpa_bwd_workspace_bytes(b, lq, lk, h, dk, dv)
+    if workspace is None:
+        workspace = torch.empty(need + 256, dtype=torch.uint8, device=device)
+    pad = (-workspace.data_ptr()) % 256
+    args = _d.TpaBwdArgs(
+        qa=_d.factor(qa), qb=_d.factor(qb), ka=_d.factor(ka), kb=_d.factor(kb), va=_d.factor(va), vb=_d.factor(vb),
+        q_segment_ids=None if qseg is None else qseg.data_ptr(),
+        kv_segment_ids=None if kvseg is None else kvseg.data_ptr(),
+        o=o.data_ptr(), lse=lse.data_ptr(), d_o=do.data_ptr(),
+        dqa=_d.grad(grads[0]), dqb=_d.grad(grads[1]), dka=_d.grad(grads[2]), dkb=_d.grad(grads[3]),
+        dva=_d.grad(grads[4]), dvb=_d.grad(grads[5]),
+        B=b, lq=lq, lk=lk, H=h, dk=dk, dv=dv, rq=rq, rk=rk,
+        dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=int(bool(causal)), kernel=_d.KERNEL_AUTO,
+        workspace=workspace.data_ptr() + pad, workspace_bytes=workspace.numel() - pad,
+    )
+    with torch.cuda.device(device):
+        _d.check("tpa_bwd", lib.tpa_bwd(args, _d.current_stream_ptr(device)))
+    return tuple(grads)
+
+
+def _bwd_concat(q, k, v, qseg, kvseg, o, lse_bhl, do, num_heads, sm_scale, causal):
+    """Gradients in the concatenated layout of q, k, v (fp32), written in place by the kernels."""
+    h = num_heads
+    dq, dk, dv = (torch.empty(t.shape, dtype=torch.float32, device=t.device) for t in (q, k, v))
+    views = (dq[..., :h], dq[..., h:], dk[..., :h], dk[..., h:], dv[..., :h], dv[..., h:])
+    tpa_factors_bwd(
+        q[..., :h], q[..., h:], k[..., :h], k[..., h:], v[..., :h], v[..., h:],
+        qseg, kvseg, o, lse_bhl, do, sm_scale, causal, grads=views,
+    )
+    return dq, dk, dv
+
+
 class _TpaFunction(torch.autograd.Function):
-    """Forward-only operator: the reference registers a vjp (tpa/tpa.py:217); this build raises."""
+    """The operator with its vjp, as tpa.defvjp(_tpa_fwd, _tpa_bwd) registers it (tpa/tpa.py:217)."""
 
     @staticmethod
     def forward(ctx, q, k, v, num_heads, qseg, kvseg, sm_scale, causal, kernel):
@@ -198,11 +267,16 @@ class _TpaFunction(torch.autograd.Function):
         va, vb = v[..., :num_heads], v[..., num_heads:]
         o, lse = tpa_factors(qa, qb, ka, kb, va, vb, qseg, kvseg, sm_scale, causal, kernel)
         ctx.mark_non_differentiable(lse)
+        ctx.save_for_backward(q, k, v, o, lse)
+        ctx.statics = (num_heads, qseg, kvseg, sm_scale, causal)
         return o, lse
 
     @staticmethod
-    def backward(ctx, *grads):
-        raise NotImplementedError("the TPA backward pass is not implemented in this build (forward only)")
+    def backward(ctx, do, _dlse):
+        q, k, v, o, lse = ctx.saved_tensors
+        num_heads, qseg, kvseg, sm_scale, causal = ctx.statics
+        dq, dk, dv = _bwd_concat(q, k, v, qseg, kvseg, o, lse, do, num_heads, sm_scale, causal)
+        return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None, None, None, None, None
 
 
 def _tpa_fwd(
@@ -260,3 +334,35 @@ def _fwd(
     q, k, v = (_as_device_tensor(x, device)[None] for x in (q, k, v))
     o, res = _tpa_fwd(q, k, v, num_heads, qs, ks, sm_scale, causal, block_sizes, nomat, debug, interpret)
     return o[0], res[-1][0]
+
+
+def _tpa_bwd(num_heads, sm_scale, causal, block_sizes, nomat, debug, interpret, residuals, do):
+    """tpa/tpa.py:168-214: (dq, dk, dv, None, None) from the residuals `_tpa_fwd` returned, in the
+    dtype and the concatenated layout of q, k, v."""
+    del block_sizes, nomat, debug, interpret
+    q, k, v, q_segment_ids, kv_segment_ids, o, l = residuals
+    device = _pick_device(q, k, v)
+    q, k, v, o, l, do = (_as_device_tensor(x, device) for x in (q, k, v, o, l, do))
+    dq, dk, dv = _bwd_concat(q, k, v, q_segment_ids, kv_segment_ids, o, l.permute(0, 2, 1), do, int(num_heads), float(sm_scale), bool(causal))
+    return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None
+
+
+def _bwd(
+    q, k, v, q_segment_ids, kv_segment_ids, o, l, do, num_heads, sm_scale, causal, block_sizes, nomat, debug, interpret
+):
+    """Per-batch-element backward (tpa/tpa.py:823-962): q[lq,rq,h+dk] ... o[lq,h,dv] l[lq,h]
+    do[lq,h,dv] -> (dq, dk, dv) shaped like q, k, v."""
+    qs = None if q_segment_ids is None else torch.as_tensor(q_segment_ids)[None]
+    ks = None if kv_segment_ids is None else torch.as_tensor(kv_segment_ids)[None]
+    device = _pick_device(q, k, v)
+    q, k, v, o, l, do = (_as_device_tensor(x, device)[None] for x in (q, k, v, o, l, do))
+    dq, dk, dv, _, _ = _tpa_bwd(num_heads, sm_scale, causal, block_sizes, nomat, debug, interpret, (q, k, v, qs, ks, o, l), do)
+    return dq[0], dk[0], dv[0]
+
+
+def _precompute_delta(out, do, lse, block_q=None, debug=False, interpret=False):
+    """tpa/tpa.py:965-995: delta[lq] = nansum(out * do, axis=1) for one head, out/do [lq, dv].
+    (The backward kernels compute it themselves; kept because callers of the reference name it.)"""
+    del block_q, debug, interpret
+    out, do = torch.as_tensor(out), torch.as_tensor(do)
+    return torch.nansum(out.float() * do.float(), dim=1).to(torch.as_tensor(lse).dtype)

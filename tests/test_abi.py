@@ -23,7 +23,8 @@ def declared_functions():
 
 def test_header_declares_the_expected_entry_points():
     names = declared_functions()
-    for f in ("tpa_fwd", "tpa_decode", "mha_fwd", "tpa_decode_workspace_bytes", "tpa_strerror", "tpa_abi_version"):
+    for f in ("tpa_fwd", "tpa_decode", "mha_fwd", "tpa_decode_workspace_bytes", "tpa_strerror", "tpa_abi_version",
+              "tpa_bwd", "mha_bwd", "tpa_bwd_workspace_bytes", "mha_bwd_workspace_bytes"):
         assert f in names, names
 
 
@@ -41,7 +42,8 @@ def test_library_exports_every_declared_symbol():
 def test_struct_layout_matches_the_c_compiler(tmp_path):
     from tpa import _dispatch as d
 
-    fields = {"TpaFactor": d.TpaFactor, "TpaFwdArgs": d.TpaFwdArgs, "MhaFwdArgs": d.MhaFwdArgs}
+    fields = {"TpaFactor": d.TpaFactor, "TpaFwdArgs": d.TpaFwdArgs, "MhaFwdArgs": d.MhaFwdArgs,
+              "TpaGrad": d.TpaGrad, "TpaBwdArgs": d.TpaBwdArgs, "MhaBwdArgs": d.MhaBwdArgs}
     lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "tpa_abi.h"', "int main(void) {"]
     for sname, cls in fields.items():
         lines.append(f'printf("{sname} %zu\\n", sizeof({sname}));')
@@ -69,6 +71,13 @@ def test_size_queries_need_no_gpu():
     assert lib.tpa_decode_workspace_bytes(64, 1, 8192, 32, 128, 0) == 64 * 4 * 32 * (128 + 2) * 4
     assert lib.tpa_decode_workspace_bytes(64, 1, 8192, 32, 128, 7) == 64 * 7 * 32 * (128 + 2) * 4
     assert lib.tpa_decode_default_splits(0, 1, 8192, 32) == 0
+    # backward: dense Q, K, V and their gradients (fp32, each rounded up to 256 bytes) plus delta
+    r = lambda n: (n + 255) // 256 * 256
+    nq, nk, nv, nd = 2 * 10 * 3 * 5 * 4, 2 * 7 * 3 * 5 * 4, 2 * 7 * 3 * 6 * 4, 2 * 3 * 10 * 4
+    assert lib.tpa_bwd_workspace_bytes(2, 10, 7, 3, 5, 6) == 2 * (r(nq) + r(nk) + r(nv)) + r(nd)
+    assert lib.mha_bwd_workspace_bytes(2, 10, 7, 3, 5, 6, 0) == r(nd)
+    assert lib.mha_bwd_workspace_bytes(2, 10, 7, 3, 5, 6, 1) == r(nd) + r(nq) + r(nk) + r(nv)
+    assert lib.tpa_bwd_workspace_bytes(2, 0, 7, 3, 5, 6) == 0
 
 
 def test_null_and_shape_errors_are_reported_before_any_launch():
@@ -89,6 +98,14 @@ def test_null_and_shape_errors_are_reported_before_any_launch():
     margs = d.MhaFwdArgs()
     assert lib.mha_fwd(ctypes.byref(margs), None) == -2
     assert lib.mha_fwd(None, None) == -1
+    bargs = d.TpaBwdArgs()
+    assert lib.tpa_bwd(None, None) == -1
+    assert lib.tpa_bwd(ctypes.byref(bargs), None) == -2
+    bargs.B = bargs.lq = bargs.lk = bargs.H = bargs.dk = bargs.dv = bargs.rq = bargs.rk = 1
+    assert lib.tpa_bwd(ctypes.byref(bargs), None) == -1  # pointers are NULL
+    mb = d.MhaBwdArgs()
+    assert lib.mha_bwd(ctypes.byref(mb), None) == -2
+    assert lib.mha_bwd(None, None) == -1
 
 
 def test_missing_library_fails_loudly(tmp_path):

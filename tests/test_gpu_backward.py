@@ -1,0 +1,175 @@
+"""GPU parity of the backward pass (tpa_bwd / mha_bwd through the C ABI) against the CPU oracle.
+
+The cases follow the reference's own backward tests: tpa/tpa_test.py:128-205 (gradients of
+nansum(o), tolerances atol 1e-3 / rtol 1e-2 there; fp32 here is held to 2e-4 of the largest
+gradient) and tpa/mha_test.py:9-41,44-118.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import make_factors, segment_ids
+from oracle import tpa_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_err(got, want):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    assert got.shape == want.shape
+    assert np.isfinite(got).all()
+    return float(np.max(np.abs(got - want)) / max(1e-30, np.max(np.abs(want))))
+
+
+# the reference's backward grid (tpa/tpa_test.py:128-141), nomat folded away: it does not change results
+@pytest.mark.parametrize("rank_q", [1, 6])
+@pytest.mark.parametrize("rank_k", [1, 4])
+@pytest.mark.parametrize(
+    "batch_size,lq,lk,h,dk,dv,segment_size",
+    [
+        (1, 8, 8, 1, 4, 6, 8),
+        (2, 1024, 128, 2, 3, 5, 42),
+        (2, 1024, 128, 2, 3, 5, None),
+        (2, 128, 1024, 2, 3, 5, 42),
+        (2, 128, 1024, 2, 3, 5, None),
+        (1, 1024, 1024, 2, 3, 5, 321),
+    ],
+)
+def test_reference_backward_grid(gpu, batch_size, rank_q, rank_k, lq, lk, h, dk, dv, segment_size):
+    """d nansum(o) / d(q, k, v) through torch.autograd on tpa(), as the reference's test takes
+    jax.grad of it; normal inputs, sm_scale = 1, not causal (tpa/tpa_test.py:155-205)."""
+    from tpa import tpa
+
+    q, k, v = make_factors(5, batch_size, lq, lk, h, dk, dv, rank_q, rank_k)
+    qseg = segment_ids(lq, segment_size, batch_size) if segment_size else None
+    kvseg = segment_ids(lk, segment_size, batch_size) if segment_size else None
+    tq, tk, tv = (torch.from_numpy(x).to(gpu).requires_grad_() for x in (q, k, v))
+    o = tpa.tpa(tq, tk, tv, num_heads=h, q_segment_ids=qseg, kv_segment_ids=kvseg, causal=False)
+    torch.nansum(o).backward()
+    want = orc.tpa_backward(q, k, v, qseg, kvseg, h, np.ones((batch_size, lq, h, dv)), sm_scale=1.0, causal=False)
+    for name, t, w in zip("qkv", (tq, tk, tv), want):
+        assert rel_err(t.grad.cpu().numpy(), w) <= 2e-4, name
+        np.testing.assert_allclose(t.grad.cpu().numpy(), w, atol=1e-3, rtol=1e-2)  # the reference's own bound
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("seg", [None, 50])
+@pytest.mark.parametrize("b,lq,lk,h,dk,dv,rq,rk", [(2, 200, 200, 3, 16, 24, 3, 2), (1, 130, 77, 4, 64, 64, 6, 2), (1, 60, 300, 2, 40, 130, 2, 3)])
+def test_backward_fp32_masks_ragged_and_random_upstream(gpu, b, lq, lk, h, dk, dv, rq, rk, seg, causal):
+    """_tpa_bwd on residuals of _tpa_fwd with a random upstream gradient."""
+    from tpa import tpa
+
+    q, k, v = make_factors(6, b, lq, lk, h, dk, dv, rq, rk, scale_by_rank=True)
+    do = np.random.default_rng(8).standard_normal((b, lq, h, dv)).astype(np.float32)
+    qseg = segment_ids(lq, seg, b) if seg else None
+    kvseg = segment_ids(lk, seg, b) if seg else None
+    scale = dk**-0.5
+    tq, tk, tv = (torch.from_numpy(x).to(gpu) for x in (q, k, v))
+    o, res = tpa._tpa_fwd(tq, tk, tv, h, qseg, kvseg, scale, causal, None, False, False, False)
+    dq, dk_, dv_, n1, n2 = tpa._tpa_bwd(h, scale, causal, None, False, False, False, res, torch.from_numpy(do).to(gpu))
+    assert n1 is None and n2 is None
+    want = orc.tpa_backward(q, k, v, qseg, kvseg, h, do, sm_scale=scale, causal=causal)
+    for name, g, w in zip("qkv", (dq, dk_, dv_), want):
+        assert g.dtype == torch.float32 and g.shape == w.shape
+        assert rel_err(g.cpu().numpy(), w) <= 2e-4, name
+
+
+def test_backward_bf16_inputs(gpu):
+    """bf16 factors: the gradients are computed in fp32 from the bf16 values and the bf16 forward
+    output, then cast to bf16; compared with the oracle on the same bf16-rounded inputs."""
+    from tpa import tpa
+
+    b, lq, lk, h, d, rq, rk = 2, 384, 384, 8, 64, 6, 2
+    q, k, v = make_factors(9, b, lq, lk, h, d, d, rq, rk, scale_by_rank=True)
+    do = np.random.default_rng(10).standard_normal((b, lq, h, d)).astype(np.float32)
+    tq, tk, tv = (torch.from_numpy(x).to(gpu).to(torch.bfloat16).requires_grad_() for x in (q, k, v))
+    tdo = torch.from_numpy(do).to(gpu).to(torch.bfloat16)
+    o = tpa.tpa(tq, tk, tv, num_heads=h, sm_scale=d**-0.5, causal=True)
+    o.backward(tdo)
+    f64 = lambda t: t.detach().float().cpu().numpy().astype(np.float64)
+    want = orc.tpa_backward(f64(tq), f64(tk), f64(tv), None, None, h, f64(tdo), sm_scale=d**-0.5, causal=True)
+    for name, t, w in zip("qkv", (tq, tk, tv), want):
+        assert t.grad.dtype == torch.bfloat16
+        assert rel_err(f64(t.grad), w) <= 2e-2, name  # bf16 output rounding (2^-9 relative) and the bf16 o in delta
+
+
+def test_backward_per_batch_entry_api(gpu):
+    """_bwd on one batch entry (tpa/tpa.py:823-962) equals the batched call."""
+    from tpa import tpa
+
+    b, lq, lk, h, dk, dv, rq, rk = 2, 40, 56, 2, 8, 8, 2, 2
+    q, k, v = make_factors(13, b, lq, lk, h, dk, dv, rq, rk)
+    do = np.random.default_rng(14).standard_normal((b, lq, h, dv)).astype(np.float32)
+    tq, tk, tv, tdo = (torch.from_numpy(x).to(gpu) for x in (q, k, v, do))
+    o, res = tpa._tpa_fwd(tq, tk, tv, h, None, None, 0.3, True, None, False, False, False)
+    dq, dk_, dv_, _, _ = tpa._tpa_bwd(h, 0.3, True, None, False, False, False, res, tdo)
+    l = res[-1]
+    one = tpa._bwd(tq[1], tk[1], tv[1], None, None, o[1], l[1], tdo[1], h, 0.3, True, None, False, False, False)
+    for g, g1 in zip((dq, dk_, dv_), one):
+        assert torch.equal(g[1], g1)
+
+
+# ---------------------------------------------------------------- dense attention (tpa/mha.py:40-65)
+@pytest.mark.parametrize("batch,lq,lk,h,dk,dv", [(2, 4, 6, 3, 8, 8), (1, 3, 5, 2, 4, 4)])
+@pytest.mark.parametrize("sm_scale", [0.5, 1.0, 2.0])
+def test_mha_gradients_match(gpu, batch, lq, lk, h, dk, dv, sm_scale):
+    """tpa/mha_test.py:9-41: random bias, do = 1."""
+    from tpa import mha
+
+    rng = np.random.default_rng(21)
+    q, k, v = (rng.standard_normal(s).astype(np.float32) for s in ((batch, lq, h, dk), (batch, lk, h, dk), (batch, lk, h, dv)))
+    bias = rng.standard_normal((batch, lq, lk)).astype(np.float32)
+    o, res = mha._mha_fwd(*(torch.from_numpy(x).to(gpu) for x in (q, k, v)), torch.from_numpy(bias).to(gpu), sm_scale)
+    dq, dk_, dv_, _, _ = mha._mha_bwd(res, torch.ones_like(o))
+    want = orc.mha_backward(q.astype(np.float64), k.astype(np.float64), v.astype(np.float64), bias.astype(np.float64), sm_scale, np.ones((batch, lq, h, dv)))
+    for g, w in zip((dq, dk_, dv_), want):
+        np.testing.assert_allclose(g.cpu().numpy(), w, atol=1e-5, rtol=1e-4)
+
+
+def test_mha_backward_known_answer(gpu):
+    """tpa/mha_test.py:44-118: the literal case with -inf bias; dq = dk = 0, dv = [[1,1],[0,0],[1,1]]."""
+    from tpa import mha
+
+    q = torch.tensor([[2.0, 1.0], [1.0, 1.0], [1.0, 1.0]], device=gpu)[None, :, None, :].requires_grad_()
+    k = torch.ones((1, 3, 1, 2), device=gpu, requires_grad=True)
+    v = torch.ones((1, 3, 1, 2), device=gpu, requires_grad=True)
+    ninf = float("-inf")
+    bias = torch.tensor([[0, ninf, 0], [0, ninf, 0], [ninf, ninf, ninf]], device=gpu)[None]
+    o = mha.mha(q, k, v, bias)
+    torch.nansum(o).backward()
+    assert torch.equal(q.grad, torch.zeros_like(q))
+    assert torch.equal(k.grad, torch.zeros_like(k))
+    np.testing.assert_allclose(v.grad[0, :, 0].cpu().numpy(), [[1, 1], [0, 0], [1, 1]], atol=1e-6)
+
+
+def test_mha_backward_bf16_causal(gpu):
+    from tpa import mha
+
+    b, l, h, d = 2, 300, 4, 64
+    rng = np.random.default_rng(22)
+    q, k, v, do = (torch.from_numpy(rng.standard_normal((b, l, h, d)).astype(np.float32)).to(gpu).to(torch.bfloat16) for _ in range(4))
+    q.requires_grad_(), k.requires_grad_(), v.requires_grad_()
+    o = mha.mha(q, k, v, None, d**-0.5, causal=True)
+    o.backward(do)
+    f64 = lambda t: t.detach().float().cpu().numpy().astype(np.float64)
+    bias = np.where(np.tril(np.ones((l, l), bool)), 0.0, -np.inf)[None].repeat(b, 0)
+    want = orc.mha_backward(f64(q), f64(k), f64(v), bias, d**-0.5, f64(do))
+    for t, w in zip((q, k, v), want):
+        assert rel_err(f64(t.grad), w) <= 2e-2
+
+
+def test_backward_error_codes(gpu):
+    """A too small workspace is refused, and there is no MFMA backward kernel to ask for."""
+    import ctypes
+
+    from tpa import _dispatch as d
+    from tpa import tpa
+
+    q, k, v = make_factors(15, 1, 16, 16, 2, 8, 8, 2, 2)
+    tq, tk, tv = (torch.from_numpy(x).to(gpu) for x in (q, k, v))
+    o, res = tpa._tpa_fwd(tq, tk, tv, 2, None, None, 1.0, False, None, False, False, False)
+    with pytest.raises(d.TpaError) as e:
+        tpa.tpa_factors_bwd(tq[..., :2], tq[..., 2:], tk[..., :2], tk[..., 2:], tv[..., :2], tv[..., 2:], None, None,
+                            o, res[-1].permute(0, 2, 1), torch.ones_like(o), workspace=torch.empty(1024, dtype=torch.uint8, device=gpu))
+    assert e.value.code == -5

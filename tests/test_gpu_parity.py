@@ -334,7 +334,7 @@ def test_mha_fp32_vs_oracle(gpu, with_bias):
         bias[rng.random((b, lq, lk)) < 0.3] = -np.inf
         bias[:, 5] = -np.inf  # one empty row
     o_ref, l_ref = orc.mha_forward(q.astype(np.float64), k.astype(np.float64), v.astype(np.float64), None if bias is None else bias.astype(np.float64), 0.5)
-    o, (lse,) = _mha_fwd(torch.from_numpy(q).to(gpu), torch.from_numpy(k).to(gpu), torch.from_numpy(v).to(gpu), bias, 0.5)
+    o, (lse, *_) = _mha_fwd(torch.from_numpy(q).to(gpu), torch.from_numpy(k).to(gpu), torch.from_numpy(v).to(gpu), bias, 0.5)
     check(o, lse, o_ref, l_ref, F32_TOL)
 
 
@@ -350,7 +350,7 @@ def test_mha_bf16_flash_vs_oracle(gpu, d, causal):
     if causal:
         bias = np.where(np.tril(np.ones((lq, lk), bool)), 0.0, -np.inf)[None].repeat(b, 0)
     o_ref, l_ref = orc.mha_forward(as_f64(q), as_f64(k), as_f64(v), bias, d**-0.5)
-    o, (lse,) = _mha_fwd(q, k, v, None, d**-0.5, causal=causal, kernel=2)
+    o, (lse, *_) = _mha_fwd(q, k, v, None, d**-0.5, causal=causal, kernel=2)
     check(o, lse, o_ref, l_ref, BF16_TOL, lse_tol=2e-3)
 
 
@@ -395,7 +395,7 @@ def test_mha_decode_bf16_vs_oracle(gpu, b, lq, lk, h, d):
     q, k, v = (torch.from_numpy(rng.standard_normal(s, dtype=np.float32)).to(torch.bfloat16).to(gpu)
                for s in ((b, lq, h, d), (b, lk, h, d), (b, lk, h, d)))
     o_ref, l_ref = orc.mha_forward(as_f64(q), as_f64(k), as_f64(v), None, d**-0.5)
-    o, (lse,) = _mha_fwd(q, k, v, None, d**-0.5, kernel=2)
+    o, (lse, *_) = _mha_fwd(q, k, v, None, d**-0.5, kernel=2)
     check(o, lse, o_ref, l_ref, BF16_TOL)
 
 
