@@ -105,12 +105,15 @@ int tpa_bwd(const TpaBwdArgs* a, void* stream) {
     if (!g->ptr) return TPA_ERR_NULL;
   if (!a->o || !a->lse || !a->d_o) return TPA_ERR_NULL;
   if ((a->q_segment_ids == nullptr) != (a->kv_segment_ids == nullptr)) return TPA_ERR_NULL;
-  if (a->kernel == TPA_KERNEL_MFMA) return TPA_ERR_UNSUPPORTED;  // there is no MFMA backward kernel
-  if (a->kernel != TPA_KERNEL_AUTO && a->kernel != TPA_KERNEL_GENERIC) return TPA_ERR_UNSUPPORTED;
+  if (a->kernel != TPA_KERNEL_AUTO && a->kernel != TPA_KERNEL_GENERIC && a->kernel != TPA_KERNEL_MFMA)
+    return TPA_ERR_UNSUPPORTED;
+  const int mfma = a->kernel != TPA_KERNEL_GENERIC &&
+                   dense_bwd_mfma_supported(a->dtype, a->dk, a->dv, a->lq, a->lk, a->H, a->sm_scale, nullptr);
+  if (a->kernel == TPA_KERNEL_MFMA && !mfma) return TPA_ERR_UNSUPPORTED;
   if (!a->workspace || a->workspace_bytes < tpa_bwd_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dk, a->dv))
     return TPA_ERR_WORKSPACE;
   if (reinterpret_cast<uintptr_t>(a->workspace) & 255) return TPA_ERR_ALIGN;
-  return tpa_bwd_generic_launch(a, static_cast<hipStream_t>(stream));
+  return tpa_bwd_launch(a, static_cast<hipStream_t>(stream), mfma);
 }
 
 size_t tpa_bwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dk, int32_t dv) {
@@ -124,12 +127,19 @@ int mha_bwd(const MhaBwdArgs* a, void* stream) {
   if (a->B <= 0 || a->lq <= 0 || a->lk <= 0 || a->H <= 0 || a->dk <= 0 || a->dv <= 0) return TPA_ERR_SHAPE;
   if (a->dk > 256 || a->dv > 256) return TPA_ERR_SHAPE;
   if (!a->q || !a->k || !a->v || !a->o || !a->lse || !a->d_o || !a->dq || !a->dk_out || !a->dv_out) return TPA_ERR_NULL;
-  if (a->kernel == TPA_KERNEL_MFMA) return TPA_ERR_UNSUPPORTED;
-  if (a->kernel != TPA_KERNEL_AUTO && a->kernel != TPA_KERNEL_GENERIC) return TPA_ERR_UNSUPPORTED;
+  if (a->kernel != TPA_KERNEL_AUTO && a->kernel != TPA_KERNEL_GENERIC && a->kernel != TPA_KERNEL_MFMA)
+    return TPA_ERR_UNSUPPORTED;
+  const int mfma = a->kernel != TPA_KERNEL_GENERIC &&
+                   dense_bwd_mfma_supported(a->dtype, a->dk, a->dv, a->lq, a->lk, a->H, a->sm_scale, a->bias) &&
+                   !(reinterpret_cast<uintptr_t>(a->q) & 15) && !(reinterpret_cast<uintptr_t>(a->k) & 15) &&
+                   !(reinterpret_cast<uintptr_t>(a->v) & 15) && !(reinterpret_cast<uintptr_t>(a->d_o) & 15) &&
+                   !(reinterpret_cast<uintptr_t>(a->dq) & 15) && !(reinterpret_cast<uintptr_t>(a->dk_out) & 15) &&
+                   !(reinterpret_cast<uintptr_t>(a->dv_out) & 15);
+  if (a->kernel == TPA_KERNEL_MFMA && !mfma) return TPA_ERR_UNSUPPORTED;
   if (!a->workspace || a->workspace_bytes < mha_bwd_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dk, a->dv, a->dtype))
     return TPA_ERR_WORKSPACE;
   if (reinterpret_cast<uintptr_t>(a->workspace) & 255) return TPA_ERR_ALIGN;
-  return mha_bwd_generic_launch(a, static_cast<hipStream_t>(stream));
+  return mha_bwd_launch(a, static_cast<hipStream_t>(stream), mfma);
 }
 
 size_t mha_bwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dk, int32_t dv, int32_t dtype) {

@@ -1,6 +1,7 @@
 // Backward pass: gradients of the attention output with respect to the rank factors
 // (tpa/tpa.py:168-214,546-995) and, for the dense baseline, with respect to q, k, v
-// (tpa/mha.py:40-65).  Any-shape fp32 arithmetic on the vector ALUs.
+// (tpa/mha.py:40-65).  Any-shape fp32 arithmetic on the vector ALUs, except stages 3 and 4, which
+// run on the matrix cores for bf16 inputs with a head size of 64 or 128.
 //
 // The factored problem is taken through dense intermediates that live in the caller's
 // workspace, so that every stage is a plain, separately checkable kernel:
@@ -24,18 +25,18 @@ constexpr int kThreads = 128;  // rows (dq) or keys (dkv) per workgroup
 constexpr int tile_of(int dmax) { return dmax > 128 ? 16 : 32; }
 
 // ------------------------------------------------------------------------------------ stage 1
-template <typename T>
-__global__ void recon_kernel(TpaFactor fa, TpaFactor fb, float* out, int L, int H, int D, int R) {
+template <typename T, typename TO>
+__global__ void recon_kernel(TpaFactor fa, TpaFactor fb, TO* out, int L, int H, int D, int R) {
   const int t = blockIdx.x, b = blockIdx.y;
   const T* ap = static_cast<const T*>(fa.ptr) + b * fa.stride_b + t * fa.stride_l;
   const T* bp = static_cast<const T*>(fb.ptr) + b * fb.stride_b + t * fb.stride_l;
-  float* op = out + ((int64_t)b * L + t) * H * D;
+  TO* op = out + ((int64_t)b * L + t) * H * D;
   const float inv = 1.f / (float)R;
   for (int idx = threadIdx.x; idx < H * D; idx += blockDim.x) {
     const int h = idx / D, d = idx - h * D;
     float acc = 0.f;
     for (int r = 0; r < R; ++r) acc += load_as_f32(ap + r * fa.stride_r + h) * load_as_f32(bp + r * fb.stride_r + d);
-    op[idx] = acc * inv;
+    store_from_f32(op + idx, acc * inv);
   }
 }
 
@@ -299,28 +300,42 @@ int launch_dense(const DenseParams& p, hipStream_t stream) {
 inline size_t align256(size_t n) { return (n + 255) & ~size_t(255); }
 
 template <typename T>
-int tpa_bwd_t(const TpaBwdArgs* a, hipStream_t stream) {
+int tpa_bwd_t(const TpaBwdArgs* a, hipStream_t stream, bool mfma) {
   const size_t nq = (size_t)a->B * a->lq * a->H * a->dk, nk = (size_t)a->B * a->lk * a->H * a->dk,
                nv = (size_t)a->B * a->lk * a->H * a->dv, nd = (size_t)a->B * a->H * a->lq;
   char* w = static_cast<char*>(a->workspace);
   auto take = [&](size_t floats) { float* ptr = reinterpret_cast<float*>(w); w += align256(floats * sizeof(float)); return ptr; };
+  // dense Q, K, V (fp32, or bf16 for the MFMA kernels: then only half of each slot is used)
   float *qd = take(nq), *kd = take(nk), *vd = take(nv), *dqd = take(nq), *dkd = take(nk), *dvd = take(nv), *delta = take(nd);
 
   const int threads = 256;
-  hipLaunchKernelGGL((recon_kernel<T>), dim3(a->lq, a->B), dim3(threads), 0, stream, a->qa, a->qb, qd, a->lq, a->H, a->dk, a->rq);
-  hipLaunchKernelGGL((recon_kernel<T>), dim3(a->lk, a->B), dim3(threads), 0, stream, a->ka, a->kb, kd, a->lk, a->H, a->dk, a->rk);
-  hipLaunchKernelGGL((recon_kernel<T>), dim3(a->lk, a->B), dim3(threads), 0, stream, a->va, a->vb, vd, a->lk, a->H, a->dv, a->rk);
+  if (mfma) {
+    uint16_t *q16 = reinterpret_cast<uint16_t*>(qd), *k16 = reinterpret_cast<uint16_t*>(kd), *v16 = reinterpret_cast<uint16_t*>(vd);
+    hipLaunchKernelGGL((recon_kernel<T, uint16_t>), dim3(a->lq, a->B), dim3(threads), 0, stream, a->qa, a->qb, q16, a->lq, a->H, a->dk, a->rq);
+    hipLaunchKernelGGL((recon_kernel<T, uint16_t>), dim3(a->lk, a->B), dim3(threads), 0, stream, a->ka, a->kb, k16, a->lk, a->H, a->dk, a->rk);
+    hipLaunchKernelGGL((recon_kernel<T, uint16_t>), dim3(a->lk, a->B), dim3(threads), 0, stream, a->va, a->vb, v16, a->lk, a->H, a->dv, a->rk);
+  } else {
+    hipLaunchKernelGGL((recon_kernel<T, float>), dim3(a->lq, a->B), dim3(threads), 0, stream, a->qa, a->qb, qd, a->lq, a->H, a->dk, a->rq);
+    hipLaunchKernelGGL((recon_kernel<T, float>), dim3(a->lk, a->B), dim3(threads), 0, stream, a->ka, a->kb, kd, a->lk, a->H, a->dk, a->rk);
+    hipLaunchKernelGGL((recon_kernel<T, float>), dim3(a->lk, a->B), dim3(threads), 0, stream, a->va, a->vb, vd, a->lk, a->H, a->dv, a->rk);
+  }
   hipLaunchKernelGGL((delta_kernel<T>), dim3((unsigned)((nd + threads - 1) / threads)), dim3(threads), 0, stream,
                      static_cast<const T*>(a->o), static_cast<const T*>(a->d_o), delta, a->B, a->lq, a->H, a->dv);
   if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
 
-  DenseParams p{};
-  p.q = qd; p.k = kd; p.v = vd; p.d_o = a->d_o; p.lse = a->lse; p.delta = delta;
-  p.qseg = a->q_segment_ids; p.kvseg = a->kv_segment_ids; p.bias = nullptr;
-  p.dq = dqd; p.dk_out = dkd; p.dv_out = dvd;
-  p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.dk = a->dk; p.dv = a->dv;
-  p.sm_scale = a->sm_scale; p.causal = a->causal;
-  const int rc = launch_dense<T>(p, stream);
+  int rc;
+  if (mfma) {
+    rc = dense_bwd_mfma_launch(qd, kd, vd, a->d_o, a->lse, delta, a->q_segment_ids, a->kv_segment_ids, dqd, dkd, dvd,
+                               a->B, a->lq, a->lk, a->H, a->dk, a->sm_scale, a->causal, stream);
+  } else {
+    DenseParams p{};
+    p.q = qd; p.k = kd; p.v = vd; p.d_o = a->d_o; p.lse = a->lse; p.delta = delta;
+    p.qseg = a->q_segment_ids; p.kvseg = a->kv_segment_ids; p.bias = nullptr;
+    p.dq = dqd; p.dk_out = dkd; p.dv_out = dvd;
+    p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.dk = a->dk; p.dv = a->dv;
+    p.sm_scale = a->sm_scale; p.causal = a->causal;
+    rc = launch_dense<T>(p, stream);
+  }
   if (rc != TPA_OK) return rc;
 
   hipLaunchKernelGGL((project_kernel<T>), dim3(a->lq, a->B), dim3(threads), 0, stream, dqd, a->qa, a->qb, a->dqa, a->dqb, a->lq, a->H, a->dk, a->rq);
@@ -330,14 +345,20 @@ int tpa_bwd_t(const TpaBwdArgs* a, hipStream_t stream) {
 }
 
 template <typename T>
-int mha_bwd_t(const MhaBwdArgs* a, hipStream_t stream) {
+int mha_bwd_t(const MhaBwdArgs* a, hipStream_t stream, bool mfma) {
   const size_t nq = (size_t)a->B * a->lq * a->H * a->dk, nk = (size_t)a->B * a->lk * a->H * a->dk,
                nv = (size_t)a->B * a->lk * a->H * a->dv, nd = (size_t)a->B * a->H * a->lq;
   char* w = static_cast<char*>(a->workspace);
   auto take = [&](size_t floats) { float* ptr = reinterpret_cast<float*>(w); w += align256(floats * sizeof(float)); return ptr; };
   float* delta = take(nd);
-  const float *qd, *kd, *vd;
   const int threads = 256;
+  hipLaunchKernelGGL((delta_kernel<T>), dim3((unsigned)((nd + threads - 1) / threads)), dim3(threads), 0, stream,
+                     static_cast<const T*>(a->o), static_cast<const T*>(a->d_o), delta, a->B, a->lq, a->H, a->dv);
+  if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
+  if (mfma)
+    return dense_bwd_mfma_launch(a->q, a->k, a->v, a->d_o, a->lse, delta, nullptr, nullptr, a->dq, a->dk_out, a->dv_out,
+                                 a->B, a->lq, a->lk, a->H, a->dk, a->sm_scale, a->causal, stream);
+  const float *qd, *kd, *vd;
   if constexpr (sizeof(T) == sizeof(float)) {
     qd = static_cast<const float*>(a->q); kd = static_cast<const float*>(a->k); vd = static_cast<const float*>(a->v);
   } else {
@@ -348,8 +369,6 @@ int mha_bwd_t(const MhaBwdArgs* a, hipStream_t stream) {
     hipLaunchKernelGGL((to_f32_kernel<T>), blocks(nv), dim3(threads), 0, stream, static_cast<const T*>(a->v), v32, (int64_t)nv);
     qd = q32; kd = k32; vd = v32;
   }
-  hipLaunchKernelGGL((delta_kernel<T>), dim3((unsigned)((nd + threads - 1) / threads)), dim3(threads), 0, stream,
-                     static_cast<const T*>(a->o), static_cast<const T*>(a->d_o), delta, a->B, a->lq, a->H, a->dv);
   if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
   DenseParams p{};
   p.q = qd; p.k = kd; p.v = vd; p.d_o = a->d_o; p.lse = a->lse; p.delta = delta;
@@ -377,16 +396,16 @@ size_t mha_bwd_workspace_size(int64_t B, int64_t lq, int64_t lk, int64_t H, int6
   return bytes;
 }
 
-int tpa_bwd_generic_launch(const TpaBwdArgs* a, hipStream_t stream) {
+int tpa_bwd_launch(const TpaBwdArgs* a, hipStream_t stream, int mfma) {
   if (a->B > 65535 || a->H > 65535) return TPA_ERR_SHAPE;
-  if (a->dtype == TPA_DTYPE_F32) return tpa::tpa_bwd_t<float>(a, stream);
-  if (a->dtype == TPA_DTYPE_BF16) return tpa::tpa_bwd_t<uint16_t>(a, stream);
+  if (a->dtype == TPA_DTYPE_F32) return tpa::tpa_bwd_t<float>(a, stream, false);
+  if (a->dtype == TPA_DTYPE_BF16) return tpa::tpa_bwd_t<uint16_t>(a, stream, mfma != 0);
   return TPA_ERR_DTYPE;
 }
 
-int mha_bwd_generic_launch(const MhaBwdArgs* a, hipStream_t stream) {
+int mha_bwd_launch(const MhaBwdArgs* a, hipStream_t stream, int mfma) {
   if (a->B > 65535 || a->H > 65535) return TPA_ERR_SHAPE;
-  if (a->dtype == TPA_DTYPE_F32) return tpa::mha_bwd_t<float>(a, stream);
-  if (a->dtype == TPA_DTYPE_BF16) return tpa::mha_bwd_t<uint16_t>(a, stream);
+  if (a->dtype == TPA_DTYPE_F32) return tpa::mha_bwd_t<float>(a, stream, false);
+  if (a->dtype == TPA_DTYPE_BF16) return tpa::mha_bwd_t<uint16_t>(a, stream, mfma != 0);
   return TPA_ERR_DTYPE;
 }

@@ -1,0 +1,525 @@
+// Backward pass of dense flash attention on the matrix cores (bf16 MFMA, fp32 accumulation),
+// used for the dense baseline (tpa/mha.py:40-65) and - between a reconstruction of dense Q, K, V
+// from the rank factors and a projection of the dense gradients back onto them - for tensor
+// product attention (tpa/tpa.py:546-962).
+//
+// The softmax matrix is recomputed from the saved logsumexp, as in the forward kernel with the
+// roles of the MFMA operands chosen so that nothing ever goes through LDS between two
+// contractions (v_mfma_f32_32x32x16_bf16; "lane" = the accumulator column a lane owns):
+//
+//   bwd_dq_kernel   one workgroup = 256 query rows of one head, a wave owns 32 rows, lane = row
+//     S^T  = K Q^T            A = K rows (LDS),      B = Q (registers, pre-scaled), addend -lse
+//     dP^T = V dO^T           A = V rows (LDS),      B = dO (registers),            addend -delta
+//     dS^T = exp2(S^T) * dP^T  in registers, packed to bf16 in place
+//     dQ^T += K^T dS^T        A = K^T (transposed LDS reads), B = dS^T
+//
+//   bwd_dkv_kernel  one workgroup = 32 keys per wave of one head, lane = key
+//     S  = Q K^T              A = Q rows (LDS),      B = K (registers, pre-scaled), addend -lse[row]
+//     dP = dO V^T             A = dO rows (LDS),     B = V (registers),             addend -delta[row]
+//     dV^T += dO^T P          A = dO^T (transposed LDS reads), B = P
+//     dK^T += Q^T dS          A = Q^T  (transposed LDS reads), B = dS
+//
+// with p = exp(x - lse), ds = sm_scale * p * (dp - delta) (tpa/tpa.py:765-781, tpa/mha.py:57-63).
+// Rows without a visible key carry lse = -inf and contribute nothing (tpa/tpa.py:675-676).
+#include <type_traits>
+#include <utility>
+
+#include "tpa_common.h"
+
+namespace tpa {
+namespace {
+
+constexpr int kTile = 64;  // keys (dq kernel) or query rows (dkv kernel) per LDS tile
+
+struct BwdParams {
+  const uint16_t* q;    // [B, lq, H, D] bf16
+  const uint16_t* k;    // [B, lk, H, D]
+  const uint16_t* v;    // [B, lk, H, D]
+  const uint16_t* d_o;  // [B, lq, H, D]
+  const float* lse;     // [B, H, lq] natural log
+  const float* delta;   // [B, H, lq]
+  const int32_t* qseg;  // [B, lq] or null
+  const int32_t* kvseg; // [B, lk] or null
+  float* dq;            // [B, lq, H, D] fp32
+  float* dk;            // [B, lk, H, D]
+  float* dv;            // [B, lk, H, D]
+  int B, lq, lk, H;
+  float sm_scale;
+  int causal;
+  int nblk;    // row blocks (dq) or key blocks (dkv) per (batch, head)
+  int npairs;  // nblk * B
+};
+
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+constexpr int kRsrcFlags = 0x00020000;  // raw 32-bit data format
+
+// A-operand fragment of rows 32 mb .. 32 mb + 31 of a row-major tile (row stride S elements),
+// contraction columns 16 kk .. 16 kk + 15: lane (i, g) reads 8 elements of row 32 mb + i.
+template <int S>
+__device__ __forceinline__ bf16x8 rows_frag(const uint16_t* tile, int mb, int kk, int i, int g) {
+  return *reinterpret_cast<const bf16x8*>(tile + (32 * mb + i) * S + 16 * kk + 8 * g);
+}
+// A-operand fragment of the TRANSPOSED tile: output rows = tile columns 32 db .. 32 db + 31,
+// contraction = tile rows 16 kk .. 16 kk + 15 in the slot order an accumulator column already has
+// (slot (g, j) = tile row 16 kk + 8 (j / 4) + 4 g + j % 4).
+template <int S>
+__device__ __forceinline__ bf16x8 cols_frag(const uint16_t* tile, int kk, int db, int g, int lp, int dhalf) {
+  const uint16_t* row = tile + (16 * kk + 4 * g + (lp >> 2)) * S + 16 * dhalf + 4 * (lp & 3) + 32 * db;
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(row));
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(row + 8 * S));
+  return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+// 16 fp32 values of one accumulator block -> two B-operand fragments (contraction steps 2 mb, 2 mb + 1)
+__device__ __forceinline__ void pack_block(const f32x16& x, bf16x8& f0, bf16x8& f1) {
+  u32x4 a, b;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    a[j] = pack_bf16(x[2 * j], x[2 * j + 1]);
+    b[j] = pack_bf16(x[8 + 2 * j], x[8 + 2 * j + 1]);
+  }
+  f0 = __builtin_bit_cast(bf16x8, a);
+  f1 = __builtin_bit_cast(bf16x8, b);
+}
+
+__device__ __forceinline__ f32x16 splat16(float x) {
+  f32x16 r;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) r[v] = x;
+  return r;
+}
+
+// ============================================================================================
+// dQ
+// ============================================================================================
+template <int D, bool SEG>
+__global__ __launch_bounds__(512) void bwd_dq_kernel(BwdParams p) {
+  constexpr int NT = 512, S = D + 8, CPR = D / 8, TPP = NT / CPR, NPASS = kTile / TPP;
+  constexpr int NKS = D / 16, NDB = D / 32, kBQ = 256;
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  uint16_t* const lds_k = smem;                  // [2][64][S]
+  uint16_t* const lds_v = smem + 2 * kTile * S;  // [2][64][S]
+  int32_t* const lds_seg = reinterpret_cast<int32_t*>(smem + 4 * kTile * S);  // [2][64]
+
+  const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
+  const int pair = (slot / p.H) * 8 + xcd, h = slot % p.H;
+  if (pair >= p.npairs) return;
+  const int qblk = p.nblk - 1 - pair / p.B, b = pair % p.B;  // heaviest causal blocks first
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
+  const int lp = l & 15, dhalf = (l >> 4) & 1;
+  const int q0 = qblk * kBQ, wrow0 = q0 + 32 * w, qrow = wrow0 + i, qrow_ld = min(qrow, p.lq - 1);
+  const float c = p.sm_scale * kLog2e;
+
+  // this lane's row: Q (scaled) and dO as B-operand fragments, -lse (log2 domain) and -delta
+  const float lse_r = p.lse[((int64_t)b * p.H + h) * p.lq + qrow_ld];
+  const bool live = qrow < p.lq && lse_r > -INFINITY;
+  const f32x16 nlse = splat16(live ? -lse_r * kLog2e : -INFINITY);
+  const f32x16 ndelta = splat16(-p.delta[((int64_t)b * p.H + h) * p.lq + qrow_ld]);
+  bf16x8 qf[NKS], gf[NKS];
+  {
+    const uint16_t* qp = p.q + (((int64_t)b * p.lq + qrow_ld) * p.H + h) * D;
+    const uint16_t* gp = p.d_o + (((int64_t)b * p.lq + qrow_ld) * p.H + h) * D;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(qp + 16 * ks + 8 * g);
+      u32x4 sc, gr = *reinterpret_cast<const u32x4*>(gp + 16 * ks + 8 * g);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        sc[j] = pack_bf16(bf16lo_to_f32(raw[j]) * c, bf16hi_to_f32(raw[j]) * c);
+        if (!live) gr[j] = 0u;  // the upstream gradient of a row without a visible key may be NaN
+      }
+      qf[ks] = __builtin_bit_cast(bf16x8, sc);
+      gf[ks] = __builtin_bit_cast(bf16x8, gr);
+    }
+  }
+  const int32_t qseg = SEG ? p.qseg[(int64_t)b * p.lq + qrow_ld] : 0;
+
+  const int kend = p.causal ? min(p.lk, min(q0 + kBQ, p.lq)) : p.lk;
+  const int ntiles = (kend + kTile - 1) / kTile, last = ntiles - 1;
+  const int wave_last_tile = p.causal ? min(last, (wrow0 + 31) / kTile) : last;
+
+  // tile loader: raw buffer loads one tile ahead (rows past kend read as zero), stored to LDS later
+  const int lt = tid / CPR, lc = tid % CPR;
+  const int64_t tok_stride = (int64_t)p.H * D;
+  const int bytes = (int)(((int64_t)(kend - 1) * tok_stride + D) * 2);
+  const __amdgpu_buffer_rsrc_t k_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.k + ((int64_t)b * p.lk * p.H + h) * D), 0, bytes, kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.v + ((int64_t)b * p.lk * p.H + h) * D), 0, bytes, kRsrcFlags);
+  const int voff = (int)((lt * tok_stride + 8 * lc) * 2);
+  u32x4 kreg[NPASS], vreg[NPASS];
+  int32_t seg_pending = 0;
+  auto issue = [&](int tile) __attribute__((always_inline)) {
+#pragma unroll
+    for (int ps = 0; ps < NPASS; ++ps) {
+      const int soff = (int)((int64_t)(tile * kTile + ps * TPP) * tok_stride * 2);
+      kreg[ps] = __builtin_amdgcn_raw_buffer_load_b128(k_rs, voff, soff, 0);
+      vreg[ps] = __builtin_amdgcn_raw_buffer_load_b128(v_rs, voff, soff, 0);
+    }
+    if constexpr (SEG)
+      if (tid < kTile) seg_pending = p.kvseg[(int64_t)b * p.lk + min(tile * kTile + tid, p.lk - 1)];
+  };
+  auto commit = [&](int tile) __attribute__((always_inline)) {
+    uint16_t* kd = lds_k + (tile & 1) * kTile * S;
+    uint16_t* vd = lds_v + (tile & 1) * kTile * S;
+#pragma unroll
+    for (int ps = 0; ps < NPASS; ++ps) {
+      const int t = ps * TPP + lt;
+      *reinterpret_cast<u32x4*>(kd + t * S + 8 * lc) = kreg[ps];
+      *reinterpret_cast<u32x4*>(vd + t * S + 8 * lc) = vreg[ps];
+    }
+    if constexpr (SEG)
+      if (tid < kTile) lds_seg[(tile & 1) * kTile + tid] = seg_pending;
+  };
+
+  f32x16 acc[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) acc[db] = splat16(0.f);
+
+  auto compute = [&](int j) __attribute__((always_inline)) {
+    const uint16_t* ks = lds_k + (j & 1) * kTile * S;
+    const uint16_t* vs = lds_v + (j & 1) * kTile * S;
+    const int k0 = j * kTile;
+    const bool need_mask = (k0 + kTile > kend) || (p.causal && (k0 + kTile - 1 > wrow0));
+    const int limit = p.causal ? min(qrow, kend - 1) : kend - 1;  // largest visible key index
+    static_for<2>([&](auto mb_c) __attribute__((always_inline)) {
+      constexpr int mb = decltype(mb_c)::value;
+      f32x16 s = nlse, dp = ndelta;
+      static_for<NKS>([&](auto kk_c) __attribute__((always_inline)) {
+        constexpr int kk = decltype(kk_c)::value;
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rows_frag<S>(ks, mb, kk, i, g), qf[kk], s, 0, 0, 0);
+      });
+      static_for<NKS>([&](auto kk_c) __attribute__((always_inline)) {
+        constexpr int kk = decltype(kk_c)::value;
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rows_frag<S>(vs, mb, kk, i, g), gf[kk], dp, 0, 0, 0);
+      });
+      if (need_mask) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          if (k0 + 32 * mb + 8 * (v >> 2) + 4 * g + (v & 3) > limit) s[v] = -INFINITY;
+      }
+      if constexpr (SEG) {
+        const int32_t* ids_p = lds_seg + (j & 1) * kTile + 32 * mb + 4 * g;
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) {
+          const int4 ids = *reinterpret_cast<const int4*>(ids_p + 8 * vq);
+          if (ids.x != qseg) s[4 * vq] = -INFINITY;
+          if (ids.y != qseg) s[4 * vq + 1] = -INFINITY;
+          if (ids.z != qseg) s[4 * vq + 2] = -INFINITY;
+          if (ids.w != qseg) s[4 * vq + 3] = -INFINITY;
+        }
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s[v] = __builtin_amdgcn_exp2f(s[v]) * dp[v];  // p * (dp - delta)
+      bf16x8 f0, f1;
+      pack_block(s, f0, f1);
+      static_for<NDB>([&](auto db_c) __attribute__((always_inline)) {
+        constexpr int db = decltype(db_c)::value;
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cols_frag<S>(ks, 2 * mb, db, g, lp, dhalf), f0, acc[db], 0, 0, 0);
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cols_frag<S>(ks, 2 * mb + 1, db, g, lp, dhalf), f1, acc[db], 0, 0, 0);
+      });
+    });
+  };
+
+  issue(0);
+  commit(0);
+  issue(min(1, last));
+  __syncthreads();
+  for (int j = 0; j < ntiles; ++j) {
+    if (j <= wave_last_tile) compute(j);
+    if (j + 1 < ntiles) {
+      commit(j + 1);
+      issue(min(j + 2, last));
+    }
+    lds_barrier();
+  }
+
+  if (qrow < p.lq) {
+    float* op = p.dq + (((int64_t)b * p.lq + qrow) * p.H + h) * D;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int vq = 0; vq < 4; ++vq) {
+        f32x4 out;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[e] = acc[db][4 * vq + e] * p.sm_scale;
+        *reinterpret_cast<f32x4*>(op + 32 * db + 8 * vq + 4 * g) = out;
+      }
+  }
+}
+
+// ============================================================================================
+// dK, dV
+// ============================================================================================
+template <int D, int NW, bool SEG>
+__global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
+  constexpr int NT = NW * 64, S = D + 8, CPR = D / 8, TPP = NT / CPR, NPASS = kTile / TPP;
+  constexpr int NKS = D / 16, NDB = D / 32, kBK = NW * 32;
+  static_assert(kTile % TPP == 0 && NPASS >= 1, "loader shape");
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  uint16_t* const lds_q = smem;                  // [2][64][S]
+  uint16_t* const lds_g = smem + 2 * kTile * S;  // [2][64][S]  upstream gradient rows
+  float* const lds_nlse = reinterpret_cast<float*>(smem + 4 * kTile * S);  // [2][64]  -lse * log2(e), -inf for dead rows
+  float* const lds_ndel = lds_nlse + 2 * kTile;                            // [2][64]  -delta
+  int32_t* const lds_seg = reinterpret_cast<int32_t*>(lds_ndel + 2 * kTile);  // [2][64]
+
+  const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
+  const int pair = (slot / p.H) * 8 + xcd, h = slot % p.H;
+  if (pair >= p.npairs) return;
+  const int kblk = pair / p.B, b = pair % p.B;  // under the causal mask the first key blocks are the heaviest
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
+  const int lp = l & 15, dhalf = (l >> 4) & 1;
+  const int k0 = kblk * kBK, wkey0 = k0 + 32 * w, key = wkey0 + i, key_ld = min(key, p.lk - 1);
+  const float c = p.sm_scale * kLog2e;
+
+  bf16x8 kf[NKS], vf[NKS];
+  {
+    const uint16_t* kp = p.k + (((int64_t)b * p.lk + key_ld) * p.H + h) * D;
+    const uint16_t* vp = p.v + (((int64_t)b * p.lk + key_ld) * p.H + h) * D;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(kp + 16 * ks + 8 * g);
+      u32x4 sc;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sc[j] = pack_bf16(bf16lo_to_f32(raw[j]) * c, bf16hi_to_f32(raw[j]) * c);
+      kf[ks] = __builtin_bit_cast(bf16x8, sc);
+      vf[ks] = *reinterpret_cast<const bf16x8*>(vp + 16 * ks + 8 * g);
+    }
+  }
+  const int32_t kseg = SEG ? p.kvseg[(int64_t)b * p.lk + key_ld] : 0;
+
+  // query tiles: under the causal mask rows before this block's first key see none of its keys
+  const int tile0 = p.causal ? k0 / kTile : 0;
+  const int ntiles = max(0, (p.lq + kTile - 1) / kTile - tile0), last = ntiles - 1;
+  const int wave_first_tile = p.causal ? wkey0 / kTile - tile0 : 0;
+
+  const int lt = tid / CPR, lc = tid % CPR;
+  const int64_t tok_stride = (int64_t)p.H * D;
+  const int bytes = (int)(((int64_t)(p.lq - 1) * tok_stride + D) * 2);
+  const __amdgpu_buffer_rsrc_t q_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.q + ((int64_t)b * p.lq * p.H + h) * D), 0, bytes, kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t g_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.d_o + ((int64_t)b * p.lq * p.H + h) * D), 0, bytes, kRsrcFlags);
+  const int voff = (int)((lt * tok_stride + 8 * lc) * 2);
+  const float* lse_b = p.lse + ((int64_t)b * p.H + h) * p.lq;
+  const float* del_b = p.delta + ((int64_t)b * p.H + h) * p.lq;
+  u32x4 qreg[NPASS], greg[NPASS];
+  float row_lse[NPASS];   // lse of the rows this thread stages (their upstream gradient is zeroed if dead)
+  float aux_pending = 0.f;
+  auto issue = [&](int tile) __attribute__((always_inline)) {
+    const int r0 = (tile0 + tile) * kTile;
+#pragma unroll
+    for (int ps = 0; ps < NPASS; ++ps) {
+      const int soff = (int)((int64_t)(r0 + ps * TPP) * tok_stride * 2);
+      qreg[ps] = __builtin_amdgcn_raw_buffer_load_b128(q_rs, voff, soff, 0);
+      greg[ps] = __builtin_amdgcn_raw_buffer_load_b128(g_rs, voff, soff, 0);
+      const int r = r0 + ps * TPP + lt;
+      row_lse[ps] = r < p.lq ? lse_b[r] : -INFINITY;
+    }
+    // threads 0..63: -lse, 64..127: -delta, 128..191: segment id of row r0 + tid % 64
+    if (tid < 3 * kTile) {
+      const int r = r0 + (tid & (kTile - 1));
+      const int rl = min(r, p.lq - 1);
+      if (tid < kTile) {
+        const float x = lse_b[rl];
+        aux_pending = (r < p.lq && x > -INFINITY) ? -x * kLog2e : -INFINITY;
+      } else if (tid < 2 * kTile) {
+        aux_pending = -del_b[rl];
+      } else if (SEG) {
+        aux_pending = __int_as_float(p.qseg[(int64_t)b * p.lq + rl]);
+      }
+    }
+  };
+  auto commit = [&](int tile) __attribute__((always_inline)) {
+    uint16_t* qd = lds_q + (tile & 1) * kTile * S;
+    uint16_t* gd = lds_g + (tile & 1) * kTile * S;
+#pragma unroll
+    for (int ps = 0; ps < NPASS; ++ps) {
+      const int t = ps * TPP + lt;
+      u32x4 gr = greg[ps];
+      if (!(row_lse[ps] > -INFINITY)) gr = u32x4{0u, 0u, 0u, 0u};  // a dead row's upstream gradient may be NaN
+      *reinterpret_cast<u32x4*>(qd + t * S + 8 * lc) = qreg[ps];
+      *reinterpret_cast<u32x4*>(gd + t * S + 8 * lc) = gr;
+    }
+    if (tid < kTile) lds_nlse[(tile & 1) * kTile + tid] = aux_pending;
+    else if (tid < 2 * kTile) lds_ndel[(tile & 1) * kTile + tid - kTile] = aux_pending;
+    else if (SEG && tid < 3 * kTile) lds_seg[(tile & 1) * kTile + tid - 2 * kTile] = __float_as_int(aux_pending);
+  };
+
+  f32x16 dk_acc[NDB], dv_acc[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) { dk_acc[db] = splat16(0.f); dv_acc[db] = splat16(0.f); }
+
+  auto compute = [&](int j) __attribute__((always_inline)) {
+    const uint16_t* qs = lds_q + (j & 1) * kTile * S;
+    const uint16_t* gs = lds_g + (j & 1) * kTile * S;
+    const float* nl = lds_nlse + (j & 1) * kTile;
+    const float* nd = lds_ndel + (j & 1) * kTile;
+    const int r0 = (tile0 + j) * kTile;
+    const bool need_mask = p.causal && (r0 < wkey0 + 31);  // a row of the tile lies before a key of this wave
+    static_for<2>([&](auto mb_c) __attribute__((always_inline)) {
+      constexpr int mb = decltype(mb_c)::value;
+      // accumulator rows of this lane: 32 mb + 8 vq + 4 g + (0..3)
+      f32x16 s, dp;
+#pragma unroll
+      for (int vq = 0; vq < 4; ++vq) {
+        const f32x4 a = *reinterpret_cast<const f32x4*>(nl + 32 * mb + 8 * vq + 4 * g);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(nd + 32 * mb + 8 * vq + 4 * g);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { s[4 * vq + e] = a[e]; dp[4 * vq + e] = d4[e]; }
+      }
+      static_for<NKS>([&](auto kk_c) __attribute__((always_inline)) {
+        constexpr int kk = decltype(kk_c)::value;
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rows_frag<S>(qs, mb, kk, i, g), kf[kk], s, 0, 0, 0);
+      });
+      static_for<NKS>([&](auto kk_c) __attribute__((always_inline)) {
+        constexpr int kk = decltype(kk_c)::value;
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rows_frag<S>(gs, mb, kk, i, g), vf[kk], dp, 0, 0, 0);
+      });
+      if (need_mask) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          if (r0 + 32 * mb + 8 * (v >> 2) + 4 * g + (v & 3) < key) s[v] = -INFINITY;
+      }
+      if constexpr (SEG) {
+        const int32_t* ids_p = lds_seg + (j & 1) * kTile + 32 * mb + 4 * g;
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) {
+          const int4 ids = *reinterpret_cast<const int4*>(ids_p + 8 * vq);
+          if (ids.x != kseg) s[4 * vq] = -INFINITY;
+          if (ids.y != kseg) s[4 * vq + 1] = -INFINITY;
+          if (ids.z != kseg) s[4 * vq + 2] = -INFINITY;
+          if (ids.w != kseg) s[4 * vq + 3] = -INFINITY;
+        }
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        s[v] = __builtin_amdgcn_exp2f(s[v]);  // p
+        dp[v] *= s[v];                        // p * (dp - delta)
+      }
+      bf16x8 p0, p1, d0, d1;
+      pack_block(s, p0, p1);
+      pack_block(dp, d0, d1);
+      static_for<NDB>([&](auto db_c) __attribute__((always_inline)) {
+        constexpr int db = decltype(db_c)::value;
+        dv_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cols_frag<S>(gs, 2 * mb, db, g, lp, dhalf), p0, dv_acc[db], 0, 0, 0);
+        dv_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cols_frag<S>(gs, 2 * mb + 1, db, g, lp, dhalf), p1, dv_acc[db], 0, 0, 0);
+      });
+      static_for<NDB>([&](auto db_c) __attribute__((always_inline)) {
+        constexpr int db = decltype(db_c)::value;
+        dk_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cols_frag<S>(qs, 2 * mb, db, g, lp, dhalf), d0, dk_acc[db], 0, 0, 0);
+        dk_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cols_frag<S>(qs, 2 * mb + 1, db, g, lp, dhalf), d1, dk_acc[db], 0, 0, 0);
+      });
+    });
+  };
+
+  if (ntiles > 0) {
+    issue(0);
+    commit(0);
+    issue(min(1, last));
+    __syncthreads();
+    for (int j = 0; j < ntiles; ++j) {
+      if (j >= wave_first_tile) compute(j);
+      if (j + 1 < ntiles) {
+        commit(j + 1);
+        issue(min(j + 2, last));
+      }
+      lds_barrier();
+    }
+  }
+
+  if (key < p.lk) {
+    float* okp = p.dk + (((int64_t)b * p.lk + key) * p.H + h) * D;
+    float* ovp = p.dv + (((int64_t)b * p.lk + key) * p.H + h) * D;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int vq = 0; vq < 4; ++vq) {
+        f32x4 ok, ov;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          ok[e] = dk_acc[db][4 * vq + e] * p.sm_scale;
+          ov[e] = dv_acc[db][4 * vq + e];
+        }
+        *reinterpret_cast<f32x4*>(okp + 32 * db + 8 * vq + 4 * g) = ok;
+        *reinterpret_cast<f32x4*>(ovp + 32 * db + 8 * vq + 4 * g) = ov;
+      }
+  }
+}
+
+template <int D, bool SEG>
+int launch_dq(const BwdParams& base, hipStream_t stream) {
+  BwdParams p = base;
+  p.nblk = (p.lq + 255) / 256;
+  p.npairs = p.nblk * p.B;
+  auto kern = bwd_dq_kernel<D, SEG>;
+  const size_t smem = (size_t)4 * kTile * (D + 8) * 2 + 2 * kTile * 4;
+  static bool configured = false;
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+      return TPA_ERR_LAUNCH;
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(((p.npairs + 7) / 8) * 8 * p.H), dim3(512), smem, stream, p);
+  return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
+}
+
+template <int D, int NW, bool SEG>
+int launch_dkv(const BwdParams& base, hipStream_t stream) {
+  BwdParams p = base;
+  p.nblk = (p.lk + NW * 32 - 1) / (NW * 32);
+  p.npairs = p.nblk * p.B;
+  auto kern = bwd_dkv_kernel<D, NW, SEG>;
+  const size_t smem = (size_t)4 * kTile * (D + 8) * 2 + 6 * kTile * 4;
+  static bool configured = false;
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+      return TPA_ERR_LAUNCH;
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(((p.npairs + 7) / 8) * 8 * p.H), dim3(NW * 64), smem, stream, p);
+  return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
+}
+
+template <int D>
+int launch_both(const BwdParams& p, hipStream_t stream) {
+  constexpr int NW = D == 128 ? 4 : 8;  // D = 128: one wave per SIMD, its accumulators need the whole register file
+  int rc;
+  if (p.qseg) {
+    rc = launch_dq<D, true>(p, stream);
+    if (rc == TPA_OK) rc = launch_dkv<D, NW, true>(p, stream);
+  } else {
+    rc = launch_dq<D, false>(p, stream);
+    if (rc == TPA_OK) rc = launch_dkv<D, NW, false>(p, stream);
+  }
+  return rc;
+}
+
+}  // namespace
+}  // namespace tpa
+
+// dense bf16 q, k, v, d_o [B, l, H, D] with D in {64, 128}; every batch entry below 2 GiB
+int dense_bwd_mfma_supported(int dtype, int dk, int dv, int64_t lq, int64_t lk, int64_t H, float sm_scale, const void* bias) {
+  if (dtype != TPA_DTYPE_BF16 || dk != dv || (dk != 64 && dk != 128) || bias) return 0;
+  if (!(sm_scale > 0.f)) return 0;
+  const int64_t big = lq > lk ? lq : lk;
+  if (big * H * dk * 2 >= (int64_t(1) << 31)) return 0;
+  return 1;
+}
+
+int dense_bwd_mfma_launch(const void* q, const void* k, const void* v, const void* d_o, const float* lse, const float* delta,
+                          const int32_t* qseg, const int32_t* kvseg, float* dq, float* dk, float* dv, int B, int lq, int lk,
+                          int H, int D, float sm_scale, int causal, hipStream_t stream) {
+  tpa::BwdParams p{};
+  p.q = static_cast<const uint16_t*>(q); p.k = static_cast<const uint16_t*>(k); p.v = static_cast<const uint16_t*>(v);
+  p.d_o = static_cast<const uint16_t*>(d_o); p.lse = lse; p.delta = delta; p.qseg = qseg; p.kvseg = kvseg;
+  p.dq = dq; p.dk = dk; p.dv = dv; p.B = B; p.lq = lq; p.lk = lk; p.H = H; p.sm_scale = sm_scale; p.causal = causal;
+  if (D == 128) return tpa::launch_both<128>(p, stream);
+  return tpa::launch_both<64>(p, stream);
+}

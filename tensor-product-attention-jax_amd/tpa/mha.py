@@ -41,7 +41,7 @@ def _mha_fwd_impl(q, k, v, bias, sm_scale, causal, kernel):
     return o, lse, (q, k, v, bias_t)
 
 
-def _mha_bwd_impl(q, k, v, bias_t, o, lse, do, sm_scale, causal):
+def _mha_bwd_impl(q, k, v, bias_t, o, lse, do, sm_scale, causal, kernel=_d.KERNEL_AUTO):
     device = q.device
     b, lq, h, dk = q.shape
     _, lk, _, dv = v.shape
@@ -59,7 +59,7 @@ def _mha_bwd_impl(q, k, v, bias_t, o, lse, do, sm_scale, causal):
         o=o.data_ptr(), lse=lse.data_ptr(), d_o=do.data_ptr(),
         dq=dq.data_ptr(), dk_out=dk_.data_ptr(), dv_out=dv_.data_ptr(),
         B=b, lq=lq, lk=lk, H=h, dk=dk, dv=dv,
-        dtype=_d.dtype_code(q.dtype), sm_scale=float(sm_scale), causal=int(bool(causal)), kernel=_d.KERNEL_AUTO,
+        dtype=_d.dtype_code(q.dtype), sm_scale=float(sm_scale), causal=int(bool(causal)), kernel=int(kernel),
         workspace=ws.data_ptr() + pad, workspace_bytes=ws.numel() - pad,
     )
     with torch.cuda.device(device):
@@ -78,11 +78,11 @@ def _mha_fwd(q, k, v, bias, sm_scale, causal: bool = False, kernel: int = _d.KER
     return o, (lse, o, q, k, v, bias_t, float(sm_scale), bool(causal))
 
 
-def _mha_bwd(res, do):
+def _mha_bwd(res, do, kernel: int = _d.KERNEL_AUTO):
     """tpa/mha.py:40-65: (dq, dk, dv, None, None) in the dtype of q, k, v.  Rows whose logits
     were all -inf contribute nothing (tpa/mha.py:52-56)."""
     lse, o, q, k, v, bias_t, sm_scale, causal = res
-    dq, dk, dv = _mha_bwd_impl(q, k, v, bias_t, o, lse, do, sm_scale, causal)
+    dq, dk, dv = _mha_bwd_impl(q, k, v, bias_t, o, lse, do, sm_scale, causal, kernel)
     return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None
 
 

@@ -14,9 +14,10 @@ reference, all on purpose:
     non-materialising form;
   * `interpret=True` (the Pallas CPU interpreter upstream) selects the plain fp32-arithmetic
     kernel instead of the MFMA kernels; `debug` is ignored;
-  * the backward pass (tpa/tpa.py:168-214,546-995) runs as fp32 vector-ALU kernels through dense
-    intermediates (there is no MFMA backward kernel); gradients are computed in fp32 and cast to
-    the input dtype; torch.autograd reaches it through `tpa()`.
+  * the backward pass (tpa/tpa.py:168-214,546-995) goes through dense Q, K, V and dense gradients
+    in a workspace (bf16 MFMA kernels for head sizes 64 and 128, fp32 vector-ALU kernels
+    otherwise); gradients are accumulated in fp32 and cast to the input dtype; torch.autograd
+    reaches it through `tpa()`.
 """
 
 from __future__ import annotations
@@ -200,6 +201,7 @@ def tpa_factors_bwd(
     causal: bool = False,
     grads=None,
     workspace: torch.Tensor | None = None,
+    kernel: int = _d.KERNEL_AUTO,
 ):
     """Backward pass on the split factor arrays: the operands of the reference's backward kernel
     launch (tpa/tpa.py:872-958) with a leading batch dimension, `lse` as [b, h, lq] fp32.
@@ -237,7 +239,7 @@ def tpa_factors_bwd(
         dqa=_d.grad(grads[0]), dqb=_d.grad(grads[1]), dka=_d.grad(grads[2]), dkb=_d.grad(grads[3]),
         dva=_d.grad(grads[4]), dvb=_d.grad(grads[5]),
         B=b, lq=lq, lk=lk, H=h, dk=dk, dv=dv, rq=rq, rk=rk,
-        dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=int(bool(causal)), kernel=_d.KERNEL_AUTO,
+        dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=int(bool(causal)), kernel=int(kernel),
         workspace=workspace.data_ptr() + pad, workspace_bytes=workspace.numel() - pad,
     )
     with torch.cuda.device(device):

@@ -173,3 +173,83 @@ def test_backward_error_codes(gpu):
         tpa.tpa_factors_bwd(tq[..., :2], tq[..., 2:], tk[..., :2], tk[..., 2:], tv[..., :2], tv[..., 2:], None, None,
                             o, res[-1].permute(0, 2, 1), torch.ones_like(o), workspace=torch.empty(1024, dtype=torch.uint8, device=gpu))
     assert e.value.code == -5
+
+
+# ---------------------------------------------------------------- bf16 MFMA backward kernels
+def _bf16_case(gpu, seed, b, lq, lk, h, d, rq, rk, seg, causal, kernel):
+    from tpa import tpa
+
+    q, k, v = make_factors(seed, b, lq, lk, h, d, d, rq, rk, scale_by_rank=True)
+    do = np.random.default_rng(seed + 1).standard_normal((b, lq, h, d)).astype(np.float32)
+    qseg = segment_ids(lq, seg, b) if seg else None
+    kvseg = segment_ids(lk, seg, b) if seg else None
+    tq, tk, tv = (torch.from_numpy(x).to(gpu).to(torch.bfloat16) for x in (q, k, v))
+    tdo = torch.from_numpy(do).to(gpu).to(torch.bfloat16)
+    sp = lambda t: (t[..., :h], t[..., h:])
+    tqs = None if qseg is None else torch.from_numpy(qseg).to(gpu)
+    tks = None if kvseg is None else torch.from_numpy(kvseg).to(gpu)
+    o, lse = tpa.tpa_factors(*sp(tq), *sp(tk), *sp(tv), tqs, tks, d**-0.5, causal)
+    grads = tpa.tpa_factors_bwd(*sp(tq), *sp(tk), *sp(tv), tqs, tks, o, lse, tdo, d**-0.5, causal, kernel=kernel)
+    f64 = lambda t: t.detach().float().cpu().numpy().astype(np.float64)
+    want = orc.tpa_backward(f64(tq), f64(tk), f64(tv), qseg, kvseg, h, f64(tdo), sm_scale=d**-0.5, causal=causal)
+    got = [np.concatenate([f64(grads[2 * n]), f64(grads[2 * n + 1])], axis=-1) for n in range(3)]
+    return got, want
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize(
+    "b,lq,lk,h,d,rq,rk,seg",
+    [
+        (2, 512, 512, 4, 128, 6, 2, None),
+        (1, 300, 300, 2, 128, 2, 2, None),   # ragged last tiles
+        (2, 200, 450, 2, 64, 3, 4, None),    # lq != lk
+        (1, 700, 333, 2, 128, 2, 1, None),
+        (2, 384, 384, 2, 64, 6, 2, 100),     # packed sequences
+        (1, 640, 384, 2, 128, 2, 2, 77),     # rows whose segment has no key: no gradient from them
+    ],
+)
+def test_backward_bf16_mfma_kernels(gpu, b, lq, lk, h, d, rq, rk, seg, causal):
+    """kernel=2 makes a fallback to the fp32 kernels an error.  bf16 P and dS in the contractions:
+    held to 1.5e-2 of the largest gradient entry."""
+    got, want = _bf16_case(gpu, 31, b, lq, lk, h, d, rq, rk, seg, causal, kernel=2)
+    for name, g, w in zip("qkv", got, want):
+        assert rel_err(g, w) <= 1.5e-2, name
+
+
+def test_backward_bf16_mfma_matches_fp32_kernels(gpu):
+    """Same inputs through the vector-ALU kernels (kernel=1) and the MFMA kernels (kernel=2)."""
+    a, want = _bf16_case(gpu, 33, 2, 320, 320, 2, 64, 4, 2, None, True, kernel=1)
+    b_, _ = _bf16_case(gpu, 33, 2, 320, 320, 2, 64, 4, 2, None, True, kernel=2)
+    for x, y, w in zip(a, b_, want):
+        assert rel_err(x, w) <= 6e-3   # the fp32 kernels are limited by the bf16 rounding of the forward output inside delta
+        assert rel_err(y, x) <= 1.5e-2
+
+
+@pytest.mark.parametrize("d,causal", [(64, False), (128, True)])
+def test_mha_backward_bf16_mfma(gpu, d, causal):
+    from tpa import mha
+
+    b, lq, lk, h = 2, 333, 333, 4
+    rng = np.random.default_rng(41)
+    mk = lambda *s: torch.from_numpy(rng.standard_normal(s).astype(np.float32)).to(gpu).to(torch.bfloat16)
+    q, k, v, do = mk(b, lq, h, d), mk(b, lk, h, d), mk(b, lk, h, d), mk(b, lq, h, d)
+    o, res = mha._mha_fwd(q, k, v, None, d**-0.5, causal=causal)
+    dq, dk, dv, _, _ = mha._mha_bwd(res, do, kernel=2)
+    f64 = lambda t: t.detach().float().cpu().numpy().astype(np.float64)
+    bias = np.where(np.tril(np.ones((lq, lk), bool)), 0.0, -np.inf)[None].repeat(b, 0) if causal else None
+    want = orc.mha_backward(f64(q), f64(k), f64(v), bias, d**-0.5, f64(do))
+    for t, w in zip((dq, dk, dv), want):
+        assert rel_err(f64(t), w) <= 2e-2
+
+
+def test_backward_mfma_refuses_what_it_cannot_run(gpu):
+    from tpa import _dispatch as d
+    from tpa import tpa
+
+    q, k, v = make_factors(15, 1, 16, 16, 2, 8, 8, 2, 2)
+    tq, tk, tv = (torch.from_numpy(x).to(gpu) for x in (q, k, v))
+    o, res = tpa._tpa_fwd(tq, tk, tv, 2, None, None, 1.0, False, None, False, False, False)
+    with pytest.raises(d.TpaError) as e:
+        tpa.tpa_factors_bwd(tq[..., :2], tq[..., 2:], tk[..., :2], tk[..., 2:], tv[..., :2], tv[..., 2:], None, None,
+                            o, res[-1].permute(0, 2, 1), torch.ones_like(o), kernel=2)
+    assert e.value.code == -6
