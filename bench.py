@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|c2p|c3p|copy] [--no-cpu] [--no-decode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|c2p|c3p|c2b|c3b|copy] [--no-cpu] [--no-decode]
 
 A step is one forward pass over one batch of synthetic, seeded inputs that are resident in HBM
 before the timed region starts.  The default workload is the prefill configuration the headline
@@ -33,6 +33,9 @@ WORKLOADS = {
     "c5": ("prefill", 8, 2048, 2048, 64, 64, 16, 8, False),
     "c4": ("decode", 64, 1, 8192, 32, 128, 6, 2, False),
     # packed sequences (segment ids, tpa/tpa.py:369-375): the c2 / c3 shapes holding documents of DOC_LEN tokens
+    # backward pass (tpa/tpa.py:168-214) at the c2 / c3 shapes: gradients of all six factor arrays
+    "c2b": ("backward", 4, 4096, 4096, 16, 128, 6, 2, True),
+    "c3b": ("backward", 1, 32768, 32768, 32, 128, 6, 2, True),
     "c2p": ("prefill", 4, 4096, 4096, 16, 128, 6, 2, True),
     "c3p": ("prefill", 1, 32768, 32768, 32, 128, 6, 2, True),
 }
@@ -120,6 +123,31 @@ def run_prefill(torch, tpa, device, name, steps, warmup):
         tflops_wall=fl / wall_ms / 1e9, tflops_kernel=fl / ev_ms / 1e9,
         shape=dict(B=B, lq=lq, lk=lk, H=H, D=D, rank_q=rq, rank_k=rk, causal=causal, **({"document_len": doc} if doc else {})),
         inputs=x, out=out,
+    )
+
+
+def run_backward(torch, tpa, device, name, steps, warmup):
+    """One step = one call of the backward entry point (all its kernels) on resident inputs, with
+    the forward's o and lse computed once beforehand."""
+    _, B, lq, lk, H, D, rq, rk, causal = WORKLOADS[name]
+    x = make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed=0)
+    scale = D**-0.5
+    o, lse = tpa.tpa_factors(*x, sm_scale=scale, causal=causal, kernel=2)
+    g = torch.Generator(device=device)
+    g.manual_seed(7)
+    do = torch.randn(o.shape, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    grads = tuple(torch.empty(t.shape, dtype=torch.float32, device=device) for t in x)
+    ws = torch.empty(tpa.bwd_workspace_bytes(B, lq, lk, H, D, D) + 256, dtype=torch.uint8, device=device)
+
+    def step(i):
+        tpa.tpa_factors_bwd(*x, None, None, o, lse, do, scale, causal, grads=grads, workspace=ws, kernel=2)
+
+    wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
+    fl = 2.5 * prefill_flops(B, lq, lk, H, D, causal)  # five contractions against the forward's two
+    return dict(
+        wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, flops=fl,
+        tflops_wall=fl / wall_ms / 1e9, tflops_kernel=fl / ev_ms / 1e9,
+        shape=dict(B=B, lq=lq, lk=lk, H=H, D=D, rank_q=rq, rank_k=rk, causal=causal),
     )
 
 
@@ -277,6 +305,19 @@ def main():
             err = float(abs(r["out"]["o"][:1].float().cpu().numpy() - o_ref).max())
             result["max_abs_err_vs_oracle_sample"] = err
             log(f"[bench] cpu {base['value']*1e3:.2f} GFLOP/s; max abs err vs oracle on the sample {err:.2e}")
+    elif kind == "backward":
+        log(f"[bench] backward {args.workload}: warmup {args.warmup}, steps {args.steps}")
+        r = run_backward(torch, tpa, device, args.workload, args.steps, args.warmup)
+        log(f"[bench] {r['kernel_ms']:.4f} ms/call (min {r['kernel_ms_min']:.4f}), {r['tflops_kernel']:.1f} TFLOP/s")
+        result.update(
+            metric="TPA causal prefill backward throughput", value=r["tflops_wall"], unit="TFLOP/s", ms_per_step=r["wall_ms"],
+            roofline=dict(bound="mfma", achieved=r["tflops_kernel"], peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
+                          frac=r["tflops_kernel"] / PEAK_BF16_TFLOPS, traffic=None,
+                          kernel="recon + delta + bwd_dq_kernel + bwd_dkv_kernel + project (whole call)",
+                          ms_per_launch=r["kernel_ms"], ms_per_launch_min=r["kernel_ms_min"],
+                          algorithmic_flops_per_launch=r["flops"]),
+            config=dict(workload=f"{args.workload}: TPA backward", **r["shape"]),
+        )
     else:
         log(f"[bench] decode {args.workload}: warmup {args.warmup}, steps {args.steps}")
         d = run_decode(torch, tpa, device, args.workload, args.steps, args.warmup)

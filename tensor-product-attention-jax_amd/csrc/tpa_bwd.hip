@@ -40,6 +40,36 @@ __global__ void recon_kernel(TpaFactor fa, TpaFactor fb, TO* out, int L, int H, 
   }
 }
 
+// bf16 factors -> dense bf16, 8 elements per thread: the thread keeps its 16-byte piece of every
+// rank's b row and walks the heads.  Needs D % 8 == 0 and 16-byte aligned b rows.
+__global__ void recon_bf16_kernel(TpaFactor fa, TpaFactor fb, uint16_t* out, int L, int H, int D, int R) {
+  const int t = blockIdx.x, b = blockIdx.y;
+  const uint16_t* ap = static_cast<const uint16_t*>(fa.ptr) + b * fa.stride_b + t * fa.stride_l;
+  const uint16_t* bp = static_cast<const uint16_t*>(fb.ptr) + b * fb.stride_b + t * fb.stride_l;
+  uint16_t* op = out + ((int64_t)b * L + t) * H * D;
+  const float inv = 1.f / (float)R;
+  const int cpr = D / 8;
+  for (int idx = threadIdx.x; idx < H * cpr; idx += blockDim.x) {
+    const int h = idx / cpr, cc = idx - h * cpr;
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+    for (int r = 0; r < R; ++r) {
+      const float av = bf16bits_to_f32(ap[r * fa.stride_r + h]);
+      const u32x4 bv = *reinterpret_cast<const u32x4*>(bp + r * fb.stride_r + 8 * cc);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc[2 * j] += av * bf16lo_to_f32(bv[j]);
+        acc[2 * j + 1] += av * bf16hi_to_f32(bv[j]);
+      }
+    }
+    u32x4 pk;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) pk[j] = pack_bf16(acc[2 * j] * inv, acc[2 * j + 1] * inv);
+    *reinterpret_cast<u32x4*>(op + h * D + 8 * cc) = pk;
+  }
+}
+
 template <typename T>
 __global__ void to_f32_kernel(const T* in, float* out, int64_t n) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
@@ -47,22 +77,46 @@ __global__ void to_f32_kernel(const T* in, float* out, int64_t n) {
 }
 
 // ------------------------------------------------------------------------------------ stage 2
-// delta[b, h, i] = sum_d o[b, i, h, d] * do[b, i, h, d], skipping NaN products (an empty row's o)
+// delta[b, h, i] = sum_d o[b, i, h, d] * do[b, i, h, d], skipping NaN products (an empty row's o).
+// Sixteen lanes share a row; with bf16 rows of a multiple of 8 elements each lane takes 16 bytes
+// per step, so a wave reads four rows with fully coalesced loads.
 template <typename T>
-__global__ void delta_kernel(const T* o, const T* d_o, float* delta, int B, int lq, int H, int dv) {
-  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // over (b, i, h)
-  if (idx >= (int64_t)B * lq * H) return;
-  const int h = idx % H;
-  const int64_t bi = idx / H;
-  const int i = bi % lq, b = bi / lq;
-  const T* op = o + idx * dv;
-  const T* gp = d_o + idx * dv;
+__global__ void delta_kernel(const T* o, const T* d_o, float* delta, int B, int lq, int H, int dv, int vec) {
+  const int64_t row = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;  // over (b, i, h)
+  const int sub = threadIdx.x & 15;
+  const bool ok = row < (int64_t)B * lq * H;
   float acc = 0.f;
-  for (int d = 0; d < dv; ++d) {
-    const float x = load_as_f32(op + d) * load_as_f32(gp + d);
-    if (x == x) acc += x;
+  if (ok) {
+    const T* op = o + row * dv;
+    const T* gp = d_o + row * dv;
+    if constexpr (sizeof(T) == 2) {
+      if (vec) {
+        for (int d = 8 * sub; d < dv; d += 128) {
+          const u32x4 a = *reinterpret_cast<const u32x4*>(op + d), g = *reinterpret_cast<const u32x4*>(gp + d);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float x0 = bf16lo_to_f32(a[j]) * bf16lo_to_f32(g[j]), x1 = bf16hi_to_f32(a[j]) * bf16hi_to_f32(g[j]);
+            if (x0 == x0) acc += x0;
+            if (x1 == x1) acc += x1;
+          }
+        }
+      }
+    }
+    if (!(sizeof(T) == 2 && vec)) {
+      for (int d = sub; d < dv; d += 16) {
+        const float x = load_as_f32(op + d) * load_as_f32(gp + d);
+        if (x == x) acc += x;
+      }
+    }
   }
-  delta[((int64_t)b * H + h) * lq + i] = acc;
+#pragma unroll
+  for (int m = 8; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 16);
+  if (ok && sub == 0) {
+    const int h = row % H;
+    const int64_t bi = row / H;
+    const int i = bi % lq, b = bi / lq;
+    delta[((int64_t)b * H + h) * lq + i] = acc;
+  }
 }
 
 struct DenseParams {
@@ -251,9 +305,12 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(DenseParams p) {
 }
 
 // ------------------------------------------------------------------------------------ stage 5
-// One workgroup per token: da[r, h] and db[r, d] from the token's dense gradient dX[h, d].
-template <typename T>
-__global__ void project_kernel(const float* dx, TpaFactor fa, TpaFactor fb, TpaGrad ga, TpaGrad gb, int L, int H, int D, int R) {
+// One workgroup (256 threads) per token: da[r, h] and db[r, d] from the token's dense gradient
+// dX[h, d].  With STAGE the token's dX (row stride D + 1), a and b sit in LDS; each da output is
+// shared by `ns` neighbouring lanes that split the sum over d and combine with lane shuffles.
+template <typename T, bool STAGE>
+__global__ __launch_bounds__(256) void project_kernel(const float* dx, TpaFactor fa, TpaFactor fb, TpaGrad ga, TpaGrad gb, int L, int H,
+                                                       int D, int R, int ns) {
   const int t = blockIdx.x, b = blockIdx.y;
   const float* xp = dx + ((int64_t)b * L + t) * H * D;
   const T* ap = static_cast<const T*>(fa.ptr) + b * fa.stride_b + t * fa.stride_l;
@@ -261,18 +318,65 @@ __global__ void project_kernel(const float* dx, TpaFactor fa, TpaFactor fb, TpaG
   float* oa = ga.ptr + b * ga.stride_b + t * ga.stride_l;
   float* ob = gb.ptr + b * gb.stride_b + t * gb.stride_l;
   const float inv = 1.f / (float)R;
-  for (int idx = threadIdx.x; idx < R * H; idx += blockDim.x) {
-    const int r = idx / H, h = idx - r * H;
-    float acc = 0.f;
-    for (int d = 0; d < D; ++d) acc += xp[h * D + d] * load_as_f32(bp + r * fb.stride_r + d);
-    oa[r * ga.stride_r + h] = acc * inv;
+  extern __shared__ float xs[];  // [H][D + 1], then b[R][D], then a[R][H]
+  if constexpr (STAGE) {
+    float* bs = xs + H * (D + 1);
+    float* as = bs + R * D;
+    for (int idx = threadIdx.x; idx < H * D; idx += 256) {
+      const int h = idx / D, d = idx - h * D;
+      xs[h * (D + 1) + d] = xp[idx];
+    }
+    for (int idx = threadIdx.x; idx < R * D; idx += 256) {
+      const int r = idx / D, d = idx - r * D;
+      bs[idx] = load_as_f32(bp + r * fb.stride_r + d);
+    }
+    for (int idx = threadIdx.x; idx < R * H; idx += 256) {
+      const int r = idx / H, h = idx - r * H;
+      as[idx] = load_as_f32(ap + r * fa.stride_r + h);
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < R * D; idx += 256) {
+      const int r = idx / D, d = idx - r * D;
+      float acc = 0.f;
+      for (int h = 0; h < H; ++h) acc += xs[h * (D + 1) + d] * as[r * H + h];
+      ob[r * gb.stride_r + d] = acc * inv;
+    }
+    const int per_pass = 256 / ns, sub = threadIdx.x % ns;
+    for (int base = 0; base < R * H; base += per_pass) {  // uniform trip count: the shuffles below need every lane
+      const int idx = base + threadIdx.x / ns;
+      const bool ok = idx < R * H;
+      const int r = ok ? idx / H : 0, h = ok ? idx - r * H : 0;
+      float acc = 0.f;
+      for (int d = sub; d < D; d += ns) acc += xs[h * (D + 1) + d] * bs[r * D + d];
+      for (int m = ns >> 1; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 64);
+      if (ok && sub == 0) oa[r * ga.stride_r + h] = acc * inv;
+    }
+  } else {
+    for (int idx = threadIdx.x; idx < R * D; idx += 256) {
+      const int r = idx / D, d = idx - r * D;
+      float acc = 0.f;
+      for (int h = 0; h < H; ++h) acc += xp[h * D + d] * load_as_f32(ap + r * fa.stride_r + h);
+      ob[r * gb.stride_r + d] = acc * inv;
+    }
+    for (int idx = threadIdx.x; idx < R * H; idx += 256) {
+      const int r = idx / H, h = idx - r * H;
+      float acc = 0.f;
+      for (int d = 0; d < D; ++d) acc += xp[h * D + d] * load_as_f32(bp + r * fb.stride_r + d);
+      oa[r * ga.stride_r + h] = acc * inv;
+    }
   }
-  for (int idx = threadIdx.x; idx < R * D; idx += blockDim.x) {
-    const int r = idx / D, d = idx - r * D;
-    float acc = 0.f;
-    for (int h = 0; h < H; ++h) acc += xp[h * D + d] * load_as_f32(ap + r * fa.stride_r + h);
-    ob[r * gb.stride_r + d] = acc * inv;
-  }
+}
+
+template <typename T>
+void launch_project(const float* dx, const TpaFactor& fa, const TpaFactor& fb, const TpaGrad& ga, const TpaGrad& gb, int B, int L,
+                    int H, int D, int R, hipStream_t stream) {
+  const size_t smem = ((size_t)H * (D + 1) + (size_t)R * D + (size_t)R * H) * sizeof(float);
+  int ns = 1;  // lanes per da output: a power of two, at most a wave, so that one pass covers the outputs if it can
+  while (ns < 64 && 2 * ns * R * H <= 256) ns *= 2;
+  if (smem <= 60 * 1024)
+    hipLaunchKernelGGL((project_kernel<T, true>), dim3(L, B), dim3(256), smem, stream, dx, fa, fb, ga, gb, L, H, D, R, ns);
+  else
+    hipLaunchKernelGGL((project_kernel<T, false>), dim3(L, B), dim3(256), 0, stream, dx, fa, fb, ga, gb, L, H, D, R, ns);
 }
 
 template <typename T, int DMAX>
@@ -311,16 +415,27 @@ int tpa_bwd_t(const TpaBwdArgs* a, hipStream_t stream, bool mfma) {
   const int threads = 256;
   if (mfma) {
     uint16_t *q16 = reinterpret_cast<uint16_t*>(qd), *k16 = reinterpret_cast<uint16_t*>(kd), *v16 = reinterpret_cast<uint16_t*>(vd);
-    hipLaunchKernelGGL((recon_kernel<T, uint16_t>), dim3(a->lq, a->B), dim3(threads), 0, stream, a->qa, a->qb, q16, a->lq, a->H, a->dk, a->rq);
-    hipLaunchKernelGGL((recon_kernel<T, uint16_t>), dim3(a->lk, a->B), dim3(threads), 0, stream, a->ka, a->kb, k16, a->lk, a->H, a->dk, a->rk);
-    hipLaunchKernelGGL((recon_kernel<T, uint16_t>), dim3(a->lk, a->B), dim3(threads), 0, stream, a->va, a->vb, v16, a->lk, a->H, a->dv, a->rk);
+    auto recon16 = [&](const TpaFactor& fa, const TpaFactor& fb, uint16_t* out, int L, int D, int R) {
+      const bool vec = sizeof(T) == 2 && !(reinterpret_cast<uintptr_t>(fb.ptr) & 15) && fb.stride_b % 8 == 0 && fb.stride_l % 8 == 0 &&
+                       fb.stride_r % 8 == 0;
+      if (vec)
+        hipLaunchKernelGGL(recon_bf16_kernel, dim3(L, a->B), dim3(threads), 0, stream, fa, fb, out, L, a->H, D, R);
+      else
+        hipLaunchKernelGGL((recon_kernel<T, uint16_t>), dim3(L, a->B), dim3(threads), 0, stream, fa, fb, out, L, a->H, D, R);
+    };
+    recon16(a->qa, a->qb, q16, a->lq, a->dk, a->rq);
+    recon16(a->ka, a->kb, k16, a->lk, a->dk, a->rk);
+    recon16(a->va, a->vb, v16, a->lk, a->dv, a->rk);
   } else {
     hipLaunchKernelGGL((recon_kernel<T, float>), dim3(a->lq, a->B), dim3(threads), 0, stream, a->qa, a->qb, qd, a->lq, a->H, a->dk, a->rq);
     hipLaunchKernelGGL((recon_kernel<T, float>), dim3(a->lk, a->B), dim3(threads), 0, stream, a->ka, a->kb, kd, a->lk, a->H, a->dk, a->rk);
     hipLaunchKernelGGL((recon_kernel<T, float>), dim3(a->lk, a->B), dim3(threads), 0, stream, a->va, a->vb, vd, a->lk, a->H, a->dv, a->rk);
   }
-  hipLaunchKernelGGL((delta_kernel<T>), dim3((unsigned)((nd + threads - 1) / threads)), dim3(threads), 0, stream,
-                     static_cast<const T*>(a->o), static_cast<const T*>(a->d_o), delta, a->B, a->lq, a->H, a->dv);
+  {
+    const int vec = a->dv % 8 == 0 && !(reinterpret_cast<uintptr_t>(a->o) & 15) && !(reinterpret_cast<uintptr_t>(a->d_o) & 15);
+    hipLaunchKernelGGL((delta_kernel<T>), dim3((unsigned)((nd * 16 + threads - 1) / threads)), dim3(threads), 0, stream,
+                       static_cast<const T*>(a->o), static_cast<const T*>(a->d_o), delta, a->B, a->lq, a->H, a->dv, vec);
+  }
   if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
 
   int rc;
@@ -338,9 +453,9 @@ int tpa_bwd_t(const TpaBwdArgs* a, hipStream_t stream, bool mfma) {
   }
   if (rc != TPA_OK) return rc;
 
-  hipLaunchKernelGGL((project_kernel<T>), dim3(a->lq, a->B), dim3(threads), 0, stream, dqd, a->qa, a->qb, a->dqa, a->dqb, a->lq, a->H, a->dk, a->rq);
-  hipLaunchKernelGGL((project_kernel<T>), dim3(a->lk, a->B), dim3(threads), 0, stream, dkd, a->ka, a->kb, a->dka, a->dkb, a->lk, a->H, a->dk, a->rk);
-  hipLaunchKernelGGL((project_kernel<T>), dim3(a->lk, a->B), dim3(threads), 0, stream, dvd, a->va, a->vb, a->dva, a->dvb, a->lk, a->H, a->dv, a->rk);
+  launch_project<T>(dqd, a->qa, a->qb, a->dqa, a->dqb, a->B, a->lq, a->H, a->dk, a->rq, stream);
+  launch_project<T>(dkd, a->ka, a->kb, a->dka, a->dkb, a->B, a->lk, a->H, a->dk, a->rk, stream);
+  launch_project<T>(dvd, a->va, a->vb, a->dva, a->dvb, a->B, a->lk, a->H, a->dv, a->rk, stream);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
 }
 
@@ -352,8 +467,11 @@ int mha_bwd_t(const MhaBwdArgs* a, hipStream_t stream, bool mfma) {
   auto take = [&](size_t floats) { float* ptr = reinterpret_cast<float*>(w); w += align256(floats * sizeof(float)); return ptr; };
   float* delta = take(nd);
   const int threads = 256;
-  hipLaunchKernelGGL((delta_kernel<T>), dim3((unsigned)((nd + threads - 1) / threads)), dim3(threads), 0, stream,
-                     static_cast<const T*>(a->o), static_cast<const T*>(a->d_o), delta, a->B, a->lq, a->H, a->dv);
+  {
+    const int vec = a->dv % 8 == 0 && !(reinterpret_cast<uintptr_t>(a->o) & 15) && !(reinterpret_cast<uintptr_t>(a->d_o) & 15);
+    hipLaunchKernelGGL((delta_kernel<T>), dim3((unsigned)((nd * 16 + threads - 1) / threads)), dim3(threads), 0, stream,
+                       static_cast<const T*>(a->o), static_cast<const T*>(a->d_o), delta, a->B, a->lq, a->H, a->dv, vec);
+  }
   if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
   if (mfma)
     return dense_bwd_mfma_launch(a->q, a->k, a->v, a->d_o, a->lse, delta, nullptr, nullptr, a->dq, a->dk_out, a->dv_out,

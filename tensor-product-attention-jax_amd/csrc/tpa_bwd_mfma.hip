@@ -63,6 +63,11 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 constexpr int kRsrcFlags = 0x00020000;  // raw 32-bit data format
 
+// Row stride (elements) of the LDS tiles.  Every tile is read both by rows (16-byte reads of 16
+// consecutive rows) and transposed (8-byte reads of 4 consecutive rows); no padding serves both
+// without bank conflicts, these leave the row reads conflict-free and the transposed ones two-way.
+constexpr int tile_stride(int d) { return d == 128 ? d + 24 : d + 8; }
+
 // A-operand fragment of rows 32 mb .. 32 mb + 31 of a row-major tile (row stride S elements),
 // contraction columns 16 kk .. 16 kk + 15: lane (i, g) reads 8 elements of row 32 mb + i.
 template <int S>
@@ -104,7 +109,7 @@ __device__ __forceinline__ f32x16 splat16(float x) {
 // ============================================================================================
 template <int D, bool SEG>
 __global__ __launch_bounds__(512) void bwd_dq_kernel(BwdParams p) {
-  constexpr int NT = 512, S = D + 8, CPR = D / 8, TPP = NT / CPR, NPASS = kTile / TPP;
+  constexpr int NT = 512, S = tile_stride(D), CPR = D / 8, TPP = NT / CPR, NPASS = kTile / TPP;
   constexpr int NKS = D / 16, NDB = D / 32, kBQ = 256;
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   uint16_t* const lds_k = smem;                  // [2][64][S]
@@ -261,7 +266,7 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(BwdParams p) {
 // ============================================================================================
 template <int D, int NW, bool SEG>
 __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
-  constexpr int NT = NW * 64, S = D + 8, CPR = D / 8, TPP = NT / CPR, NPASS = kTile / TPP;
+  constexpr int NT = NW * 64, S = tile_stride(D), CPR = D / 8, TPP = NT / CPR, NPASS = kTile / TPP;
   constexpr int NKS = D / 16, NDB = D / 32, kBK = NW * 32;
   static_assert(kTile % TPP == 0 && NPASS >= 1, "loader shape");
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
@@ -459,7 +464,7 @@ int launch_dq(const BwdParams& base, hipStream_t stream) {
   p.nblk = (p.lq + 255) / 256;
   p.npairs = p.nblk * p.B;
   auto kern = bwd_dq_kernel<D, SEG>;
-  const size_t smem = (size_t)4 * kTile * (D + 8) * 2 + 2 * kTile * 4;
+  const size_t smem = (size_t)4 * kTile * tile_stride(D) * 2 + 2 * kTile * 4;
   static bool configured = false;
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
@@ -476,7 +481,7 @@ int launch_dkv(const BwdParams& base, hipStream_t stream) {
   p.nblk = (p.lk + NW * 32 - 1) / (NW * 32);
   p.npairs = p.nblk * p.B;
   auto kern = bwd_dkv_kernel<D, NW, SEG>;
-  const size_t smem = (size_t)4 * kTile * (D + 8) * 2 + 6 * kTile * 4;
+  const size_t smem = (size_t)4 * kTile * tile_stride(D) * 2 + 6 * kTile * 4;
   static bool configured = false;
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
@@ -489,7 +494,7 @@ int launch_dkv(const BwdParams& base, hipStream_t stream) {
 
 template <int D>
 int launch_both(const BwdParams& p, hipStream_t stream) {
-  constexpr int NW = D == 128 ? 4 : 8;  // D = 128: one wave per SIMD, its accumulators need the whole register file
+  constexpr int NW = 8;
   int rc;
   if (p.qseg) {
     rc = launch_dq<D, true>(p, stream);

@@ -247,6 +247,10 @@ def tpa_factors_bwd(
     return tuple(grads)
 
 
+def bwd_workspace_bytes(b: int, lq: int, lk: int, h: int, dk: int, dv: int) -> int:
+    return int(_d.load_library().tpa_bwd_workspace_bytes(b, lq, lk, h, dk, dv))
+
+
 def _bwd_concat(q, k, v, qseg, kvseg, o, lse_bhl, do, num_heads, sm_scale, causal):
     """Gradients in the concatenated layout of q, k, v (fp32), written in place by the kernels."""
     h = num_heads
