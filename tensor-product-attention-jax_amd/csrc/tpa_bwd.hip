@@ -318,13 +318,16 @@ __global__ __launch_bounds__(256) void project_kernel(const float* dx, TpaFactor
   float* oa = ga.ptr + b * ga.stride_b + t * ga.stride_l;
   float* ob = gb.ptr + b * gb.stride_b + t * gb.stride_l;
   const float inv = 1.f / (float)R;
-  extern __shared__ float xs[];  // [H][D + 1], then b[R][D], then a[R][H]
+  extern __shared__ __attribute__((aligned(16))) float xs[];  // [H][XS], then b[R][D], then a[R][H]
   if constexpr (STAGE) {
-    float* bs = xs + H * (D + 1);
+    // D % 4 == 0 here; rows 16 bytes apart in the banks, so that lanes that read 16 bytes of
+    // different rows (the da part) spread over the banks
+    const int XS = D + 4;
+    float* bs = xs + H * XS;
     float* as = bs + R * D;
-    for (int idx = threadIdx.x; idx < H * D; idx += 256) {
-      const int h = idx / D, d = idx - h * D;
-      xs[h * (D + 1) + d] = xp[idx];
+    for (int idx = threadIdx.x; idx < H * D / 4; idx += 256) {
+      const int h = idx / (D / 4), d4 = idx - h * (D / 4);
+      *reinterpret_cast<f32x4*>(xs + h * XS + 4 * d4) = *reinterpret_cast<const f32x4*>(xp + 4 * idx);
     }
     for (int idx = threadIdx.x; idx < R * D; idx += 256) {
       const int r = idx / D, d = idx - r * D;
@@ -338,7 +341,7 @@ __global__ __launch_bounds__(256) void project_kernel(const float* dx, TpaFactor
     for (int idx = threadIdx.x; idx < R * D; idx += 256) {
       const int r = idx / D, d = idx - r * D;
       float acc = 0.f;
-      for (int h = 0; h < H; ++h) acc += xs[h * (D + 1) + d] * as[r * H + h];
+      for (int h = 0; h < H; ++h) acc += xs[h * XS + d] * as[r * H + h];
       ob[r * gb.stride_r + d] = acc * inv;
     }
     const int per_pass = 256 / ns, sub = threadIdx.x % ns;
@@ -347,7 +350,11 @@ __global__ __launch_bounds__(256) void project_kernel(const float* dx, TpaFactor
       const bool ok = idx < R * H;
       const int r = ok ? idx / H : 0, h = ok ? idx - r * H : 0;
       float acc = 0.f;
-      for (int d = sub; d < D; d += ns) acc += xs[h * (D + 1) + d] * bs[r * D + d];
+      for (int d = 4 * sub; d < D; d += 4 * ns) {
+        const f32x4 xv = *reinterpret_cast<const f32x4*>(xs + h * XS + d);
+        const f32x4 bv = *reinterpret_cast<const f32x4*>(bs + r * D + d);
+        acc += xv[0] * bv[0] + xv[1] * bv[1] + xv[2] * bv[2] + xv[3] * bv[3];
+      }
       for (int m = ns >> 1; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 64);
       if (ok && sub == 0) oa[r * ga.stride_r + h] = acc * inv;
     }
@@ -370,10 +377,10 @@ __global__ __launch_bounds__(256) void project_kernel(const float* dx, TpaFactor
 template <typename T>
 void launch_project(const float* dx, const TpaFactor& fa, const TpaFactor& fb, const TpaGrad& ga, const TpaGrad& gb, int B, int L,
                     int H, int D, int R, hipStream_t stream) {
-  const size_t smem = ((size_t)H * (D + 1) + (size_t)R * D + (size_t)R * H) * sizeof(float);
+  const size_t smem = ((size_t)H * (D + 4) + (size_t)R * D + (size_t)R * H) * sizeof(float);
   int ns = 1;  // lanes per da output: a power of two, at most a wave, so that one pass covers the outputs if it can
-  while (ns < 64 && 2 * ns * R * H <= 256) ns *= 2;
-  if (smem <= 60 * 1024)
+  while (ns < 64 && 2 * ns * R * H <= 256 && 8 * ns <= D) ns *= 2;
+  if (smem <= 60 * 1024 && D % 4 == 0)
     hipLaunchKernelGGL((project_kernel<T, true>), dim3(L, B), dim3(256), smem, stream, dx, fa, fb, ga, gb, L, H, D, R, ns);
   else
     hipLaunchKernelGGL((project_kernel<T, false>), dim3(L, B), dim3(256), 0, stream, dx, fa, fb, ga, gb, L, H, D, R, ns);

@@ -264,10 +264,11 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(BwdParams p) {
 // ============================================================================================
 // dK, dV
 // ============================================================================================
-template <int D, int NW, bool SEG>
+template <int D, int NW, int NB, bool SEG>
 __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
+  // a wave owns NB blocks of 32 keys: every operand fragment read from LDS feeds NB MFMAs
   constexpr int NT = NW * 64, S = tile_stride(D), CPR = D / 8, TPP = NT / CPR, NPASS = kTile / TPP;
-  constexpr int NKS = D / 16, NDB = D / 32, kBK = NW * 32;
+  constexpr int NKS = D / 16, NDB = D / 32, kWK = 32 * NB, kBK = NW * kWK;
   static_assert(kTile % TPP == 0 && NPASS >= 1, "loader shape");
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   uint16_t* const lds_q = smem;                  // [2][64][S]
@@ -282,11 +283,14 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
   const int kblk = pair / p.B, b = pair % p.B;  // under the causal mask the first key blocks are the heaviest
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
   const int lp = l & 15, dhalf = (l >> 4) & 1;
-  const int k0 = kblk * kBK, wkey0 = k0 + 32 * w, key = wkey0 + i, key_ld = min(key, p.lk - 1);
+  const int k0 = kblk * kBK, wkey0 = k0 + kWK * w;
   const float c = p.sm_scale * kLog2e;
 
-  bf16x8 kf[NKS], vf[NKS];
-  {
+  bf16x8 kf[NB][NKS], vf[NB][NKS];
+  int32_t kseg[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int key_ld = min(wkey0 + 32 * nb + i, p.lk - 1);
     const uint16_t* kp = p.k + (((int64_t)b * p.lk + key_ld) * p.H + h) * D;
     const uint16_t* vp = p.v + (((int64_t)b * p.lk + key_ld) * p.H + h) * D;
 #pragma unroll
@@ -295,11 +299,11 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
       u32x4 sc;
 #pragma unroll
       for (int j = 0; j < 4; ++j) sc[j] = pack_bf16(bf16lo_to_f32(raw[j]) * c, bf16hi_to_f32(raw[j]) * c);
-      kf[ks] = __builtin_bit_cast(bf16x8, sc);
-      vf[ks] = *reinterpret_cast<const bf16x8*>(vp + 16 * ks + 8 * g);
+      kf[nb][ks] = __builtin_bit_cast(bf16x8, sc);
+      vf[nb][ks] = *reinterpret_cast<const bf16x8*>(vp + 16 * ks + 8 * g);
     }
+    kseg[nb] = SEG ? p.kvseg[(int64_t)b * p.lk + key_ld] : 0;
   }
-  const int32_t kseg = SEG ? p.kvseg[(int64_t)b * p.lk + key_ld] : 0;
 
   // query tiles: under the causal mask rows before this block's first key see none of its keys
   const int tile0 = p.causal ? k0 / kTile : 0;
@@ -357,9 +361,11 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
     else if (SEG && tid < 3 * kTile) lds_seg[(tile & 1) * kTile + tid - 2 * kTile] = __float_as_int(aux_pending);
   };
 
-  f32x16 dk_acc[NDB], dv_acc[NDB];
+  f32x16 dk_acc[NB][NDB], dv_acc[NB][NDB];
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) { dk_acc[db] = splat16(0.f); dv_acc[db] = splat16(0.f); }
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) { dk_acc[nb][db] = splat16(0.f); dv_acc[nb][db] = splat16(0.f); }
 
   auto compute = [&](int j) __attribute__((always_inline)) {
     const uint16_t* qs = lds_q + (j & 1) * kTile * S;
@@ -367,59 +373,71 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
     const float* nl = lds_nlse + (j & 1) * kTile;
     const float* nd = lds_ndel + (j & 1) * kTile;
     const int r0 = (tile0 + j) * kTile;
-    const bool need_mask = p.causal && (r0 < wkey0 + 31);  // a row of the tile lies before a key of this wave
+    const bool need_mask = p.causal && (r0 < wkey0 + kWK - 1);  // a row of the tile lies before a key of this wave
     static_for<2>([&](auto mb_c) __attribute__((always_inline)) {
       constexpr int mb = decltype(mb_c)::value;
       // accumulator rows of this lane: 32 mb + 8 vq + 4 g + (0..3)
-      f32x16 s, dp;
+      f32x16 s[NB], dp[NB];
 #pragma unroll
       for (int vq = 0; vq < 4; ++vq) {
         const f32x4 a = *reinterpret_cast<const f32x4*>(nl + 32 * mb + 8 * vq + 4 * g);
         const f32x4 d4 = *reinterpret_cast<const f32x4*>(nd + 32 * mb + 8 * vq + 4 * g);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { s[4 * vq + e] = a[e]; dp[4 * vq + e] = d4[e]; }
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { s[nb][4 * vq + e] = a[e]; dp[nb][4 * vq + e] = d4[e]; }
       }
       static_for<NKS>([&](auto kk_c) __attribute__((always_inline)) {
         constexpr int kk = decltype(kk_c)::value;
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rows_frag<S>(qs, mb, kk, i, g), kf[kk], s, 0, 0, 0);
+        const bf16x8 a = rows_frag<S>(qs, mb, kk, i, g);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, kf[nb][kk], s[nb], 0, 0, 0);
       });
       static_for<NKS>([&](auto kk_c) __attribute__((always_inline)) {
         constexpr int kk = decltype(kk_c)::value;
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rows_frag<S>(gs, mb, kk, i, g), vf[kk], dp, 0, 0, 0);
+        const bf16x8 a = rows_frag<S>(gs, mb, kk, i, g);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) dp[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, vf[nb][kk], dp[nb], 0, 0, 0);
       });
-      if (need_mask) {
+      bf16x8 pf[NB][2], df[NB][2];
 #pragma unroll
-        for (int v = 0; v < 16; ++v)
-          if (r0 + 32 * mb + 8 * (v >> 2) + 4 * g + (v & 3) < key) s[v] = -INFINITY;
-      }
-      if constexpr (SEG) {
-        const int32_t* ids_p = lds_seg + (j & 1) * kTile + 32 * mb + 4 * g;
+      for (int nb = 0; nb < NB; ++nb) {
+        if (need_mask) {
+          const int key = wkey0 + 32 * nb + i;
 #pragma unroll
-        for (int vq = 0; vq < 4; ++vq) {
-          const int4 ids = *reinterpret_cast<const int4*>(ids_p + 8 * vq);
-          if (ids.x != kseg) s[4 * vq] = -INFINITY;
-          if (ids.y != kseg) s[4 * vq + 1] = -INFINITY;
-          if (ids.z != kseg) s[4 * vq + 2] = -INFINITY;
-          if (ids.w != kseg) s[4 * vq + 3] = -INFINITY;
+          for (int v = 0; v < 16; ++v)
+            if (r0 + 32 * mb + 8 * (v >> 2) + 4 * g + (v & 3) < key) s[nb][v] = -INFINITY;
         }
-      }
+        if constexpr (SEG) {
+          const int32_t* ids_p = lds_seg + (j & 1) * kTile + 32 * mb + 4 * g;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        s[v] = __builtin_amdgcn_exp2f(s[v]);  // p
-        dp[v] *= s[v];                        // p * (dp - delta)
+          for (int vq = 0; vq < 4; ++vq) {
+            const int4 ids = *reinterpret_cast<const int4*>(ids_p + 8 * vq);
+            if (ids.x != kseg[nb]) s[nb][4 * vq] = -INFINITY;
+            if (ids.y != kseg[nb]) s[nb][4 * vq + 1] = -INFINITY;
+            if (ids.z != kseg[nb]) s[nb][4 * vq + 2] = -INFINITY;
+            if (ids.w != kseg[nb]) s[nb][4 * vq + 3] = -INFINITY;
+          }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          s[nb][v] = __builtin_amdgcn_exp2f(s[nb][v]);  // p
+          dp[nb][v] *= s[nb][v];                        // p * (dp - delta)
+        }
+        pack_block(s[nb], pf[nb][0], pf[nb][1]);
+        pack_block(dp[nb], df[nb][0], df[nb][1]);
       }
-      bf16x8 p0, p1, d0, d1;
-      pack_block(s, p0, p1);
-      pack_block(dp, d0, d1);
-      static_for<NDB>([&](auto db_c) __attribute__((always_inline)) {
-        constexpr int db = decltype(db_c)::value;
-        dv_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cols_frag<S>(gs, 2 * mb, db, g, lp, dhalf), p0, dv_acc[db], 0, 0, 0);
-        dv_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cols_frag<S>(gs, 2 * mb + 1, db, g, lp, dhalf), p1, dv_acc[db], 0, 0, 0);
+      static_for<2 * NDB>([&](auto n_c) __attribute__((always_inline)) {
+        constexpr int db = decltype(n_c)::value / 2, half = decltype(n_c)::value % 2;
+        const bf16x8 a = cols_frag<S>(gs, 2 * mb + half, db, g, lp, dhalf);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) dv_acc[nb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[nb][half], dv_acc[nb][db], 0, 0, 0);
       });
-      static_for<NDB>([&](auto db_c) __attribute__((always_inline)) {
-        constexpr int db = decltype(db_c)::value;
-        dk_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cols_frag<S>(qs, 2 * mb, db, g, lp, dhalf), d0, dk_acc[db], 0, 0, 0);
-        dk_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cols_frag<S>(qs, 2 * mb + 1, db, g, lp, dhalf), d1, dk_acc[db], 0, 0, 0);
+      static_for<2 * NDB>([&](auto n_c) __attribute__((always_inline)) {
+        constexpr int db = decltype(n_c)::value / 2, half = decltype(n_c)::value % 2;
+        const bf16x8 a = cols_frag<S>(qs, 2 * mb + half, db, g, lp, dhalf);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) dk_acc[nb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, df[nb][half], dk_acc[nb][db], 0, 0, 0);
       });
     });
   };
@@ -439,22 +457,26 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
     }
   }
 
-  if (key < p.lk) {
-    float* okp = p.dk + (((int64_t)b * p.lk + key) * p.H + h) * D;
-    float* ovp = p.dv + (((int64_t)b * p.lk + key) * p.H + h) * D;
 #pragma unroll
-    for (int db = 0; db < NDB; ++db)
+  for (int nb = 0; nb < NB; ++nb) {
+    const int key = wkey0 + 32 * nb + i;
+    if (key < p.lk) {
+      float* okp = p.dk + (((int64_t)b * p.lk + key) * p.H + h) * D;
+      float* ovp = p.dv + (((int64_t)b * p.lk + key) * p.H + h) * D;
 #pragma unroll
-      for (int vq = 0; vq < 4; ++vq) {
-        f32x4 ok, ov;
+      for (int db = 0; db < NDB; ++db)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          ok[e] = dk_acc[db][4 * vq + e] * p.sm_scale;
-          ov[e] = dv_acc[db][4 * vq + e];
+        for (int vq = 0; vq < 4; ++vq) {
+          f32x4 ok, ov;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            ok[e] = dk_acc[nb][db][4 * vq + e] * p.sm_scale;
+            ov[e] = dv_acc[nb][db][4 * vq + e];
+          }
+          *reinterpret_cast<f32x4*>(okp + 32 * db + 8 * vq + 4 * g) = ok;
+          *reinterpret_cast<f32x4*>(ovp + 32 * db + 8 * vq + 4 * g) = ov;
         }
-        *reinterpret_cast<f32x4*>(okp + 32 * db + 8 * vq + 4 * g) = ok;
-        *reinterpret_cast<f32x4*>(ovp + 32 * db + 8 * vq + 4 * g) = ov;
-      }
+    }
   }
 }
 
@@ -475,12 +497,12 @@ int launch_dq(const BwdParams& base, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
 }
 
-template <int D, int NW, bool SEG>
+template <int D, int NW, int NB, bool SEG>
 int launch_dkv(const BwdParams& base, hipStream_t stream) {
   BwdParams p = base;
-  p.nblk = (p.lk + NW * 32 - 1) / (NW * 32);
+  p.nblk = (p.lk + NW * NB * 32 - 1) / (NW * NB * 32);
   p.npairs = p.nblk * p.B;
-  auto kern = bwd_dkv_kernel<D, NW, SEG>;
+  auto kern = bwd_dkv_kernel<D, NW, NB, SEG>;
   const size_t smem = (size_t)4 * kTile * tile_stride(D) * 2 + 6 * kTile * 4;
   static bool configured = false;
   if (!configured) {
@@ -494,14 +516,16 @@ int launch_dkv(const BwdParams& base, hipStream_t stream) {
 
 template <int D>
 int launch_both(const BwdParams& p, hipStream_t stream) {
-  constexpr int NW = 8;
+  // dK/dV: 8 waves of 32 keys.  (64 keys per wave would halve the LDS reads per MFMA, which bound
+  // this kernel, but its 384 stationary registers at D = 128 leave the compiler spilling.)
+  constexpr int NW = 8, NB = 1;
   int rc;
   if (p.qseg) {
     rc = launch_dq<D, true>(p, stream);
-    if (rc == TPA_OK) rc = launch_dkv<D, NW, true>(p, stream);
+    if (rc == TPA_OK) rc = launch_dkv<D, NW, NB, true>(p, stream);
   } else {
     rc = launch_dq<D, false>(p, stream);
-    if (rc == TPA_OK) rc = launch_dkv<D, NW, false>(p, stream);
+    if (rc == TPA_OK) rc = launch_dkv<D, NW, NB, false>(p, stream);
   }
   return rc;
 }
