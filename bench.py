@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|c2p|c3p|c2b|c3b|copy] [--no-cpu] [--no-decode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|c2p|c3p|c2b|c3b|c2pb|copy] [--no-cpu] [--no-decode]
 
 A step is one forward pass over one batch of synthetic, seeded inputs that are resident in HBM
 before the timed region starts.  The default workload is the prefill configuration the headline
@@ -36,6 +36,7 @@ WORKLOADS = {
     # backward pass (tpa/tpa.py:168-214) at the c2 / c3 shapes: gradients of all six factor arrays
     "c2b": ("backward", 4, 4096, 4096, 16, 128, 6, 2, True),
     "c3b": ("backward", 1, 32768, 32768, 32, 128, 6, 2, True),
+    "c2pb": ("backward", 4, 4096, 4096, 16, 128, 6, 2, True),   # packed documents, as c2p
     "c2p": ("prefill", 4, 4096, 4096, 16, 128, 6, 2, True),
     "c3p": ("prefill", 1, 32768, 32768, 32, 128, 6, 2, True),
 }
@@ -69,7 +70,7 @@ def make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed):
     )
 
 
-DOC_LEN = {"c2p": 1024, "c3p": 4096}
+DOC_LEN = {"c2p": 1024, "c3p": 4096, "c2pb": 1024}
 
 
 def prefill_flops(B, lq, lk, H, D, causal):
@@ -132,7 +133,9 @@ def run_backward(torch, tpa, device, name, steps, warmup):
     _, B, lq, lk, H, D, rq, rk, causal = WORKLOADS[name]
     x = make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed=0)
     scale = D**-0.5
-    o, lse = tpa.tpa_factors(*x, sm_scale=scale, causal=causal, kernel=2)
+    doc = DOC_LEN.get(name)
+    seg = (torch.arange(lq, device=device, dtype=torch.int32) // doc).repeat(B, 1).contiguous() if doc else None
+    o, lse = tpa.tpa_factors(*x, seg, seg, sm_scale=scale, causal=causal, kernel=2)
     g = torch.Generator(device=device)
     g.manual_seed(7)
     do = torch.randn(o.shape, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
@@ -140,14 +143,15 @@ def run_backward(torch, tpa, device, name, steps, warmup):
     ws = torch.empty(tpa.bwd_workspace_bytes(B, lq, lk, H, D, D) + 256, dtype=torch.uint8, device=device)
 
     def step(i):
-        tpa.tpa_factors_bwd(*x, None, None, o, lse, do, scale, causal, grads=grads, workspace=ws, kernel=2)
+        tpa.tpa_factors_bwd(*x, seg, seg, o, lse, do, scale, causal, grads=grads, workspace=ws, kernel=2)
 
     wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
-    fl = 2.5 * prefill_flops(B, lq, lk, H, D, causal)  # five contractions against the forward's two
+    # five contractions against the forward's two; packed: only pairs inside a document count
+    fl = 2.5 * (prefill_flops(B * (lq // doc), doc, doc, H, D, causal) if doc else prefill_flops(B, lq, lk, H, D, causal))
     return dict(
         wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, flops=fl,
         tflops_wall=fl / wall_ms / 1e9, tflops_kernel=fl / ev_ms / 1e9,
-        shape=dict(B=B, lq=lq, lk=lk, H=H, D=D, rank_q=rq, rank_k=rk, causal=causal),
+        shape=dict(B=B, lq=lq, lk=lk, H=H, D=D, rank_q=rq, rank_k=rk, causal=causal, **({"document_len": doc} if doc else {})),
     )
 
 

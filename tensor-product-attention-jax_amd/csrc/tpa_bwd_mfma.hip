@@ -104,6 +104,39 @@ __device__ __forceinline__ f32x16 splat16(float x) {
   return r;
 }
 
+
+// Packed sequences (tpa/tpa.py:369-375 compares ids pairwise): an element of `other` can only
+// pair with this workgroup's elements if its id lies within [min, max] of the workgroup's own ids
+// `mine[0 .. n_mine)`.  Returns the first and last such index of other[0 .. n_other) (last = -1 if
+// there is none): exact for ids that do not decrease along the sequence, conservative otherwise
+// (the per-pair mask still decides).  `red` = 4 ints of LDS; every thread of the workgroup calls.
+template <int NT>
+__device__ __forceinline__ void id_window(const int32_t* mine, int n_mine, const int32_t* other, int n_other, int32_t* red,
+                                          int tid, int& first, int& last) {
+  if (tid == 0) { red[0] = INT32_MAX; red[1] = INT32_MIN; red[2] = INT32_MAX; red[3] = -1; }
+  __syncthreads();
+  for (int t = tid; t < n_mine; t += NT) {
+    const int32_t sid = mine[t];
+    __hip_atomic_fetch_min(&red[0], sid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __hip_atomic_fetch_max(&red[1], sid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+  __syncthreads();
+  const int32_t lo_id = red[0], hi_id = red[1];
+  int lo = INT32_MAX, hi = -1;
+  for (int t = tid; t < n_other; t += NT) {
+    const int32_t sid = other[t];
+    if (sid >= lo_id && sid <= hi_id) { lo = min(lo, t); hi = max(hi, t); }
+  }
+  if (hi >= 0) {
+    __hip_atomic_fetch_min(&red[2], lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __hip_atomic_fetch_max(&red[3], hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+  __syncthreads();
+  first = red[2];
+  last = red[3];
+  __syncthreads();  // the tiles reuse this memory
+}
+
 // ============================================================================================
 // dQ
 // ============================================================================================
@@ -149,16 +182,25 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(BwdParams p) {
   }
   const int32_t qseg = SEG ? p.qseg[(int64_t)b * p.lq + qrow_ld] : 0;
 
-  const int kend = p.causal ? min(p.lk, min(q0 + kBQ, p.lq)) : p.lk;
-  const int ntiles = (kend + kTile - 1) / kTile, last = ntiles - 1;
-  const int wave_last_tile = p.causal ? min(last, (wrow0 + 31) / kTile) : last;
+  // keys [kpos0, kend) are visited; tiles and key positions below count from kpos0
+  int kpos0 = 0, kend = p.causal ? min(p.lk, min(q0 + kBQ, p.lq)) : p.lk;
+  if constexpr (SEG) {
+    int first, lastk;
+    id_window<NT>(p.qseg + (int64_t)b * p.lq + q0, min(kBQ, p.lq - q0), p.kvseg + (int64_t)b * p.lk, kend,
+                  reinterpret_cast<int32_t*>(smem), tid, first, lastk);
+    if (lastk >= 0) { kpos0 = first / kTile * kTile; kend = lastk + 1; }
+    else kend = min(kend, kTile);  // nothing visible: one fully masked tile
+  }
+  const int lk_r = kend - kpos0, wrow_r = wrow0 - kpos0, qrow_r = qrow - kpos0;
+  const int ntiles = (lk_r + kTile - 1) / kTile, last = ntiles - 1;
+  const int wave_last_tile = p.causal ? min(last, max(wrow_r + 31, 0) / kTile) : last;
 
   // tile loader: raw buffer loads one tile ahead (rows past kend read as zero), stored to LDS later
   const int lt = tid / CPR, lc = tid % CPR;
   const int64_t tok_stride = (int64_t)p.H * D;
-  const int bytes = (int)(((int64_t)(kend - 1) * tok_stride + D) * 2);
-  const __amdgpu_buffer_rsrc_t k_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.k + ((int64_t)b * p.lk * p.H + h) * D), 0, bytes, kRsrcFlags);
-  const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.v + ((int64_t)b * p.lk * p.H + h) * D), 0, bytes, kRsrcFlags);
+  const int bytes = (int)(((int64_t)(lk_r - 1) * tok_stride + D) * 2);
+  const __amdgpu_buffer_rsrc_t k_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.k + (((int64_t)b * p.lk + kpos0) * p.H + h) * D), 0, bytes, kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.v + (((int64_t)b * p.lk + kpos0) * p.H + h) * D), 0, bytes, kRsrcFlags);
   const int voff = (int)((lt * tok_stride + 8 * lc) * 2);
   u32x4 kreg[NPASS], vreg[NPASS];
   int32_t seg_pending = 0;
@@ -170,7 +212,7 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(BwdParams p) {
       vreg[ps] = __builtin_amdgcn_raw_buffer_load_b128(v_rs, voff, soff, 0);
     }
     if constexpr (SEG)
-      if (tid < kTile) seg_pending = p.kvseg[(int64_t)b * p.lk + min(tile * kTile + tid, p.lk - 1)];
+      if (tid < kTile) seg_pending = p.kvseg[(int64_t)b * p.lk + kpos0 + min(tile * kTile + tid, lk_r - 1)];
   };
   auto commit = [&](int tile) __attribute__((always_inline)) {
     uint16_t* kd = lds_k + (tile & 1) * kTile * S;
@@ -193,8 +235,8 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(BwdParams p) {
     const uint16_t* ks = lds_k + (j & 1) * kTile * S;
     const uint16_t* vs = lds_v + (j & 1) * kTile * S;
     const int k0 = j * kTile;
-    const bool need_mask = (k0 + kTile > kend) || (p.causal && (k0 + kTile - 1 > wrow0));
-    const int limit = p.causal ? min(qrow, kend - 1) : kend - 1;  // largest visible key index
+    const bool need_mask = (k0 + kTile > lk_r) || (p.causal && (k0 + kTile - 1 > wrow_r));
+    const int limit = p.causal ? min(qrow_r, lk_r - 1) : lk_r - 1;  // largest visible key index
     static_for<2>([&](auto mb_c) __attribute__((always_inline)) {
       constexpr int mb = decltype(mb_c)::value;
       f32x16 s = nlse, dp = ndelta;
@@ -305,14 +347,23 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
     kseg[nb] = SEG ? p.kvseg[(int64_t)b * p.lk + key_ld] : 0;
   }
 
-  // query tiles: under the causal mask rows before this block's first key see none of its keys
-  const int tile0 = p.causal ? k0 / kTile : 0;
-  const int ntiles = max(0, (p.lq + kTile - 1) / kTile - tile0), last = ntiles - 1;
-  const int wave_first_tile = p.causal ? wkey0 / kTile - tile0 : 0;
+  // query tiles tile0 .. : under the causal mask rows before this block's first key see none of
+  // its keys; rows from lq_r on are not visited
+  int tile0 = p.causal ? k0 / kTile : 0, lq_r = p.lq;
+  if constexpr (SEG) {
+    int first, lastq;
+    const int rbeg = min(tile0 * kTile, p.lq);
+    id_window<NT>(p.kvseg + (int64_t)b * p.lk + k0, min(kBK, p.lk - k0), p.qseg + (int64_t)b * p.lq + rbeg, p.lq - rbeg,
+                  reinterpret_cast<int32_t*>(smem), tid, first, lastq);
+    if (lastq >= 0) { tile0 = (rbeg + first) / kTile; lq_r = rbeg + lastq + 1; }
+    else lq_r = 0;  // no row can see a key of this block
+  }
+  const int ntiles = max(0, (lq_r + kTile - 1) / kTile - tile0), last = ntiles - 1;
+  const int wave_first_tile = p.causal ? max(wkey0 / kTile - tile0, 0) : 0;
 
   const int lt = tid / CPR, lc = tid % CPR;
   const int64_t tok_stride = (int64_t)p.H * D;
-  const int bytes = (int)(((int64_t)(p.lq - 1) * tok_stride + D) * 2);
+  const int bytes = (int)(((int64_t)(max(lq_r, 1) - 1) * tok_stride + D) * 2);
   const __amdgpu_buffer_rsrc_t q_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.q + ((int64_t)b * p.lq * p.H + h) * D), 0, bytes, kRsrcFlags);
   const __amdgpu_buffer_rsrc_t g_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.d_o + ((int64_t)b * p.lq * p.H + h) * D), 0, bytes, kRsrcFlags);
   const int voff = (int)((lt * tok_stride + 8 * lc) * 2);
@@ -329,7 +380,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
       qreg[ps] = __builtin_amdgcn_raw_buffer_load_b128(q_rs, voff, soff, 0);
       greg[ps] = __builtin_amdgcn_raw_buffer_load_b128(g_rs, voff, soff, 0);
       const int r = r0 + ps * TPP + lt;
-      row_lse[ps] = r < p.lq ? lse_b[r] : -INFINITY;
+      row_lse[ps] = r < lq_r ? lse_b[r] : -INFINITY;
     }
     // threads 0..63: -lse, 64..127: -delta, 128..191: segment id of row r0 + tid % 64
     if (tid < 3 * kTile) {
@@ -337,7 +388,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
       const int rl = min(r, p.lq - 1);
       if (tid < kTile) {
         const float x = lse_b[rl];
-        aux_pending = (r < p.lq && x > -INFINITY) ? -x * kLog2e : -INFINITY;
+        aux_pending = (r < lq_r && x > -INFINITY) ? -x * kLog2e : -INFINITY;
       } else if (tid < 2 * kTile) {
         aux_pending = -del_b[rl];
       } else if (SEG) {

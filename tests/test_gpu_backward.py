@@ -253,3 +253,32 @@ def test_backward_mfma_refuses_what_it_cannot_run(gpu):
         tpa.tpa_factors_bwd(tq[..., :2], tq[..., 2:], tk[..., :2], tk[..., 2:], tv[..., :2], tv[..., 2:], None, None,
                             o, res[-1].permute(0, 2, 1), torch.ones_like(o), kernel=2)
     assert e.value.code == -6
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("pattern", ["long_runs", "shuffled", "island", "island_with_hole", "absent", "descending"])
+def test_backward_bf16_segment_id_patterns(gpu, pattern, causal):
+    """The MFMA backward kernels visit only the tiles between the first and last key (row) whose id
+    lies in the id range of a workgroup's rows (keys); the gradients must not depend on how the ids
+    are laid out."""
+    from test_gpu_parity import _id_pattern
+    from tpa import tpa
+
+    b, lq, lk, h, d = 2, 1536, 1536, 4, 128
+    q, k, v = make_factors(81, b, lq, lk, h, d, d, 3, 2, scale_by_rank=True)
+    do = np.random.default_rng(82).standard_normal((b, lq, h, d)).astype(np.float32)
+    qseg, kvseg = _id_pattern(pattern, b, lq, lk)
+    tq, tk, tv = (torch.from_numpy(x).to(gpu).to(torch.bfloat16) for x in (q, k, v))
+    tdo = torch.from_numpy(do).to(gpu).to(torch.bfloat16)
+    tqs, tks = torch.from_numpy(qseg).to(gpu), torch.from_numpy(kvseg).to(gpu)
+    sp = lambda t: (t[..., :h], t[..., h:])
+    o, lse = tpa.tpa_factors(*sp(tq), *sp(tk), *sp(tv), tqs, tks, d**-0.5, causal)
+    grads = tpa.tpa_factors_bwd(*sp(tq), *sp(tk), *sp(tv), tqs, tks, o, lse, tdo, d**-0.5, causal, kernel=2)
+    f64 = lambda t: t.detach().float().cpu().numpy().astype(np.float64)
+    want = orc.tpa_backward(f64(tq), f64(tk), f64(tv), qseg, kvseg, h, f64(tdo), sm_scale=d**-0.5, causal=causal)
+    got = [np.concatenate([f64(grads[2 * n]), f64(grads[2 * n + 1])], axis=-1) for n in range(3)]
+    for name, g, w in zip("qkv", got, want):
+        if pattern == "absent":
+            assert not np.any(g) and not np.any(w), name  # no pair is visible: every gradient is zero
+        else:
+            assert rel_err(g, w) <= 1.5e-2, name
