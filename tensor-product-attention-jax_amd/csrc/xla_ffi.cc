@@ -114,7 +114,84 @@ ffi::Error MhaFwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ff
   return rc == TPA_OK ? ffi::Error::Success() : fail(rc);
 }
 
+// Backward (replaces _tpa_bwd, tpa/tpa.py:168-214): operands q, k, v, o, lse[b, h, lq] (fp32, as
+// TpaFwd returned it) and do; results dq, dk, dv as fp32 arrays shaped like q, k, v, plus a u8
+// workspace of tpa_bwd_workspace_bytes(...) bytes that XLA allocates (256-byte aligned, as XLA's
+// buffers are).  Segment ids, when used, are two more operands (TpaBwdSeg).
+void split_grad(ffi::Result<ffi::AnyBuffer>& x, int h, TpaGrad* a, TpaGrad* b) {
+  const auto d = x->dimensions();
+  const int64_t sr = d[3], sl = d[2] * sr, sb = d[1] * sl;
+  float* base = static_cast<float*>(x->untyped_data());
+  *a = TpaGrad{base, sb, sl, sr};
+  *b = TpaGrad{base + h, sb, sl, sr};
+}
+
+ffi::Error TpaBwdCommon(hipStream_t stream, const ffi::AnyBuffer& q, const ffi::AnyBuffer& k, const ffi::AnyBuffer& v,
+                        const int32_t* qseg, const int32_t* kvseg, const ffi::AnyBuffer& o, const ffi::AnyBuffer& lse,
+                        const ffi::AnyBuffer& d_o, ffi::Result<ffi::AnyBuffer>& dq, ffi::Result<ffi::AnyBuffer>& dk,
+                        ffi::Result<ffi::AnyBuffer>& dv, ffi::Result<ffi::AnyBuffer>& workspace, int32_t num_heads,
+                        float sm_scale, bool causal) {
+  const auto qd = q.dimensions(), kd = k.dimensions(), vd = v.dimensions();
+  if (qd.size() != 4 || kd.size() != 4 || vd.size() != 4) return ffi::Error::InvalidArgument("q, k, v must be [b, l, r, h+d]");
+  const int code = dtype_code(q.element_type());
+  if (code < 0 || k.element_type() != q.element_type() || v.element_type() != q.element_type() ||
+      o.element_type() != q.element_type() || d_o.element_type() != q.element_type())
+    return ffi::Error::InvalidArgument("q, k, v, o, do must share one of f32 / bf16");
+  if (lse.element_type() != ffi::DataType::F32 || dq->element_type() != ffi::DataType::F32 ||
+      dk->element_type() != ffi::DataType::F32 || dv->element_type() != ffi::DataType::F32)
+    return ffi::Error::InvalidArgument("lse and the gradients are f32");
+  TpaBwdArgs a{};
+  split(q, num_heads, code, &a.qa, &a.qb);
+  split(k, num_heads, code, &a.ka, &a.kb);
+  split(v, num_heads, code, &a.va, &a.vb);
+  split_grad(dq, num_heads, &a.dqa, &a.dqb);
+  split_grad(dk, num_heads, &a.dka, &a.dkb);
+  split_grad(dv, num_heads, &a.dva, &a.dvb);
+  a.q_segment_ids = qseg; a.kv_segment_ids = kvseg;
+  a.o = o.untyped_data(); a.lse = static_cast<const float*>(lse.untyped_data()); a.d_o = d_o.untyped_data();
+  a.B = (int32_t)qd[0]; a.lq = (int32_t)qd[1]; a.lk = (int32_t)kd[1]; a.H = num_heads;
+  a.dk = (int32_t)qd[3] - num_heads; a.dv = (int32_t)vd[3] - num_heads;
+  a.rq = (int32_t)qd[2]; a.rk = (int32_t)kd[2];
+  a.dtype = code; a.sm_scale = sm_scale; a.causal = causal ? 1 : 0; a.kernel = TPA_KERNEL_AUTO;
+  a.workspace = workspace->untyped_data(); a.workspace_bytes = workspace->size_bytes();
+  const int rc = tpa_bwd(&a, stream);
+  return rc == TPA_OK ? ffi::Error::Success() : fail(rc);
+}
+
+ffi::Error TpaBwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v, ffi::AnyBuffer o,
+                      ffi::AnyBuffer lse, ffi::AnyBuffer d_o, ffi::Result<ffi::AnyBuffer> dq, ffi::Result<ffi::AnyBuffer> dk,
+                      ffi::Result<ffi::AnyBuffer> dv, ffi::Result<ffi::AnyBuffer> workspace, int32_t num_heads,
+                      float sm_scale, bool causal) {
+  return TpaBwdCommon(stream, q, k, v, nullptr, nullptr, o, lse, d_o, dq, dk, dv, workspace, num_heads, sm_scale, causal);
+}
+
+ffi::Error TpaBwdSegImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v,
+                         ffi::Buffer<ffi::DataType::S32> q_segment_ids, ffi::Buffer<ffi::DataType::S32> kv_segment_ids,
+                         ffi::AnyBuffer o, ffi::AnyBuffer lse, ffi::AnyBuffer d_o, ffi::Result<ffi::AnyBuffer> dq,
+                         ffi::Result<ffi::AnyBuffer> dk, ffi::Result<ffi::AnyBuffer> dv,
+                         ffi::Result<ffi::AnyBuffer> workspace, int32_t num_heads, float sm_scale, bool causal) {
+  return TpaBwdCommon(stream, q, k, v, q_segment_ids.typed_data(), kv_segment_ids.typed_data(), o, lse, d_o, dq, dk, dv,
+                      workspace, num_heads, sm_scale, causal);
+}
+
 }  // namespace
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(TpaBwd, TpaBwdImpl,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
+                                  .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
+                                  .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
+                                  .Attr<int32_t>("num_heads").Attr<float>("sm_scale").Attr<bool>("causal"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(TpaBwdSeg, TpaBwdSegImpl,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
+                                  .Arg<ffi::Buffer<ffi::DataType::S32>>().Arg<ffi::Buffer<ffi::DataType::S32>>()
+                                  .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
+                                  .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
+                                  .Attr<int32_t>("num_heads").Attr<float>("sm_scale").Attr<bool>("causal"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(TpaFwd, TpaFwdImpl,
                               ffi::Ffi::Bind()
