@@ -68,6 +68,19 @@ int tpa_fwd(const TpaFwdArgs* a, void* stream) {
   return tpa_generic_launch(a, s);
 }
 
+size_t tpa_fwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dk, int32_t dv, int32_t rq, int32_t rk) {
+  (void)rq;
+  if (B <= 0 || lq <= 0 || lk <= 0 || H <= 0 || dk <= 0 || dv <= 0 || rk <= 0) return 0;
+  if (dk != dv || (dk != 64 && dk != 128)) return 0;  // the kernels that use a workspace take these head sizes only
+  size_t need = 0;
+  if (lq <= 16 && lk >= 1024) need = tpa_decode_workspace_bytes(B, lq, lk, H, dv, 0);
+  if (rk != 2 && lq > 256) {
+    const size_t dense = tpa_prefill_dense_kv_bytes(B, lk, H, dk);
+    if (dense > need) need = dense;
+  }
+  return need;
+}
+
 int tpa_decode(const TpaFwdArgs* a, void* stream) {
   const int rc = validate_tpa(a);
   if (rc != TPA_OK) return rc;

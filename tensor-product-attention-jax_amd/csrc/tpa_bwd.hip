@@ -507,6 +507,17 @@ int mha_bwd_t(const MhaBwdArgs* a, hipStream_t stream, bool mfma) {
 }  // namespace
 }  // namespace tpa
 
+int tpa_recon_dense_bf16(const TpaFactor* fa, const TpaFactor* fb, uint16_t* out, int B, int L, int H, int D, int R, hipStream_t stream) {
+  if (B > 65535) return TPA_ERR_SHAPE;
+  const bool vec = D % 8 == 0 && !(reinterpret_cast<uintptr_t>(fb->ptr) & 15) && fb->stride_b % 8 == 0 && fb->stride_l % 8 == 0 &&
+                   fb->stride_r % 8 == 0;
+  if (vec)
+    hipLaunchKernelGGL(tpa::recon_bf16_kernel, dim3(L, B), dim3(256), 0, stream, *fa, *fb, out, L, H, D, R);
+  else
+    hipLaunchKernelGGL((tpa::recon_kernel<uint16_t, uint16_t>), dim3(L, B), dim3(256), 0, stream, *fa, *fb, out, L, H, D, R);
+  return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
+}
+
 size_t tpa_bwd_workspace_size(int64_t B, int64_t lq, int64_t lk, int64_t H, int64_t dk, int64_t dv) {
   using tpa::align256;
   const size_t nq = (size_t)(B * lq * H * dk), nk = (size_t)(B * lk * H * dk), nv = (size_t)(B * lk * H * dv), nd = (size_t)(B * H * lq);

@@ -47,6 +47,7 @@ struct PrefillParams {
   int causal;
   int nqb;     // query blocks per (batch, head)
   int npairs;  // nqb * B
+  int q_factors;  // dense K/V loader only: 1 = Q is still given by its rank factors qa, qb
 };
 
 template <int D>
@@ -96,9 +97,9 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   // scalars out of the argument block (never take the address of the block itself)
   struct Fac { const uint16_t* ptr; int64_t stride_b; int stride_l, stride_r; };
   auto fac = [](const TpaFactor& f) { return Fac{static_cast<const uint16_t*>(f.ptr), f.stride_b, (int)f.stride_l, (int)f.stride_r}; };
-  struct { Fac qa, qb, ka, kb, va, vb; const int32_t* qseg; const int32_t* kvseg; uint16_t* o; float* lse; int B, lq, lk, H, rq, rk; float sm_scale; int causal, nqb, npairs; } const p = {
+  struct { Fac qa, qb, ka, kb, va, vb; const int32_t* qseg; const int32_t* kvseg; uint16_t* o; float* lse; int B, lq, lk, H, rq, rk; float sm_scale; int causal, nqb, npairs, q_factors; } const p = {
       fac(pp.qa), fac(pp.qb), fac(pp.ka), fac(pp.kb), fac(pp.va), fac(pp.vb), pp.qseg, pp.kvseg, pp.o, pp.lse, pp.B, pp.lq, pp.lk, pp.H, pp.rq, pp.rk,
-      pp.sm_scale, pp.causal, pp.nqb, pp.npairs};
+      pp.sm_scale, pp.causal, pp.nqb, pp.npairs, pp.q_factors};
 
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   uint16_t* const lds_k = smem;                                  // [2][kTK][KS]
@@ -129,7 +130,10 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   // c * Q[qrow][16ks + 8g + 0..7]
   bf16x8 qf[NKS];
   auto build_q = [&]() __attribute__((always_inline)) {
-    if constexpr (LOADER == LOAD_DENSE) {
+    // the dense loader serves dense attention (Q dense too) and factored attention whose K and V
+    // were reconstructed beforehand (Q still in factors)
+    const bool dense_q = LOADER == LOAD_DENSE && !p.q_factors;
+    if (dense_q) {
       const uint16_t* qp = p.qb.ptr + b * p.qb.stride_b + (int64_t)qrow_ld * p.qb.stride_l + (int64_t)h * D;
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
@@ -888,6 +892,13 @@ int tpa_prefill_mfma_supported(const TpaFwdArgs* a) {
   return 1;
 }
 
+// bytes of workspace that let the prefill kernel run on dense K and V (both bf16 [B, lk, H, D]);
+// 0 if a batch entry would not fit the kernel's 32-bit tile offsets
+size_t tpa_prefill_dense_kv_bytes(int64_t B, int64_t lk, int64_t H, int64_t D) {
+  if (lk * H * D * 2 >= (int64_t(1) << 31)) return 0;
+  return (size_t)(2 * ((B * lk * H * D * 2 + 255) / 256 * 256));
+}
+
 int tpa_prefill_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
   using namespace tpa;
   PrefillParams p{};
@@ -898,6 +909,28 @@ int tpa_prefill_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
   p.sm_scale = a->sm_scale; p.causal = a->causal;
   p.nqb = (a->lq + kBQ - 1) / kBQ;
   p.npairs = p.nqb * a->B;
+  // Ranks other than 2: every workgroup of the fused kernel would rebuild the K/V tiles of its
+  // head from all ranks again (once per 256 query rows).  With a workspace the dense K and V are
+  // built once and the kernel runs with its plain tile loader, Q still coming from its factors.
+  const size_t dense_bytes = tpa_prefill_dense_kv_bytes(a->B, a->lk, a->H, a->dk);
+  if (a->rk != 2 && a->lq > kBQ && a->workspace && dense_bytes && a->workspace_bytes >= dense_bytes &&
+      !(reinterpret_cast<uintptr_t>(a->workspace) & 255)) {
+    uint16_t* kd = static_cast<uint16_t*>(a->workspace);
+    uint16_t* vd = kd + dense_bytes / 4;
+    int rc = tpa_recon_dense_bf16(&a->ka, &a->kb, kd, a->B, a->lk, a->H, a->dk, a->rk, stream);
+    if (rc == TPA_OK) rc = tpa_recon_dense_bf16(&a->va, &a->vb, vd, a->B, a->lk, a->H, a->dv, a->rk, stream);
+    if (rc != TPA_OK) return rc;
+    const int64_t hd = (int64_t)a->H * a->dk;
+    p.kb = TpaFactor{kd, a->lk * hd, hd, 0};
+    p.vb = TpaFactor{vd, a->lk * hd, hd, 0};
+    p.q_factors = 1;
+    if (p.kvseg) {
+      if (a->dk == 128) return launch_prefill<128, LOAD_DENSE, true>(p, stream);
+      return launch_prefill<64, LOAD_DENSE, true>(p, stream);
+    }
+    if (a->dk == 128) return launch_prefill<128, LOAD_DENSE>(p, stream);
+    return launch_prefill<64, LOAD_DENSE>(p, stream);
+  }
   if (p.kvseg) {
     if (a->dk == 128) {
       if (a->rk == 2) return launch_prefill<128, LOAD_TPA_R2, true>(p, stream);

@@ -196,6 +196,8 @@ def load_library(path: str | None = None) -> ctypes.CDLL:
         lib.tpa_decode_default_splits.argtypes = [ctypes.c_int32] * 4
         lib.mha_fwd_workspace_bytes.restype = ctypes.c_size_t
         lib.mha_fwd_workspace_bytes.argtypes = [ctypes.c_int32] * 6
+        lib.tpa_fwd_workspace_bytes.restype = ctypes.c_size_t
+        lib.tpa_fwd_workspace_bytes.argtypes = [ctypes.c_int32] * 8
         lib.tpa_bwd.restype = ctypes.c_int
         lib.tpa_bwd.argtypes = [ctypes.POINTER(TpaBwdArgs), ctypes.c_void_p]
         lib.mha_bwd.restype = ctypes.c_int

@@ -98,6 +98,7 @@ def tpa_factors(
     causal: bool = False,
     kernel: int = _d.KERNEL_AUTO,
     return_lse: bool = True,
+    use_workspace: bool = True,
 ):
     """Forward pass on the six split factor arrays, the operands of the reference's kernel
     launch (tpa/tpa.py:246-251,543) with a leading batch dimension:
@@ -106,6 +107,8 @@ def tpa_factors(
 
     Returns (o[b,lq,h,dv] in the input dtype, lse[b,h,lq] fp32 or None).  The arrays may be
     views (e.g. slices of the concatenated tensors); only the last dimension must be contiguous.
+    `use_workspace=False` withholds the optional scratch memory, which keeps the call on the
+    fused prefill kernel whatever the problem.
     """
     device = _pick_device(qa, qb, ka, kb, va, vb)
     qa, qb, ka, kb, va, vb = (_as_device_tensor(x, device) for x in (qa, qb, ka, kb, va, vb))
@@ -129,11 +132,16 @@ def tpa_factors(
     o = torch.empty((b, lq, h, dv), dtype=dtype, device=device)
     lse = torch.empty((b, h, lq), dtype=torch.float32, device=device) if return_lse else None
     lib = _d.load_library()
-    # decode through the reference's own entry point (lq = 1 over a long cache): hand the library
-    # the workspace its split-key kernel needs; it decides whether the problem qualifies
-    ws = None
-    if lq <= 16 and lk >= 1024 and not causal and qseg is None and dtype == torch.bfloat16 and kernel != _d.KERNEL_GENERIC:
-        ws = torch.empty(max(lib.tpa_decode_workspace_bytes(b, lq, lk, h, dv, 0), 16), dtype=torch.uint8, device=device)
+    # hand the library the workspace with which it can pick its fastest kernel (split partials for
+    # a decode through this entry point, dense K and V for ranks other than 2); it decides whether
+    # the problem qualifies
+    ws, ws_ptr, ws_bytes = None, None, 0
+    if use_workspace and dtype == torch.bfloat16 and kernel != _d.KERNEL_GENERIC:
+        need = lib.tpa_fwd_workspace_bytes(b, lq, lk, h, dk, dv, rq, rk)
+        if need:
+            ws = torch.empty(need + 256, dtype=torch.uint8, device=device)
+            pad = (-ws.data_ptr()) % 256
+            ws_ptr, ws_bytes = ws.data_ptr() + pad, need
     args = _d.TpaFwdArgs(
         qa=_d.factor(qa), qb=_d.factor(qb), ka=_d.factor(ka), kb=_d.factor(kb), va=_d.factor(va), vb=_d.factor(vb),
         q_segment_ids=qseg.data_ptr() if qseg is not None else None,
@@ -141,7 +149,7 @@ def tpa_factors(
         o=o.data_ptr(), lse=lse.data_ptr() if lse is not None else None,
         B=b, lq=lq, lk=lk, H=h, dk=dk, dv=dv, rq=rq, rk=rk,
         dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=int(bool(causal)), kernel=int(kernel),
-        workspace=ws.data_ptr() if ws is not None else None, workspace_bytes=ws.numel() if ws is not None else 0, num_splits=0,
+        workspace=ws_ptr, workspace_bytes=ws_bytes, num_splits=0,
     )
     with torch.cuda.device(device):
         _d.check("tpa_fwd", lib.tpa_fwd(args, _d.current_stream_ptr(device)))

@@ -71,6 +71,11 @@ def test_size_queries_need_no_gpu():
     assert lib.tpa_decode_workspace_bytes(64, 1, 8192, 32, 128, 0) == 64 * 4 * 32 * (128 + 2) * 4
     assert lib.tpa_decode_workspace_bytes(64, 1, 8192, 32, 128, 7) == 64 * 7 * 32 * (128 + 2) * 4
     assert lib.tpa_decode_default_splits(0, 1, 8192, 32) == 0
+    # optional forward workspace: decode partials, or dense bf16 K and V when the rank is not 2
+    assert lib.tpa_fwd_workspace_bytes(64, 1, 8192, 32, 128, 128, 6, 2) == lib.tpa_decode_workspace_bytes(64, 1, 8192, 32, 128, 0)
+    assert lib.tpa_fwd_workspace_bytes(8, 2048, 2048, 64, 64, 64, 16, 8) == 2 * 8 * 2048 * 64 * 64 * 2
+    assert lib.tpa_fwd_workspace_bytes(4, 4096, 4096, 16, 128, 128, 6, 2) == 0   # rank 2: the fused kernel
+    assert lib.tpa_fwd_workspace_bytes(2, 512, 512, 4, 48, 48, 6, 4) == 0        # not an MFMA head size
     # backward: dense Q, K, V and their gradients (fp32, each rounded up to 256 bytes) plus delta
     r = lambda n: (n + 255) // 256 * 256
     nq, nk, nv, nd = 2 * 10 * 3 * 5 * 4, 2 * 7 * 3 * 5 * 4, 2 * 7 * 3 * 6 * 4, 2 * 3 * 10 * 4

@@ -635,3 +635,29 @@ def test_prefill_bf16_segment_runs_other_instances(gpu, d, rk):
     o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), tqs, tks, d**-0.5, True, 2)
     o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), qseg, kvseg, h, sm_scale=d**-0.5, causal=True)
     check(o, lse, o_ref, l_ref, BF16_TOL)
+
+
+@pytest.mark.parametrize("d,rk,causal,seg", [(64, 8, False, None), (128, 4, True, None), (128, 3, True, 300), (64, 1, False, 150)])
+def test_prefill_high_rank_through_dense_kv(gpu, d, rk, causal, seg):
+    """Ranks other than 2: with the optional workspace K and V are reconstructed once and the flash
+    kernel runs on dense tiles; without it every workgroup rebuilds its tiles from all ranks.  Both
+    round K and V to bf16 after an fp32 sum over the ranks, so the two routes agree far inside
+    the bf16 tolerance."""
+    from tpa import tpa
+
+    b, lq, lk, h, rq = 2, 700, 900, 8, 5
+    q, k, v = make_factors(91, b, lq, lk, h, d, d, rq, rk, scale_by_rank=True)
+    qseg = segment_ids(lq, seg, b) if seg else None
+    kvseg = segment_ids(lk, seg, b) if seg else None
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    tqs = torch.from_numpy(qseg).to(gpu) if seg else None
+    tks = torch.from_numpy(kvseg).to(gpu) if seg else None
+    from tpa import _dispatch as dd
+    assert dd.load_library().tpa_fwd_workspace_bytes(b, lq, lk, h, d, d, rq, rk) > 0
+    o1, l1 = tpa.tpa_factors(*split(tq, tk, tv, h), tqs, tks, d**-0.5, causal, 2)
+    o2, l2 = tpa.tpa_factors(*split(tq, tk, tv, h), tqs, tks, d**-0.5, causal, 2, use_workspace=False)
+    o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), qseg, kvseg, h, sm_scale=d**-0.5, causal=causal)
+    check(o1, l1, o_ref, l_ref, BF16_TOL)
+    check(o2, l2, o_ref, l_ref, BF16_TOL)
+    diff = (torch.nan_to_num(o1.float()) - torch.nan_to_num(o2.float())).abs().max().item()
+    assert diff <= 0.25 * BF16_TOL * max(1.0, float(np.nanmax(np.abs(o_ref))))
