@@ -184,8 +184,13 @@ int launch_generic(const GenericParams& p, hipStream_t stream) {
     hipLaunchKernelGGL((generic_fwd_kernel<T, 64>), grid, block, smem, stream, p);
   else if (dmax <= 128)
     hipLaunchKernelGGL((generic_fwd_kernel<T, 128>), grid, block, smem, stream, p);
-  else if (dmax <= 256)
+  else if (dmax <= 256) {
+    // two 256-wide tiles are a few bytes over the 64 KB a kernel gets without asking
+    if (smem > 64 * 1024 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(generic_fwd_kernel<T, 256>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+      return TPA_ERR_LAUNCH;
     hipLaunchKernelGGL((generic_fwd_kernel<T, 256>), grid, block, smem, stream, p);
+  }
   else
     return TPA_ERR_SHAPE;
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;

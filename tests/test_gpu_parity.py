@@ -661,3 +661,21 @@ def test_prefill_high_rank_through_dense_kv(gpu, d, rk, causal, seg):
     check(o2, l2, o_ref, l_ref, BF16_TOL)
     diff = (torch.nan_to_num(o1.float()) - torch.nan_to_num(o2.float())).abs().max().item()
     assert diff <= 0.25 * BF16_TOL * max(1.0, float(np.nanmax(np.abs(o_ref))))
+
+
+def test_fp32_widest_heads(gpu):
+    """dk = dv = 256, the widest head the library takes (forward and backward, fp32 kernels)."""
+    from tpa import tpa
+
+    b, lq, lk, h, d = 1, 70, 90, 2, 256
+    q, k, v = make_factors(95, b, lq, lk, h, d, d, 2, 2, scale_by_rank=True)
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu).requires_grad_() for x in (q, k, v))
+    o, res = tpa._tpa_fwd(tq, tk, tv, h, None, None, d**-0.5, True, None, False, False, False)
+    o_ref, l_ref = orc.tpa_reference(q, k, v, None, None, h, sm_scale=d**-0.5, causal=True)
+    check(o, res[-1].permute(0, 2, 1), o_ref, l_ref, F32_TOL)
+    do = np.random.default_rng(96).standard_normal(o_ref.shape).astype(np.float32)
+    o.backward(torch.from_numpy(do).to(gpu))
+    want = orc.tpa_backward(q, k, v, None, None, h, do, sm_scale=d**-0.5, causal=True)
+    for t, w in zip((tq, tk, tv), want):
+        g = t.grad.cpu().numpy().astype(np.float64)
+        assert np.max(np.abs(g - w)) <= 2e-4 * np.max(np.abs(w))
