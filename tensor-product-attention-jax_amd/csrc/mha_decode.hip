@@ -87,8 +87,8 @@ __global__ __launch_bounds__(kWaves * 64) void mha_decode_kernel(MhaDecodeParams
 #pragma unroll
       for (int i = 0; i < kNL; ++i)
         if (slot_ok[i]) {
-          kr[u][i] = *reinterpret_cast<const u32x4*>(kb + t * row + i * HPL * D);
-          vr[u][i] = *reinterpret_cast<const u32x4*>(vb + t * row + i * HPL * D);
+          kr[u][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kb + t * row + i * HPL * D));
+          vr[u][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vb + t * row + i * HPL * D));
         }
     }
   };

@@ -103,7 +103,9 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   const int lb_row = l / CPR, lb_c = l % CPR;             // B tiles: row within the instruction, chunk
   const int la_row = l >> 2, la_c = min(l & 3, a_chunks - 1);  // A tiles: 16 rows per instruction
 
-  // two register sets: while one block is staged and consumed, two more are in flight
+  // two register sets: while one block is staged and consumed, two more are in flight.  The cache
+  // is read exactly once per call, so the loads are marked non-temporal (measured on the whole
+  // call: 5.1 -> 5.75 TB/s)
   u32x4 rbk[2][NLB], rbv[2][NLB], rak[2][2], rav[2][2];
   auto issue = [&](auto set_c, int blk) {
     constexpr int set = decltype(set_c)::value;
@@ -111,14 +113,14 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
 #pragma unroll
     for (int n = 0; n < NLB; ++n) {
       const int row = min(row0 + n * RPI + lb_row, last_row);
-      rbk[set][n] = *reinterpret_cast<const u32x4*>(kb_base + (int64_t)row * p.kb.stride_r + 8 * lb_c);
-      rbv[set][n] = *reinterpret_cast<const u32x4*>(vb_base + (int64_t)row * p.vb.stride_r + 8 * lb_c);
+      rbk[set][n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kb_base + (int64_t)row * p.kb.stride_r + 8 * lb_c));
+      rbv[set][n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vb_base + (int64_t)row * p.vb.stride_r + 8 * lb_c));
     }
 #pragma unroll
     for (int n = 0; n < 2; ++n) {
       const int row = min(row0 + 16 * n + la_row, last_row);
-      rak[set][n] = *reinterpret_cast<const u32x4*>(ka_base + (int64_t)row * p.ka.stride_r + 8 * la_c);
-      rav[set][n] = *reinterpret_cast<const u32x4*>(va_base + (int64_t)row * p.va.stride_r + 8 * la_c);
+      rak[set][n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(ka_base + (int64_t)row * p.ka.stride_r + 8 * la_c));
+      rav[set][n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(va_base + (int64_t)row * p.va.stride_r + 8 * la_c));
     }
   };
   auto stage = [&](auto set_c) {
