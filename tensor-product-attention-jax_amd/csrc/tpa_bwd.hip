@@ -92,7 +92,8 @@ __global__ void delta_kernel(const T* o, const T* d_o, float* delta, int B, int 
     if constexpr (sizeof(T) == 2) {
       if (vec) {
         for (int d = 8 * sub; d < dv; d += 128) {
-          const u32x4 a = *reinterpret_cast<const u32x4*>(op + d), g = *reinterpret_cast<const u32x4*>(gp + d);
+          const u32x4 a = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(op + d));
+          const u32x4 g = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(gp + d));
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const float x0 = bf16lo_to_f32(a[j]) * bf16lo_to_f32(g[j]), x1 = bf16hi_to_f32(a[j]) * bf16hi_to_f32(g[j]);
@@ -327,7 +328,7 @@ __global__ __launch_bounds__(256) void project_kernel(const float* dx, TpaFactor
     float* as = bs + R * D;
     for (int idx = threadIdx.x; idx < H * D / 4; idx += 256) {
       const int h = idx / (D / 4), d4 = idx - h * (D / 4);
-      *reinterpret_cast<f32x4*>(xs + h * XS + 4 * d4) = *reinterpret_cast<const f32x4*>(xp + 4 * idx);
+      *reinterpret_cast<f32x4*>(xs + h * XS + 4 * d4) = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xp + 4 * idx));
     }
     for (int idx = threadIdx.x; idx < R * D; idx += 256) {
       const int r = idx / D, d = idx - r * D;
