@@ -140,10 +140,12 @@ __device__ __forceinline__ void id_window(const int32_t* mine, int n_mine, const
 // ============================================================================================
 // dQ
 // ============================================================================================
-template <int D, bool SEG>
-__global__ __launch_bounds__(512) void bwd_dq_kernel(BwdParams p) {
-  constexpr int NT = 512, S = tile_stride(D), CPR = D / 8, TPP = NT / CPR, NPASS = kTile / TPP;
-  constexpr int NKS = D / 16, NDB = D / 32, kBQ = 256;
+template <int D, int NW, int NB, bool SEG>
+__global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(BwdParams p) {
+  // a wave owns NB blocks of 32 query rows: every operand fragment read from LDS feeds NB MFMAs
+  constexpr int NT = NW * 64, S = tile_stride(D), CPR = D / 8, TPP = NT / CPR, NPASS = kTile / TPP;
+  constexpr int NKS = D / 16, NDB = D / 32, kWQ = 32 * NB, kBQ = NW * kWQ;
+  static_assert(kTile % TPP == 0 && NPASS >= 1, "loader shape");
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   uint16_t* const lds_k = smem;                  // [2][64][S]
   uint16_t* const lds_v = smem + 2 * kTile * S;  // [2][64][S]
@@ -155,16 +157,20 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(BwdParams p) {
   const int qblk = p.nblk - 1 - pair / p.B, b = pair % p.B;  // heaviest causal blocks first
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
   const int lp = l & 15, dhalf = (l >> 4) & 1;
-  const int q0 = qblk * kBQ, wrow0 = q0 + 32 * w, qrow = wrow0 + i, qrow_ld = min(qrow, p.lq - 1);
+  const int q0 = qblk * kBQ, wrow0 = q0 + kWQ * w;
   const float c = p.sm_scale * kLog2e;
 
-  // this lane's row: Q (scaled) and dO as B-operand fragments, -lse (log2 domain) and -delta
-  const float lse_r = p.lse[((int64_t)b * p.H + h) * p.lq + qrow_ld];
-  const bool live = qrow < p.lq && lse_r > -INFINITY;
-  const f32x16 nlse = splat16(live ? -lse_r * kLog2e : -INFINITY);
-  const f32x16 ndelta = splat16(-p.delta[((int64_t)b * p.H + h) * p.lq + qrow_ld]);
-  bf16x8 qf[NKS], gf[NKS];
-  {
+  // this lane's rows: Q (scaled) and dO as B-operand fragments, -lse (log2 domain) and -delta
+  f32x16 nlse[NB], ndelta[NB];
+  bf16x8 qf[NB][NKS], gf[NB][NKS];
+  int32_t qseg[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int qrow = wrow0 + 32 * nb + i, qrow_ld = min(qrow, p.lq - 1);
+    const float lse_r = p.lse[((int64_t)b * p.H + h) * p.lq + qrow_ld];
+    const bool live = qrow < p.lq && lse_r > -INFINITY;
+    nlse[nb] = splat16(live ? -lse_r * kLog2e : -INFINITY);
+    ndelta[nb] = splat16(-p.delta[((int64_t)b * p.H + h) * p.lq + qrow_ld]);
     const uint16_t* qp = p.q + (((int64_t)b * p.lq + qrow_ld) * p.H + h) * D;
     const uint16_t* gp = p.d_o + (((int64_t)b * p.lq + qrow_ld) * p.H + h) * D;
 #pragma unroll
@@ -176,11 +182,11 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(BwdParams p) {
         sc[j] = pack_bf16(bf16lo_to_f32(raw[j]) * c, bf16hi_to_f32(raw[j]) * c);
         if (!live) gr[j] = 0u;  // the upstream gradient of a row without a visible key may be NaN
       }
-      qf[ks] = __builtin_bit_cast(bf16x8, sc);
-      gf[ks] = __builtin_bit_cast(bf16x8, gr);
+      qf[nb][ks] = __builtin_bit_cast(bf16x8, sc);
+      gf[nb][ks] = __builtin_bit_cast(bf16x8, gr);
     }
+    qseg[nb] = SEG ? p.qseg[(int64_t)b * p.lq + qrow_ld] : 0;
   }
-  const int32_t qseg = SEG ? p.qseg[(int64_t)b * p.lq + qrow_ld] : 0;
 
   // keys [kpos0, kend) are visited; tiles and key positions below count from kpos0
   int kpos0 = 0, kend = p.causal ? min(p.lk, min(q0 + kBQ, p.lq)) : p.lk;
@@ -191,9 +197,9 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(BwdParams p) {
     if (lastk >= 0) { kpos0 = first / kTile * kTile; kend = lastk + 1; }
     else kend = min(kend, kTile);  // nothing visible: one fully masked tile
   }
-  const int lk_r = kend - kpos0, wrow_r = wrow0 - kpos0, qrow_r = qrow - kpos0;
+  const int lk_r = kend - kpos0, wrow_r = wrow0 - kpos0;
   const int ntiles = (lk_r + kTile - 1) / kTile, last = ntiles - 1;
-  const int wave_last_tile = p.causal ? min(last, max(wrow_r + 31, 0) / kTile) : last;
+  const int wave_last_tile = p.causal ? min(last, max(wrow_r + kWQ - 1, 0) / kTile) : last;
 
   // tile loader: raw buffer loads one tile ahead (rows past kend read as zero), stored to LDS later
   const int lt = tid / CPR, lc = tid % CPR;
@@ -227,51 +233,64 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(BwdParams p) {
       if (tid < kTile) lds_seg[(tile & 1) * kTile + tid] = seg_pending;
   };
 
-  f32x16 acc[NDB];
+  f32x16 acc[NB][NDB];
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) acc[db] = splat16(0.f);
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) acc[nb][db] = splat16(0.f);
 
   auto compute = [&](int j) __attribute__((always_inline)) {
     const uint16_t* ks = lds_k + (j & 1) * kTile * S;
     const uint16_t* vs = lds_v + (j & 1) * kTile * S;
     const int k0 = j * kTile;
     const bool need_mask = (k0 + kTile > lk_r) || (p.causal && (k0 + kTile - 1 > wrow_r));
-    const int limit = p.causal ? min(qrow_r, lk_r - 1) : lk_r - 1;  // largest visible key index
     static_for<2>([&](auto mb_c) __attribute__((always_inline)) {
       constexpr int mb = decltype(mb_c)::value;
-      f32x16 s = nlse, dp = ndelta;
+      f32x16 s[NB], dp[NB];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) { s[nb] = nlse[nb]; dp[nb] = ndelta[nb]; }
       static_for<NKS>([&](auto kk_c) __attribute__((always_inline)) {
         constexpr int kk = decltype(kk_c)::value;
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rows_frag<S>(ks, mb, kk, i, g), qf[kk], s, 0, 0, 0);
+        const bf16x8 a = rows_frag<S>(ks, mb, kk, i, g);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[nb][kk], s[nb], 0, 0, 0);
       });
       static_for<NKS>([&](auto kk_c) __attribute__((always_inline)) {
         constexpr int kk = decltype(kk_c)::value;
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rows_frag<S>(vs, mb, kk, i, g), gf[kk], dp, 0, 0, 0);
+        const bf16x8 a = rows_frag<S>(vs, mb, kk, i, g);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) dp[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, gf[nb][kk], dp[nb], 0, 0, 0);
       });
-      if (need_mask) {
+      bf16x8 df[NB][2];
 #pragma unroll
-        for (int v = 0; v < 16; ++v)
-          if (k0 + 32 * mb + 8 * (v >> 2) + 4 * g + (v & 3) > limit) s[v] = -INFINITY;
-      }
-      if constexpr (SEG) {
-        const int32_t* ids_p = lds_seg + (j & 1) * kTile + 32 * mb + 4 * g;
+      for (int nb = 0; nb < NB; ++nb) {
+        if (need_mask) {
+          const int qrow_r = wrow_r + 32 * nb + i;
+          const int limit = p.causal ? min(qrow_r, lk_r - 1) : lk_r - 1;  // largest visible key index
 #pragma unroll
-        for (int vq = 0; vq < 4; ++vq) {
-          const int4 ids = *reinterpret_cast<const int4*>(ids_p + 8 * vq);
-          if (ids.x != qseg) s[4 * vq] = -INFINITY;
-          if (ids.y != qseg) s[4 * vq + 1] = -INFINITY;
-          if (ids.z != qseg) s[4 * vq + 2] = -INFINITY;
-          if (ids.w != qseg) s[4 * vq + 3] = -INFINITY;
+          for (int v = 0; v < 16; ++v)
+            if (k0 + 32 * mb + 8 * (v >> 2) + 4 * g + (v & 3) > limit) s[nb][v] = -INFINITY;
         }
-      }
+        if constexpr (SEG) {
+          const int32_t* ids_p = lds_seg + (j & 1) * kTile + 32 * mb + 4 * g;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) s[v] = __builtin_amdgcn_exp2f(s[v]) * dp[v];  // p * (dp - delta)
-      bf16x8 f0, f1;
-      pack_block(s, f0, f1);
-      static_for<NDB>([&](auto db_c) __attribute__((always_inline)) {
-        constexpr int db = decltype(db_c)::value;
-        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cols_frag<S>(ks, 2 * mb, db, g, lp, dhalf), f0, acc[db], 0, 0, 0);
-        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cols_frag<S>(ks, 2 * mb + 1, db, g, lp, dhalf), f1, acc[db], 0, 0, 0);
+          for (int vq = 0; vq < 4; ++vq) {
+            const int4 ids = *reinterpret_cast<const int4*>(ids_p + 8 * vq);
+            if (ids.x != qseg[nb]) s[nb][4 * vq] = -INFINITY;
+            if (ids.y != qseg[nb]) s[nb][4 * vq + 1] = -INFINITY;
+            if (ids.z != qseg[nb]) s[nb][4 * vq + 2] = -INFINITY;
+            if (ids.w != qseg[nb]) s[nb][4 * vq + 3] = -INFINITY;
+          }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[nb][v] = __builtin_amdgcn_exp2f(s[nb][v]) * dp[nb][v];  // p * (dp - delta)
+        pack_block(s[nb], df[nb][0], df[nb][1]);
+      }
+      static_for<2 * NDB>([&](auto n_c) __attribute__((always_inline)) {
+        constexpr int db = decltype(n_c)::value / 2, half = decltype(n_c)::value % 2;
+        const bf16x8 a = cols_frag<S>(ks, 2 * mb + half, db, g, lp, dhalf);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[nb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, df[nb][half], acc[nb][db], 0, 0, 0);
       });
     });
   };
@@ -289,17 +308,21 @@ __global__ __launch_bounds__(512) void bwd_dq_kernel(BwdParams p) {
     lds_barrier();
   }
 
-  if (qrow < p.lq) {
-    float* op = p.dq + (((int64_t)b * p.lq + qrow) * p.H + h) * D;
 #pragma unroll
-    for (int db = 0; db < NDB; ++db)
+  for (int nb = 0; nb < NB; ++nb) {
+    const int qrow = wrow0 + 32 * nb + i;
+    if (qrow < p.lq) {
+      float* op = p.dq + (((int64_t)b * p.lq + qrow) * p.H + h) * D;
 #pragma unroll
-      for (int vq = 0; vq < 4; ++vq) {
-        f32x4 out;
+      for (int db = 0; db < NDB; ++db)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) out[e] = acc[db][4 * vq + e] * p.sm_scale;
-        *reinterpret_cast<f32x4*>(op + 32 * db + 8 * vq + 4 * g) = out;
-      }
+        for (int vq = 0; vq < 4; ++vq) {
+          f32x4 out;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) out[e] = acc[nb][db][4 * vq + e] * p.sm_scale;
+          *reinterpret_cast<f32x4*>(op + 32 * db + 8 * vq + 4 * g) = out;
+        }
+    }
   }
 }
 
@@ -531,12 +554,12 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
   }
 }
 
-template <int D, bool SEG>
+template <int D, int NW, int NB, bool SEG>
 int launch_dq(const BwdParams& base, hipStream_t stream) {
   BwdParams p = base;
-  p.nblk = (p.lq + 255) / 256;
+  p.nblk = (p.lq + NW * NB * 32 - 1) / (NW * NB * 32);
   p.npairs = p.nblk * p.B;
-  auto kern = bwd_dq_kernel<D, SEG>;
+  auto kern = bwd_dq_kernel<D, NW, NB, SEG>;
   const size_t smem = (size_t)4 * kTile * tile_stride(D) * 2 + 2 * kTile * 4;
   static bool configured = false;
   if (!configured) {
@@ -544,7 +567,7 @@ int launch_dq(const BwdParams& base, hipStream_t stream) {
       return TPA_ERR_LAUNCH;
     configured = true;
   }
-  hipLaunchKernelGGL(kern, dim3(((p.npairs + 7) / 8) * 8 * p.H), dim3(512), smem, stream, p);
+  hipLaunchKernelGGL(kern, dim3(((p.npairs + 7) / 8) * 8 * p.H), dim3(NW * 64), smem, stream, p);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
 }
 
@@ -569,13 +592,16 @@ template <int D>
 int launch_both(const BwdParams& p, hipStream_t stream) {
   // dK/dV: 8 waves of 32 keys.  (64 keys per wave would halve the LDS reads per MFMA, which bound
   // this kernel, but its 384 stationary registers at D = 128 leave the compiler spilling.)
+  // (measured at D = 128: the dQ kernel with 4 waves of 64 rows, one wave per SIMD and 512 registers, takes
+  // 922 us where 8 waves of 32 rows take 401 us)
   constexpr int NW = 8, NB = 1;
+  constexpr int QNW = 8, QNB = 1;
   int rc;
   if (p.qseg) {
-    rc = launch_dq<D, true>(p, stream);
+    rc = launch_dq<D, QNW, QNB, true>(p, stream);
     if (rc == TPA_OK) rc = launch_dkv<D, NW, NB, true>(p, stream);
   } else {
-    rc = launch_dq<D, false>(p, stream);
+    rc = launch_dq<D, QNW, QNB, false>(p, stream);
     if (rc == TPA_OK) rc = launch_dkv<D, NW, NB, false>(p, stream);
   }
   return rc;
