@@ -311,7 +311,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(DenseParams p) {
 // shared by `ns` neighbouring lanes that split the sum over d and combine with lane shuffles.
 template <typename T, bool STAGE>
 __global__ __launch_bounds__(256) void project_kernel(const float* dx, TpaFactor fa, TpaFactor fb, TpaGrad ga, TpaGrad gb, int L, int H,
-                                                       int D, int R, int ns) {
+                                                       int D, int R, int dsh, int nsh) {
   const int t = blockIdx.x, b = blockIdx.y;
   const float* xp = dx + ((int64_t)b * L + t) * H * D;
   const T* ap = static_cast<const T*>(fa.ptr) + b * fa.stride_b + t * fa.stride_l;
@@ -321,17 +321,17 @@ __global__ __launch_bounds__(256) void project_kernel(const float* dx, TpaFactor
   const float inv = 1.f / (float)R;
   extern __shared__ __attribute__((aligned(16))) float xs[];  // [H][XS], then b[R][D], then a[R][H]
   if constexpr (STAGE) {
-    // D % 4 == 0 here; rows 16 bytes apart in the banks, so that lanes that read 16 bytes of
-    // different rows (the da part) spread over the banks
-    const int XS = D + 4;
+    // D = 1 << dsh here (indices by shifts, not divisions); rows 16 bytes apart in the banks, so
+    // that lanes that read 16 bytes of different rows (the da part) spread over the banks
+    const int XS = D + 4, d4sh = dsh - 2, d4mask = (D >> 2) - 1;
     float* bs = xs + H * XS;
     float* as = bs + R * D;
-    for (int idx = threadIdx.x; idx < H * D / 4; idx += 256) {
-      const int h = idx / (D / 4), d4 = idx - h * (D / 4);
+    for (int idx = threadIdx.x; idx < (H << d4sh); idx += 256) {
+      const int h = idx >> d4sh, d4 = idx & d4mask;
       *reinterpret_cast<f32x4*>(xs + h * XS + 4 * d4) = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xp + 4 * idx));
     }
-    for (int idx = threadIdx.x; idx < R * D; idx += 256) {
-      const int r = idx / D, d = idx - r * D;
+    for (int idx = threadIdx.x; idx < (R << dsh); idx += 256) {
+      const int r = idx >> dsh, d = idx & (D - 1);
       bs[idx] = load_as_f32(bp + r * fb.stride_r + d);
     }
     for (int idx = threadIdx.x; idx < R * H; idx += 256) {
@@ -339,24 +339,32 @@ __global__ __launch_bounds__(256) void project_kernel(const float* dx, TpaFactor
       as[idx] = load_as_f32(ap + r * fa.stride_r + h);
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < R * D; idx += 256) {
-      const int r = idx / D, d = idx - r * D;
-      float acc = 0.f;
-      for (int h = 0; h < H; ++h) acc += xs[h * XS + d] * as[r * H + h];
-      ob[r * gb.stride_r + d] = acc * inv;
+    // db: four neighbouring d per thread
+    for (int idx = threadIdx.x; idx < (R << d4sh); idx += 256) {
+      const int r = idx >> d4sh, d4 = idx & d4mask;
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      for (int h = 0; h < H; ++h) {
+        const f32x4 xv = *reinterpret_cast<const f32x4*>(xs + h * XS + 4 * d4);
+        const float av = as[r * H + h];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] += xv[e] * av;
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ob[r * gb.stride_r + 4 * d4 + e] = acc[e] * inv;
     }
-    const int per_pass = 256 / ns, sub = threadIdx.x % ns;
+    // da: ns = 1 << nsh neighbouring lanes share an output
+    const int per_pass = 256 >> nsh, sub = threadIdx.x & ((1 << nsh) - 1);
     for (int base = 0; base < R * H; base += per_pass) {  // uniform trip count: the shuffles below need every lane
-      const int idx = base + threadIdx.x / ns;
+      const int idx = base + (threadIdx.x >> nsh);
       const bool ok = idx < R * H;
       const int r = ok ? idx / H : 0, h = ok ? idx - r * H : 0;
       float acc = 0.f;
-      for (int d = 4 * sub; d < D; d += 4 * ns) {
+      for (int d = 4 * sub; d < D; d += 4 << nsh) {
         const f32x4 xv = *reinterpret_cast<const f32x4*>(xs + h * XS + d);
         const f32x4 bv = *reinterpret_cast<const f32x4*>(bs + r * D + d);
         acc += xv[0] * bv[0] + xv[1] * bv[1] + xv[2] * bv[2] + xv[3] * bv[3];
       }
-      for (int m = ns >> 1; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 64);
+      for (int m = (1 << nsh) >> 1; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 64);
       if (ok && sub == 0) oa[r * ga.stride_r + h] = acc * inv;
     }
   } else {
@@ -379,12 +387,14 @@ template <typename T>
 void launch_project(const float* dx, const TpaFactor& fa, const TpaFactor& fb, const TpaGrad& ga, const TpaGrad& gb, int B, int L,
                     int H, int D, int R, hipStream_t stream) {
   const size_t smem = ((size_t)H * (D + 4) + (size_t)R * D + (size_t)R * H) * sizeof(float);
-  int ns = 1;  // lanes per da output: a power of two, at most a wave, so that one pass covers the outputs if it can
-  while (ns < 64 && 2 * ns * R * H <= 256 && 8 * ns <= D) ns *= 2;
-  if (smem <= 60 * 1024 && D % 4 == 0)
-    hipLaunchKernelGGL((project_kernel<T, true>), dim3(L, B), dim3(256), smem, stream, dx, fa, fb, ga, gb, L, H, D, R, ns);
+  int dsh = 0;
+  while ((1 << dsh) < D) ++dsh;
+  int nsh = 0;  // lanes per da output: a power of two, at most a wave, so that one pass covers the outputs if it can
+  while (nsh < 6 && (4 << nsh) * R * H <= 512 && (16 << nsh) <= D) ++nsh;
+  if (smem <= 60 * 1024 && (1 << dsh) == D && D >= 4)
+    hipLaunchKernelGGL((project_kernel<T, true>), dim3(L, B), dim3(256), smem, stream, dx, fa, fb, ga, gb, L, H, D, R, dsh, nsh);
   else
-    hipLaunchKernelGGL((project_kernel<T, false>), dim3(L, B), dim3(256), 0, stream, dx, fa, fb, ga, gb, L, H, D, R, ns);
+    hipLaunchKernelGGL((project_kernel<T, false>), dim3(L, B), dim3(256), 0, stream, dx, fa, fb, ga, gb, L, H, D, R, dsh, nsh);
 }
 
 template <typename T, int DMAX>
