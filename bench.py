@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|c2p|c3p|c2b|c3b|c2pb|copy] [--no-cpu] [--no-decode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|copy] [--no-cpu] [--no-decode]
 
 A step is one forward pass over one batch of synthetic, seeded inputs that are resident in HBM
 before the timed region starts.  The default workload is the prefill configuration the headline
@@ -32,6 +32,10 @@ WORKLOADS = {
     "c3": ("prefill", 1, 32768, 32768, 32, 128, 6, 2, True),
     "c5": ("prefill", 8, 2048, 2048, 64, 64, 16, 8, False),
     "c4": ("decode", 64, 1, 8192, 32, 128, 6, 2, False),
+    # dense flash attention (tpa/mha.py) at the prefill shapes: the same-shape baseline
+    "c2m": ("dense", 4, 4096, 4096, 16, 128, 0, 0, True),
+    "c3m": ("dense", 1, 32768, 32768, 32, 128, 0, 0, True),
+    "c5m": ("dense", 8, 2048, 2048, 64, 64, 0, 0, False),
     # packed sequences (segment ids, tpa/tpa.py:369-375): the c2 / c3 shapes holding documents of DOC_LEN tokens
     # backward pass (tpa/tpa.py:168-214) at the c2 / c3 shapes: gradients of all six factor arrays
     "c2b": ("backward", 4, 4096, 4096, 16, 128, 6, 2, True),
@@ -124,6 +128,27 @@ def run_prefill(torch, tpa, device, name, steps, warmup):
         tflops_wall=fl / wall_ms / 1e9, tflops_kernel=fl / ev_ms / 1e9,
         shape=dict(B=B, lq=lq, lk=lk, H=H, D=D, rank_q=rq, rank_k=rk, causal=causal, **({"document_len": doc} if doc else {})),
         inputs=x, out=out,
+    )
+
+
+def run_dense_prefill(torch, mha, device, name, steps, warmup):
+    """Dense multi-head flash attention (tpa/mha.py:23-37) on q, k, v [B, T, H, D] bf16."""
+    _, B, lq, lk, H, D, _, _, causal = WORKLOADS[name]
+    g = torch.Generator(device=device)
+    g.manual_seed(5)
+    draw = lambda l: torch.randn((B, l, H, D), generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    q, k, v = draw(lq), draw(lk), draw(lk)
+    scale = D**-0.5
+
+    def step(i):
+        mha._mha_fwd(q, k, v, None, scale, causal=causal, kernel=2)
+
+    wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
+    fl = prefill_flops(B, lq, lk, H, D, causal)
+    return dict(
+        wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, flops=fl,
+        tflops_wall=fl / wall_ms / 1e9, tflops_kernel=fl / ev_ms / 1e9,
+        shape=dict(B=B, lq=lq, lk=lk, H=H, D=D, causal=causal),
     )
 
 
@@ -309,6 +334,20 @@ def main():
             err = float(abs(r["out"]["o"][:1].float().cpu().numpy() - o_ref).max())
             result["max_abs_err_vs_oracle_sample"] = err
             log(f"[bench] cpu {base['value']*1e3:.2f} GFLOP/s; max abs err vs oracle on the sample {err:.2e}")
+    elif kind == "dense":
+        from tpa import mha
+
+        log(f"[bench] dense flash attention {args.workload}: warmup {args.warmup}, steps {args.steps}")
+        r = run_dense_prefill(torch, mha, device, args.workload, args.steps, args.warmup)
+        log(f"[bench] {r['kernel_ms']:.4f} ms/launch (min {r['kernel_ms_min']:.4f}), {r['tflops_kernel']:.1f} TFLOP/s")
+        result.update(
+            metric="dense flash attention forward throughput", value=r["tflops_wall"], unit="TFLOP/s", ms_per_step=r["wall_ms"],
+            roofline=dict(bound="mfma", achieved=r["tflops_kernel"], peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
+                          frac=r["tflops_kernel"] / PEAK_BF16_TFLOPS, traffic=None, kernel="prefill_kernel (dense loader)",
+                          ms_per_launch=r["kernel_ms"], ms_per_launch_min=r["kernel_ms_min"],
+                          algorithmic_flops_per_launch=r["flops"]),
+            config=dict(workload=f"{args.workload}: dense flash attention (tpa/mha.py) at the prefill shape", **r["shape"]),
+        )
     elif kind == "backward":
         log(f"[bench] backward {args.workload}: warmup {args.warmup}, steps {args.steps}")
         r = run_backward(torch, tpa, device, args.workload, args.steps, args.warmup)
