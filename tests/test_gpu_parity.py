@@ -377,9 +377,10 @@ def test_abi_error_codes(gpu):
         tpa.tpa(x, x[:, :4], x, num_heads=4)
     with pytest.raises(TypeError):
         tpa.tpa(x.half(), x.half(), x.half(), num_heads=4)
-    with pytest.raises(NotImplementedError):
-        xr = x.clone().requires_grad_(True)
-        tpa.tpa(xr, x, x, num_heads=4).nansum().backward()
+    # the operator is differentiable (tpa.defvjp, tpa/tpa.py:217): gradients arrive in the input's dtype and shape
+    xr = x.clone().requires_grad_(True)
+    tpa.tpa(xr, x, x, num_heads=4).nansum().backward()
+    assert xr.grad is not None and xr.grad.shape == x.shape and xr.grad.dtype == x.dtype and torch.isfinite(xr.grad).all()
     # MFMA kernel requested for a problem it cannot run -> TPA_ERR_UNSUPPORTED, nothing launched
     with pytest.raises(d.TpaError) as e:
         tpa.tpa_factors(x[..., :4], x[..., 4:], x[..., :4], x[..., 4:], x[..., :4], x[..., 4:], kernel=d.KERNEL_MFMA)
