@@ -121,7 +121,8 @@ int tpa_bwd(const TpaBwdArgs* a, void* stream) {
   if (a->kernel != TPA_KERNEL_AUTO && a->kernel != TPA_KERNEL_GENERIC && a->kernel != TPA_KERNEL_MFMA)
     return TPA_ERR_UNSUPPORTED;
   const int mfma = a->kernel != TPA_KERNEL_GENERIC &&
-                   dense_bwd_mfma_supported(a->dtype, a->dk, a->dv, a->lq, a->lk, a->H, a->sm_scale, nullptr);
+                   dense_bwd_mfma_supported(a->dtype, a->dk, a->dv, a->lq, a->lk, a->H, a->sm_scale, nullptr) &&
+                   !(reinterpret_cast<uintptr_t>(a->d_o) & 15);  // the MFMA kernels read do with 16-byte loads
   if (a->kernel == TPA_KERNEL_MFMA && !mfma) return TPA_ERR_UNSUPPORTED;
   if (!a->workspace || a->workspace_bytes < tpa_bwd_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dk, a->dv))
     return TPA_ERR_WORKSPACE;
