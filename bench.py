@@ -1,13 +1,14 @@
 #!/usr/bin/env python3
 """Benchmark of the TPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|copy] [--no-cpu] [--no-decode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|copy] [--no-cpu] [--no-decode] [--no-backward]
 
 A step is one forward pass over one batch of synthetic, seeded inputs that are resident in HBM
 before the timed region starts.  The default workload is the prefill configuration the headline
 metric is quoted on (c2: B=4, T=4096, H=16, D=128, Rq=6, Rk=Rv=2, bf16, causal); the same run
 also times the decode configuration (c4: B=64, cache 8192, H=32, D=128) and reports it in the
-"decode" object, and times the CPU oracle on a bounded sample of c2 ("cpu_baseline").
+"decode" object, the backward pass at the c2 shape ("backward"), and times the CPU oracle on a bounded
+sample of c2 ("cpu_baseline").
 One JSON line is printed on stdout; progress goes to stderr.
 """
 
@@ -269,6 +270,7 @@ def main():
                     help="copy = a plain device copy of known size, the yardstick for the HBM byte counters")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the secondary decode measurement")
+    ap.add_argument("--no-backward", action="store_true", help="skip the secondary backward measurement")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives are built); use --gpus 1")
@@ -326,6 +328,19 @@ def main():
             result["decode"]["dense_mha_same_shape"] = dict(
                 ms_per_launch=dd["kernel_ms"], achieved=dd["gbs_kernel"], unit="GB/s", frac=dd["gbs_kernel"] / PEAK_HBM_GBS,
                 algorithmic_bytes_per_launch=dd["bytes"], speedup_of_factored_cache=dd["kernel_ms"] / d["kernel_ms"])
+        if not args.no_backward and args.workload == "c2":
+            log("[bench] backward at the c2 shape")
+            bw = run_backward(torch, tpa, device, "c2b", max(10, args.steps // 2), 5)
+            log(f"[bench] {bw['kernel_ms']:.4f} ms/call, {bw['tflops_kernel']:.1f} TFLOP/s")
+            result["backward"] = dict(
+                metric="TPA causal prefill backward throughput", value=bw["tflops_wall"], unit="TFLOP/s", ms_per_step=bw["wall_ms"],
+                roofline=dict(bound="mfma", achieved=bw["tflops_kernel"], peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
+                              frac=bw["tflops_kernel"] / PEAK_BF16_TFLOPS, traffic=None,
+                              kernel="recon + delta + bwd_dq_kernel + bwd_dkv_kernel + project (whole call)",
+                              ms_per_launch=bw["kernel_ms"], ms_per_launch_min=bw["kernel_ms_min"],
+                              algorithmic_flops_per_launch=bw["flops"]),
+                config=dict(workload="c2b: TPA backward", **bw["shape"]),
+            )
         if not args.no_cpu and args.workload == "c2":
             log("[bench] cpu baseline (numpy oracle on a sample)")
             base, o_ref, _ = cpu_baseline_prefill(torch, r["inputs"], r["shape"])
