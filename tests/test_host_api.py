@@ -11,9 +11,9 @@ def test_module_layout_mirrors_the_reference():
     from tpa import mha, tpa
 
     # names other code reaches for (tpa/ring_tpa.py:82,241,244; tpa/mha_test.py:6)
-    for name in ("tpa", "BlockSizes", "_fwd", "_tpa_fwd", "_lse", "_lse_accum"):
+    for name in ("tpa", "BlockSizes", "_fwd", "_tpa_fwd", "_bwd", "_tpa_bwd", "_precompute_delta", "_lse", "_lse_accum"):
         assert hasattr(tpa, name), name
-    for name in ("mha", "_mha_fwd"):
+    for name in ("mha", "_mha_fwd", "_mha_bwd"):
         assert hasattr(mha, name), name
     bs = tpa.BlockSizes()
     assert (bs.block_q, bs.block_kv, bs.block_h) == (128, 128, 4)  # tpa/tpa.py:39-70
@@ -45,6 +45,26 @@ def test_lse_helpers_match_the_oracle():
     a = torch.tensor([0.3, -np.inf, -np.inf, 2.0])
     b = torch.tensor([1.1, -np.inf, 0.5, -np.inf])
     np.testing.assert_allclose(tpa._lse_accum(a, b).numpy(), orc.lse_accum(a.numpy().astype(np.float64), b.numpy().astype(np.float64)), rtol=1e-6)
+
+
+def test_backward_signatures_and_delta():
+    import inspect
+
+    from tpa import tpa
+
+    # tpa/tpa.py:168-178 and tpa/tpa.py:823-839
+    assert list(inspect.signature(tpa._tpa_bwd).parameters) == [
+        "num_heads", "sm_scale", "causal", "block_sizes", "nomat", "debug", "interpret", "residuals", "do"]
+    assert list(inspect.signature(tpa._bwd).parameters) == [
+        "q", "k", "v", "q_segment_ids", "kv_segment_ids", "o", "l", "do", "num_heads", "sm_scale", "causal",
+        "block_sizes", "nomat", "debug", "interpret"]
+    # tpa/tpa.py:965-995: nansum(out * do) per row, NaN rows of an empty query contribute 0
+    rng = np.random.default_rng(2)
+    out, do = rng.standard_normal((6, 5)).astype(np.float32), rng.standard_normal((6, 5)).astype(np.float32)
+    out[3] = np.nan
+    got = tpa._precompute_delta(torch.from_numpy(out), torch.from_numpy(do), torch.zeros(6)).numpy()
+    np.testing.assert_allclose(got, np.nansum(out * do, axis=1), rtol=1e-6)
+    assert got[3] == 0.0
 
 
 def test_no_gpu_means_an_error_not_a_fallback():
