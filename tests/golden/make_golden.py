@@ -11,6 +11,9 @@ small_cases.npz  inputs and full outputs of small problems, among them the upstr
                  (1, 8, 8, 1, 4, 6) of tpa/tpa_test.py:66 and the literal case of tpa/mha_test.py
 sampled_rows.npz for larger seeded problems: the seed recipe, a checksum of the inputs and the
                  outputs of a few query rows
+backward_cases.npz  for the small problems: a seeded upstream gradient and the gradients of the three
+                 factor arrays (what _tpa_bwd returns, tpa/tpa.py:168-214), and the literal gradients
+                 upstream keeps in tpa/mha_test.py:87-118
 """
 import os
 import sys
@@ -65,6 +68,20 @@ def main():
     small["upstream_mha_literal.bias"] = np.array([[0, ninf, 0], [0, ninf, 0], [ninf, ninf, ninf]])[None]
     small["upstream_mha_literal.o"] = np.array([[1.0, 1.0], [1.0, 1.0], [np.nan, np.nan]])[None, :, None, :]
     np.savez_compressed(os.path.join(HERE, "small_cases.npz"), **small)
+
+    back = {}
+    for name, (seed, b, lq, lk, h, dk, dv, rq, rk, seg, causal, scale, dist) in SMALL.items():
+        q, k, v = make_factors(seed, b, lq, lk, h, dk, dv, rq, rk, dist=dist)
+        qs = segment_ids(lq, seg, b) if seg else None
+        ks = segment_ids(lk, seg, b) if seg else None
+        do = np.random.Generator(np.random.Philox(seed + 1000)).standard_normal((b, lq, h, dv)).astype(np.float32)
+        dq, dk_, dv_ = orc.tpa_backward(q, k, v, qs, ks, h, do, sm_scale=scale, causal=causal)
+        back.update({f"{name}.do": do, f"{name}.dq": dq, f"{name}.dk": dk_, f"{name}.dv": dv_})
+    # tpa/mha_test.py:87-118: gradients of nansum(o) on the literal case
+    back["upstream_mha_literal.dq"] = np.zeros((1, 3, 1, 2))
+    back["upstream_mha_literal.dk"] = np.zeros((1, 3, 1, 2))
+    back["upstream_mha_literal.dv"] = np.array([[1.0, 1.0], [0.0, 0.0], [1.0, 1.0]])[None, :, None, :]
+    np.savez_compressed(os.path.join(HERE, "backward_cases.npz"), **back)
 
     sampled = {}
     for name, (seed, b, lq, lk, h, dk, dv, rq, rk, causal, scale, dist, sbr, rows) in SAMPLED.items():

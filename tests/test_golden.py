@@ -121,3 +121,38 @@ def test_kernel_reproduces_sampled_fixture(gpu, name):
     else:
         same(o, SAMPLED[f"{name}.o"], otol)
         same(lse, SAMPLED[f"{name}.lse"], ltol)
+
+
+# ------------------------------------------------------------------------------------ backward
+BACK = np.load(os.path.join(GOLDEN, "backward_cases.npz"))
+
+
+@pytest.mark.parametrize("name", SMALL_NAMES)
+def test_oracle_reproduces_backward_fixture(name):
+    q, k, v, qs, ks, h, scale, causal = small_case(name)
+    got = orc.tpa_backward(q, k, v, qs, ks, h, BACK[f"{name}.do"], sm_scale=scale, causal=causal)
+    for g, key in zip(got, ("dq", "dk", "dv")):
+        np.testing.assert_allclose(g, BACK[f"{name}.{key}"], rtol=0, atol=1e-13)
+
+
+def test_oracle_reproduces_upstream_literal_gradients():
+    """tpa/mha_test.py:87-118: dq = dk = 0, dv = [[1, 1], [0, 0], [1, 1]] for nansum(o)."""
+    got = orc.mha_backward(SMALL["upstream_mha_literal.q"], SMALL["upstream_mha_literal.k"], SMALL["upstream_mha_literal.v"],
+                           SMALL["upstream_mha_literal.bias"], 1.0, np.ones((1, 3, 1, 2)))
+    for g, key in zip(got, ("dq", "dk", "dv")):
+        np.testing.assert_allclose(g, BACK[f"upstream_mha_literal.{key}"], atol=1e-15)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", SMALL_NAMES)
+def test_kernel_reproduces_backward_fixture(gpu, name):
+    import torch
+    from tpa import tpa
+
+    q, k, v, qs, ks, h, scale, causal = small_case(name)
+    tq, tk, tv = (torch.from_numpy(x).to(gpu) for x in (q, k, v))
+    o, res = tpa._tpa_fwd(tq, tk, tv, h, qs, ks, scale, causal, None, False, False, False)
+    grads = tpa._tpa_bwd(h, scale, causal, None, False, False, False, res, torch.from_numpy(BACK[f"{name}.do"]).to(gpu))
+    for g, key in zip(grads[:3], ("dq", "dk", "dv")):
+        want = BACK[f"{name}.{key}"]
+        assert np.max(np.abs(g.double().cpu().numpy() - want)) <= 2e-4 * max(1.0, float(np.max(np.abs(want))))
