@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define TPA_ABI_VERSION 2
+#define TPA_ABI_VERSION 3
 
 /* element types of the factor / output arrays */
 enum { TPA_DTYPE_F32 = 0, TPA_DTYPE_BF16 = 1 };
@@ -95,6 +95,10 @@ typedef struct TpaFwdArgs {
   void* workspace;        /* required by tpa_decode (split partials); optional for tpa_fwd (tpa_fwd_workspace_bytes) */
   size_t workspace_bytes; /* size of workspace */
   int32_t num_splits;     /* tpa_decode only: 0 = choose; otherwise the number of key ranges */
+  const int32_t* kv_lengths; /* [B] or NULL: batch entry b attends to its first min(kv_lengths[b], lk) keys only,
+                                the rest of its k / v arrays is not read (sequences of different lengths in one
+                                padded cache; 0 = no key: o = NaN, lse = -inf).  No counterpart in the reference,
+                                which would express this with segment ids (tpa/tpa.py:369-375). */
 } TpaFwdArgs;
 
 /*

@@ -31,9 +31,9 @@ struct DecodeParams {
   float* part_o;  // [B, lq, S, H, D] fp32, unnormalised
   float* part_m;  // [B, lq, S, H] running max (log2 domain)
   float* part_l;  // [B, lq, S, H] sum of exp2
+  const int32_t* kvlen;  // [B] keys per batch entry, or null (= lk)
   int B, lq, lk, H, rq;
   int S;           // key ranges
-  int nblocks;     // 32-row blocks in the cache: ceil(lk * rk / 32)
   float qscale;    // sm_scale * log2(e) / (rq * rk)
 };
 
@@ -87,10 +87,11 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   // waves of the grid, which advance in step, read neighbouring addresses at any one time)
   const int nparts = S * kWaves;
   const int part = split * kWaves + w;
+  const int len_b = p.kvlen ? max(0, min(p.kvlen[b], p.lk)) : p.lk;  // keys of this batch entry
   const int blk_begin = part;
-  const int blk_end = p.nblocks;
+  const int blk_end = (len_b * RK + kRowsPerBlock - 1) / kRowsPerBlock;  // 32-row blocks of its cache
   const int blk_step = nparts;
-  const int last_row = p.lk * RK - 1;
+  const int last_row = len_b * RK - 1;
 
   // rows of the cache matrices: row = token * RK + rank, row stride = stride_r
   const uint16_t* kb_base = static_cast<const uint16_t*>(p.kb.ptr) + b * p.kb.stride_b;
@@ -359,7 +360,7 @@ int launch_decode(const TpaFwdArgs* a, int S, hipStream_t stream) {
   const size_t nm = (size_t)a->B * a->lq * S * a->H;
   p.part_o = ws; p.part_m = ws + no; p.part_l = ws + no + nm;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.S = S;
-  p.nblocks = (int)(((int64_t)a->lk * RK + kRowsPerBlock - 1) / kRowsPerBlock);
+  p.kvlen = a->kv_lengths;
   p.qscale = a->sm_scale * kLog2e / ((float)a->rq * (float)RK);
   auto kern = decode_kernel<D, RK>;
   static bool configured = false;

@@ -20,6 +20,7 @@ struct GenericParams {
   const int32_t* qseg;
   const int32_t* kvseg;
   const float* bias;  // [B, lq, lk] or null
+  const int32_t* kvlen;  // [B] keys per batch entry, or null (= lk)
   void* o;
   float* lse;
   int B, lq, lk, H, dk, dv, rq, rk;
@@ -74,10 +75,10 @@ __global__ __launch_bounds__(kRows) void generic_fwd_kernel(GenericParams p) {
   float l = 0.f;        // running sum of exp(x - m)
 
   // keys this workgroup has to visit
-  int k_end = p.lk;
+  int k_end = p.kvlen ? max(0, min(p.kvlen[b], p.lk)) : p.lk;
   if (p.causal) {
     const int last_row = min(p.lq, (int)(blockIdx.x + 1) * kRows) - 1;
-    k_end = min(p.lk, last_row + 1);
+    k_end = min(k_end, last_row + 1);
   }
 
   for (int k0 = 0; k0 < k_end; k0 += kTile) {
@@ -202,7 +203,7 @@ int launch_generic(const GenericParams& p, hipStream_t stream) {
 int tpa_generic_launch(const TpaFwdArgs* a, hipStream_t stream) {
   tpa::GenericParams p{};
   p.qa = a->qa; p.qb = a->qb; p.ka = a->ka; p.kb = a->kb; p.va = a->va; p.vb = a->vb;
-  p.qseg = a->q_segment_ids; p.kvseg = a->kv_segment_ids; p.bias = nullptr;
+  p.qseg = a->q_segment_ids; p.kvseg = a->kv_segment_ids; p.bias = nullptr; p.kvlen = a->kv_lengths;
   p.o = a->o; p.lse = a->lse;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.dk = a->dk; p.dv = a->dv; p.rq = a->rq; p.rk = a->rk;
   p.sm_scale = a->sm_scale; p.causal = a->causal; p.dense = 0;

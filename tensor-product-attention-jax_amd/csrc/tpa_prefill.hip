@@ -40,6 +40,7 @@ struct PrefillParams {
   TpaFactor qa, qb, ka, kb, va, vb;  // dense: qb/kb/vb hold q/k/v with stride_l = H*D, ptr at head 0
   const int32_t* qseg;   // [B, lq] or null
   const int32_t* kvseg;  // [B, lk] or null (both or neither)
+  const int32_t* kvlen;  // [B] keys per batch entry, or null (= lk)
   uint16_t* o;
   float* lse;
   int B, lq, lk, H, rq, rk;
@@ -97,8 +98,8 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   // scalars out of the argument block (never take the address of the block itself)
   struct Fac { const uint16_t* ptr; int64_t stride_b; int stride_l, stride_r; };
   auto fac = [](const TpaFactor& f) { return Fac{static_cast<const uint16_t*>(f.ptr), f.stride_b, (int)f.stride_l, (int)f.stride_r}; };
-  struct { Fac qa, qb, ka, kb, va, vb; const int32_t* qseg; const int32_t* kvseg; uint16_t* o; float* lse; int B, lq, lk, H, rq, rk; float sm_scale; int causal, nqb, npairs, q_factors; } const p = {
-      fac(pp.qa), fac(pp.qb), fac(pp.ka), fac(pp.kb), fac(pp.va), fac(pp.vb), pp.qseg, pp.kvseg, pp.o, pp.lse, pp.B, pp.lq, pp.lk, pp.H, pp.rq, pp.rk,
+  struct { Fac qa, qb, ka, kb, va, vb; const int32_t* qseg; const int32_t* kvseg; const int32_t* kvlen; uint16_t* o; float* lse; int B, lq, lk, H, rq, rk; float sm_scale; int causal, nqb, npairs, q_factors; } const p = {
+      fac(pp.qa), fac(pp.qb), fac(pp.ka), fac(pp.kb), fac(pp.va), fac(pp.vb), pp.qseg, pp.kvseg, pp.kvlen, pp.o, pp.lse, pp.B, pp.lq, pp.lk, pp.H, pp.rq, pp.rk,
       pp.sm_scale, pp.causal, pp.nqb, pp.npairs, pp.q_factors};
 
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
@@ -205,7 +206,18 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
 
   // ---- key range [kpos0, kend) this workgroup visits; tiles are counted from kpos0
   int kpos0 = 0;
-  int kend = p.causal ? min(p.lk, min(q0 + kBQ, p.lq)) : p.lk;
+  const int len_b = p.kvlen ? max(0, min(p.kvlen[b], p.lk)) : p.lk;  // keys of this batch entry
+  int kend = p.causal ? min(len_b, min(q0 + kBQ, p.lq)) : len_b;
+  if (kend <= 0) {  // no key at all: the rows end as NaN / -inf (tpa/tpa.py:437-439)
+    if (qrow < p.lq) {
+      uint16_t* op = p.o + (((int64_t)b * p.lq + qrow) * p.H + h) * D;
+      const u32x4 nan4 = {0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u};
+#pragma unroll
+      for (int cch = 0; cch < D / 16; ++cch) *reinterpret_cast<u32x4*>(op + 16 * cch + 8 * g) = nan4;
+      if (p.lse && g == 0) p.lse[((int64_t)b * p.H + h) * p.lq + qrow] = -INFINITY;
+    }
+    return;
+  }
   bool seg_pure = false;  // every visited key from the second tile on carries the rows' one segment id
   if constexpr (SEG) {
     // Packed sequences: a key can only be visible to this block if its id lies within the
@@ -903,7 +915,7 @@ int tpa_prefill_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
   using namespace tpa;
   PrefillParams p{};
   p.qa = a->qa; p.qb = a->qb; p.ka = a->ka; p.kb = a->kb; p.va = a->va; p.vb = a->vb;
-  p.qseg = a->q_segment_ids; p.kvseg = a->kv_segment_ids;
+  p.qseg = a->q_segment_ids; p.kvseg = a->kv_segment_ids; p.kvlen = a->kv_lengths;
   p.o = static_cast<uint16_t*>(a->o); p.lse = a->lse;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.rk = a->rk;
   p.sm_scale = a->sm_scale; p.causal = a->causal;

@@ -22,7 +22,7 @@ KERNEL_AUTO = 0
 KERNEL_GENERIC = 1
 KERNEL_MFMA = 2
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class TpaFactor(ctypes.Structure):
@@ -61,6 +61,7 @@ class TpaFwdArgs(ctypes.Structure):
         ("workspace", ctypes.c_void_p),
         ("workspace_bytes", ctypes.c_size_t),
         ("num_splits", ctypes.c_int32),
+        ("kv_lengths", ctypes.c_void_p),
     ]
 
 

@@ -90,6 +90,15 @@ def _segment_ids(ids, batch: int, length: int, device) -> torch.Tensor | None:
     return t.contiguous()
 
 
+def _lengths(kv_lengths, batch: int, device) -> torch.Tensor | None:
+    if kv_lengths is None:
+        return None
+    t = _as_device_tensor(kv_lengths, device).to(torch.int32).contiguous()
+    if tuple(t.shape) != (batch,):
+        raise ValueError(f"kv_lengths must have shape {(batch,)}, got {tuple(t.shape)}")
+    return t
+
+
 def tpa_factors(
     qa, qb, ka, kb, va, vb,
     q_segment_ids=None,
@@ -99,6 +108,7 @@ def tpa_factors(
     kernel: int = _d.KERNEL_AUTO,
     return_lse: bool = True,
     use_workspace: bool = True,
+    kv_lengths=None,
 ):
     """Forward pass on the six split factor arrays, the operands of the reference's kernel
     launch (tpa/tpa.py:246-251,543) with a leading batch dimension:
@@ -108,7 +118,9 @@ def tpa_factors(
     Returns (o[b,lq,h,dv] in the input dtype, lse[b,h,lq] fp32 or None).  The arrays may be
     views (e.g. slices of the concatenated tensors); only the last dimension must be contiguous.
     `use_workspace=False` withholds the optional scratch memory, which keeps the call on the
-    fused prefill kernel whatever the problem.
+    fused prefill kernel whatever the problem.  `kv_lengths` (int32 [b], an addition): batch
+    entry i attends to its first kv_lengths[i] keys only; the rest of its k / v rows is padding
+    that is never read.
     """
     device = _pick_device(qa, qb, ka, kb, va, vb)
     qa, qb, ka, kb, va, vb = (_as_device_tensor(x, device) for x in (qa, qb, ka, kb, va, vb))
@@ -129,6 +141,7 @@ def tpa_factors(
     if (qseg is None) != (kvseg is None):
         raise ValueError("q_segment_ids and kv_segment_ids must be given together")
 
+    kvlen = _lengths(kv_lengths, b, device)
     o = torch.empty((b, lq, h, dv), dtype=dtype, device=device)
     lse = torch.empty((b, h, lq), dtype=torch.float32, device=device) if return_lse else None
     lib = _d.load_library()
@@ -150,6 +163,7 @@ def tpa_factors(
         B=b, lq=lq, lk=lk, H=h, dk=dk, dv=dv, rq=rq, rk=rk,
         dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=int(bool(causal)), kernel=int(kernel),
         workspace=ws_ptr, workspace_bytes=ws_bytes, num_splits=0,
+        kv_lengths=kvlen.data_ptr() if kvlen is not None else None,
     )
     with torch.cuda.device(device):
         _d.check("tpa_fwd", lib.tpa_fwd(args, _d.current_stream_ptr(device)))
@@ -162,13 +176,16 @@ def tpa_decode(
     num_splits: int = 0,
     workspace: torch.Tensor | None = None,
     kernel: int = _d.KERNEL_AUTO,
+    kv_lengths=None,
 ):
     """Few query tokens against a long factored KV cache (no mask), split over key ranges.
 
     The reference has no separate entry point for this: it is tpa() with lq = 1
     (block_q = min(128, lq), tpa/tpa.py:485).  Same operands as `tpa_factors`; the cache is
     ka/kb/va/vb.  `workspace` (uint8, at least `decode_workspace_bytes(...)`) may be passed to
-    avoid the allocation.  Returns (o[b,lq,h,dv], lse[b,h,lq]).
+    avoid the allocation.  `kv_lengths` (int32 [b]): how many tokens of each batch entry's cache
+    are filled (sequences of different lengths in one padded cache); the rest is not read.
+    Returns (o[b,lq,h,dv], lse[b,h,lq]).
     """
     device = _pick_device(qa, qb, ka, kb, va, vb)
     qa, qb, ka, kb, va, vb = (_as_device_tensor(x, device) for x in (qa, qb, ka, kb, va, vb))
@@ -178,6 +195,7 @@ def tpa_decode(
     dk = qb.shape[-1]
     assert tuple(kb.shape) == (b, lk, rk, dk), kb.shape
     assert tuple(ka.shape) == (b, lk, rk, h) and tuple(va.shape) == (b, lk, rk, h)
+    kvlen = _lengths(kv_lengths, b, device)
     lib = _d.load_library()
     need = lib.tpa_decode_workspace_bytes(b, lq, lk, h, dv, num_splits)
     if workspace is None:
@@ -191,6 +209,7 @@ def tpa_decode(
         dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=0, kernel=int(kernel),
         workspace=workspace.data_ptr(), workspace_bytes=workspace.numel() * workspace.element_size(),
         num_splits=int(num_splits),
+        kv_lengths=kvlen.data_ptr() if kvlen is not None else None,
     )
     with torch.cuda.device(device):
         _d.check("tpa_decode", lib.tpa_decode(args, _d.current_stream_ptr(device)))

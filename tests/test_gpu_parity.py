@@ -680,3 +680,55 @@ def test_fp32_widest_heads(gpu):
     for t, w in zip((tq, tk, tv), want):
         g = t.grad.cpu().numpy().astype(np.float64)
         assert np.max(np.abs(g - w)) <= 2e-4 * np.max(np.abs(w))
+
+
+# ---------------------------------------------------------------- sequences of different lengths in one padded batch
+def _varlen_reference(q, k, v, lengths, h, sm_scale, causal):
+    """Per batch entry: the oracle on the first lengths[b] keys (the padding is never visible)."""
+    os_, ls_ = [], []
+    for bi, n in enumerate(lengths):
+        if n == 0:
+            os_.append(np.full((1, q.shape[1], h, v.shape[-1] - h), np.nan))
+            ls_.append(np.full((1, q.shape[1], h), -np.inf))
+            continue
+        o, l_ = orc.tpa_reference(q[bi : bi + 1], k[bi : bi + 1, :n], v[bi : bi + 1, :n], None, None, h, sm_scale=sm_scale, causal=causal)
+        os_.append(o)
+        ls_.append(l_)
+    return np.concatenate(os_), np.concatenate(ls_)
+
+
+@pytest.mark.parametrize("d,rk,h", [(128, 2, 32), (64, 4, 16)])
+def test_decode_with_per_sequence_cache_lengths(gpu, d, rk, h):
+    """tpa_decode over a padded cache: entry b reads only its first kv_lengths[b] tokens (one of
+    them not a multiple of anything, one shorter than a block, one full, one empty)."""
+    from tpa import tpa
+
+    b, lk = 5, 3000
+    lengths = [3000, 1777, 9, 640, 0]
+    q, k, v = make_factors(101, b, 1, lk, h, d, d, 6, rk, scale_by_rank=True)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    # poison the padding: it must not be read
+    for bi, n in enumerate(lengths):
+        tk[bi, n:] = float("nan")
+        tv[bi, n:] = float("nan")
+    o, lse = tpa.tpa_decode(*tpa_split(tq, tk, tv, h), sm_scale=d**-0.5, kv_lengths=torch.tensor(lengths, dtype=torch.int32), kernel=2)
+    o_ref, l_ref = _varlen_reference(as_f64(tq), np.nan_to_num(as_f64(tk)), np.nan_to_num(as_f64(tv)), lengths, h, d**-0.5, False)
+    check(o, lse, o_ref, l_ref, BF16_TOL)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("kernel,dt", [(2, torch.bfloat16), (1, torch.float32)])
+def test_prefill_with_per_sequence_key_lengths(gpu, kernel, dt, causal):
+    """tpa_fwd (MFMA prefill kernel and fp32 kernel) on a padded batch."""
+    from tpa import tpa
+
+    b, lq, lk, h, d = 4, 400, 700, 8, 64
+    lengths = [700, 333, 64, 0]
+    q, k, v = make_factors(102, b, lq, lk, h, d, d, 3, 2, scale_by_rank=True)
+    tq, tk, tv = (to_gpu(x, dt, gpu) for x in (q, k, v))
+    for bi, n in enumerate(lengths):
+        tk[bi, n:] = float("nan")
+        tv[bi, n:] = float("nan")
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), None, None, d**-0.5, causal, kernel, kv_lengths=lengths)
+    o_ref, l_ref = _varlen_reference(as_f64(tq), np.nan_to_num(as_f64(tk)), np.nan_to_num(as_f64(tv)), lengths, h, d**-0.5, causal)
+    check(o, lse, o_ref, l_ref, BF16_TOL if dt == torch.bfloat16 else F32_TOL)
