@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|copy] [--no-cpu] [--no-decode] [--no-backward]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c4pg|c5|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|copy] [--no-cpu] [--no-decode] [--no-backward]
 
 A step is one forward pass over one batch of synthetic, seeded inputs that are resident in HBM
 before the timed region starts.  The default workload is the prefill configuration the headline
@@ -33,6 +33,7 @@ WORKLOADS = {
     "c3": ("prefill", 1, 32768, 32768, 32, 128, 6, 2, True),
     "c5": ("prefill", 8, 2048, 2048, 64, 64, 16, 8, False),
     "c4": ("decode", 64, 1, 8192, 32, 128, 6, 2, False),
+    "c4pg": ("decode", 64, 1, 8192, 32, 128, 6, 2, False),  # the c4 cache as a pool of shuffled 64-token pages
     # dense flash attention (tpa/mha.py) at the prefill shapes: the same-shape baseline
     "c2m": ("dense", 4, 4096, 4096, 16, 128, 0, 0, True),
     "c3m": ("dense", 1, 32768, 32768, 32, 128, 0, 0, True),
@@ -188,9 +189,17 @@ def run_decode(torch, tpa, device, name, steps, warmup):
     scale = D**-0.5
     ws = torch.empty(max(tpa.decode_workspace_bytes(B, lq, lk, H, D), 16), dtype=torch.uint8, device=device)
     out = {}
+    table = None
+    if name == "c4pg":
+        page = 64
+        g = torch.Generator(device=device)
+        g.manual_seed(11)
+        table = torch.randperm(B * lk // page, generator=g, device=device).to(torch.int32).reshape(B, lk // page)
+        # a pool holds the same bytes; which page holds what does not matter for the timing
+        xs = [x[:2] + tuple(t.reshape(B * lk // page, page, rk, t.shape[-1]) for t in x[2:]) for x in xs]
 
     def step(i):
-        out["o"], out["lse"] = tpa.tpa_decode(*xs[i & 1], sm_scale=scale, workspace=ws, kernel=2)
+        out["o"], out["lse"] = tpa.tpa_decode(*xs[i & 1], sm_scale=scale, workspace=ws, kernel=2, page_table=table)
 
     wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
     nbytes = decode_bytes(B, lq, lk, H, D, rq, rk)

@@ -99,6 +99,13 @@ typedef struct TpaFwdArgs {
                                 the rest of its k / v arrays is not read (sequences of different lengths in one
                                 padded cache; 0 = no key: o = NaN, lse = -inf).  No counterpart in the reference,
                                 which would express this with segment ids (tpa/tpa.py:369-375). */
+  /* Paged cache (tpa_decode's split-key kernel only; TPA_ERR_UNSUPPORTED elsewhere).  With page_table != NULL
+     ka / kb / va / vb are page pools [page, token_in_page, rank, x] (stride_b = elements between pages) and token
+     t of batch entry b lives in page page_table[b * pages_per_seq + t / page_size] at slot t % page_size.
+     page_size * rk must be a multiple of 32 and pages_per_seq * page_size >= lk.  No counterpart in the reference. */
+  const int32_t* page_table; /* [B, pages_per_seq] or NULL */
+  int32_t page_size;         /* tokens per page */
+  int32_t pages_per_seq;     /* entries per row of page_table */
 } TpaFwdArgs;
 
 /*

@@ -56,6 +56,7 @@ const char* tpa_strerror(int code) {
 int tpa_fwd(const TpaFwdArgs* a, void* stream) {
   const int rc = validate_tpa(a);
   if (rc != TPA_OK) return rc;
+  if (a->page_table) return TPA_ERR_UNSUPPORTED;  // paged caches are read by tpa_decode only
   hipStream_t s = static_cast<hipStream_t>(stream);
   // few query tokens over a long cache (the reference's decode is this same call with lq = 1,
   // tpa/tpa.py:485): split over keys, if the caller brought the workspace for it
@@ -87,7 +88,7 @@ int tpa_decode(const TpaFwdArgs* a, void* stream) {
   if (a->causal || a->q_segment_ids) return TPA_ERR_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (a->kernel != TPA_KERNEL_GENERIC && tpa_decode_mfma_supported(a)) return tpa_decode_mfma_launch(a, s);
-  if (a->kernel == TPA_KERNEL_MFMA) return TPA_ERR_UNSUPPORTED;
+  if (a->kernel == TPA_KERNEL_MFMA || a->page_table) return TPA_ERR_UNSUPPORTED;  // only the split-key kernel reads page pools
   return tpa_generic_launch(a, s);
 }
 

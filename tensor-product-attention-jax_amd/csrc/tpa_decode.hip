@@ -32,6 +32,8 @@ struct DecodeParams {
   float* part_m;  // [B, lq, S, H] running max (log2 domain)
   float* part_l;  // [B, lq, S, H] sum of exp2
   const int32_t* kvlen;  // [B] keys per batch entry, or null (= lk)
+  const int32_t* page_table;  // paged cache: [B, pages_per_seq] physical page of each logical page
+  int page_size, pages_per_seq;  // tokens per page; table row length
   int B, lq, lk, H, rq;
   int S;           // key ranges
   float qscale;    // sm_scale * log2(e) / (rq * rk)
@@ -48,7 +50,7 @@ struct DecodeLds {
   static constexpr size_t kBytes = (size_t)kWaves * kPerWave * sizeof(uint16_t);
 };
 
-template <int D, int RK>
+template <int D, int RK, bool PAGED>
 __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   constexpr int CPR = D / 8;               // 16-byte chunks per B row
   constexpr int RPI = 64 / CPR;            // B rows per load instruction
@@ -94,10 +96,14 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   const int last_row = len_b * RK - 1;
 
   // rows of the cache matrices: row = token * RK + rank, row stride = stride_r
-  const uint16_t* kb_base = static_cast<const uint16_t*>(p.kb.ptr) + b * p.kb.stride_b;
-  const uint16_t* vb_base = static_cast<const uint16_t*>(p.vb.ptr) + b * p.vb.stride_b;
-  const uint16_t* ka_base = static_cast<const uint16_t*>(p.ka.ptr) + b * p.ka.stride_b + h0;
-  const uint16_t* va_base = static_cast<const uint16_t*>(p.va.ptr) + b * p.va.stride_b + h0;
+  // (paged cache: the arrays are page pools, stride_b = elements between pages, and a block of 32
+  // rows lies inside one page, which the page table of this batch entry locates)
+  const int64_t boff = PAGED ? 0 : b;
+  const uint16_t* kb_base = static_cast<const uint16_t*>(p.kb.ptr) + boff * p.kb.stride_b;
+  const uint16_t* vb_base = static_cast<const uint16_t*>(p.vb.ptr) + boff * p.vb.stride_b;
+  const uint16_t* ka_base = static_cast<const uint16_t*>(p.ka.ptr) + boff * p.ka.stride_b + h0;
+  const uint16_t* va_base = static_cast<const uint16_t*>(p.va.ptr) + boff * p.va.stride_b + h0;
+  const int rpp = PAGED ? p.page_size * RK : 1;  // rows per page
   const int a_chunks = min(4, (p.H - h0) / 8);  // valid 16-byte chunks of an A row in this head block
 
   // loader lane roles
@@ -111,17 +117,28 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   auto issue = [&](auto set_c, int blk) {
     constexpr int set = decltype(set_c)::value;
     const int row0 = blk * kRowsPerBlock;
+    // element offsets that take a logical row of this block to its place in the page pool
+    int64_t pkb = 0, pvb = 0, pka = 0, pva = 0;
+    if constexpr (PAGED) {
+      const int page = row0 / rpp;
+      const int64_t phys = p.page_table[(int64_t)b * p.pages_per_seq + page];
+      const int64_t first = (int64_t)page * rpp;  // first logical row of the page
+      pkb = phys * p.kb.stride_b - first * p.kb.stride_r;
+      pvb = phys * p.vb.stride_b - first * p.vb.stride_r;
+      pka = phys * p.ka.stride_b - first * p.ka.stride_r;
+      pva = phys * p.va.stride_b - first * p.va.stride_r;
+    }
 #pragma unroll
     for (int n = 0; n < NLB; ++n) {
       const int row = min(row0 + n * RPI + lb_row, last_row);
-      rbk[set][n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kb_base + (int64_t)row * p.kb.stride_r + 8 * lb_c));
-      rbv[set][n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vb_base + (int64_t)row * p.vb.stride_r + 8 * lb_c));
+      rbk[set][n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kb_base + pkb + (int64_t)row * p.kb.stride_r + 8 * lb_c));
+      rbv[set][n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vb_base + pvb + (int64_t)row * p.vb.stride_r + 8 * lb_c));
     }
 #pragma unroll
     for (int n = 0; n < 2; ++n) {
       const int row = min(row0 + 16 * n + la_row, last_row);
-      rak[set][n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(ka_base + (int64_t)row * p.ka.stride_r + 8 * la_c));
-      rav[set][n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(va_base + (int64_t)row * p.va.stride_r + 8 * la_c));
+      rak[set][n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(ka_base + pka + (int64_t)row * p.ka.stride_r + 8 * la_c));
+      rav[set][n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(va_base + pva + (int64_t)row * p.va.stride_r + 8 * la_c));
     }
   };
   auto stage = [&](auto set_c) {
@@ -351,8 +368,8 @@ size_t workspace_bytes(int B, int lq, int H, int D, int S) {
   return (size_t)B * lq * S * H * (D + 2) * sizeof(float);
 }
 
-template <int D, int RK>
-int launch_decode(const TpaFwdArgs* a, int S, hipStream_t stream) {
+template <int D, int RK, bool PAGED>
+int launch_decode_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   DecodeParams p{};
   p.qa = a->qa; p.qb = a->qb; p.ka = a->ka; p.kb = a->kb; p.va = a->va; p.vb = a->vb;
   float* ws = static_cast<float*>(a->workspace);
@@ -361,8 +378,9 @@ int launch_decode(const TpaFwdArgs* a, int S, hipStream_t stream) {
   p.part_o = ws; p.part_m = ws + no; p.part_l = ws + no + nm;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.S = S;
   p.kvlen = a->kv_lengths;
+  p.page_table = a->page_table; p.page_size = a->page_size; p.pages_per_seq = a->pages_per_seq;
   p.qscale = a->sm_scale * kLog2e / ((float)a->rq * (float)RK);
-  auto kern = decode_kernel<D, RK>;
+  auto kern = decode_kernel<D, RK, PAGED>;
   static bool configured = false;
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)DecodeLds<D>::kBytes) != hipSuccess)
@@ -375,6 +393,18 @@ int launch_decode(const TpaFwdArgs* a, int S, hipStream_t stream) {
   hipLaunchKernelGGL(decode_merge_kernel<D>, dim3(a->B * a->lq, a->H), dim3(D), 0, stream, p.part_o, p.part_m, p.part_l,
                      static_cast<uint16_t*>(a->o), a->lse, S, a->H, a->lq, 1.f / (float)RK);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
+}
+
+template <int D, int RK>
+int launch_decode(const TpaFwdArgs* a, int S, hipStream_t stream) {
+  if (a->page_table) {
+    // a block of 32 (token, rank) rows must not straddle pages, and the table must cover lk
+    if (a->page_size <= 0 || (a->page_size * RK) % kRowsPerBlock != 0 ||
+        (int64_t)a->pages_per_seq * a->page_size < a->lk)
+      return TPA_ERR_SHAPE;
+    return launch_decode_t<D, RK, true>(a, S, stream);
+  }
+  return launch_decode_t<D, RK, false>(a, S, stream);
 }
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }

@@ -62,6 +62,9 @@ class TpaFwdArgs(ctypes.Structure):
         ("workspace_bytes", ctypes.c_size_t),
         ("num_splits", ctypes.c_int32),
         ("kv_lengths", ctypes.c_void_p),
+        ("page_table", ctypes.c_void_p),
+        ("page_size", ctypes.c_int32),
+        ("pages_per_seq", ctypes.c_int32),
     ]
 
 

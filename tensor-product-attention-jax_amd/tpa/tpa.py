@@ -177,6 +177,7 @@ def tpa_decode(
     workspace: torch.Tensor | None = None,
     kernel: int = _d.KERNEL_AUTO,
     kv_lengths=None,
+    page_table=None,
 ):
     """Few query tokens against a long factored KV cache (no mask), split over key ranges.
 
@@ -185,16 +186,29 @@ def tpa_decode(
     ka/kb/va/vb.  `workspace` (uint8, at least `decode_workspace_bytes(...)`) may be passed to
     avoid the allocation.  `kv_lengths` (int32 [b]): how many tokens of each batch entry's cache
     are filled (sequences of different lengths in one padded cache); the rest is not read.
+    `page_table` (int32 [b, pages_per_seq]): the cache arrays are then page pools
+    [pages, page_size, rk, x] shared by all sequences, and token t of entry i lives in page
+    page_table[i, t // page_size]; the logical cache length is pages_per_seq * page_size.
     Returns (o[b,lq,h,dv], lse[b,h,lq]).
     """
     device = _pick_device(qa, qb, ka, kb, va, vb)
     qa, qb, ka, kb, va, vb = (_as_device_tensor(x, device) for x in (qa, qb, ka, kb, va, vb))
     dtype = qa.dtype
     b, lq, rq, h = qa.shape
-    _, lk, rk, dv = vb.shape
     dk = qb.shape[-1]
-    assert tuple(kb.shape) == (b, lk, rk, dk), kb.shape
-    assert tuple(ka.shape) == (b, lk, rk, h) and tuple(va.shape) == (b, lk, rk, h)
+    pt, page_size, pages_per_seq = None, 0, 0
+    if page_table is None:
+        _, lk, rk, dv = vb.shape
+        assert tuple(kb.shape) == (b, lk, rk, dk), kb.shape
+        assert tuple(ka.shape) == (b, lk, rk, h) and tuple(va.shape) == (b, lk, rk, h)
+    else:
+        pt = _as_device_tensor(page_table, device).to(torch.int32).contiguous()
+        assert pt.dim() == 2 and pt.shape[0] == b, pt.shape
+        npages, page_size, rk, dv = vb.shape
+        pages_per_seq = pt.shape[1]
+        lk = pages_per_seq * page_size
+        assert tuple(kb.shape) == (npages, page_size, rk, dk), kb.shape
+        assert tuple(ka.shape) == (npages, page_size, rk, h) and tuple(va.shape) == (npages, page_size, rk, h)
     kvlen = _lengths(kv_lengths, b, device)
     lib = _d.load_library()
     need = lib.tpa_decode_workspace_bytes(b, lq, lk, h, dv, num_splits)
@@ -210,6 +224,7 @@ def tpa_decode(
         workspace=workspace.data_ptr(), workspace_bytes=workspace.numel() * workspace.element_size(),
         num_splits=int(num_splits),
         kv_lengths=kvlen.data_ptr() if kvlen is not None else None,
+        page_table=pt.data_ptr() if pt is not None else None, page_size=int(page_size), pages_per_seq=int(pages_per_seq),
     )
     with torch.cuda.device(device):
         _d.check("tpa_decode", lib.tpa_decode(args, _d.current_stream_ptr(device)))

@@ -732,3 +732,53 @@ def test_prefill_with_per_sequence_key_lengths(gpu, kernel, dt, causal):
     o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), None, None, d**-0.5, causal, kernel, kv_lengths=lengths)
     o_ref, l_ref = _varlen_reference(as_f64(tq), np.nan_to_num(as_f64(tk)), np.nan_to_num(as_f64(tv)), lengths, h, d**-0.5, causal)
     check(o, lse, o_ref, l_ref, BF16_TOL if dt == torch.bfloat16 else F32_TOL)
+
+
+@pytest.mark.parametrize("d,rk,page_size", [(128, 2, 16), (128, 2, 256), (64, 4, 8), (64, 1, 32)])
+def test_decode_over_a_paged_cache(gpu, d, rk, page_size):
+    """The same cache, once contiguous per sequence and once scattered over a shuffled page pool:
+    the split-key kernel does the same arithmetic in the same order, so the results are equal
+    bit for bit; the contiguous one is checked against the oracle."""
+    from tpa import tpa
+
+    b, h = 3, 16
+    pages_per_seq = max(4, 2048 // page_size)
+    lk = pages_per_seq * page_size
+    lengths = [lk, lk - page_size - 3, 5]
+    q, k, v = make_factors(111, b, 1, lk, h, d, d, 6, rk, scale_by_rank=True)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    kv_len = torch.tensor(lengths, dtype=torch.int32)
+    o1, l1 = tpa.tpa_decode(*tpa_split(tq, tk, tv, h), sm_scale=d**-0.5, kv_lengths=kv_len, kernel=2)
+    # scatter the pages of all sequences over a pool twice as large, in random order
+    npages = 2 * b * pages_per_seq
+    perm = torch.from_numpy(np.random.default_rng(112).permutation(npages)[: b * pages_per_seq].astype(np.int32)).reshape(b, pages_per_seq)
+    pool_k = torch.full((npages, page_size, rk, h + d), float("nan"), dtype=torch.bfloat16, device=gpu)
+    pool_v = torch.full_like(pool_k, float("nan"))
+    for bi in range(b):
+        for pg in range(pages_per_seq):
+            pool_k[perm[bi, pg]] = tk[bi, pg * page_size : (pg + 1) * page_size]
+            pool_v[perm[bi, pg]] = tv[bi, pg * page_size : (pg + 1) * page_size]
+    qa, qb = tq[..., :h].contiguous(), tq[..., h:].contiguous()
+    o2, l2 = tpa.tpa_decode(qa, qb, pool_k[..., :h].contiguous(), pool_k[..., h:].contiguous(), pool_v[..., :h].contiguous(),
+                            pool_v[..., h:].contiguous(), sm_scale=d**-0.5, kv_lengths=kv_len, page_table=perm, kernel=2)
+    assert torch.equal(o1, o2) and torch.equal(l1, l2)
+    o_ref, l_ref = _varlen_reference(as_f64(tq), as_f64(tk), as_f64(tv), lengths, h, d**-0.5, False)
+    check(o1, l1, o_ref, l_ref, BF16_TOL)
+
+
+def test_paged_cache_is_refused_where_no_kernel_reads_it(gpu):
+    from tpa import _dispatch as dd
+    from tpa import tpa
+
+    q, k, v = make_factors(113, 1, 1, 72, 8, 64, 64, 2, 2)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    qa, qb, ka, kb, va, vb = tpa_split(tq, tk, tv, 8)
+    table = torch.tensor([[0, 1, 2]], dtype=torch.int32)
+    with pytest.raises(dd.TpaError) as e:  # 24 tokens per page * rank 2 = 48 rows: not a multiple of 32
+        tpa.tpa_decode(qa, qb, ka.reshape(3, 24, 2, 8), kb.reshape(3, 24, 2, 64), va.reshape(3, 24, 2, 8),
+                       vb.reshape(3, 24, 2, 64), page_table=table, kernel=2)
+    assert e.value.code == -2
+    with pytest.raises(dd.TpaError) as e:  # the fp32 kernel does not read page pools
+        tpa.tpa_decode(qa.float(), qb.float(), ka.reshape(3, 24, 2, 8).float(), kb.reshape(3, 24, 2, 64).float(),
+                       va.reshape(3, 24, 2, 8).float(), vb.reshape(3, 24, 2, 64).float(), page_table=table)
+    assert e.value.code == -6
