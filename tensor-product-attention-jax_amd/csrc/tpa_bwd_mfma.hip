@@ -561,12 +561,8 @@ int launch_dq(const BwdParams& base, hipStream_t stream) {
   p.npairs = p.nblk * p.B;
   auto kern = bwd_dq_kernel<D, NW, NB, SEG>;
   const size_t smem = (size_t)4 * kTile * tile_stride(D) * 2 + 2 * kTile * 4;
-  static bool configured = false;
-  if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
-      return TPA_ERR_LAUNCH;
-    configured = true;
-  }
+  static bool configured[kMaxDevices] = {};
+  if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), smem); rc != TPA_OK) return rc;
   hipLaunchKernelGGL(kern, dim3(((p.npairs + 7) / 8) * 8 * p.H), dim3(NW * 64), smem, stream, p);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
 }
@@ -578,12 +574,8 @@ int launch_dkv(const BwdParams& base, hipStream_t stream) {
   p.npairs = p.nblk * p.B;
   auto kern = bwd_dkv_kernel<D, NW, NB, SEG>;
   const size_t smem = (size_t)4 * kTile * tile_stride(D) * 2 + 6 * kTile * 4;
-  static bool configured = false;
-  if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
-      return TPA_ERR_LAUNCH;
-    configured = true;
-  }
+  static bool configured[kMaxDevices] = {};
+  if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), smem); rc != TPA_OK) return rc;
   hipLaunchKernelGGL(kern, dim3(((p.npairs + 7) / 8) * 8 * p.H), dim3(NW * 64), smem, stream, p);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
 }

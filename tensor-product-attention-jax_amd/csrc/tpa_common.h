@@ -111,6 +111,19 @@ __device__ __forceinline__ void build_q_fragments(const uint16_t* ap, int64_t a_
   }
 }
 
+// Raise a kernel's dynamic LDS limit above the 64 KB a kernel gets without asking.  The attribute
+// belongs to one device's copy of the code, so it is set once per device (`done` is the calling
+// launcher's own table; a race between two first launches only repeats the same call).
+constexpr int kMaxDevices = 64;
+inline int raise_lds_limit(bool (&done)[kMaxDevices], const void* kern, size_t bytes) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) return TPA_ERR_LAUNCH;
+  if (dev < kMaxDevices && done[dev]) return TPA_OK;
+  if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) return TPA_ERR_LAUNCH;
+  if (dev < kMaxDevices) done[dev] = true;
+  return TPA_OK;
+}
+
 }  // namespace tpa
 
 // host-side entry points of the individual kernel files (launchers return TPA_* codes)

@@ -381,12 +381,8 @@ int launch_decode_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   p.page_table = a->page_table; p.page_size = a->page_size; p.pages_per_seq = a->pages_per_seq;
   p.qscale = a->sm_scale * kLog2e / ((float)a->rq * (float)RK);
   auto kern = decode_kernel<D, RK, PAGED>;
-  static bool configured = false;
-  if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)DecodeLds<D>::kBytes) != hipSuccess)
-      return TPA_ERR_LAUNCH;
-    configured = true;
-  }
+  static bool configured[kMaxDevices] = {};
+  if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), DecodeLds<D>::kBytes); rc != TPA_OK) return rc;
   dim3 grid(a->B * S, a->lq, (a->H + 31) / 32);
   hipLaunchKernelGGL(kern, grid, dim3(kWaves * 64), DecodeLds<D>::kBytes, stream, p);
   if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;

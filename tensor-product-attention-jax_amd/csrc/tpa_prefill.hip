@@ -865,12 +865,8 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
 template <int D, int LOADER, bool SEG = false>
 int launch_prefill(const PrefillParams& p, hipStream_t stream) {
   auto kern = prefill_kernel<D, LOADER, SEG>;
-  static bool configured = false;  // idempotent attribute; a race only repeats the same call
-  if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)Lds<D>::kBytes) != hipSuccess)
-      return TPA_ERR_LAUNCH;
-    configured = true;
-  }
+  static bool configured[kMaxDevices] = {};
+  if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), Lds<D>::kBytes); rc != TPA_OK) return rc;
   const int groups = (p.npairs + 7) / 8;
   dim3 grid(groups * 8 * p.H);
   hipLaunchKernelGGL(kern, grid, dim3(kNW * 64), Lds<D>::kBytes, stream, p);
