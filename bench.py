@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c4pg|c5|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|copy] [--no-cpu] [--no-decode] [--no-backward]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c4pg|c5|c2f|c3f|c2fb|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|copy] [--no-cpu] [--no-decode] [--no-backward]
 
 A step is one forward pass over one batch of synthetic, seeded inputs that are resident in HBM
 before the timed region starts.  The default workload is the prefill configuration the headline
@@ -25,6 +25,7 @@ sys.path.insert(0, os.path.join(ROOT, "tensor-product-attention-jax_amd"))
 sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2516.6  # MI355X dense bf16 MFMA
+PEAK_F32_TFLOPS = 157.3    # MI355X dense fp32 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
 WORKLOADS = {
@@ -45,7 +46,12 @@ WORKLOADS = {
     "c2pb": ("backward", 4, 4096, 4096, 16, 128, 6, 2, True),   # packed documents, as c2p
     "c2p": ("prefill", 4, 4096, 4096, 16, 128, 6, 2, True),
     "c3p": ("prefill", 1, 32768, 32768, 32, 128, 6, 2, True),
+    # fp32 inputs (the reference's default dtype) at the c2 shape and at a quarter of c3's length: the fp32 MFMA kernel
+    "c2f": ("prefill", 4, 4096, 4096, 16, 128, 6, 2, True),
+    "c3f": ("prefill", 1, 16384, 16384, 32, 128, 6, 2, True),
+    "c2fb": ("backward", 4, 4096, 4096, 16, 128, 6, 2, True),
 }
+F32_WORKLOADS = ("c2f", "c3f", "c2fb")
 COPY_BYTES = 1 << 30  # --workload copy: bytes read (and bytes written) by each plain copy launch
 
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counters (profiles/), each scaled by what
@@ -61,13 +67,13 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed):
-    """Split factor arrays, i.i.d. N(0,1) / sqrt(R), bf16, generated on the device."""
+def make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed, dtype=None):
+    """Split factor arrays, i.i.d. N(0,1) / sqrt(R), bf16 unless `dtype` says otherwise, generated on the device."""
     g = torch.Generator(device=device)
     g.manual_seed(seed)
 
     def draw(shape, r):
-        return (torch.randn(shape, generator=g, device=device, dtype=torch.float32) / r**0.5).to(torch.bfloat16)
+        return (torch.randn(shape, generator=g, device=device, dtype=torch.float32) / r**0.5).to(dtype or torch.bfloat16)
 
     return (
         draw((B, lq, rq, H), rq), draw((B, lq, rq, D), rq),
@@ -111,7 +117,7 @@ def time_steps(torch, fn, steps, warmup):
 
 def run_prefill(torch, tpa, device, name, steps, warmup):
     _, B, lq, lk, H, D, rq, rk, causal = WORKLOADS[name]
-    x = make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed=0)
+    x = make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed=0, dtype=torch.float32 if name in F32_WORKLOADS else None)
     scale = D**-0.5
     out = {}
     doc = DOC_LEN.get(name)
@@ -158,14 +164,15 @@ def run_backward(torch, tpa, device, name, steps, warmup):
     """One step = one call of the backward entry point (all its kernels) on resident inputs, with
     the forward's o and lse computed once beforehand."""
     _, B, lq, lk, H, D, rq, rk, causal = WORKLOADS[name]
-    x = make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed=0)
+    dtype = torch.float32 if name in F32_WORKLOADS else torch.bfloat16
+    x = make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed=0, dtype=dtype)
     scale = D**-0.5
     doc = DOC_LEN.get(name)
     seg = (torch.arange(lq, device=device, dtype=torch.int32) // doc).repeat(B, 1).contiguous() if doc else None
     o, lse = tpa.tpa_factors(*x, seg, seg, sm_scale=scale, causal=causal, kernel=2)
     g = torch.Generator(device=device)
     g.manual_seed(7)
-    do = torch.randn(o.shape, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    do = torch.randn(o.shape, generator=g, device=device, dtype=torch.float32).to(dtype)
     grads = tuple(torch.empty(t.shape, dtype=torch.float32, device=device) for t in x)
     ws = torch.empty(tpa.bwd_workspace_bytes(B, lq, lk, H, D, D) + 256, dtype=torch.uint8, device=device)
 
@@ -305,18 +312,20 @@ def main():
     result = {}
     if kind == "prefill":
         log(f"[bench] prefill {args.workload}: warmup {args.warmup}, steps {args.steps}")
+        f32 = args.workload in F32_WORKLOADS
+        peak = PEAK_F32_TFLOPS if f32 else PEAK_BF16_TFLOPS
         r = run_prefill(torch, tpa, device, args.workload, args.steps, args.warmup)
         log(f"[bench] {r['kernel_ms']:.4f} ms/launch (min {r['kernel_ms_min']:.4f}), {r['tflops_kernel']:.1f} TFLOP/s")
         result.update(
             metric="TPA causal prefill forward throughput" if r["shape"]["causal"] else "TPA prefill forward throughput",
             value=r["tflops_wall"], unit="TFLOP/s", ms_per_step=r["wall_ms"],
-            roofline=dict(bound="mfma", achieved=r["tflops_kernel"], peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                          frac=r["tflops_kernel"] / PEAK_BF16_TFLOPS, traffic=MEASURED_TRAFFIC.get(args.workload),
-                          kernel="prefill_kernel", ms_per_launch=r["kernel_ms"], ms_per_launch_min=r["kernel_ms_min"],
-                          algorithmic_flops_per_launch=r["flops"]),
-            config=dict(workload=f"{args.workload}: TPA prefill", **r["shape"]),
+            roofline=dict(bound="mfma", achieved=r["tflops_kernel"], peak=peak, unit="TFLOP/s",
+                          frac=r["tflops_kernel"] / peak, traffic=MEASURED_TRAFFIC.get(args.workload),
+                          kernel="prefill_f32_kernel" if f32 else "prefill_kernel", ms_per_launch=r["kernel_ms"],
+                          ms_per_launch_min=r["kernel_ms_min"], algorithmic_flops_per_launch=r["flops"]),
+            config=dict(workload=f"{args.workload}: TPA prefill" + (", fp32 inputs" if f32 else ""), **r["shape"]),
         )
-        if not args.no_decode:
+        if not args.no_decode and not f32:
             log("[bench] decode c4")
             d = run_decode(torch, tpa, device, "c4", args.steps, args.warmup)
             log(f"[bench] {d['kernel_ms']*1e3:.1f} us/launch (min {d['kernel_ms_min']*1e3:.1f}), {d['gbs_kernel']:.0f} GB/s")
@@ -376,14 +385,17 @@ def main():
         log(f"[bench] backward {args.workload}: warmup {args.warmup}, steps {args.steps}")
         r = run_backward(torch, tpa, device, args.workload, args.steps, args.warmup)
         log(f"[bench] {r['kernel_ms']:.4f} ms/call (min {r['kernel_ms_min']:.4f}), {r['tflops_kernel']:.1f} TFLOP/s")
+        f32 = args.workload in F32_WORKLOADS
+        peak = PEAK_F32_TFLOPS if f32 else PEAK_BF16_TFLOPS
         result.update(
             metric="TPA causal prefill backward throughput", value=r["tflops_wall"], unit="TFLOP/s", ms_per_step=r["wall_ms"],
-            roofline=dict(bound="mfma", achieved=r["tflops_kernel"], peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                          frac=r["tflops_kernel"] / PEAK_BF16_TFLOPS, traffic=None,
-                          kernel="recon + delta + bwd_dq_kernel + bwd_dkv_kernel + project (whole call)",
+            roofline=dict(bound="mfma", achieved=r["tflops_kernel"], peak=peak, unit="TFLOP/s",
+                          frac=r["tflops_kernel"] / peak, traffic=None,
+                          kernel=("recon + delta + bwd_f32_dq_kernel + bwd_f32_dkv_kernel + project (whole call)" if f32 else
+                                  "recon + delta + bwd_dq_kernel + bwd_dkv_kernel + project (whole call)"),
                           ms_per_launch=r["kernel_ms"], ms_per_launch_min=r["kernel_ms_min"],
                           algorithmic_flops_per_launch=r["flops"]),
-            config=dict(workload=f"{args.workload}: TPA backward", **r["shape"]),
+            config=dict(workload=f"{args.workload}: TPA backward" + (", fp32 inputs" if f32 else ""), **r["shape"]),
         )
     else:
         log(f"[bench] decode {args.workload}: warmup {args.warmup}, steps {args.steps}")
@@ -400,7 +412,7 @@ def main():
         )
     result.update(
         n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True, scaling="weak",
-        vs_baseline=None, dtype="bf16", data="synthetic",
+        vs_baseline=None, dtype="f32" if args.workload in F32_WORKLOADS else "bf16", data="synthetic",
     )
     print(json.dumps(result), flush=True)
 

@@ -65,6 +65,7 @@ int tpa_fwd(const TpaFwdArgs* a, void* stream) {
       a->workspace_bytes >= tpa_decode_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dv, a->num_splits))
     return tpa_decode_mfma_launch(a, s);
   if (a->kernel != TPA_KERNEL_GENERIC && tpa_prefill_mfma_supported(a)) return tpa_prefill_mfma_launch(a, s);
+  if (a->kernel != TPA_KERNEL_GENERIC && tpa_prefill_f32_supported(a)) return tpa_prefill_f32_launch(a, s);
   if (a->kernel == TPA_KERNEL_MFMA) return TPA_ERR_UNSUPPORTED;
   return tpa_generic_launch(a, s);
 }
@@ -100,6 +101,7 @@ int mha_fwd(const MhaFwdArgs* a, void* stream) {
     // few query tokens over a long cache: split over keys, if the caller brought the workspace
     if (mha_decode_supported(a) && a->workspace) return mha_decode_launch(a, s);
     if (mha_prefill_mfma_supported(a)) return mha_prefill_mfma_launch(a, s);
+    if (mha_prefill_f32_supported(a)) return mha_prefill_f32_launch(a, s);
   }
   if (a->kernel == TPA_KERNEL_MFMA) return TPA_ERR_UNSUPPORTED;
   return mha_generic_launch(a, s);
@@ -121,9 +123,11 @@ int tpa_bwd(const TpaBwdArgs* a, void* stream) {
   if ((a->q_segment_ids == nullptr) != (a->kv_segment_ids == nullptr)) return TPA_ERR_NULL;
   if (a->kernel != TPA_KERNEL_AUTO && a->kernel != TPA_KERNEL_GENERIC && a->kernel != TPA_KERNEL_MFMA)
     return TPA_ERR_UNSUPPORTED;
+  // matrix-core kernels: bf16 ones for bf16 inputs, fp32 ones for fp32 inputs; both read do with 16-byte loads
   const int mfma = a->kernel != TPA_KERNEL_GENERIC &&
-                   dense_bwd_mfma_supported(a->dtype, a->dk, a->dv, a->lq, a->lk, a->H, a->sm_scale, nullptr) &&
-                   !(reinterpret_cast<uintptr_t>(a->d_o) & 15);  // the MFMA kernels read do with 16-byte loads
+                   (dense_bwd_mfma_supported(a->dtype, a->dk, a->dv, a->lq, a->lk, a->H, a->sm_scale, nullptr) ||
+                    dense_bwd_f32_supported(a->dtype, a->dk, a->dv, a->lq, a->lk, nullptr)) &&
+                   !(reinterpret_cast<uintptr_t>(a->d_o) & 15);
   if (a->kernel == TPA_KERNEL_MFMA && !mfma) return TPA_ERR_UNSUPPORTED;
   if (!a->workspace || a->workspace_bytes < tpa_bwd_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dk, a->dv))
     return TPA_ERR_WORKSPACE;
@@ -145,7 +149,8 @@ int mha_bwd(const MhaBwdArgs* a, void* stream) {
   if (a->kernel != TPA_KERNEL_AUTO && a->kernel != TPA_KERNEL_GENERIC && a->kernel != TPA_KERNEL_MFMA)
     return TPA_ERR_UNSUPPORTED;
   const int mfma = a->kernel != TPA_KERNEL_GENERIC &&
-                   dense_bwd_mfma_supported(a->dtype, a->dk, a->dv, a->lq, a->lk, a->H, a->sm_scale, a->bias) &&
+                   (dense_bwd_mfma_supported(a->dtype, a->dk, a->dv, a->lq, a->lk, a->H, a->sm_scale, a->bias) ||
+                    dense_bwd_f32_supported(a->dtype, a->dk, a->dv, a->lq, a->lk, a->bias)) &&
                    !(reinterpret_cast<uintptr_t>(a->q) & 15) && !(reinterpret_cast<uintptr_t>(a->k) & 15) &&
                    !(reinterpret_cast<uintptr_t>(a->v) & 15) && !(reinterpret_cast<uintptr_t>(a->d_o) & 15) &&
                    !(reinterpret_cast<uintptr_t>(a->dq) & 15) && !(reinterpret_cast<uintptr_t>(a->dk_out) & 15) &&

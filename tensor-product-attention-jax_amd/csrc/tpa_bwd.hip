@@ -431,6 +431,9 @@ int tpa_bwd_t(const TpaBwdArgs* a, hipStream_t stream, bool mfma) {
   float *qd = take(nq), *kd = take(nk), *vd = take(nv), *dqd = take(nq), *dkd = take(nk), *dvd = take(nv), *delta = take(nd);
 
   const int threads = 256;
+  // the matrix-core kernels: bf16 ones on bf16 copies of Q, K, V; fp32 ones on the fp32 copies
+  const bool mfma32 = mfma && sizeof(T) == sizeof(float);
+  mfma = mfma && !mfma32;
   if (mfma) {
     uint16_t *q16 = reinterpret_cast<uint16_t*>(qd), *k16 = reinterpret_cast<uint16_t*>(kd), *v16 = reinterpret_cast<uint16_t*>(vd);
     auto recon16 = [&](const TpaFactor& fa, const TpaFactor& fb, uint16_t* out, int L, int D, int R) {
@@ -460,6 +463,9 @@ int tpa_bwd_t(const TpaBwdArgs* a, hipStream_t stream, bool mfma) {
   if (mfma) {
     rc = dense_bwd_mfma_launch(qd, kd, vd, a->d_o, a->lse, delta, a->q_segment_ids, a->kv_segment_ids, dqd, dkd, dvd,
                                a->B, a->lq, a->lk, a->H, a->dk, a->sm_scale, a->causal, stream);
+  } else if (mfma32) {
+    rc = dense_bwd_f32_launch(qd, kd, vd, static_cast<const float*>(a->d_o), a->lse, delta, a->q_segment_ids, a->kv_segment_ids,
+                              dqd, dkd, dvd, a->B, a->lq, a->lk, a->H, a->dk, a->sm_scale, a->causal, stream);
   } else {
     DenseParams p{};
     p.q = qd; p.k = kd; p.v = vd; p.d_o = a->d_o; p.lse = a->lse; p.delta = delta;
@@ -491,6 +497,10 @@ int mha_bwd_t(const MhaBwdArgs* a, hipStream_t stream, bool mfma) {
                        static_cast<const T*>(a->o), static_cast<const T*>(a->d_o), delta, a->B, a->lq, a->H, a->dv, vec);
   }
   if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
+  if (mfma && sizeof(T) == sizeof(float))
+    return dense_bwd_f32_launch(static_cast<const float*>(a->q), static_cast<const float*>(a->k), static_cast<const float*>(a->v),
+                                static_cast<const float*>(a->d_o), a->lse, delta, nullptr, nullptr, a->dq, a->dk_out, a->dv_out,
+                                a->B, a->lq, a->lk, a->H, a->dk, a->sm_scale, a->causal, stream);
   if (mfma)
     return dense_bwd_mfma_launch(a->q, a->k, a->v, a->d_o, a->lse, delta, nullptr, nullptr, a->dq, a->dk_out, a->dv_out,
                                  a->B, a->lq, a->lk, a->H, a->dk, a->sm_scale, a->causal, stream);
@@ -545,14 +555,14 @@ size_t mha_bwd_workspace_size(int64_t B, int64_t lq, int64_t lk, int64_t H, int6
 
 int tpa_bwd_launch(const TpaBwdArgs* a, hipStream_t stream, int mfma) {
   if (a->B > 65535 || a->H > 65535) return TPA_ERR_SHAPE;
-  if (a->dtype == TPA_DTYPE_F32) return tpa::tpa_bwd_t<float>(a, stream, false);
+  if (a->dtype == TPA_DTYPE_F32) return tpa::tpa_bwd_t<float>(a, stream, mfma != 0);
   if (a->dtype == TPA_DTYPE_BF16) return tpa::tpa_bwd_t<uint16_t>(a, stream, mfma != 0);
   return TPA_ERR_DTYPE;
 }
 
 int mha_bwd_launch(const MhaBwdArgs* a, hipStream_t stream, int mfma) {
   if (a->B > 65535 || a->H > 65535) return TPA_ERR_SHAPE;
-  if (a->dtype == TPA_DTYPE_F32) return tpa::mha_bwd_t<float>(a, stream, false);
+  if (a->dtype == TPA_DTYPE_F32) return tpa::mha_bwd_t<float>(a, stream, mfma != 0);
   if (a->dtype == TPA_DTYPE_BF16) return tpa::mha_bwd_t<uint16_t>(a, stream, mfma != 0);
   return TPA_ERR_DTYPE;
 }

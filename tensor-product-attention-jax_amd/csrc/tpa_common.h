@@ -133,6 +133,10 @@ int tpa_prefill_mfma_supported(const TpaFwdArgs* a);
 int tpa_prefill_mfma_launch(const TpaFwdArgs* a, hipStream_t stream);
 int mha_prefill_mfma_supported(const MhaFwdArgs* a);
 int mha_prefill_mfma_launch(const MhaFwdArgs* a, hipStream_t stream);
+int tpa_prefill_f32_supported(const TpaFwdArgs* a);
+int tpa_prefill_f32_launch(const TpaFwdArgs* a, hipStream_t stream);
+int mha_prefill_f32_supported(const MhaFwdArgs* a);
+int mha_prefill_f32_launch(const MhaFwdArgs* a, hipStream_t stream);
 int tpa_decode_mfma_supported(const TpaFwdArgs* a);
 int tpa_decode_mfma_launch(const TpaFwdArgs* a, hipStream_t stream);
 int mha_decode_supported(const MhaFwdArgs* a);
@@ -143,6 +147,10 @@ int dense_bwd_mfma_supported(int dtype, int dk, int dv, int64_t lq, int64_t lk, 
 int dense_bwd_mfma_launch(const void* q, const void* k, const void* v, const void* d_o, const float* lse, const float* delta,
                           const int32_t* qseg, const int32_t* kvseg, float* dq, float* dk, float* dv, int B, int lq, int lk,
                           int H, int D, float sm_scale, int causal, hipStream_t stream);
+int dense_bwd_f32_supported(int dtype, int dk, int dv, int64_t lq, int64_t lk, const void* bias);
+int dense_bwd_f32_launch(const float* q, const float* k, const float* v, const float* d_o, const float* lse, const float* delta,
+                         const int32_t* qseg, const int32_t* kvseg, float* dq, float* dk, float* dv, int B, int lq, int lk,
+                         int H, int D, float sm_scale, int causal, hipStream_t stream);
 size_t tpa_bwd_workspace_size(int64_t B, int64_t lq, int64_t lk, int64_t H, int64_t dk, int64_t dv);
 size_t mha_bwd_workspace_size(int64_t B, int64_t lq, int64_t lk, int64_t H, int64_t dk, int64_t dv, int dtype);
 size_t tpa_prefill_dense_kv_bytes(int64_t B, int64_t lk, int64_t H, int64_t D);

@@ -1,0 +1,141 @@
+"""Parity of the fp32 MFMA prefill kernel (fp32 inputs, the reference's default dtype) against the
+CPU oracle, through the Python API -> C ABI.  kernel=2 makes a fall-back to the vector-ALU kernel
+an error, so every case here really runs the matrix-core kernel.  Tolerance: 1e-4 on outputs,
+1e-3 on the logsumexp, as for every fp32 path.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import make_factors, segment_ids
+from oracle import tpa_oracle as orc
+from test_gpu_parity import F32_TOL, _varlen_reference, as_f64, check, split, to_gpu
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize(
+    "b,lq,lk,h,rq,rk",
+    [
+        (2, 512, 512, 4, 6, 2),   # the benchmark ranks
+        (1, 300, 300, 2, 6, 2),   # ragged tails in both directions
+        (1, 257, 130, 2, 1, 1),   # lq > lk, rank 1
+        (1, 100, 700, 3, 3, 4),   # lk > lq
+        (1, 256, 256, 2, 16, 8),  # the high-rank configuration's ranks
+    ],
+)
+def test_prefill_f32_mfma(gpu, d, causal, b, lq, lk, h, rq, rk):
+    from tpa import tpa
+
+    q, k, v = make_factors(12, b, lq, lk, h, d, d, rq, rk)
+    scale = d**-0.5
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=scale, causal=causal, kernel=2)
+    o_ref, l_ref = orc.tpa_reference(q, k, v, None, None, h, sm_scale=scale, causal=causal)
+    check(o, lse, o_ref, l_ref, F32_TOL)
+
+
+def test_prefill_f32_mfma_concatenated_layout_in_place(gpu):
+    """The reference's q[b, l, r, h + d] arrays read in place (A = base, B = base + h), default
+    kernel choice: identical to the explicit MFMA request on split copies."""
+    from tpa import tpa
+
+    b, t, h, d = 2, 384, 8, 64
+    q, k, v = make_factors(13, b, t, t, h, d, d, 6, 2)
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    o, res = tpa._tpa_fwd(tq, tk, tv, h, None, None, d**-0.5, True, None, False, False, False)
+    o2, lse2 = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=d**-0.5, causal=True, kernel=2)
+    assert torch.equal(o, o2) and torch.equal(res[-1].permute(0, 2, 1), lse2)
+    o_ref, l_ref = orc.tpa_reference(q, k, v, None, None, h, sm_scale=d**-0.5, causal=True)
+    check(o, res[-1].permute(0, 2, 1), o_ref, l_ref, F32_TOL)
+
+
+@pytest.mark.parametrize(
+    "b,lq,lk,h,d,rk,seg,causal",
+    [
+        (2, 512, 512, 4, 128, 2, 100, True),
+        (2, 640, 384, 2, 64, 2, 77, False),    # query rows whose segment has no key at all: NaN / -inf
+        (1, 1024, 1024, 2, 128, 2, 321, True),  # the segment size of tpa/tpa_test.py:72
+        (1, 256, 1024, 2, 64, 4, 42, False),    # tpa/tpa_test.py:69-70 style: lq != lk
+    ],
+)
+def test_prefill_f32_mfma_segment_ids(gpu, b, lq, lk, h, d, rk, seg, causal):
+    from tpa import tpa
+
+    q, k, v = make_factors(14, b, lq, lk, h, d, d, 6, rk)
+    qseg, kvseg = segment_ids(lq, seg, b), segment_ids(lk, seg, b)
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    tqs, tks = torch.from_numpy(qseg).to(gpu), torch.from_numpy(kvseg).to(gpu)
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), tqs, tks, d**-0.5, causal, 2)
+    o_ref, l_ref = orc.tpa_reference(q, k, v, qseg, kvseg, h, sm_scale=d**-0.5, causal=causal)
+    check(o, lse, o_ref, l_ref, F32_TOL)
+    if lq > lk:
+        assert np.isnan(o_ref).any()  # the case really has empty rows
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_prefill_f32_mfma_per_sequence_key_lengths(gpu, causal):
+    """A padded batch: keys past kv_lengths[b] are never read as values (they are NaN here)."""
+    from tpa import tpa
+
+    b, lq, lk, h, d = 4, 400, 700, 8, 64
+    lengths = [700, 333, 64, 0]
+    q, k, v = make_factors(15, b, lq, lk, h, d, d, 3, 2)
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    for bi, n in enumerate(lengths):
+        tk[bi, n:] = float("nan")
+        tv[bi, n:] = float("nan")
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), None, None, d**-0.5, causal, 2, kv_lengths=lengths)
+    o_ref, l_ref = _varlen_reference(as_f64(tq), np.nan_to_num(as_f64(tk)), np.nan_to_num(as_f64(tv)), lengths, h, d**-0.5, causal)
+    check(o, lse, o_ref, l_ref, F32_TOL)
+
+
+def test_prefill_f32_mfma_sharp_softmax_large_logits(gpu):
+    """sm_scale = 1 on N(0,1) factors: logits of order ten and more, row maxima that keep moving
+    from tile to tile (the rescale path), still within the fp32 tolerance."""
+    from tpa import tpa
+
+    b, t, h, d = 1, 640, 2, 64
+    q, k, v = make_factors(16, b, t, t, h, d, d, 2, 2)
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=1.0, causal=False, kernel=2)
+    o_ref, l_ref = orc.tpa_reference(q, k, v, None, None, h, sm_scale=1.0, causal=False)
+    check(o, lse, o_ref, l_ref, F32_TOL)
+    assert np.abs(l_ref).max() > 10  # the logits really are large
+
+
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("causal", [False, True])
+def test_mha_f32_mfma_vs_oracle(gpu, d, causal):
+    """The dense baseline (tpa/mha.py:23-37) through the same kernel."""
+    from tpa.mha import _mha_fwd
+
+    b, lq, lk, h = 2, 320, 450, 3
+    rng = np.random.Generator(np.random.Philox(17))
+    q = rng.standard_normal((b, lq, h, d))
+    k = rng.standard_normal((b, lk, h, d))
+    v = rng.standard_normal((b, lk, h, d))
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    o, (lse, *_) = _mha_fwd(tq, tk, tv, None, d**-0.5, causal=causal, kernel=2)
+    bias = np.where(np.tril(np.ones((lq, lk), bool)), 0.0, -np.inf)[None].repeat(b, 0) if causal else None
+    o_ref, l_ref = orc.mha_forward(as_f64(tq), as_f64(tk), as_f64(tv), bias, d**-0.5)
+    check(o, lse, o_ref, l_ref, F32_TOL)
+
+
+def test_f32_mfma_refuses_what_it_cannot_run(gpu):
+    from tpa import _dispatch as dsp
+    from tpa import tpa
+
+    # too few query rows for a 256-row block per head: the vector-ALU kernel serves these, and an
+    # explicit request for the matrix-core kernel is an error
+    q, k, v = make_factors(18, 1, 8, 512, 2, 64, 64, 2, 2)
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    with pytest.raises(dsp.TpaError) as e:
+        tpa.tpa_factors(*split(tq, tk, tv, 2), sm_scale=0.125, kernel=2)
+    assert e.value.code == -6
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, 2), sm_scale=0.125)
+    o_ref, l_ref = orc.tpa_reference(q, k, v, None, None, 2, sm_scale=0.125)
+    check(o, lse, o_ref, l_ref, F32_TOL)
