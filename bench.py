@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c4pg|c5|c2f|c3f|c2fb|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|copy] [--no-cpu] [--no-decode] [--no-backward]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c4pg|c5|c2f|c3f|c2fb|c4f|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|copy] [--no-cpu] [--no-decode] [--no-backward]
 
 A step is one forward pass over one batch of synthetic, seeded inputs that are resident in HBM
 before the timed region starts.  The default workload is the prefill configuration the headline
@@ -50,8 +50,9 @@ WORKLOADS = {
     "c2f": ("prefill", 4, 4096, 4096, 16, 128, 6, 2, True),
     "c3f": ("prefill", 1, 16384, 16384, 32, 128, 6, 2, True),
     "c2fb": ("backward", 4, 4096, 4096, 16, 128, 6, 2, True),
+    "c4f": ("decode", 64, 1, 8192, 32, 128, 6, 2, False),
 }
-F32_WORKLOADS = ("c2f", "c3f", "c2fb")
+F32_WORKLOADS = ("c2f", "c3f", "c2fb", "c4f")
 COPY_BYTES = 1 << 30  # --workload copy: bytes read (and bytes written) by each plain copy launch
 
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counters (profiles/), each scaled by what
@@ -90,10 +91,10 @@ def prefill_flops(B, lq, lk, H, D, causal):
     return 2.0 * B * H * (D + D) * pairs
 
 
-def decode_bytes(B, lq, lk, H, D, rq, rk):
-    cache = B * lk * (rk + rk) * (H + D) * 2
-    qf = B * lq * rq * (H + D) * 2
-    out = B * lq * H * D * 2 + B * H * lq * 4
+def decode_bytes(B, lq, lk, H, D, rq, rk, elem=2):
+    cache = B * lk * (rk + rk) * (H + D) * elem
+    qf = B * lq * rq * (H + D) * elem
+    out = B * lq * H * D * elem + B * H * lq * 4
     return cache + qf + out
 
 
@@ -192,7 +193,8 @@ def run_backward(torch, tpa, device, name, steps, warmup):
 def run_decode(torch, tpa, device, name, steps, warmup):
     _, B, lq, lk, H, D, rq, rk, _ = WORKLOADS[name]
     # two distinct caches, alternated, so that no launch finds its cache in the 256 MB last-level cache
-    xs = [make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed=s) for s in (0, 1)]
+    f32 = name in F32_WORKLOADS
+    xs = [make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed=s, dtype=torch.float32 if f32 else None) for s in (0, 1)]
     scale = D**-0.5
     ws = torch.empty(max(tpa.decode_workspace_bytes(B, lq, lk, H, D), 16), dtype=torch.uint8, device=device)
     out = {}
@@ -209,7 +211,7 @@ def run_decode(torch, tpa, device, name, steps, warmup):
         out["o"], out["lse"] = tpa.tpa_decode(*xs[i & 1], sm_scale=scale, workspace=ws, kernel=2, page_table=table)
 
     wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
-    nbytes = decode_bytes(B, lq, lk, H, D, rq, rk)
+    nbytes = decode_bytes(B, lq, lk, H, D, rq, rk, elem=4 if f32 else 2)
     return dict(
         wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, bytes=nbytes,
         gbs_wall=nbytes / wall_ms / 1e6, gbs_kernel=nbytes / ev_ms / 1e6,
@@ -405,10 +407,11 @@ def main():
             metric="TPA decode effective HBM bandwidth", value=d["gbs_wall"], unit="GB/s", ms_per_step=d["wall_ms"],
             roofline=dict(bound="hbm", achieved=d["gbs_kernel"], peak=PEAK_HBM_GBS, unit="GB/s",
                           frac=d["gbs_kernel"] / PEAK_HBM_GBS, traffic=MEASURED_TRAFFIC.get(args.workload),
-                          kernel="decode_kernel + decode_merge_kernel",
+                          kernel=("decode_f32_kernel" if args.workload in F32_WORKLOADS else "decode_kernel") + " + decode_merge_kernel",
                           ms_per_launch=d["kernel_ms"], ms_per_launch_min=d["kernel_ms_min"],
                           algorithmic_bytes_per_launch=d["bytes"]),
-            config=dict(workload=f"{args.workload}: TPA decode over the factored KV cache", **d["shape"]),
+            config=dict(workload=f"{args.workload}: TPA decode over the factored KV cache" +
+                        (", fp32 cache" if args.workload in F32_WORKLOADS else ""), **d["shape"]),
         )
     result.update(
         n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True, scaling="weak",

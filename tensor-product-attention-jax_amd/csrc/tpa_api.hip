@@ -61,9 +61,10 @@ int tpa_fwd(const TpaFwdArgs* a, void* stream) {
   // few query tokens over a long cache (the reference's decode is this same call with lq = 1,
   // tpa/tpa.py:485): split over keys, if the caller brought the workspace for it
   if (a->kernel != TPA_KERNEL_GENERIC && a->workspace && a->lq <= 16 && a->lk >= 1024 && !a->causal &&
-      !a->q_segment_ids && tpa_decode_mfma_supported(a) &&
-      a->workspace_bytes >= tpa_decode_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dv, a->num_splits))
-    return tpa_decode_mfma_launch(a, s);
+      !a->q_segment_ids && a->workspace_bytes >= tpa_decode_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dv, a->num_splits)) {
+    if (tpa_decode_mfma_supported(a)) return tpa_decode_mfma_launch(a, s);
+    if (tpa_decode_f32_supported(a)) return tpa_decode_f32_launch(a, s);
+  }
   if (a->kernel != TPA_KERNEL_GENERIC && tpa_prefill_mfma_supported(a)) return tpa_prefill_mfma_launch(a, s);
   if (a->kernel != TPA_KERNEL_GENERIC && tpa_prefill_f32_supported(a)) return tpa_prefill_f32_launch(a, s);
   if (a->kernel == TPA_KERNEL_MFMA) return TPA_ERR_UNSUPPORTED;
@@ -89,6 +90,7 @@ int tpa_decode(const TpaFwdArgs* a, void* stream) {
   if (a->causal || a->q_segment_ids) return TPA_ERR_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (a->kernel != TPA_KERNEL_GENERIC && tpa_decode_mfma_supported(a)) return tpa_decode_mfma_launch(a, s);
+  if (a->kernel != TPA_KERNEL_GENERIC && tpa_decode_f32_supported(a)) return tpa_decode_f32_launch(a, s);
   if (a->kernel == TPA_KERNEL_MFMA || a->page_table) return TPA_ERR_UNSUPPORTED;  // only the split-key kernel reads page pools
   return tpa_generic_launch(a, s);
 }

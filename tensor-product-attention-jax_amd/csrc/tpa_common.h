@@ -139,6 +139,8 @@ int mha_prefill_f32_supported(const MhaFwdArgs* a);
 int mha_prefill_f32_launch(const MhaFwdArgs* a, hipStream_t stream);
 int tpa_decode_mfma_supported(const TpaFwdArgs* a);
 int tpa_decode_mfma_launch(const TpaFwdArgs* a, hipStream_t stream);
+int tpa_decode_f32_supported(const TpaFwdArgs* a);
+int tpa_decode_f32_launch(const TpaFwdArgs* a, hipStream_t stream);
 int mha_decode_supported(const MhaFwdArgs* a);
 int mha_decode_launch(const MhaFwdArgs* a, hipStream_t stream);
 int tpa_bwd_launch(const TpaBwdArgs* a, hipStream_t stream, int mfma);

@@ -323,10 +323,243 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   }
 }
 
-// Merge the key ranges: o = sum_s f_s O_s / (Rk sum_s f_s l_s), f_s = 2^(m_s - max m); lse = ln of the total.
+// ---------------------------------------------------------------------------------------------
+// The same decode for an fp32 cache (the reference's default dtype): fp32 MFMA contractions
+// (v_mfma_f32_32x32x2_f32) on fp32 rows.  Same decomposition and the same workspace; what differs
+// is the operand order a two-index fp32 step asks for: over d, wave half g takes d = 8m + 4g + e
+// (one 16-byte LDS read feeds four steps); over the block's rows, half g takes the row its S'^T
+// register belongs to, and the 32 rows of block db of O^T are d = (D/32) i + db, so one 16-byte
+// read of B_v[row][(D/32) i ...] feeds every block.  One block of loads is in flight in registers
+// (128 of them for D = 128) while the previous block is consumed; the head factors a_k, a_v are
+// read straight into the registers of the logits they multiply.
 template <int D>
+struct DecodeF32Lds {
+  static constexpr int RS = D + 4;                   // row stride (floats)
+  static constexpr int kTile = kRowsPerBlock * RS;   // one B tile
+  static constexpr int kPerWave = 2 * kTile;         // B_k and B_v; the wave merge reuses it (32 x RS + 64 floats)
+  static constexpr size_t kBytes = (size_t)kWaves * kPerWave * sizeof(float);
+};
+
+template <int D, int RK>
+__global__ __launch_bounds__(kWaves * 64) void decode_f32_kernel(DecodeParams p) {
+  constexpr int CPR = D / 4;               // 16-byte chunks per B row
+  constexpr int RPI = 64 / CPR;            // B rows per load instruction
+  constexpr int NLB = kRowsPerBlock / RPI; // load instructions per B tile
+  constexpr int NDB = D / 32;
+  constexpr int TPQ = 4 / RK;              // tokens per 4-row group
+  constexpr int RS = DecodeF32Lds<D>::RS;
+  static_assert(RK == 1 || RK == 2 || RK == 4, "rank must divide 4");
+  typedef __attribute__((ext_vector_type(NDB))) float f32xN;
+
+  extern __shared__ __attribute__((aligned(16))) float smem_dec_f32[];
+
+  const int S = p.S;
+  const int b = blockIdx.x / S, split = blockIdx.x % S;
+  const int qi = blockIdx.y;
+  const int h0 = blockIdx.z * 32;
+  const int tid = threadIdx.x;
+  const int w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
+  const int hl = min(h0 + i, p.H - 1);  // this lane's head (clamped: lanes past H idle along)
+
+  float* const lds = smem_dec_f32 + w * DecodeF32Lds<D>::kPerWave;
+  float* const lds_bk = lds;
+  float* const lds_bv = lds + DecodeF32Lds<D>::kTile;
+
+  const int nparts = S * kWaves;
+  const int part = split * kWaves + w;
+  const int len_b = p.kvlen ? max(0, min(p.kvlen[b], p.lk)) : p.lk;
+  const int blk_begin = part;
+  const int blk_end = (len_b * RK + kRowsPerBlock - 1) / kRowsPerBlock;
+  const int blk_step = nparts;
+  const int last_row = len_b * RK - 1;
+
+  const float* const kb_base = static_cast<const float*>(p.kb.ptr) + b * p.kb.stride_b;
+  const float* const vb_base = static_cast<const float*>(p.vb.ptr) + b * p.vb.stride_b;
+  const float* const ka_base = static_cast<const float*>(p.ka.ptr) + b * p.ka.stride_b + hl;
+  const float* const va_base = static_cast<const float*>(p.va.ptr) + b * p.va.stride_b + hl;
+  const int lb_row = l / CPR, lb_c = l % CPR;
+
+  // one register set: the block after the one being consumed
+  f32x4 rbk[NLB], rbv[NLB];
+  float rak[16], rav[16];
+  auto issue = [&](int blk) {
+    const int row0 = blk * kRowsPerBlock;
+#pragma unroll
+    for (int n = 0; n < NLB; ++n) {
+      const int row = min(row0 + n * RPI + lb_row, last_row);
+      rbk[n] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(kb_base + (int64_t)row * p.kb.stride_r + 4 * lb_c));
+      rbv[n] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(vb_base + (int64_t)row * p.vb.stride_r + 4 * lb_c));
+    }
+    // a[row][head of this lane] for the 16 rows this lane's S'^T registers belong to
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = min(row0 + 8 * (v >> 2) + 4 * g + (v & 3), last_row);
+      rak[v] = ka_base[(int64_t)row * p.ka.stride_r];
+      rav[v] = va_base[(int64_t)row * p.va.stride_r];
+    }
+  };
+  float ak[16], av[16];
+  auto stage = [&]() {
+#pragma unroll
+    for (int n = 0; n < NLB; ++n) {
+      const int row = n * RPI + lb_row;
+      *reinterpret_cast<f32x4*>(lds_bk + row * RS + 4 * lb_c) = rbk[n];
+      *reinterpret_cast<f32x4*>(lds_bv + row * RS + 4 * lb_c) = rbv[n];
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) { ak[v] = rak[v]; av[v] = rav[v]; }
+  };
+
+  if (blk_begin < blk_end) issue(blk_begin);
+
+  // ---- Qm (B operand of S'^T = B_k Qm^T): qf[4m + e] = qscale * sum_r qa[r][h] qb[r][8m + 4g + e]
+  float qf[D / 2];
+#pragma unroll
+  for (int j = 0; j < D / 2; ++j) qf[j] = 0.f;
+  {
+    const float* ap = static_cast<const float*>(p.qa.ptr) + b * p.qa.stride_b + (int64_t)qi * p.qa.stride_l + hl;
+    const float* bp = static_cast<const float*>(p.qb.ptr) + b * p.qb.stride_b + (int64_t)qi * p.qb.stride_l + 4 * g;
+    for (int r = 0; r < p.rq; ++r) {
+      const float a = ap[r * p.qa.stride_r];
+#pragma unroll
+      for (int m = 0; m < D / 8; ++m) {
+        const f32x4 bv = *reinterpret_cast<const f32x4*>(bp + r * p.qb.stride_r + 8 * m);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) qf[4 * m + e] += a * bv[e];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < D / 2; ++j) qf[j] *= p.qscale;
+  }
+
+  f32x16 o[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
+  float m = -INFINITY, lsum = 0.f;
+
+  auto compute = [&](int blk) {
+    // ---- S'^T[row, h] = sum_d B_k[row, d] Qm[h, d]; two accumulation chains, added at the end
+    f32x16 sp, sp2;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) { sp[v] = 0.f; sp2[v] = 0.f; }
+#pragma unroll
+    for (int mm = 0; mm < D / 8; ++mm) {
+      const f32x4 kf = *reinterpret_cast<const f32x4*>(lds_bk + i * RS + 8 * mm + 4 * g);
+      sp = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[0], qf[4 * mm], sp, 0, 0, 0);
+      sp2 = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[1], qf[4 * mm + 1], sp2, 0, 0, 0);
+      sp = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[2], qf[4 * mm + 2], sp, 0, 0, 0);
+      sp2 = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[3], qf[4 * mm + 3], sp2, 0, 0, 0);
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) sp[v] += sp2[v];
+
+    // ---- logits per token (log2 domain), masked past the end of the cache
+    float st[4 * TPQ];
+    float tmax = -INFINITY;
+    const int row0 = blk * kRowsPerBlock;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int e = 0; e < TPQ; ++e) {
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < RK; ++j) acc += ak[4 * q + e * RK + j] * sp[4 * q + e * RK + j];
+        const int row = row0 + 8 * q + 4 * g + e * RK;
+        if (row > last_row) acc = -INFINITY;
+        st[q * TPQ + e] = acc;
+        tmax = fmaxf(tmax, acc);
+      }
+    tmax = halves_max(tmax);
+    const float m_new = fmaxf(m, tmax);  // finite: row0 itself is always inside the cache
+    if (__any(m_new > m)) {
+      const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+      lsum *= alpha;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+      m = m_new;
+    }
+
+    // ---- P'^T[row, h] = p[h, token(row)] * a_v[row, h], in place of the logits' registers
+    float pp[16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int e = 0; e < TPQ; ++e) {
+        const float pt = __builtin_amdgcn_exp2f(st[q * TPQ + e] - m);
+        lsum += pt;
+#pragma unroll
+        for (int j = 0; j < RK; ++j) pp[4 * q + e * RK + j] = pt * av[4 * q + e * RK + j];
+      }
+
+    // ---- O^T[d, h] += sum_row B_v[row, d] P'^T[row, h]
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = 8 * (v >> 2) + 4 * g + (v & 3);
+      const f32xN vf = *reinterpret_cast<const f32xN*>(lds_bv + row * RS + NDB * i);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf[db], pp[v], o[db], 0, 0, 0);
+    }
+  };
+
+  for (int blk = blk_begin; blk < blk_end; blk += blk_step) {
+    stage();  // waits for this block's loads; its registers are then free again
+    if (blk + blk_step < blk_end) issue(blk + blk_step);
+    compute(blk);
+  }
+
+  // ---- merge the 4 waves through LDS (each wave reuses its own staging region)
+  const float ltot = halves_sum(lsum);
+  float* red_o = lds;  // [32 heads][RS]: row 8 (v/4) + 4 g + v%4 of block db is d = NDB * row + db
+  float* red_m = red_o + 32 * RS;
+  float* red_l = red_m + 32;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int row = 8 * (v >> 2) + 4 * g + (v & 3);
+    f32xN out;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) out[db] = o[db][v];
+    *reinterpret_cast<f32xN*>(red_o + i * RS + NDB * row) = out;
+  }
+  if (g == 0) {
+    red_m[i] = m;
+    red_l[i] = ltot;
+  }
+  __syncthreads();
+
+  const int nh = min(32, p.H - h0);
+  const int64_t pbase = (((int64_t)b * p.lq + qi) * S + split) * p.H + h0;
+  for (int idx = tid; idx < nh * D; idx += kWaves * 64) {
+    const int hh = idx / D, d = idx % D;
+    float mw[kWaves], mmax = -INFINITY;
+#pragma unroll
+    for (int ww = 0; ww < kWaves; ++ww) {
+      mw[ww] = (smem_dec_f32 + ww * DecodeF32Lds<D>::kPerWave)[32 * RS + hh];
+      mmax = fmaxf(mmax, mw[ww]);
+    }
+    float acc = 0.f, lacc = 0.f;
+#pragma unroll
+    for (int ww = 0; ww < kWaves; ++ww) {
+      const float* ro = smem_dec_f32 + ww * DecodeF32Lds<D>::kPerWave;
+      const float f = mw[ww] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw[ww] - mmax);
+      acc += f * ro[hh * RS + d];
+      lacc += f * ro[32 * RS + 32 + hh];
+    }
+    p.part_o[(pbase + hh) * D + d] = acc;
+    if (d == 0) {
+      p.part_m[pbase + hh] = mmax;
+      p.part_l[pbase + hh] = lacc;
+    }
+  }
+}
+
+// Merge the key ranges: o = sum_s f_s O_s / (Rk sum_s f_s l_s), f_s = 2^(m_s - max m); lse = ln of the total.
+template <int D, typename TO>
 __global__ __launch_bounds__(D) void decode_merge_kernel(const float* part_o, const float* part_m, const float* part_l,
-                                                         uint16_t* o, float* lse, int S, int H, int lq, float inv_rk) {
+                                                         TO* o, float* lse, int S, int H, int lq, float inv_rk) {
   const int bq = blockIdx.x;  // b * lq + qi
   const int h = blockIdx.y;
   const int d = threadIdx.x;
@@ -386,8 +619,29 @@ int launch_decode_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   dim3 grid(a->B * S, a->lq, (a->H + 31) / 32);
   hipLaunchKernelGGL(kern, grid, dim3(kWaves * 64), DecodeLds<D>::kBytes, stream, p);
   if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
-  hipLaunchKernelGGL(decode_merge_kernel<D>, dim3(a->B * a->lq, a->H), dim3(D), 0, stream, p.part_o, p.part_m, p.part_l,
+  hipLaunchKernelGGL((decode_merge_kernel<D, uint16_t>), dim3(a->B * a->lq, a->H), dim3(D), 0, stream, p.part_o, p.part_m, p.part_l,
                      static_cast<uint16_t*>(a->o), a->lse, S, a->H, a->lq, 1.f / (float)RK);
+  return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
+}
+
+template <int D, int RK>
+int launch_decode_f32(const TpaFwdArgs* a, int S, hipStream_t stream) {
+  DecodeParams p{};
+  p.qa = a->qa; p.qb = a->qb; p.ka = a->ka; p.kb = a->kb; p.va = a->va; p.vb = a->vb;
+  float* ws = static_cast<float*>(a->workspace);
+  const size_t no = (size_t)a->B * a->lq * S * a->H * D, nm = (size_t)a->B * a->lq * S * a->H;
+  p.part_o = ws; p.part_m = ws + no; p.part_l = ws + no + nm;
+  p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.S = S;
+  p.kvlen = a->kv_lengths;
+  p.qscale = a->sm_scale * kLog2e / ((float)a->rq * (float)RK);
+  auto kern = decode_f32_kernel<D, RK>;
+  static bool configured[kMaxDevices] = {};
+  if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), DecodeF32Lds<D>::kBytes); rc != TPA_OK) return rc;
+  dim3 grid(a->B * S, a->lq, (a->H + 31) / 32);
+  hipLaunchKernelGGL(kern, grid, dim3(kWaves * 64), DecodeF32Lds<D>::kBytes, stream, p);
+  if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
+  hipLaunchKernelGGL((decode_merge_kernel<D, float>), dim3(a->B * a->lq, a->H), dim3(D), 0, stream, p.part_o, p.part_m, p.part_l,
+                     static_cast<float*>(a->o), a->lse, S, a->H, a->lq, 1.f / (float)RK);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
 }
 
@@ -463,4 +717,37 @@ int tpa_decode_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
   if (a->rk == 1) return launch_decode<64, 1>(a, S, stream);
   if (a->rk == 2) return launch_decode<64, 2>(a, S, stream);
   return launch_decode<64, 4>(a, S, stream);
+}
+
+int tpa_decode_f32_supported(const TpaFwdArgs* a) {
+  using namespace tpa;
+  if (a->dtype != TPA_DTYPE_F32) return 0;
+  if (a->dk != a->dv || (a->dk != 64 && a->dk != 128)) return 0;
+  if (a->rk != 1 && a->rk != 2 && a->rk != 4) return 0;
+  if (a->lq > 64) return 0;
+  if (a->causal || a->q_segment_ids || a->kv_segment_ids || a->page_table) return 0;
+  // rows (token, rank) must be uniformly strided: stride_l == rk * stride_r; B rows are read as 16-byte vectors
+  const TpaFactor* fs[4] = {&a->ka, &a->kb, &a->va, &a->vb};
+  for (const TpaFactor* f : fs)
+    if (f->stride_l != (int64_t)a->rk * f->stride_r) return 0;
+  const TpaFactor* bs[3] = {&a->kb, &a->vb, &a->qb};
+  for (const TpaFactor* f : bs)
+    if (!aligned16(f->ptr) || f->stride_r % 4 != 0 || f->stride_l % 4 != 0 || f->stride_b % 4 != 0) return 0;
+  return 1;
+}
+
+int tpa_decode_f32_launch(const TpaFwdArgs* a, hipStream_t stream) {
+  using namespace tpa;
+  const int S = a->num_splits > 0 ? a->num_splits : default_splits(a->B, a->lq, a->lk, a->H);
+  if (S > 65535 || (int64_t)a->B * S > 2147483647LL) return TPA_ERR_SHAPE;
+  if (!a->workspace || a->workspace_bytes < workspace_bytes(a->B, a->lq, a->H, a->dv, S)) return TPA_ERR_WORKSPACE;
+  if (!aligned16(a->workspace)) return TPA_ERR_ALIGN;
+  if (a->dk == 128) {
+    if (a->rk == 1) return launch_decode_f32<128, 1>(a, S, stream);
+    if (a->rk == 2) return launch_decode_f32<128, 2>(a, S, stream);
+    return launch_decode_f32<128, 4>(a, S, stream);
+  }
+  if (a->rk == 1) return launch_decode_f32<64, 1>(a, S, stream);
+  if (a->rk == 2) return launch_decode_f32<64, 2>(a, S, stream);
+  return launch_decode_f32<64, 4>(a, S, stream);
 }

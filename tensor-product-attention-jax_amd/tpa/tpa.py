@@ -15,9 +15,9 @@ reference, all on purpose:
   * `interpret=True` (the Pallas CPU interpreter upstream) selects the plain fp32-arithmetic
     kernel instead of the MFMA kernels; `debug` is ignored;
   * the backward pass (tpa/tpa.py:168-214,546-995) goes through dense Q, K, V and dense gradients
-    in a workspace (bf16 MFMA kernels for head sizes 64 and 128, fp32 vector-ALU kernels
-    otherwise); gradients are accumulated in fp32 and cast to the input dtype; torch.autograd
-    reaches it through `tpa()`.
+    in a workspace (bf16 MFMA kernels for bf16 inputs and fp32 MFMA kernels for fp32 inputs of
+    head sizes 64 and 128, fp32 vector-ALU kernels otherwise); gradients are accumulated in fp32
+    and cast to the input dtype; torch.autograd reaches it through `tpa()`.
 """
 
 from __future__ import annotations
@@ -149,7 +149,8 @@ def tpa_factors(
     # a decode through this entry point, dense K and V for ranks other than 2); it decides whether
     # the problem qualifies
     ws, ws_ptr, ws_bytes = None, None, 0
-    if use_workspace and dtype == torch.bfloat16 and kernel != _d.KERNEL_GENERIC:
+    # (fp32 inputs: only the split-key decode kernel takes a workspace)
+    if use_workspace and kernel != _d.KERNEL_GENERIC and (dtype == torch.bfloat16 or lq <= 16):
         need = lib.tpa_fwd_workspace_bytes(b, lq, lk, h, dk, dv, rq, rk)
         if need:
             ws = torch.empty(need + 256, dtype=torch.uint8, device=device)

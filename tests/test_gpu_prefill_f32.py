@@ -139,3 +139,80 @@ def test_f32_mfma_refuses_what_it_cannot_run(gpu):
     o, lse = tpa.tpa_factors(*split(tq, tk, tv, 2), sm_scale=0.125)
     o_ref, l_ref = orc.tpa_reference(q, k, v, None, None, 2, sm_scale=0.125)
     check(o, lse, o_ref, l_ref, F32_TOL)
+
+
+# ---------------------------------------------------------------- fp32 decode over the factored cache
+def _decode_f32(gpu, q, k, v, h, sm_scale, num_splits=0, kernel=2, **kw):
+    from tpa import tpa
+
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    o, lse = tpa.tpa_decode(*split(tq, tk, tv, h), sm_scale=sm_scale, num_splits=num_splits, kernel=kernel, **kw)
+    return (tq, tk, tv), o, lse
+
+
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize(
+    "b,lq,lk,h,rq,rk",
+    [
+        (3, 1, 1024, 32, 6, 2),
+        (2, 1, 1000, 32, 6, 2),  # cache length not a multiple of the block
+        (2, 1, 37, 32, 6, 2),    # shorter than one block per wave
+        (1, 2, 777, 16, 3, 1),   # two query tokens, 16 heads, rank 1
+        (1, 1, 515, 64, 2, 4),   # two head blocks, rank 4
+        (2, 1, 640, 5, 6, 2),    # a head count that is no multiple of anything
+    ],
+)
+def test_decode_f32_mfma(gpu, d, b, lq, lk, h, rq, rk):
+    q, k, v = make_factors(26, b, lq, lk, h, d, d, rq, rk)
+    scale = d**-0.5
+    _, o, lse = _decode_f32(gpu, q, k, v, h, scale)
+    assert o.dtype == torch.float32
+    o_ref, l_ref = orc.tpa_reference(q, k, v, None, None, h, sm_scale=scale)
+    check(o, lse, o_ref, l_ref, F32_TOL)
+
+
+def test_decode_f32_split_invariance_and_vector_kernel(gpu):
+    b, lk, h, d = 2, 2048, 32, 128
+    q, k, v = make_factors(28, b, 1, lk, h, d, d, 6, 2)
+    scale = d**-0.5
+    o_ref, l_ref = orc.tpa_reference(q, k, v, None, None, h, sm_scale=scale)
+    results = []
+    for s in (1, 2, 3, 8):
+        _, o, lse = _decode_f32(gpu, q, k, v, h, scale, num_splits=s)
+        check(o, lse, o_ref, l_ref, F32_TOL)
+        results.append((as_f64(o), as_f64(lse)))
+    for o, lse in results[1:]:  # any number of key ranges: the same answer up to fp32 re-association
+        assert np.abs(o - results[0][0]).max() <= 1e-5 and np.abs(lse - results[0][1]).max() <= 1e-5
+    _, og, lg = _decode_f32(gpu, q, k, v, h, scale, kernel=1)  # the vector-ALU kernel on the same inputs
+    assert np.abs(as_f64(og) - results[0][0]).max() <= F32_TOL and np.abs(as_f64(lg) - results[0][1]).max() <= F32_TOL
+
+
+def test_decode_f32_per_sequence_cache_lengths(gpu):
+    """A padded fp32 cache: entry b reads only its first kv_lengths[b] tokens (the padding is NaN)."""
+    from tpa import tpa
+
+    b, lk, h, d, rk = 5, 3000, 32, 128, 2
+    lengths = [3000, 1777, 9, 640, 0]
+    q, k, v = make_factors(29, b, 1, lk, h, d, d, 6, rk)
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    for bi, n in enumerate(lengths):
+        tk[bi, n:] = float("nan")
+        tv[bi, n:] = float("nan")
+    o, lse = tpa.tpa_decode(*split(tq, tk, tv, h), sm_scale=d**-0.5, kv_lengths=torch.tensor(lengths, dtype=torch.int32), kernel=2)
+    o_ref, l_ref = _varlen_reference(as_f64(tq), np.nan_to_num(as_f64(tk)), np.nan_to_num(as_f64(tv)), lengths, h, d**-0.5, False)
+    check(o, lse, o_ref, l_ref, F32_TOL)
+
+
+def test_tpa_entry_point_serves_fp32_decode_with_the_split_key_kernel(gpu):
+    """tpa() with one query token over a long fp32 cache: the library's decode route (it gets a
+    workspace from the wrapper); the result equals the explicit tpa_decode call bit for bit."""
+    from tpa import tpa
+
+    b, lk, h, d = 2, 4096, 32, 128
+    q, k, v = make_factors(30, b, 1, lk, h, d, d, 6, 2)
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    o = tpa.tpa(tq, tk, tv, num_heads=h, sm_scale=d**-0.5)
+    o2, _ = tpa.tpa_decode(*split(tq, tk, tv, h), sm_scale=d**-0.5, kernel=2)
+    assert torch.equal(o, o2)
+    o_ref, _ = orc.tpa_reference(q, k, v, None, None, h, sm_scale=d**-0.5)
+    assert np.abs(as_f64(o) - o_ref).max() <= F32_TOL
