@@ -168,7 +168,7 @@ typedef struct TpaBwdArgs {
   int32_t dtype;
   float sm_scale;
   int32_t causal;
-  int32_t kernel;         /* TPA_KERNEL_*: the MFMA kernels take bf16 with dk == dv in {64, 128}; d_o must be 16-byte aligned */
+  int32_t kernel;         /* TPA_KERNEL_*: the MFMA kernels take bf16 or fp32 with dk == dv in {64, 128}; d_o must be 16-byte aligned */
   void* workspace;        /* required: at least tpa_bwd_workspace_bytes(...) bytes, 256-byte aligned */
   size_t workspace_bytes;
 } TpaBwdArgs;
