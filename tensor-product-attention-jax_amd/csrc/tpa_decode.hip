@@ -57,8 +57,9 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   constexpr int NLB = kRowsPerBlock / RPI; // load instructions per B tile
   constexpr int NKS = D / 16;
   constexpr int NDB = D / 32;
-  constexpr int TPQ = 4 / RK;              // tokens per 4-row group
-  static_assert(RK == 1 || RK == 2 || RK == 4, "rank must divide 4");
+  constexpr int NTOK = RK <= 4 ? 16 / RK : 32 / RK;  // tokens whose rows this lane holds, per block
+  constexpr int NV = RK <= 4 ? RK : RK / 2;          // rows of one token held by this half of the wave
+  static_assert(RK == 1 || RK == 2 || RK == 4 || RK == 8 || RK == 16 || RK == 32, "a block of 32 rows holds whole tokens");
 
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
 
@@ -202,21 +203,23 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
     }
 
     // ---- logits per token (log2 domain), masked past the end of the cache
-    float st[4 * TPQ];
+    // (a token's RK rows are registers v0 .. v0 + NV - 1; from rank 8 on they span both halves of
+    // the wave, which then hold the same tokens and exchange their partial sums)
+    float st[NTOK];
     float tmax = -INFINITY;
     const int row0 = blk * kRowsPerBlock;
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
+    for (int t = 0; t < NTOK; ++t) {
+      const int v0 = t * NV;
+      float acc = 0.f;
 #pragma unroll
-      for (int e = 0; e < TPQ; ++e) {
-        float acc = 0.f;
-#pragma unroll
-        for (int j = 0; j < RK; ++j) acc += ak[4 * q + e * RK + j] * sp[4 * q + e * RK + j];
-        const int row = row0 + 8 * q + 4 * g + e * RK;
-        if (row > last_row) acc = -INFINITY;
-        st[q * TPQ + e] = acc;
-        tmax = fmaxf(tmax, acc);
-      }
+      for (int j = 0; j < NV; ++j) acc += ak[v0 + j] * sp[v0 + j];
+      if constexpr (RK >= 8) acc = halves_sum(acc);
+      const int row = RK >= 8 ? row0 + RK * t : row0 + 8 * (v0 >> 2) + 4 * g + (v0 & 3);  // the token's first row
+      if (row > last_row) acc = -INFINITY;
+      st[t] = acc;
+      tmax = fmaxf(tmax, acc);
+    }
     tmax = halves_max(tmax);
     const float m_new = fmaxf(m, tmax);  // finite: row0 itself is always inside the cache
     if (__any(m_new > m)) {
@@ -232,14 +235,12 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
     // ---- P'^T[row, h] = p[h, token(row)] * a_v[row, h], packed as the B operand of the PV product
     float pp[16];
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
+    for (int t = 0; t < NTOK; ++t) {
+      const float pt = __builtin_amdgcn_exp2f(st[t] - m);
+      lsum += RK >= 8 ? 0.5f * pt : pt;  // both halves hold the token: each adds half of it
 #pragma unroll
-      for (int e = 0; e < TPQ; ++e) {
-        const float pt = __builtin_amdgcn_exp2f(st[q * TPQ + e] - m);
-        lsum += pt;
-#pragma unroll
-        for (int j = 0; j < RK; ++j) pp[4 * q + e * RK + j] = pt * av[4 * q + e * RK + j];
-      }
+      for (int j = 0; j < NV; ++j) pp[t * NV + j] = pt * av[t * NV + j];
+    }
     bf16x8 pf[2];
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
@@ -346,9 +347,10 @@ __global__ __launch_bounds__(kWaves * 64) void decode_f32_kernel(DecodeParams p)
   constexpr int RPI = 64 / CPR;            // B rows per load instruction
   constexpr int NLB = kRowsPerBlock / RPI; // load instructions per B tile
   constexpr int NDB = D / 32;
-  constexpr int TPQ = 4 / RK;              // tokens per 4-row group
+  constexpr int NTOK = RK <= 4 ? 16 / RK : 32 / RK;  // tokens whose rows this lane holds, per block
+  constexpr int NV = RK <= 4 ? RK : RK / 2;          // rows of one token held by this half of the wave
   constexpr int RS = DecodeF32Lds<D>::RS;
-  static_assert(RK == 1 || RK == 2 || RK == 4, "rank must divide 4");
+  static_assert(RK == 1 || RK == 2 || RK == 4 || RK == 8 || RK == 16 || RK == 32, "a block of 32 rows holds whole tokens");
   typedef __attribute__((ext_vector_type(NDB))) float f32xN;
 
   extern __shared__ __attribute__((aligned(16))) float smem_dec_f32[];
@@ -456,21 +458,23 @@ __global__ __launch_bounds__(kWaves * 64) void decode_f32_kernel(DecodeParams p)
     for (int v = 0; v < 16; ++v) sp[v] += sp2[v];
 
     // ---- logits per token (log2 domain), masked past the end of the cache
-    float st[4 * TPQ];
+    // (a token's RK rows are registers v0 .. v0 + NV - 1; from rank 8 on they span both halves of
+    // the wave, which then hold the same tokens and exchange their partial sums)
+    float st[NTOK];
     float tmax = -INFINITY;
     const int row0 = blk * kRowsPerBlock;
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
+    for (int t = 0; t < NTOK; ++t) {
+      const int v0 = t * NV;
+      float acc = 0.f;
 #pragma unroll
-      for (int e = 0; e < TPQ; ++e) {
-        float acc = 0.f;
-#pragma unroll
-        for (int j = 0; j < RK; ++j) acc += ak[4 * q + e * RK + j] * sp[4 * q + e * RK + j];
-        const int row = row0 + 8 * q + 4 * g + e * RK;
-        if (row > last_row) acc = -INFINITY;
-        st[q * TPQ + e] = acc;
-        tmax = fmaxf(tmax, acc);
-      }
+      for (int j = 0; j < NV; ++j) acc += ak[v0 + j] * sp[v0 + j];
+      if constexpr (RK >= 8) acc = halves_sum(acc);
+      const int row = RK >= 8 ? row0 + RK * t : row0 + 8 * (v0 >> 2) + 4 * g + (v0 & 3);  // the token's first row
+      if (row > last_row) acc = -INFINITY;
+      st[t] = acc;
+      tmax = fmaxf(tmax, acc);
+    }
     tmax = halves_max(tmax);
     const float m_new = fmaxf(m, tmax);  // finite: row0 itself is always inside the cache
     if (__any(m_new > m)) {
@@ -486,14 +490,12 @@ __global__ __launch_bounds__(kWaves * 64) void decode_f32_kernel(DecodeParams p)
     // ---- P'^T[row, h] = p[h, token(row)] * a_v[row, h], in place of the logits' registers
     float pp[16];
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
+    for (int t = 0; t < NTOK; ++t) {
+      const float pt = __builtin_amdgcn_exp2f(st[t] - m);
+      lsum += RK >= 8 ? 0.5f * pt : pt;  // both halves hold the token: each adds half of it
 #pragma unroll
-      for (int e = 0; e < TPQ; ++e) {
-        const float pt = __builtin_amdgcn_exp2f(st[q * TPQ + e] - m);
-        lsum += pt;
-#pragma unroll
-        for (int j = 0; j < RK; ++j) pp[4 * q + e * RK + j] = pt * av[4 * q + e * RK + j];
-      }
+      for (int j = 0; j < NV; ++j) pp[t * NV + j] = pt * av[t * NV + j];
+    }
 
     // ---- O^T[d, h] += sum_row B_v[row, d] P'^T[row, h]
 #pragma unroll
@@ -689,7 +691,7 @@ int tpa_decode_mfma_supported(const TpaFwdArgs* a) {
   using namespace tpa;
   if (a->dtype != TPA_DTYPE_BF16) return 0;
   if (a->dk != a->dv || (a->dk != 64 && a->dk != 128)) return 0;
-  if (a->rk != 1 && a->rk != 2 && a->rk != 4) return 0;
+  if (a->rk != 1 && a->rk != 2 && a->rk != 4 && a->rk != 8 && a->rk != 16 && a->rk != 32) return 0;
   if (a->H % 8 != 0) return 0;
   if (a->lq > 64) return 0;
   if (a->causal || a->q_segment_ids || a->kv_segment_ids) return 0;
@@ -710,20 +712,30 @@ int tpa_decode_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
   if (!a->workspace || a->workspace_bytes < workspace_bytes(a->B, a->lq, a->H, a->dv, S)) return TPA_ERR_WORKSPACE;
   if (!aligned16(a->workspace)) return TPA_ERR_ALIGN;
   if (a->dk == 128) {
-    if (a->rk == 1) return launch_decode<128, 1>(a, S, stream);
-    if (a->rk == 2) return launch_decode<128, 2>(a, S, stream);
-    return launch_decode<128, 4>(a, S, stream);
+    switch (a->rk) {
+      case 1: return launch_decode<128, 1>(a, S, stream);
+      case 2: return launch_decode<128, 2>(a, S, stream);
+      case 4: return launch_decode<128, 4>(a, S, stream);
+      case 8: return launch_decode<128, 8>(a, S, stream);
+      case 16: return launch_decode<128, 16>(a, S, stream);
+      default: return launch_decode<128, 32>(a, S, stream);
+    }
   }
-  if (a->rk == 1) return launch_decode<64, 1>(a, S, stream);
-  if (a->rk == 2) return launch_decode<64, 2>(a, S, stream);
-  return launch_decode<64, 4>(a, S, stream);
+  switch (a->rk) {
+    case 1: return launch_decode<64, 1>(a, S, stream);
+    case 2: return launch_decode<64, 2>(a, S, stream);
+    case 4: return launch_decode<64, 4>(a, S, stream);
+    case 8: return launch_decode<64, 8>(a, S, stream);
+    case 16: return launch_decode<64, 16>(a, S, stream);
+    default: return launch_decode<64, 32>(a, S, stream);
+  }
 }
 
 int tpa_decode_f32_supported(const TpaFwdArgs* a) {
   using namespace tpa;
   if (a->dtype != TPA_DTYPE_F32) return 0;
   if (a->dk != a->dv || (a->dk != 64 && a->dk != 128)) return 0;
-  if (a->rk != 1 && a->rk != 2 && a->rk != 4) return 0;
+  if (a->rk != 1 && a->rk != 2 && a->rk != 4 && a->rk != 8 && a->rk != 16 && a->rk != 32) return 0;
   if (a->lq > 64) return 0;
   if (a->causal || a->q_segment_ids || a->kv_segment_ids || a->page_table) return 0;
   // rows (token, rank) must be uniformly strided: stride_l == rk * stride_r; B rows are read as 16-byte vectors
@@ -743,11 +755,21 @@ int tpa_decode_f32_launch(const TpaFwdArgs* a, hipStream_t stream) {
   if (!a->workspace || a->workspace_bytes < workspace_bytes(a->B, a->lq, a->H, a->dv, S)) return TPA_ERR_WORKSPACE;
   if (!aligned16(a->workspace)) return TPA_ERR_ALIGN;
   if (a->dk == 128) {
-    if (a->rk == 1) return launch_decode_f32<128, 1>(a, S, stream);
-    if (a->rk == 2) return launch_decode_f32<128, 2>(a, S, stream);
-    return launch_decode_f32<128, 4>(a, S, stream);
+    switch (a->rk) {
+      case 1: return launch_decode_f32<128, 1>(a, S, stream);
+      case 2: return launch_decode_f32<128, 2>(a, S, stream);
+      case 4: return launch_decode_f32<128, 4>(a, S, stream);
+      case 8: return launch_decode_f32<128, 8>(a, S, stream);
+      case 16: return launch_decode_f32<128, 16>(a, S, stream);
+      default: return launch_decode_f32<128, 32>(a, S, stream);
+    }
   }
-  if (a->rk == 1) return launch_decode_f32<64, 1>(a, S, stream);
-  if (a->rk == 2) return launch_decode_f32<64, 2>(a, S, stream);
-  return launch_decode_f32<64, 4>(a, S, stream);
+  switch (a->rk) {
+    case 1: return launch_decode_f32<64, 1>(a, S, stream);
+    case 2: return launch_decode_f32<64, 2>(a, S, stream);
+    case 4: return launch_decode_f32<64, 4>(a, S, stream);
+    case 8: return launch_decode_f32<64, 8>(a, S, stream);
+    case 16: return launch_decode_f32<64, 16>(a, S, stream);
+    default: return launch_decode_f32<64, 32>(a, S, stream);
+  }
 }

@@ -254,6 +254,22 @@ def test_decode_bf16_mfma(gpu, d, b, lq, lk, h, rq, rk):
     check(o, lse, o_ref, l_ref, BF16_TOL)
 
 
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("d,rk,h,lk", [(64, 8, 64, 2048), (128, 8, 32, 1001), (128, 16, 16, 515), (64, 32, 8, 300)])
+def test_decode_high_ranks(gpu, dt, d, rk, h, lk):
+    """Ranks 8, 16, 32 (the high-rank configuration caches rank 8): a token's rows span both halves of
+    a wave in the split-key kernels.  lk = 1001 / 515 / 300 end inside a block."""
+    from tpa import tpa
+
+    b = 2
+    q, k, v = make_factors(110 + rk, b, 1, lk, h, d, d, 16, rk, scale_by_rank=True)
+    tq, tk, tv = (to_gpu(x, dt, gpu) for x in (q, k, v))
+    lengths = torch.tensor([lk, lk - rk - 3], dtype=torch.int32)
+    o, lse = tpa.tpa_decode(*split(tq, tk, tv, h), sm_scale=d**-0.5, kv_lengths=lengths, kernel=2)
+    o_ref, l_ref = _varlen_reference(as_f64(tq), as_f64(tk), as_f64(tv), lengths.tolist(), h, d**-0.5, False)
+    check(o, lse, o_ref, l_ref, BF16_TOL if dt == torch.bfloat16 else F32_TOL)
+
+
 def test_decode_sharp_softmax_and_split_invariance(gpu):
     b, lk, h, d = 2, 2048, 32, 128
     q, k, v = make_factors(8, b, 1, lk, h, d, d, 6, 2)
