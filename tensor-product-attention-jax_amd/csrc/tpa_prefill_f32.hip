@@ -256,7 +256,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_f32_kernel(F32Params pp) {
   // middle of it, so the SIMD always has a wave with matrix work and both end the tile together.
   const bool rebuild_first = w < kNW / 2;
   for (int j = 0; j < ntiles; ++j) {
-    const bool more = j + 1 < ntiles, mine = j <= wave_last_tile;
+    const bool more = j + 1 < ntiles, mine = j <= wave_last_tile && wrow0 < p.lq;  // waves past the last row only help rebuild
     if (rebuild_first && more) rebuild(j + 1);
     if (mine) logits_softmax(j);
     if (!rebuild_first && more) rebuild(j + 1);
@@ -299,17 +299,12 @@ bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15)
 bool rows_ok(const TpaFactor& f) {  // rows of 4-float vectors
   return aligned16(f.ptr) && f.stride_b % 4 == 0 && f.stride_l % 4 == 0 && f.stride_r % 4 == 0;
 }
-// The kernel spends a 256-row block on every (batch, head) however few rows there are; below this
-// many query rows the vector-ALU kernel, which spreads the keys instead, is the better one.
-constexpr int kMinRows = 64;
-
 }  // namespace
 }  // namespace tpa
 
 int tpa_prefill_f32_supported(const TpaFwdArgs* a) {
   if (a->dtype != TPA_DTYPE_F32) return 0;
   if (a->dk != a->dv || (a->dk != 64 && a->dk != 128)) return 0;
-  if (a->lq < tpa::kMinRows) return 0;
   if (!tpa::rows_ok(a->qb) || !tpa::rows_ok(a->kb) || !tpa::rows_ok(a->vb) || !tpa::aligned16(a->o)) return 0;
   return 1;
 }
@@ -331,7 +326,6 @@ int mha_prefill_f32_supported(const MhaFwdArgs* a) {
   if (a->dtype != TPA_DTYPE_F32) return 0;
   if (a->dk != a->dv || (a->dk != 64 && a->dk != 128)) return 0;
   if (a->bias) return 0;
-  if (a->lq < tpa::kMinRows) return 0;
   if (!tpa::aligned16(a->q) || !tpa::aligned16(a->k) || !tpa::aligned16(a->v) || !tpa::aligned16(a->o)) return 0;
   return 1;
 }

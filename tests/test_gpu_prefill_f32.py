@@ -125,13 +125,19 @@ def test_mha_f32_mfma_vs_oracle(gpu, d, causal):
     check(o, lse, o_ref, l_ref, F32_TOL)
 
 
-def test_f32_mfma_refuses_what_it_cannot_run(gpu):
+def test_f32_mfma_few_query_rows_and_refusals(gpu):
     from tpa import _dispatch as dsp
     from tpa import tpa
 
-    # too few query rows for a 256-row block per head: the vector-ALU kernel serves these, and an
-    # explicit request for the matrix-core kernel is an error
-    q, k, v = make_factors(18, 1, 8, 512, 2, 64, 64, 2, 2)
+    # a handful of query rows over a short cache (no decode route below 1024 keys): still the
+    # matrix-core kernel, whose waves without rows only help rebuild the tiles
+    q, k, v = make_factors(18, 2, 3, 500, 2, 64, 64, 2, 2)
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, 2), sm_scale=0.125, kernel=2, use_workspace=False)
+    o_ref, l_ref = orc.tpa_reference(q, k, v, None, None, 2, sm_scale=0.125)
+    check(o, lse, o_ref, l_ref, F32_TOL)
+    # a head size the matrix-core kernels do not take: explicit request refused, default falls back
+    q, k, v = make_factors(19, 1, 70, 90, 2, 32, 32, 2, 2)
     tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
     with pytest.raises(dsp.TpaError) as e:
         tpa.tpa_factors(*split(tq, tk, tv, 2), sm_scale=0.125, kernel=2)
