@@ -222,3 +222,36 @@ def test_tpa_entry_point_serves_fp32_decode_with_the_split_key_kernel(gpu):
     assert torch.equal(o, o2)
     o_ref, _ = orc.tpa_reference(q, k, v, None, None, h, sm_scale=d**-0.5)
     assert np.abs(as_f64(o) - o_ref).max() <= F32_TOL
+
+
+# ---------------------------------------------------------------- random problems
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_f32_mfma_forward_and_backward(gpu, seed):
+    """Random problems the fp32 matrix-core kernels take, forward and backward (kernel=2 makes a
+    silent fallback an error): any lengths, head counts, ranks, masks."""
+    from tpa import tpa
+
+    rng = np.random.default_rng(7000 + seed)
+    b, lq, lk = int(rng.integers(1, 4)), int(rng.integers(64, 700)), int(rng.integers(64, 700))
+    h, d = int(rng.integers(1, 6)), int(rng.choice([64, 128]))
+    rq, rk = int(rng.integers(1, 7)), int(rng.integers(1, 6))
+    causal = bool(rng.integers(0, 2))
+    seg = int(rng.integers(20, 400)) if rng.integers(0, 3) == 0 else None
+    q, k, v = make_factors(8000 + seed, b, lq, lk, h, d, d, rq, rk)
+    do = rng.standard_normal((b, lq, h, d)).astype(np.float32)
+    qseg = segment_ids(lq, seg, b) if seg else None
+    kvseg = segment_ids(lk, seg, b) if seg else None
+    tq, tk, tv, tdo = (to_gpu(x, torch.float32, gpu) for x in (q, k, v, do))
+    tqs = torch.from_numpy(qseg).to(gpu) if seg else None
+    tks = torch.from_numpy(kvseg).to(gpu) if seg else None
+    # the head factors sit at 4 h bytes into a row: split copies keep the B factors 16-byte aligned
+    parts = split(tq, tk, tv, h)
+    o, lse = tpa.tpa_factors(*parts, tqs, tks, d**-0.5, causal, 2)
+    o_ref, l_ref = orc.tpa_reference(q, k, v, qseg, kvseg, h, sm_scale=d**-0.5, causal=causal)
+    check(o, lse, o_ref, l_ref, F32_TOL)
+    grads = tpa.tpa_factors_bwd(*parts, tqs, tks, o, lse, tdo, d**-0.5, causal, kernel=2)
+    want = orc.tpa_backward(q, k, v, qseg, kvseg, h, do, sm_scale=d**-0.5, causal=causal)
+    for n, w in enumerate(want):
+        g = np.concatenate([x.cpu().numpy() for x in grads[2 * n : 2 * n + 2]], axis=-1).astype(np.float64)
+        assert np.isfinite(g).all()
+        assert np.max(np.abs(g - w)) <= 2e-4 * max(1e-30, np.max(np.abs(w))), "qkv"[n]
