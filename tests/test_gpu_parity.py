@@ -798,3 +798,51 @@ def test_paged_cache_is_refused_where_no_kernel_reads_it(gpu):
         tpa.tpa_decode(qa.float(), qb.float(), ka.reshape(3, 24, 2, 8).float(), kb.reshape(3, 24, 2, 64).float(),
                        va.reshape(3, 24, 2, 8).float(), vb.reshape(3, 24, 2, 64).float(), page_table=table)
     assert e.value.code == -6
+
+
+# ---------------------------------------------------------------- few query rows through the vector-ALU kernels
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("seg", [None, 137])
+@pytest.mark.parametrize("b,lq,lk,h,dk,dv,rq,rk", [(2, 3, 1500, 3, 20, 12, 3, 3), (1, 1, 2600, 5, 96, 96, 6, 2), (2, 16, 300, 2, 256, 40, 2, 1)])
+def test_few_rows_over_many_keys_any_head_size(gpu, dt, causal, seg, b, lq, lk, h, dk, dv, rq, rk):
+    """A decode the matrix-core kernels do not take (head sizes, masks, rank 3): the vector-ALU
+    kernel that spreads the keys of one query row over a workgroup."""
+    from tpa import tpa
+
+    q, k, v = make_factors(120, b, lq, lk, h, dk, dv, rq, rk, scale_by_rank=True)
+    qseg = segment_ids(lq, seg, b) if seg else None
+    kvseg = segment_ids(lk, seg, b) if seg else None
+    lengths = [lk - 7 * i for i in range(b)]
+    tq, tk, tv = (to_gpu(x, dt, gpu) for x in (q, k, v))
+    for bi, n in enumerate(lengths):
+        tk[bi, n:] = float("nan")
+        tv[bi, n:] = float("nan")
+    tqs = torch.from_numpy(qseg).to(gpu) if seg else None
+    tks = torch.from_numpy(kvseg).to(gpu) if seg else None
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), tqs, tks, dk**-0.5, causal, kv_lengths=lengths)
+    os_, ls_ = [], []
+    for bi, n in enumerate(lengths):  # the oracle on the first lengths[b] keys of each entry
+        o1, l1 = orc.tpa_reference(as_f64(tq[bi : bi + 1]), as_f64(tk[bi : bi + 1, :n]), as_f64(tv[bi : bi + 1, :n]),
+                                   None if qseg is None else qseg[bi : bi + 1], None if kvseg is None else kvseg[bi : bi + 1, :n],
+                                   h, sm_scale=dk**-0.5, causal=causal)
+        os_.append(o1)
+        ls_.append(l1)
+    check(o, lse, np.concatenate(os_), np.concatenate(ls_), BF16_TOL if dt == torch.bfloat16 else F32_TOL)
+
+
+def test_mha_few_rows_with_bias(gpu):
+    """Dense attention with an additive bias (tpa/mha.py:23-37), two query rows over 700 keys."""
+    from tpa.mha import _mha_fwd
+
+    rng = np.random.Generator(np.random.Philox(121))
+    b, lq, lk, h, dk, dv = 2, 2, 700, 3, 24, 40
+    q = rng.standard_normal((b, lq, h, dk), dtype=np.float32)
+    k = rng.standard_normal((b, lk, h, dk), dtype=np.float32)
+    v = rng.standard_normal((b, lk, h, dv), dtype=np.float32)
+    bias = rng.standard_normal((b, lq, lk), dtype=np.float32)
+    bias[rng.random((b, lq, lk)) < 0.3] = -np.inf
+    bias[1, 1] = -np.inf  # one empty row
+    o_ref, l_ref = orc.mha_forward(q.astype(np.float64), k.astype(np.float64), v.astype(np.float64), bias.astype(np.float64), 0.5)
+    o, (lse, *_) = _mha_fwd(torch.from_numpy(q).to(gpu), torch.from_numpy(k).to(gpu), torch.from_numpy(v).to(gpu), bias, 0.5)
+    check(o, lse, o_ref, l_ref, F32_TOL)
