@@ -847,8 +847,12 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   // ---- epilogue: normalise, store O[b, qrow, h, :] and LSE[b, h, qrow]
   const float ltot = halves_sum(lsum);
   const float inv = 1.f / ltot;
-  if (qrow < p.lq) {
-    uint16_t* op = p.o + (((int64_t)b * p.lq + qrow) * p.H + h) * D;
+  // The wave's 32 output rows go through its own slice of LDS (free after the last barrier), so
+  // that they leave as whole 16-byte chunks of whole rows instead of 8-byte pieces of 32 rows.
+  {
+    constexpr int OS = D + 8;  // row stride (elements)
+    uint16_t* const ot = smem + w * 32 * OS;
+    static_assert(kNW * 32 * OS * sizeof(uint16_t) <= Lds<D>::kBytes, "output staging fits");
 #pragma unroll
     for (int db = 0; db < NDB; ++db)
 #pragma unroll
@@ -856,10 +860,20 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
         u32x2 pk;
         pk[0] = pack_bf16(o[db][4 * vq] * inv, o[db][4 * vq + 1] * inv);
         pk[1] = pack_bf16(o[db][4 * vq + 2] * inv, o[db][4 * vq + 3] * inv);
-        *reinterpret_cast<u32x2*>(op + 32 * db + 8 * vq + 4 * g) = pk;
+        *reinterpret_cast<u32x2*>(ot + i * OS + 32 * db + 8 * vq + 4 * g) = pk;
       }
-    if (p.lse && g == 0) p.lse[((int64_t)b * p.H + h) * p.lq + qrow] = (mref + __builtin_amdgcn_logf(ltot)) * kLn2;
+    __builtin_amdgcn_wave_barrier();
+    constexpr int CPRO = D / 8, RPI = 64 / CPRO;  // 16-byte chunks per row, rows per store instruction
+    const int orow_l = l / CPRO, ochunk = l % CPRO;
+#pragma unroll
+    for (int n = 0; n < 32 / RPI; ++n) {
+      const int r = n * RPI + orow_l;
+      const u32x4 val = *reinterpret_cast<const u32x4*>(ot + r * OS + 8 * ochunk);
+      if (wrow0 + r < p.lq)
+        *reinterpret_cast<u32x4*>(p.o + (((int64_t)b * p.lq + wrow0 + r) * p.H + h) * D + 8 * ochunk) = val;
+    }
   }
+  if (qrow < p.lq && p.lse && g == 0) p.lse[((int64_t)b * p.H + h) * p.lq + qrow] = (mref + __builtin_amdgcn_logf(ltot)) * kLn2;
 }
 
 template <int D, int LOADER, bool SEG = false>
