@@ -44,9 +44,12 @@ struct BwdLds {
 };
 
 // which (block, batch, head): heads of one (block, batch) pair on one XCD, pairs in launch order
+// (the eight pairs of a round go to the XCDs in alternating direction, so that no XCD collects the
+// heaviest pair of every round)
 __device__ __forceinline__ bool decode_block(int npairs, int H, int& pair, int& h) {
   const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
-  pair = (slot / H) * 8 + xcd;
+  const int round = slot / H;
+  pair = round * 8 + ((round & 1) ? 7 - xcd : xcd);  // alternating direction: every XCD gets the same load
   h = slot % H;
   return pair < npairs;
 }
