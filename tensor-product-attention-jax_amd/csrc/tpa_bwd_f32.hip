@@ -44,12 +44,10 @@ struct BwdLds {
 };
 
 // which (block, batch, head): heads of one (block, batch) pair on one XCD, pairs in launch order
-// (the eight pairs of a round go to the XCDs in alternating direction, so that no XCD collects the
-// heaviest pair of every round)
-__device__ __forceinline__ bool decode_block(int npairs, int H, int& pair, int& h) {
+__device__ __forceinline__ bool decode_block(int npairs, int H, int B, int& pair, int& h) {
   const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
   const int round = slot / H;
-  pair = round * 8 + ((round & 1) ? 7 - xcd : xcd);  // alternating direction: every XCD gets the same load
+  pair = round * 8 + xcd_pair_slot(round, xcd, B);
   h = slot % H;
   return pair < npairs;
 }
@@ -156,7 +154,7 @@ __global__ __launch_bounds__(kThreads) void bwd_f32_dq_kernel(BwdF32Params p) {
   int32_t* const lds_seg = reinterpret_cast<int32_t*>(smem_bwd_f32 + 4 * kMat);  // [2][kTile] key segment ids
 
   int pair, h;
-  if (!decode_block(p.npairs, p.H, pair, h)) return;
+  if (!decode_block(p.npairs, p.H, p.B, pair, h)) return;
   const int blk = p.nblk - 1 - pair / p.B;  // heaviest causal blocks first
   const int b = pair % p.B;
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
@@ -250,7 +248,7 @@ __global__ __launch_bounds__(kThreads) void bwd_f32_dkv_kernel(BwdF32Params p) {
   float* const lds_row = smem_bwd_f32 + 4 * kMat;  // [2][lse2 | delta | segment id][kTile]
 
   int pair, h;
-  if (!decode_block(p.npairs, p.H, pair, h)) return;
+  if (!decode_block(p.npairs, p.H, p.B, pair, h)) return;
   const int blk = pair / p.B;  // under the causal mask the first key blocks see the most rows: heaviest first
   const int b = pair % p.B;
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;

@@ -153,7 +153,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(BwdParams p) {
 
   const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
   const int round = slot / p.H, h = slot % p.H;
-  const int pair = round * 8 + ((round & 1) ? 7 - xcd : xcd);  // alternating direction: every XCD gets the same load
+  const int pair = round * 8 + xcd_pair_slot(round, xcd, p.B);
   if (pair >= p.npairs) return;
   const int qblk = p.nblk - 1 - pair / p.B, b = pair % p.B;  // heaviest causal blocks first
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
@@ -345,7 +345,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
 
   const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
   const int round = slot / p.H, h = slot % p.H;
-  const int pair = round * 8 + ((round & 1) ? 7 - xcd : xcd);  // alternating direction: every XCD gets the same load
+  const int pair = round * 8 + xcd_pair_slot(round, xcd, p.B);
   if (pair >= p.npairs) return;
   const int kblk = pair / p.B, b = pair % p.B;  // under the causal mask the first key blocks are the heaviest
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;

@@ -111,6 +111,18 @@ __device__ __forceinline__ void build_q_fragments(const uint16_t* ap, int64_t a_
   }
 }
 
+// Which of the eight (block, batch) pairs of round `round` the workgroups on XCD `xcd` take, with
+// pair = block_rank * B + batch.  Workgroup ids map to XCDs statically, so with a fixed direction
+// one XCD would collect the heaviest causal block of every round; odd rounds therefore reverse the
+// order of the blocks.  Where B divides 8 only the block rank is reversed and the batch entry is
+// kept, so that an XCD keeps meeting the same batch entries (their K/V factors stay in its L2);
+// where B is a multiple of 8 a round holds one block rank only and nothing needs to move.
+__device__ __forceinline__ int xcd_pair_slot(int round, int xcd, int B) {
+  if (!(round & 1) || B % 8 == 0) return xcd;
+  if (8 % B == 0) return (8 / B - 1 - xcd / B) * B + xcd % B;
+  return 7 - xcd;
+}
+
 // Raise a kernel's dynamic LDS limit above the 64 KB a kernel gets without asking.  The attribute
 // belongs to one device's copy of the code, so it is set once per device (`done` is the calling
 // launcher's own table; a race between two first launches only repeats the same call).

@@ -113,10 +113,8 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   // that XCD's L2; pairs are ordered heaviest (last causal block) first.
   const int id = blockIdx.x;
   const int xcd = id & 7, slot = id >> 3;
-  // (the eight pairs of a round are dealt to the XCDs in alternating direction: with a fixed
-  // direction XCD 0 would get the heaviest pair of every round and XCD 7 the lightest)
   const int round = slot / p.H;
-  const int pair = round * 8 + ((round & 1) ? 7 - xcd : xcd);
+  const int pair = round * 8 + xcd_pair_slot(round, xcd, p.B);
   const int h = slot % p.H;
   if (pair >= p.npairs) return;
   const int qblk = p.nqb - 1 - pair / p.B;

@@ -73,7 +73,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_f32_kernel(F32Params pp) {
   const int id = blockIdx.x;
   const int xcd = id & 7, slot = id >> 3;
   const int round = slot / p.H;
-  const int pair = round * 8 + ((round & 1) ? 7 - xcd : xcd);  // alternating direction: every XCD gets the same load
+  const int pair = round * 8 + xcd_pair_slot(round, xcd, p.B);
   const int h = slot % p.H;
   if (pair >= p.npairs) return;
   const int qblk = p.nqb - 1 - pair / p.B;
