@@ -59,7 +59,7 @@ COPY_BYTES = 1 << 30  # --workload copy: bytes read (and bytes written) by each 
 # the same counter reads for the 1 GiB copy of `--workload copy`; None where no counter run exists.
 # FETCH_SIZE reads 0.5 KiB per KiB the copy fetches (scale 2.0), WRITE_SIZE 1.0 per KiB (scale 1.0).
 MEASURED_TRAFFIC = {
-    "c2": (2.0 * 56729.0 + 1.0 * 66560.0) * 1024,                     # prefill_kernel<128,0,false>
+    "c2": (2.0 * 56386.7 + 1.0 * 66560.0) * 1024,                     # prefill_kernel<128,0,false>
     "c4": (2.0 * (328100.3 + 2135.5) + 1.0 * (4160.0 + 520.0)) * 1024,  # decode_kernel + decode_merge_kernel
 }
 
