@@ -209,18 +209,18 @@ const char* tpa_strerror(int code);
  * tpa/tpa.py:492-543 for all batch entries at once (the reference vmaps it, tpa/tpa.py:144-163).
  * If `workspace` holds at least tpa_decode_workspace_bytes(...) bytes and the problem is a
  * decode (lq <= 16, lk >= 1024, no mask) that tpa_decode's kernel takes, the call is served by
- * it; if the rank of k, v is not 2 and `workspace` holds tpa_fwd_workspace_bytes(...) bytes, K and
- * V are reconstructed into it once.  Without a workspace the same problems run on the fused
- * prefill kernel.
+ * it; if the rank of k, v is not 2 (or the sequence is long, 16384 rows and more) and `workspace`
+ * holds tpa_fwd_workspace_bytes(...) bytes, K and V are reconstructed into it once.  Without a
+ * workspace the same problems run on the fused prefill kernel.
  */
 int tpa_fwd(const TpaFwdArgs* args, void* stream);
 
 /*
  * Bytes of optional workspace (256-byte aligned) with which tpa_fwd can pick a faster kernel for
  * this problem, 0 if none would be used: the split partials of the decode kernel (lq <= 16 over
- * a long cache), or room for dense bf16 K and V when the rank of k and v is not 2 - then K and V
- * are reconstructed once (tpa/tpa.py:364,417 do it per query block) and the flash kernel runs
- * with its plain tile loader.
+ * a long cache), or room for dense bf16 K and V when the rank of k and v is not 2 or there are
+ * 16384 query rows and more - then K and V are reconstructed once (tpa/tpa.py:364,417 do it per
+ * query block) and the flash kernel runs with its plain tile loader.
  */
 size_t tpa_fwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dk, int32_t dv, int32_t rq, int32_t rk);
 

@@ -922,6 +922,15 @@ size_t tpa_prefill_dense_kv_bytes(int64_t B, int64_t lk, int64_t H, int64_t D) {
   return (size_t)(2 * ((B * lk * H * D * 2 + 255) / 256 * 256));
 }
 
+// Whether reconstructing dense K and V once (two HBM-bound launches) and running the plain tile
+// loader beats rebuilding every tile in the flash loop.  Ranks other than 2: from the second
+// query block on (the loop over ranks has no tuned rebuild).  Rank 2: the tuned rebuild costs the
+// loop about 9 % and the reconstruction grows with the length only, so it pays for long sequences.
+int tpa_prefill_wants_dense_kv(int64_t lq, int64_t rk) {
+  if (rk != 2) return lq > tpa::kBQ;
+  return lq >= 16384;
+}
+
 int tpa_prefill_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
   using namespace tpa;
   PrefillParams p{};
@@ -936,7 +945,7 @@ int tpa_prefill_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
   // head from all ranks again (once per 256 query rows).  With a workspace the dense K and V are
   // built once and the kernel runs with its plain tile loader, Q still coming from its factors.
   const size_t dense_bytes = tpa_prefill_dense_kv_bytes(a->B, a->lk, a->H, a->dk);
-  if (a->rk != 2 && a->lq > kBQ && a->workspace && dense_bytes && a->workspace_bytes >= dense_bytes &&
+  if (tpa_prefill_wants_dense_kv(a->lq, a->rk) && a->workspace && dense_bytes && a->workspace_bytes >= dense_bytes &&
       !(reinterpret_cast<uintptr_t>(a->workspace) & 255)) {
     uint16_t* kd = static_cast<uint16_t*>(a->workspace);
     uint16_t* vd = kd + dense_bytes / 4;
