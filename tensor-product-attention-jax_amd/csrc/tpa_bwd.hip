@@ -40,33 +40,49 @@ __global__ void recon_kernel(TpaFactor fa, TpaFactor fb, TO* out, int L, int H, 
   }
 }
 
-// bf16 factors -> dense bf16, 8 elements per thread: the thread keeps its 16-byte piece of every
-// rank's b row and walks the heads.  Needs D % 8 == 0 and 16-byte aligned b rows.
-__global__ void recon_bf16_kernel(TpaFactor fa, TpaFactor fb, uint16_t* out, int L, int H, int D, int R) {
-  const int t = blockIdx.x, b = blockIdx.y;
-  const uint16_t* ap = static_cast<const uint16_t*>(fa.ptr) + b * fa.stride_b + t * fa.stride_l;
-  const uint16_t* bp = static_cast<const uint16_t*>(fb.ptr) + b * fb.stride_b + t * fb.stride_l;
-  uint16_t* op = out + ((int64_t)b * L + t) * H * D;
+// bf16 factors -> dense bf16, 8 elements per thread and token.  A workgroup takes kReconTokens
+// consecutive tokens and every thread works on the same (head, 16-byte piece) of all of them at
+// once, so that several independent load chains are in flight (one token per workgroup left the
+// kernel waiting for one small load after the other).  Needs D % 8 == 0 and 16-byte aligned b rows.
+constexpr int kReconTokens = 4;
+__global__ __launch_bounds__(256) void recon_bf16_kernel(TpaFactor fa, TpaFactor fb, uint16_t* out, int L, int H, int D, int R) {
+  const int t0 = blockIdx.x * kReconTokens, b = blockIdx.y;
+  const uint16_t* ap = static_cast<const uint16_t*>(fa.ptr) + b * fa.stride_b;
+  const uint16_t* bp = static_cast<const uint16_t*>(fb.ptr) + b * fb.stride_b;
   const float inv = 1.f / (float)R;
   const int cpr = D / 8;
   for (int idx = threadIdx.x; idx < H * cpr; idx += blockDim.x) {
     const int h = idx / cpr, cc = idx - h * cpr;
-    float acc[8];
+    float acc[kReconTokens][8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+    for (int u = 0; u < kReconTokens; ++u)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[u][j] = 0.f;
     for (int r = 0; r < R; ++r) {
-      const float av = bf16bits_to_f32(ap[r * fa.stride_r + h]);
-      const u32x4 bv = *reinterpret_cast<const u32x4*>(bp + r * fb.stride_r + 8 * cc);
+      float av[kReconTokens];
+      u32x4 bv[kReconTokens];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        acc[2 * j] += av * bf16lo_to_f32(bv[j]);
-        acc[2 * j + 1] += av * bf16hi_to_f32(bv[j]);
+      for (int u = 0; u < kReconTokens; ++u) {
+        const int64_t t = min(t0 + u, L - 1);
+        av[u] = bf16bits_to_f32(ap[t * fa.stride_l + r * fa.stride_r + h]);
+        bv[u] = *reinterpret_cast<const u32x4*>(bp + t * fb.stride_l + r * fb.stride_r + 8 * cc);
       }
-    }
-    u32x4 pk;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) pk[j] = pack_bf16(acc[2 * j] * inv, acc[2 * j + 1] * inv);
-    *reinterpret_cast<u32x4*>(op + h * D + 8 * cc) = pk;
+      for (int u = 0; u < kReconTokens; ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[u][2 * j] += av[u] * bf16lo_to_f32(bv[u][j]);
+          acc[u][2 * j + 1] += av[u] * bf16hi_to_f32(bv[u][j]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kReconTokens; ++u) {
+      if (t0 + u >= L) break;
+      u32x4 pk;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pk[j] = pack_bf16(acc[u][2 * j] * inv, acc[u][2 * j + 1] * inv);
+      *reinterpret_cast<u32x4*>(out + (((int64_t)b * L + t0 + u) * H + h) * D + 8 * cc) = pk;
+    }
   }
 }
 
@@ -440,7 +456,7 @@ int tpa_bwd_t(const TpaBwdArgs* a, hipStream_t stream, bool mfma) {
       const bool vec = sizeof(T) == 2 && !(reinterpret_cast<uintptr_t>(fb.ptr) & 15) && fb.stride_b % 8 == 0 && fb.stride_l % 8 == 0 &&
                        fb.stride_r % 8 == 0;
       if (vec)
-        hipLaunchKernelGGL(recon_bf16_kernel, dim3(L, a->B), dim3(threads), 0, stream, fa, fb, out, L, a->H, D, R);
+        hipLaunchKernelGGL(recon_bf16_kernel, dim3((L + kReconTokens - 1) / kReconTokens, a->B), dim3(threads), 0, stream, fa, fb, out, L, a->H, D, R);
       else
         hipLaunchKernelGGL((recon_kernel<T, uint16_t>), dim3(L, a->B), dim3(threads), 0, stream, fa, fb, out, L, a->H, D, R);
     };
@@ -533,7 +549,7 @@ int tpa_recon_dense_bf16(const TpaFactor* fa, const TpaFactor* fb, uint16_t* out
   const bool vec = D % 8 == 0 && !(reinterpret_cast<uintptr_t>(fb->ptr) & 15) && fb->stride_b % 8 == 0 && fb->stride_l % 8 == 0 &&
                    fb->stride_r % 8 == 0;
   if (vec)
-    hipLaunchKernelGGL(tpa::recon_bf16_kernel, dim3(L, B), dim3(256), 0, stream, *fa, *fb, out, L, H, D, R);
+    hipLaunchKernelGGL(tpa::recon_bf16_kernel, dim3((L + tpa::kReconTokens - 1) / tpa::kReconTokens, B), dim3(256), 0, stream, *fa, *fb, out, L, H, D, R);
   else
     hipLaunchKernelGGL((tpa::recon_kernel<uint16_t, uint16_t>), dim3(L, B), dim3(256), 0, stream, *fa, *fb, out, L, H, D, R);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
