@@ -69,6 +69,10 @@ __device__ __forceinline__ float dot2_bf16(uint32_t pair, uint32_t aa) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pair), __builtin_bit_cast(bf16x2, aa), 0.f, false);
 }
 
+__device__ __forceinline__ float dot2_bf16_acc(uint32_t pair, uint32_t aa, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pair), __builtin_bit_cast(bf16x2, aa), c, false);
+}
+
 // Workgroup barrier that waits for this wave's LDS traffic only.  __syncthreads() would also
 // wait for the global loads of the next tile's factors, which are meant to stay in flight.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
@@ -182,14 +186,18 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
         if (tid < kBQ) qas[tid] = (uint16_t)a_nxt;
         if (r + 1 < p.rq) load_rank(r + 1);
         lds_barrier();
-        const float a = bf16bits_to_f32(qas[32 * w + i]);
+        // a * b[d] for a packed pair (b[d], b[d+1]) is one dot instruction with (a, 0) or (0, a):
+        // no unpacking, and the dot unit is idle here anyway
+        const uint32_t a_lo = qas[32 * w + i], a_hi = a_lo << 16;
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
           const u32x4 bv = *reinterpret_cast<const u32x4*>(qs + (32 * w + i) * QS + 16 * ks + 8 * g);
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            acc[ks][2 * j] += a * bf16lo_to_f32(bv[j]);
-            acc[ks][2 * j + 1] += a * bf16hi_to_f32(bv[j]);
+            uint32_t pair = bv[j];
+            asm volatile("" : "+v"(pair));  // keeps the compiler from taking element 0 of the vector for every j
+            acc[ks][2 * j] = dot2_bf16_acc(pair, a_lo, acc[ks][2 * j]);
+            acc[ks][2 * j + 1] = dot2_bf16_acc(pair, a_hi, acc[ks][2 * j + 1]);
           }
         }
         lds_barrier();  // everyone has read this rank before the next one overwrites it
