@@ -341,7 +341,7 @@ struct DecodeF32Lds {
   static constexpr size_t kBytes = (size_t)kWaves * kPerWave * sizeof(float);
 };
 
-template <int D, int RK>
+template <int D, int RK, bool PAGED>
 __global__ __launch_bounds__(kWaves * 64) void decode_f32_kernel(DecodeParams p) {
   constexpr int CPR = D / 4;               // 16-byte chunks per B row
   constexpr int RPI = 64 / CPR;            // B rows per load instruction
@@ -375,10 +375,14 @@ __global__ __launch_bounds__(kWaves * 64) void decode_f32_kernel(DecodeParams p)
   const int blk_step = nparts;
   const int last_row = len_b * RK - 1;
 
-  const float* const kb_base = static_cast<const float*>(p.kb.ptr) + b * p.kb.stride_b;
-  const float* const vb_base = static_cast<const float*>(p.vb.ptr) + b * p.vb.stride_b;
-  const float* const ka_base = static_cast<const float*>(p.ka.ptr) + b * p.ka.stride_b + hl;
-  const float* const va_base = static_cast<const float*>(p.va.ptr) + b * p.va.stride_b + hl;
+  // (paged cache: the arrays are page pools, stride_b = elements between pages, and a block of 32
+  // rows lies inside one page, which the page table of this batch entry locates)
+  const int64_t boff = PAGED ? 0 : b;
+  const float* const kb_base = static_cast<const float*>(p.kb.ptr) + boff * p.kb.stride_b;
+  const float* const vb_base = static_cast<const float*>(p.vb.ptr) + boff * p.vb.stride_b;
+  const float* const ka_base = static_cast<const float*>(p.ka.ptr) + boff * p.ka.stride_b + hl;
+  const float* const va_base = static_cast<const float*>(p.va.ptr) + boff * p.va.stride_b + hl;
+  const int rpp = PAGED ? p.page_size * RK : 1;  // rows per page
   const int lb_row = l / CPR, lb_c = l % CPR;
 
   // one register set: the block after the one being consumed
@@ -386,18 +390,29 @@ __global__ __launch_bounds__(kWaves * 64) void decode_f32_kernel(DecodeParams p)
   float rak[16], rav[16];
   auto issue = [&](int blk) {
     const int row0 = blk * kRowsPerBlock;
+    // element offsets that take a logical row of this block to its place in the page pool
+    int64_t pkb = 0, pvb = 0, pka = 0, pva = 0;
+    if constexpr (PAGED) {
+      const int page = row0 / rpp;
+      const int64_t phys = p.page_table[(int64_t)b * p.pages_per_seq + page];
+      const int64_t first = (int64_t)page * rpp;  // first logical row of the page
+      pkb = phys * p.kb.stride_b - first * p.kb.stride_r;
+      pvb = phys * p.vb.stride_b - first * p.vb.stride_r;
+      pka = phys * p.ka.stride_b - first * p.ka.stride_r;
+      pva = phys * p.va.stride_b - first * p.va.stride_r;
+    }
 #pragma unroll
     for (int n = 0; n < NLB; ++n) {
       const int row = min(row0 + n * RPI + lb_row, last_row);
-      rbk[n] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(kb_base + (int64_t)row * p.kb.stride_r + 4 * lb_c));
-      rbv[n] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(vb_base + (int64_t)row * p.vb.stride_r + 4 * lb_c));
+      rbk[n] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(kb_base + pkb + (int64_t)row * p.kb.stride_r + 4 * lb_c));
+      rbv[n] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(vb_base + pvb + (int64_t)row * p.vb.stride_r + 4 * lb_c));
     }
     // a[row][head of this lane] for the 16 rows this lane's S'^T registers belong to
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int row = min(row0 + 8 * (v >> 2) + 4 * g + (v & 3), last_row);
-      rak[v] = ka_base[(int64_t)row * p.ka.stride_r];
-      rav[v] = va_base[(int64_t)row * p.va.stride_r];
+      rak[v] = ka_base[pka + (int64_t)row * p.ka.stride_r];
+      rav[v] = va_base[pva + (int64_t)row * p.va.stride_r];
     }
   };
   float ak[16], av[16];
@@ -626,8 +641,8 @@ int launch_decode_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
 }
 
-template <int D, int RK>
-int launch_decode_f32(const TpaFwdArgs* a, int S, hipStream_t stream) {
+template <int D, int RK, bool PAGED>
+int launch_decode_f32_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   DecodeParams p{};
   p.qa = a->qa; p.qb = a->qb; p.ka = a->ka; p.kb = a->kb; p.va = a->va; p.vb = a->vb;
   float* ws = static_cast<float*>(a->workspace);
@@ -635,8 +650,9 @@ int launch_decode_f32(const TpaFwdArgs* a, int S, hipStream_t stream) {
   p.part_o = ws; p.part_m = ws + no; p.part_l = ws + no + nm;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.S = S;
   p.kvlen = a->kv_lengths;
+  p.page_table = a->page_table; p.page_size = a->page_size; p.pages_per_seq = a->pages_per_seq;
   p.qscale = a->sm_scale * kLog2e / ((float)a->rq * (float)RK);
-  auto kern = decode_f32_kernel<D, RK>;
+  auto kern = decode_f32_kernel<D, RK, PAGED>;
   static bool configured[kMaxDevices] = {};
   if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), DecodeF32Lds<D>::kBytes); rc != TPA_OK) return rc;
   dim3 grid(a->B * S, a->lq, (a->H + 31) / 32);
@@ -645,6 +661,17 @@ int launch_decode_f32(const TpaFwdArgs* a, int S, hipStream_t stream) {
   hipLaunchKernelGGL((decode_merge_kernel<D, float>), dim3(a->B * a->lq, a->H), dim3(D), 0, stream, p.part_o, p.part_m, p.part_l,
                      static_cast<float*>(a->o), a->lse, S, a->H, a->lq, 1.f / (float)RK);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
+}
+
+template <int D, int RK>
+int launch_decode_f32(const TpaFwdArgs* a, int S, hipStream_t stream) {
+  if (a->page_table) {
+    if (a->page_size <= 0 || (a->page_size * RK) % kRowsPerBlock != 0 ||
+        (int64_t)a->pages_per_seq * a->page_size < a->lk)
+      return TPA_ERR_SHAPE;
+    return launch_decode_f32_t<D, RK, true>(a, S, stream);
+  }
+  return launch_decode_f32_t<D, RK, false>(a, S, stream);
 }
 
 template <int D, int RK>
@@ -737,7 +764,7 @@ int tpa_decode_f32_supported(const TpaFwdArgs* a) {
   if (a->dk != a->dv || (a->dk != 64 && a->dk != 128)) return 0;
   if (a->rk != 1 && a->rk != 2 && a->rk != 4 && a->rk != 8 && a->rk != 16 && a->rk != 32) return 0;
   if (a->lq > 64) return 0;
-  if (a->causal || a->q_segment_ids || a->kv_segment_ids || a->page_table) return 0;
+  if (a->causal || a->q_segment_ids || a->kv_segment_ids) return 0;
   // rows (token, rank) must be uniformly strided: stride_l == rk * stride_r; B rows are read as 16-byte vectors
   const TpaFactor* fs[4] = {&a->ka, &a->kb, &a->va, &a->vb};
   for (const TpaFactor* f : fs)

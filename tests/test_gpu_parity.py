@@ -751,7 +751,8 @@ def test_prefill_with_per_sequence_key_lengths(gpu, kernel, dt, causal):
 
 
 @pytest.mark.parametrize("d,rk,page_size", [(128, 2, 16), (128, 2, 256), (64, 4, 8), (64, 1, 32)])
-def test_decode_over_a_paged_cache(gpu, d, rk, page_size):
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
+def test_decode_over_a_paged_cache(gpu, dt, d, rk, page_size):
     """The same cache, once contiguous per sequence and once scattered over a shuffled page pool:
     the split-key kernel does the same arithmetic in the same order, so the results are equal
     bit for bit; the contiguous one is checked against the oracle."""
@@ -762,13 +763,13 @@ def test_decode_over_a_paged_cache(gpu, d, rk, page_size):
     lk = pages_per_seq * page_size
     lengths = [lk, lk - page_size - 3, 5]
     q, k, v = make_factors(111, b, 1, lk, h, d, d, 6, rk, scale_by_rank=True)
-    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    tq, tk, tv = (to_gpu(x, dt, gpu) for x in (q, k, v))
     kv_len = torch.tensor(lengths, dtype=torch.int32)
     o1, l1 = tpa.tpa_decode(*tpa_split(tq, tk, tv, h), sm_scale=d**-0.5, kv_lengths=kv_len, kernel=2)
     # scatter the pages of all sequences over a pool twice as large, in random order
     npages = 2 * b * pages_per_seq
     perm = torch.from_numpy(np.random.default_rng(112).permutation(npages)[: b * pages_per_seq].astype(np.int32)).reshape(b, pages_per_seq)
-    pool_k = torch.full((npages, page_size, rk, h + d), float("nan"), dtype=torch.bfloat16, device=gpu)
+    pool_k = torch.full((npages, page_size, rk, h + d), float("nan"), dtype=dt, device=gpu)
     pool_v = torch.full_like(pool_k, float("nan"))
     for bi in range(b):
         for pg in range(pages_per_seq):
@@ -779,7 +780,7 @@ def test_decode_over_a_paged_cache(gpu, d, rk, page_size):
                             pool_v[..., h:].contiguous(), sm_scale=d**-0.5, kv_lengths=kv_len, page_table=perm, kernel=2)
     assert torch.equal(o1, o2) and torch.equal(l1, l2)
     o_ref, l_ref = _varlen_reference(as_f64(tq), as_f64(tk), as_f64(tv), lengths, h, d**-0.5, False)
-    check(o1, l1, o_ref, l_ref, BF16_TOL)
+    check(o1, l1, o_ref, l_ref, BF16_TOL if dt == torch.bfloat16 else F32_TOL)
 
 
 def test_paged_cache_is_refused_where_no_kernel_reads_it(gpu):
@@ -794,9 +795,17 @@ def test_paged_cache_is_refused_where_no_kernel_reads_it(gpu):
         tpa.tpa_decode(qa, qb, ka.reshape(3, 24, 2, 8), kb.reshape(3, 24, 2, 64), va.reshape(3, 24, 2, 8),
                        vb.reshape(3, 24, 2, 64), page_table=table, kernel=2)
     assert e.value.code == -2
-    with pytest.raises(dd.TpaError) as e:  # the fp32 kernel does not read page pools
+    with pytest.raises(dd.TpaError) as e:  # the same through the fp32 split-key kernel
         tpa.tpa_decode(qa.float(), qb.float(), ka.reshape(3, 24, 2, 8).float(), kb.reshape(3, 24, 2, 64).float(),
                        va.reshape(3, 24, 2, 8).float(), vb.reshape(3, 24, 2, 64).float(), page_table=table)
+    assert e.value.code == -2
+    # a head size only the vector-ALU kernel takes: it does not read page pools
+    q, k, v = make_factors(114, 1, 1, 64, 8, 32, 32, 2, 2)
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    qa, qb, ka, kb, va, vb = tpa_split(tq, tk, tv, 8)
+    with pytest.raises(dd.TpaError) as e:
+        tpa.tpa_decode(qa, qb, ka.reshape(2, 32, 2, 8), kb.reshape(2, 32, 2, 32), va.reshape(2, 32, 2, 8),
+                       vb.reshape(2, 32, 2, 32), page_table=torch.tensor([[0, 1]], dtype=torch.int32))
     assert e.value.code == -6
 
 
