@@ -855,3 +855,42 @@ def test_mha_few_rows_with_bias(gpu):
     o_ref, l_ref = orc.mha_forward(q.astype(np.float64), k.astype(np.float64), v.astype(np.float64), bias.astype(np.float64), 0.5)
     o, (lse, *_) = _mha_fwd(torch.from_numpy(q).to(gpu), torch.from_numpy(k).to(gpu), torch.from_numpy(v).to(gpu), bias, 0.5)
     check(o, lse, o_ref, l_ref, F32_TOL)
+
+
+# ---------------------------------------------------------------- the ring schedule, one GPU standing in for all shards
+@pytest.mark.parametrize("dt,shards", [(torch.float32, 4), (torch.bfloat16, 3)])
+def test_ring_schedule_emulated_on_one_gpu(gpu, dt, shards):
+    """tpa/ring_tpa.py:41-112 with the devices replaced by a loop: every query shard meets every
+    K/V shard once, each meeting is one block call (o_, l_) of this library, and the partial
+    results are merged with _lse_accum exactly as the reference's scan body does.  The merged
+    result equals the unsharded call: what each GPU of a ring would run is already here."""
+    from tpa import tpa
+
+    b, h, d, per = 2, 8, 64, 320
+    t = shards * per
+    q, k, v = make_factors(130, b, t, t, h, d, d, 6, 2, scale_by_rank=True)
+    seg = segment_ids(t, 450, b)  # documents that straddle the shard boundaries
+    tq, tk, tv = (to_gpu(x, dt, gpu) for x in (q, k, v))
+    tseg = torch.from_numpy(seg).to(gpu)
+    o_full, res = tpa._tpa_fwd(tq, tk, tv, h, tseg, tseg, d**-0.5, False, None, False, False, False)
+    outs = []
+    for s in range(shards):
+        qs, qseg = tq[:, s * per : (s + 1) * per], tseg[:, s * per : (s + 1) * per]
+        o = torch.zeros((b, per, h, d), dtype=torch.float32, device=gpu)
+        l = torch.full((b, per, h), float("-inf"), dtype=torch.float32, device=gpu)
+        for i in range(shards):
+            j = (s - i) % shards  # the shard that has rotated onto this device at step i
+            sl = slice(j * per, (j + 1) * per)
+            o_, r_ = tpa._tpa_fwd(qs, tk[:, sl], tv[:, sl], h, qseg, tseg[:, sl], d**-0.5, False, None, False, False, False)
+            l_ = r_[-1].float()
+            l_next = tpa._lse_accum(l, l_)
+            o = torch.nan_to_num(o * torch.exp(l - l_next)[..., None], nan=0.0)
+            o = o + torch.nan_to_num(o_.float() * torch.exp(l_ - l_next)[..., None], nan=0.0)
+            l = l_next
+        outs.append(torch.where(torch.isneginf(l)[..., None], torch.full_like(o, float("nan")), o))
+    o_ring = torch.cat(outs, dim=1)
+    tol = F32_TOL if dt == torch.float32 else BF16_TOL
+    assert torch.equal(torch.isnan(o_ring), torch.isnan(o_full.float()))
+    assert (torch.nan_to_num(o_ring) - torch.nan_to_num(o_full.float())).abs().max().item() <= tol
+    o_ref, _ = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), seg, seg, h, sm_scale=d**-0.5)
+    assert np.nanmax(np.abs(as_f64(o_ring) - o_ref)) <= tol
