@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define TPA_ABI_VERSION 3
+#define TPA_ABI_VERSION 4
 
 /* element types of the factor / output arrays */
 enum { TPA_DTYPE_F32 = 0, TPA_DTYPE_BF16 = 1 };
@@ -106,6 +106,12 @@ typedef struct TpaFwdArgs {
   const int32_t* page_table; /* [B, pages_per_seq] or NULL */
   int32_t page_size;         /* tokens per page */
   int32_t pages_per_seq;     /* entries per row of page_table */
+  /* With causal != 0: key index <= query index + causal_offset.  0 is the reference's top-left alignment
+     (tpa/tpa.py:377-379); lk - lq aligns the last query with the last key (a chunk of new tokens over a
+     cache); a sequence shard passes the distance between its first query and the first key of the key shard
+     it meets (tpa/ring_tpa.py:73-79 calls the block function with local indices only).  Rows that see no key
+     end as NaN / -inf like any other empty row.  tpa_fwd only; ignored when causal == 0. */
+  int32_t causal_offset;
 } TpaFwdArgs;
 
 /*

@@ -123,6 +123,14 @@ __device__ __forceinline__ int xcd_pair_slot(int round, int xcd, int B) {
   return 7 - xcd;
 }
 
+// Causal offset of a forward call as the kernels take it: row i sees keys <= i + offset.  Offsets
+// of lk and more mask nothing and offsets of -lq and less mask everything, so the value is clamped
+// to that range (keeps the kernels' index arithmetic far from overflow); 0 without the causal mask.
+inline int causal_offset_of(const TpaFwdArgs* a) {
+  if (!a->causal) return 0;
+  return a->causal_offset < -a->lq ? -a->lq : (a->causal_offset > a->lk ? a->lk : a->causal_offset);
+}
+
 // Raise a kernel's dynamic LDS limit above the 64 KB a kernel gets without asking.  The attribute
 // belongs to one device's copy of the code, so it is set once per device (`done` is the calling
 // launcher's own table; a race between two first launches only repeats the same call).

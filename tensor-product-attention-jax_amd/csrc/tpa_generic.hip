@@ -26,6 +26,7 @@ struct GenericParams {
   int B, lq, lk, H, dk, dv, rq, rk;
   float sm_scale;
   int causal;
+  int coff;  // with causal: row i sees keys <= i + coff
   int dense;
 };
 
@@ -78,7 +79,7 @@ __global__ __launch_bounds__(kRows) void generic_fwd_kernel(GenericParams p) {
   int k_end = p.kvlen ? max(0, min(p.kvlen[b], p.lk)) : p.lk;
   if (p.causal) {
     const int last_row = min(p.lq, (int)(blockIdx.x + 1) * kRows) - 1;
-    k_end = min(k_end, last_row + 1);
+    k_end = min(k_end, last_row + 1 + p.coff);
   }
 
   for (int k0 = 0; k0 < k_end; k0 += kTile) {
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(kRows) void generic_fwd_kernel(GenericParams p) {
         if (p.bias) x += p.bias[((int64_t)b * p.lq + row) * p.lk + k0 + t];
         bool keep = true;
         if (p.kvseg) keep = segs[t] == qseg;
-        if (p.causal) keep = keep && (k0 + t <= row);
+        if (p.causal) keep = keep && (k0 + t <= row + p.coff);
         if (!keep) x = -INFINITY;
       }
       s[t] = x;
@@ -215,7 +216,7 @@ __global__ __launch_bounds__(kFewThreads) void generic_fewrows_kernel(GenericPar
   }
   const int qseg = p.qseg ? p.qseg[(int64_t)b * p.lq + row] : 0;
   int k_end = p.kvlen ? max(0, min(p.kvlen[b], p.lk)) : p.lk;
-  if (p.causal) k_end = min(k_end, row + 1);
+  if (p.causal) k_end = min(k_end, row + 1 + p.coff);
   const float inv_rk = 1.f / (float)p.rk;
 
   float m = -INFINITY, l = 0.f, acc = 0.f;  // acc: o[tid] for tid < dv
@@ -355,7 +356,7 @@ int tpa_generic_launch(const TpaFwdArgs* a, hipStream_t stream) {
   p.qseg = a->q_segment_ids; p.kvseg = a->kv_segment_ids; p.bias = nullptr; p.kvlen = a->kv_lengths;
   p.o = a->o; p.lse = a->lse;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.dk = a->dk; p.dv = a->dv; p.rq = a->rq; p.rk = a->rk;
-  p.sm_scale = a->sm_scale; p.causal = a->causal; p.dense = 0;
+  p.sm_scale = a->sm_scale; p.causal = a->causal; p.coff = tpa::causal_offset_of(a); p.dense = 0;
   if (a->B > 65535 || a->H > 65535) return TPA_ERR_SHAPE;
   if (a->dtype == TPA_DTYPE_F32) return tpa::launch_generic<float>(p, stream);
   if (a->dtype == TPA_DTYPE_BF16) return tpa::launch_generic<uint16_t>(p, stream);

@@ -46,6 +46,7 @@ struct PrefillParams {
   int B, lq, lk, H, rq, rk;
   float sm_scale;
   int causal;
+  int coff;         // with causal: row i sees keys <= i + coff (0 = top-left aligned)
   int nqb;     // query blocks per (batch, head)
   int npairs;  // nqb * B
   int q_factors;  // dense K/V loader only: 1 = Q is still given by its rank factors qa, qb
@@ -102,9 +103,9 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   // scalars out of the argument block (never take the address of the block itself)
   struct Fac { const uint16_t* ptr; int64_t stride_b; int stride_l, stride_r; };
   auto fac = [](const TpaFactor& f) { return Fac{static_cast<const uint16_t*>(f.ptr), f.stride_b, (int)f.stride_l, (int)f.stride_r}; };
-  struct { Fac qa, qb, ka, kb, va, vb; const int32_t* qseg; const int32_t* kvseg; const int32_t* kvlen; uint16_t* o; float* lse; int B, lq, lk, H, rq, rk; float sm_scale; int causal, nqb, npairs, q_factors; } const p = {
+  struct { Fac qa, qb, ka, kb, va, vb; const int32_t* qseg; const int32_t* kvseg; const int32_t* kvlen; uint16_t* o; float* lse; int B, lq, lk, H, rq, rk; float sm_scale; int causal, coff, nqb, npairs, q_factors; } const p = {
       fac(pp.qa), fac(pp.qb), fac(pp.ka), fac(pp.kb), fac(pp.va), fac(pp.vb), pp.qseg, pp.kvseg, pp.kvlen, pp.o, pp.lse, pp.B, pp.lq, pp.lk, pp.H, pp.rq, pp.rk,
-      pp.sm_scale, pp.causal, pp.nqb, pp.npairs, pp.q_factors};
+      pp.sm_scale, pp.causal, pp.causal ? pp.coff : 0, pp.nqb, pp.npairs, pp.q_factors};
 
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   uint16_t* const lds_k = smem;                                  // [2][kTK][KS]
@@ -216,7 +217,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   // ---- key range [kpos0, kend) this workgroup visits; tiles are counted from kpos0
   int kpos0 = 0;
   const int len_b = p.kvlen ? max(0, min(p.kvlen[b], p.lk)) : p.lk;  // keys of this batch entry
-  int kend = p.causal ? min(len_b, min(q0 + kBQ, p.lq)) : len_b;
+  int kend = p.causal ? min(len_b, min(q0 + kBQ, p.lq) + p.coff) : len_b;
   if (kend <= 0) {  // no key at all: the rows end as NaN / -inf (tpa/tpa.py:437-439)
     if (qrow < p.lq) {
       uint16_t* op = p.o + (((int64_t)b * p.lq + qrow) * p.H + h) * D;
@@ -284,8 +285,10 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     }
   }
   const int lk_r = kend - kpos0;          // keys counted from kpos0
-  const int wrow_r = wrow0 - kpos0;       // this wave's first row, and this lane's row, on that scale
-  const int qrow_r = qrow - kpos0;
+  // this wave's first row and this lane's row on that scale, shifted by the causal offset: row r
+  // sees keys up to r_r, which is negative for a row that sees none
+  const int wrow_r = wrow0 + p.coff - kpos0;
+  const int qrow_r = qrow + p.coff - kpos0;
   const int ntiles = (lk_r + kTK - 1) / kTK;
   const int last = ntiles - 1;
   // last tile this wave needs under the causal mask (its rows: wrow0 .. wrow0 + 31)
@@ -946,7 +949,7 @@ int tpa_prefill_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
   p.qseg = a->q_segment_ids; p.kvseg = a->kv_segment_ids; p.kvlen = a->kv_lengths;
   p.o = static_cast<uint16_t*>(a->o); p.lse = a->lse;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.rk = a->rk;
-  p.sm_scale = a->sm_scale; p.causal = a->causal;
+  p.sm_scale = a->sm_scale; p.causal = a->causal; p.coff = tpa::causal_offset_of(a);
   p.nqb = (a->lq + kBQ - 1) / kBQ;
   p.npairs = p.nqb * a->B;
   // Ranks other than 2: every workgroup of the fused kernel would rebuild the K/V tiles of its
@@ -1007,7 +1010,7 @@ int mha_prefill_mfma_launch(const MhaFwdArgs* a, hipStream_t stream) {
   p.qa = p.ka = p.va = TpaFactor{nullptr, 0, 0, 0};
   p.o = static_cast<uint16_t*>(a->o); p.lse = a->lse;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = 1; p.rk = 1;
-  p.sm_scale = a->sm_scale; p.causal = a->causal;
+  p.sm_scale = a->sm_scale; p.causal = a->causal; p.coff = 0;
   p.nqb = (a->lq + kBQ - 1) / kBQ;
   p.npairs = p.nqb * a->B;
   if (a->dk == 128) return launch_prefill<128, LOAD_DENSE>(p, stream);

@@ -36,7 +36,7 @@ struct F32Params {
   float* lse;
   int B, lq, lk, H, rq, rk;
   float sm_scale;
-  int causal, nqb, npairs;
+  int causal, coff, nqb, npairs;  // coff: with causal, row i sees keys <= i + coff
 };
 
 template <int D>
@@ -59,9 +59,9 @@ __global__ __launch_bounds__(kNW * 64) void prefill_f32_kernel(F32Params pp) {
 
   struct Fac { const float* ptr; int64_t stride_b, stride_l, stride_r; };
   auto fac = [](const TpaFactor& f) { return Fac{static_cast<const float*>(f.ptr), f.stride_b, f.stride_l, f.stride_r}; };
-  struct { Fac qa, qb, ka, kb, va, vb; const int32_t* qseg; const int32_t* kvseg; const int32_t* kvlen; float* o; float* lse; int B, lq, lk, H, rq, rk; float sm_scale; int causal, nqb, npairs; } const p = {
+  struct { Fac qa, qb, ka, kb, va, vb; const int32_t* qseg; const int32_t* kvseg; const int32_t* kvlen; float* o; float* lse; int B, lq, lk, H, rq, rk; float sm_scale; int causal, coff, nqb, npairs; } const p = {
       fac(pp.qa), fac(pp.qb), fac(pp.ka), fac(pp.kb), fac(pp.va), fac(pp.vb), pp.qseg, pp.kvseg, pp.kvlen, pp.o, pp.lse,
-      pp.B, pp.lq, pp.lk, pp.H, pp.rq, pp.rk, pp.sm_scale, pp.causal, pp.nqb, pp.npairs};
+      pp.B, pp.lq, pp.lk, pp.H, pp.rq, pp.rk, pp.sm_scale, pp.causal, pp.causal ? pp.coff : 0, pp.nqb, pp.npairs};
 
   extern __shared__ __attribute__((aligned(16))) float smem_f32[];
   float* const lds_k = smem_f32;                                         // [2][kTK][RS]
@@ -89,7 +89,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_f32_kernel(F32Params pp) {
 
   // ---- key range
   const int len_b = p.kvlen ? max(0, min(p.kvlen[b], p.lk)) : p.lk;
-  const int kend = p.causal ? min(len_b, min(q0 + kBQ, p.lq)) : len_b;
+  const int kend = p.causal ? min(len_b, min(q0 + kBQ, p.lq) + p.coff) : len_b;
   float* const orow = p.o + (((int64_t)b * p.lq + qrow) * p.H + h) * D;
   if (kend <= 0) {  // no key at all: the rows end as NaN / -inf (tpa/tpa.py:437-439)
     if (qrow < p.lq) {
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_f32_kernel(F32Params pp) {
     return;
   }
   const int ntiles = (kend + kTK - 1) / kTK;
-  const int wave_last_tile = p.causal ? min(ntiles - 1, (wrow0 + 31) / kTK) : ntiles - 1;
+  const int wave_last_tile = p.causal ? min(ntiles - 1, max(wrow0 + p.coff + 31, 0) / kTK) : ntiles - 1;
 
   // ---- Q (B operand of S^T = K Q^T), scaled: qf[4m + e] = c * Q[qrow][8m + 4g + e]
   float qf[NQ];
@@ -186,9 +186,9 @@ __global__ __launch_bounds__(kNW * 64) void prefill_f32_kernel(F32Params pp) {
       }
     }
     // register v of block mb, wave half g  <->  key k0 + 32 mb + 8 (v / 4) + 4 g + v % 4
-    const bool need_mask = (k0 + kTK > kend) || (p.causal && (k0 + kTK - 1 > wrow0));
+    const bool need_mask = (k0 + kTK > kend) || (p.causal && (k0 + kTK - 1 > wrow0 + p.coff));
     if (need_mask) {
-      const int limit = p.causal ? min(qrow, kend - 1) : kend - 1;  // largest visible key index
+      const int limit = p.causal ? min(qrow + p.coff, kend - 1) : kend - 1;  // largest visible key index
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
@@ -317,7 +317,7 @@ int tpa_prefill_f32_launch(const TpaFwdArgs* a, hipStream_t stream) {
   p.qseg = a->q_segment_ids; p.kvseg = a->kv_segment_ids; p.kvlen = a->kv_lengths;
   p.o = static_cast<float*>(a->o); p.lse = a->lse;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.rk = a->rk;
-  p.sm_scale = a->sm_scale; p.causal = a->causal;
+  p.sm_scale = a->sm_scale; p.causal = a->causal; p.coff = causal_offset_of(a);
   p.nqb = (a->lq + kBQ - 1) / kBQ;
   p.npairs = p.nqb * a->B;
   return launch_any(p, a->dk, stream);

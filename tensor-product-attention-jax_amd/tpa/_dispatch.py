@@ -22,7 +22,7 @@ KERNEL_AUTO = 0
 KERNEL_GENERIC = 1
 KERNEL_MFMA = 2
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class TpaFactor(ctypes.Structure):
@@ -65,6 +65,7 @@ class TpaFwdArgs(ctypes.Structure):
         ("page_table", ctypes.c_void_p),
         ("page_size", ctypes.c_int32),
         ("pages_per_seq", ctypes.c_int32),
+        ("causal_offset", ctypes.c_int32),
     ]
 
 

@@ -109,6 +109,7 @@ def tpa_factors(
     return_lse: bool = True,
     use_workspace: bool = True,
     kv_lengths=None,
+    causal_offset: int = 0,
 ):
     """Forward pass on the six split factor arrays, the operands of the reference's kernel
     launch (tpa/tpa.py:246-251,543) with a leading batch dimension:
@@ -120,7 +121,11 @@ def tpa_factors(
     `use_workspace=False` withholds the optional scratch memory, which keeps the call on the
     fused prefill kernel whatever the problem.  `kv_lengths` (int32 [b], an addition): batch
     entry i attends to its first kv_lengths[i] keys only; the rest of its k / v rows is padding
-    that is never read.
+    that is never read.  `causal_offset` (an addition, forward only): with `causal`, query i
+    sees keys up to i + causal_offset; 0 is the reference's top-left alignment
+    (tpa/tpa.py:377-379), lk - lq aligns the last query with the last key (new tokens over a
+    cache), and a sequence shard of a ring (tpa/ring_tpa.py:73-79) passes the distance from the
+    first key of the shard it meets to its own first query.
     """
     device = _pick_device(qa, qb, ka, kb, va, vb)
     qa, qb, ka, kb, va, vb = (_as_device_tensor(x, device) for x in (qa, qb, ka, kb, va, vb))
@@ -165,6 +170,7 @@ def tpa_factors(
         dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=int(bool(causal)), kernel=int(kernel),
         workspace=ws_ptr, workspace_bytes=ws_bytes, num_splits=0,
         kv_lengths=kvlen.data_ptr() if kvlen is not None else None,
+        causal_offset=int(causal_offset),
     )
     with torch.cuda.device(device):
         _d.check("tpa_fwd", lib.tpa_fwd(args, _d.current_stream_ptr(device)))

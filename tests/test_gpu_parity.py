@@ -857,13 +857,78 @@ def test_mha_few_rows_with_bias(gpu):
     check(o, lse, o_ref, l_ref, F32_TOL)
 
 
+# ---------------------------------------------------------------- causal mask with an offset between query and key positions
+def _offset_reference(q, k, v, h, sm_scale, offset, qseg=None, kvseg=None):
+    """Oracle attention under the bias `key <= query + offset` (np.tril with that diagonal), built
+    here from the oracle's parts: reconstruction, segment bias, dense attention."""
+    q, k, v = (np.asarray(x, dtype=np.float64) for x in (q, k, v))
+    b, lq, lk = q.shape[0], q.shape[1], k.shape[1]
+    bias = orc.attention_bias(b, lq, lk, qseg, kvseg, False)
+    bias = bias + np.where(np.tril(np.ones((lq, lk), dtype=bool), k=offset), 0.0, -np.inf)[None]
+    dense = [orc.reconstruct(*orc.split_factors(x, h)) for x in (q, k, v)]
+    return orc.mha_forward(*dense, bias=bias, sm_scale=sm_scale)
+
+
+@pytest.mark.parametrize(
+    "dt,kernel,b,lq,lk,h,d,rq,rk,offset,seg",
+    [
+        (torch.bfloat16, 2, 2, 512, 1024, 4, 128, 6, 2, 512, None),   # new tokens over a cache: last query sees the last key
+        (torch.bfloat16, 2, 1, 300, 700, 2, 128, 6, 2, 400, None),    # ragged, same alignment
+        (torch.bfloat16, 2, 1, 600, 600, 2, 128, 2, 2, -130, None),   # negative: the first 130 rows see nothing
+        (torch.bfloat16, 2, 1, 600, 600, 2, 64, 2, 2, -259, None),    # whole first query block empty, second one partly
+        (torch.bfloat16, 2, 1, 384, 500, 2, 128, 2, 2, 77, None),     # the diagonal cuts tiles off their boundaries
+        (torch.bfloat16, 2, 1, 320, 320, 2, 64, 3, 4, 64, None),      # any-rank loader
+        (torch.bfloat16, 2, 1, 640, 900, 2, 128, 2, 4, 260, None),    # ranks other than 2 through dense K and V
+        (torch.bfloat16, 2, 2, 512, 768, 2, 128, 2, 2, 256, 200),     # with packed documents
+        (torch.bfloat16, 2, 1, 256, 256, 2, 128, 2, 2, 100000, None), # beyond lk: nothing is masked
+        (torch.bfloat16, 2, 1, 256, 256, 2, 128, 2, 2, -100000, None),  # beyond -lq: everything is
+        (torch.float32, 2, 2, 320, 640, 2, 64, 6, 2, 320, None),      # fp32 matrix-core kernel
+        (torch.float32, 2, 1, 400, 400, 2, 128, 2, 2, -97, 150),
+        (torch.float32, 1, 2, 130, 200, 3, 24, 2, 3, 70, None),       # vector-ALU kernel, odd head size
+        (torch.float32, 1, 1, 130, 200, 3, 24, 2, 3, -40, 50),
+        (torch.bfloat16, 0, 2, 4, 2000, 4, 128, 2, 2, 1996, None),    # few rows over many keys
+        (torch.float32, 1, 1, 3, 1500, 2, 40, 2, 2, 1000, None),      # the few-rows vector kernel
+    ],
+)
+def test_causal_offset(gpu, dt, kernel, b, lq, lk, h, d, rq, rk, offset, seg):
+    from tpa import tpa
+
+    q, k, v = make_factors(140, b, lq, lk, h, d, d, rq, rk, scale_by_rank=dt == torch.bfloat16)
+    qseg = segment_ids(lq, seg, b) if seg else None
+    kvseg = segment_ids(lk, seg, b) if seg else None
+    tq, tk, tv = (to_gpu(x, dt, gpu) for x in (q, k, v))
+    sm_scale = d**-0.5
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), qseg, kvseg, sm_scale=sm_scale, causal=True, kernel=kernel, causal_offset=offset)
+    o_ref, l_ref = _offset_reference(as_f64(tq), as_f64(tk), as_f64(tv), h, sm_scale, offset, qseg, kvseg)
+    check(o, lse, o_ref, l_ref, F32_TOL if dt == torch.float32 else BF16_TOL)
+
+
+def test_causal_offset_rows_equal_the_tail_of_the_full_causal_call(gpu):
+    """The last 256 rows of a causal call over 1024 tokens, and those 256 rows alone as queries with
+    causal_offset = 768 over the same keys: the same launch-level arithmetic, equal results."""
+    from tpa import tpa
+
+    b, t, h, d, n = 2, 1024, 4, 128, 256
+    q, k, v = make_factors(141, b, t, t, h, d, d, 6, 2, scale_by_rank=True)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    o_full, lse_full = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=d**-0.5, causal=True)
+    o_tail, lse_tail = tpa.tpa_factors(*split(tq[:, t - n :], tk, tv, h), sm_scale=d**-0.5, causal=True, causal_offset=t - n)
+    assert torch.equal(o_tail, o_full[:, t - n :])
+    assert torch.equal(lse_tail, lse_full[:, :, t - n :])
+
+
 # ---------------------------------------------------------------- the ring schedule, one GPU standing in for all shards
+@pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dt,shards", [(torch.float32, 4), (torch.bfloat16, 3)])
-def test_ring_schedule_emulated_on_one_gpu(gpu, dt, shards):
+def test_ring_schedule_emulated_on_one_gpu(gpu, dt, shards, causal):
     """tpa/ring_tpa.py:41-112 with the devices replaced by a loop: every query shard meets every
     K/V shard once, each meeting is one block call (o_, l_) of this library, and the partial
     results are merged with _lse_accum exactly as the reference's scan body does.  The merged
-    result equals the unsharded call: what each GPU of a ring would run is already here."""
+    result equals the unsharded call: what each GPU of a ring would run is already here.  Under the
+    causal mask a block call gets the distance between the two shards as its offset (the reference
+    hands its block function local indices only, tpa/ring_tpa.py:73-79, which is right for the
+    diagonal block alone); key shards that lie after the query shard come back empty (-inf) and
+    drop out of the merge."""
     from tpa import tpa
 
     b, h, d, per = 2, 8, 64, 320
@@ -872,7 +937,7 @@ def test_ring_schedule_emulated_on_one_gpu(gpu, dt, shards):
     seg = segment_ids(t, 450, b)  # documents that straddle the shard boundaries
     tq, tk, tv = (to_gpu(x, dt, gpu) for x in (q, k, v))
     tseg = torch.from_numpy(seg).to(gpu)
-    o_full, res = tpa._tpa_fwd(tq, tk, tv, h, tseg, tseg, d**-0.5, False, None, False, False, False)
+    o_full, res = tpa._tpa_fwd(tq, tk, tv, h, tseg, tseg, d**-0.5, causal, None, False, False, False)
     outs = []
     for s in range(shards):
         qs, qseg = tq[:, s * per : (s + 1) * per], tseg[:, s * per : (s + 1) * per]
@@ -881,8 +946,11 @@ def test_ring_schedule_emulated_on_one_gpu(gpu, dt, shards):
         for i in range(shards):
             j = (s - i) % shards  # the shard that has rotated onto this device at step i
             sl = slice(j * per, (j + 1) * per)
-            o_, r_ = tpa._tpa_fwd(qs, tk[:, sl], tv[:, sl], h, qseg, tseg[:, sl], d**-0.5, False, None, False, False, False)
-            l_ = r_[-1].float()
+            o_, l_ = tpa.tpa_factors(
+                qs[..., :h], qs[..., h:], tk[:, sl, :, :h], tk[:, sl, :, h:], tv[:, sl, :, :h], tv[:, sl, :, h:],
+                qseg, tseg[:, sl], d**-0.5, causal, causal_offset=(s - j) * per,
+            )
+            l_ = l_.permute(0, 2, 1)
             l_next = tpa._lse_accum(l, l_)
             o = torch.nan_to_num(o * torch.exp(l - l_next)[..., None], nan=0.0)
             o = o + torch.nan_to_num(o_.float() * torch.exp(l_ - l_next)[..., None], nan=0.0)
@@ -892,5 +960,5 @@ def test_ring_schedule_emulated_on_one_gpu(gpu, dt, shards):
     tol = F32_TOL if dt == torch.float32 else BF16_TOL
     assert torch.equal(torch.isnan(o_ring), torch.isnan(o_full.float()))
     assert (torch.nan_to_num(o_ring) - torch.nan_to_num(o_full.float())).abs().max().item() <= tol
-    o_ref, _ = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), seg, seg, h, sm_scale=d**-0.5)
+    o_ref, _ = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), seg, seg, h, sm_scale=d**-0.5, causal=causal)
     assert np.nanmax(np.abs(as_f64(o_ring) - o_ref)) <= tol
