@@ -110,7 +110,8 @@ typedef struct TpaFwdArgs {
      (tpa/tpa.py:377-379); lk - lq aligns the last query with the last key (a chunk of new tokens over a
      cache); a sequence shard passes the distance between its first query and the first key of the key shard
      it meets (tpa/ring_tpa.py:73-79 calls the block function with local indices only).  Rows that see no key
-     end as NaN / -inf like any other empty row.  tpa_fwd only; ignored when causal == 0. */
+     end as NaN / -inf like any other empty row.  tpa_fwd and tpa_decode; ignored when causal == 0; the
+     backward does not take it. */
   int32_t causal_offset;
 } TpaFwdArgs;
 
@@ -214,7 +215,7 @@ const char* tpa_strerror(int code);
  * Forward pass for any lq (prefill).  Replaces pl.pallas_call(..., name="tpa_fwd") at
  * tpa/tpa.py:492-543 for all batch entries at once (the reference vmaps it, tpa/tpa.py:144-163).
  * If `workspace` holds at least tpa_decode_workspace_bytes(...) bytes and the problem is a
- * decode (lq <= 16, lk >= 1024, no mask) that tpa_decode's kernel takes, the call is served by
+ * decode (lq <= 16, lk >= 1024, no segment ids) that tpa_decode's kernel takes, the call is served by
  * it; if the rank of k, v is not 2 (or the sequence is long, 16384 rows and more) and `workspace`
  * holds tpa_fwd_workspace_bytes(...) bytes, K and V are reconstructed into it once.  Without a
  * workspace the same problems run on the fused prefill kernel.
@@ -234,8 +235,9 @@ size_t tpa_fwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int
  * Forward pass for few query tokens over a long factored cache (the reference reaches this as
  * the same call with lq = 1: block_q = min(128, lq), tpa/tpa.py:485).  Keys are split into
  * ranges whose partial (o, lse) are merged with the rule of _lse_accum (tpa/tpa.py:228-242).
- * Needs `workspace` of at least tpa_decode_workspace_bytes(...) bytes.  Masks are not
- * supported (causal must be 0 and segment ids NULL): TPA_ERR_UNSUPPORTED otherwise.
+ * Needs `workspace` of at least tpa_decode_workspace_bytes(...) bytes.  The causal mask is a
+ * key count per query row (row i reads its first i + causal_offset + 1 keys); segment ids are
+ * not supported (must be NULL): TPA_ERR_UNSUPPORTED otherwise.
  */
 int tpa_decode(const TpaFwdArgs* args, void* stream);
 

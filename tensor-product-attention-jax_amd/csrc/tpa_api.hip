@@ -60,7 +60,7 @@ int tpa_fwd(const TpaFwdArgs* a, void* stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   // few query tokens over a long cache (the reference's decode is this same call with lq = 1,
   // tpa/tpa.py:485): split over keys, if the caller brought the workspace for it
-  if (a->kernel != TPA_KERNEL_GENERIC && a->workspace && a->lq <= 16 && a->lk >= 1024 && !a->causal &&
+  if (a->kernel != TPA_KERNEL_GENERIC && a->workspace && a->lq <= 16 && a->lk >= 1024 &&
       !a->q_segment_ids && a->workspace_bytes >= tpa_decode_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dv, a->num_splits)) {
     if (tpa_decode_mfma_supported(a)) return tpa_decode_mfma_launch(a, s);
     if (tpa_decode_f32_supported(a)) return tpa_decode_f32_launch(a, s);
@@ -87,7 +87,7 @@ size_t tpa_fwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int
 int tpa_decode(const TpaFwdArgs* a, void* stream) {
   const int rc = validate_tpa(a);
   if (rc != TPA_OK) return rc;
-  if (a->causal || a->q_segment_ids) return TPA_ERR_UNSUPPORTED;
+  if (a->q_segment_ids) return TPA_ERR_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (a->kernel != TPA_KERNEL_GENERIC && tpa_decode_mfma_supported(a)) return tpa_decode_mfma_launch(a, s);
   if (a->kernel != TPA_KERNEL_GENERIC && tpa_decode_f32_supported(a)) return tpa_decode_f32_launch(a, s);

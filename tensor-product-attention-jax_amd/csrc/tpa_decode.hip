@@ -35,6 +35,7 @@ struct DecodeParams {
   const int32_t* page_table;  // paged cache: [B, pages_per_seq] physical page of each logical page
   int page_size, pages_per_seq;  // tokens per page; table row length
   int B, lq, lk, H, rq;
+  int climit;      // query row qi sees its first qi + climit keys (causal: offset + 1; otherwise lk, no limit)
   int S;           // key ranges
   float qscale;    // sm_scale * log2(e) / (rq * rk)
 };
@@ -90,7 +91,8 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   // waves of the grid, which advance in step, read neighbouring addresses at any one time)
   const int nparts = S * kWaves;
   const int part = split * kWaves + w;
-  const int len_b = p.kvlen ? max(0, min(p.kvlen[b], p.lk)) : p.lk;  // keys of this batch entry
+  // keys of this batch entry that this query row sees
+  const int len_b = max(0, min(p.kvlen ? min(p.kvlen[b], p.lk) : p.lk, qi + p.climit));
   const int blk_begin = part;
   const int blk_end = (len_b * RK + kRowsPerBlock - 1) / kRowsPerBlock;  // 32-row blocks of its cache
   const int blk_step = nparts;
@@ -369,7 +371,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_f32_kernel(DecodeParams p)
 
   const int nparts = S * kWaves;
   const int part = split * kWaves + w;
-  const int len_b = p.kvlen ? max(0, min(p.kvlen[b], p.lk)) : p.lk;
+  const int len_b = max(0, min(p.kvlen ? min(p.kvlen[b], p.lk) : p.lk, qi + p.climit));
   const int blk_begin = part;
   const int blk_end = (len_b * RK + kRowsPerBlock - 1) / kRowsPerBlock;
   const int blk_step = nparts;
@@ -628,6 +630,7 @@ int launch_decode_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   p.part_o = ws; p.part_m = ws + no; p.part_l = ws + no + nm;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.S = S;
   p.kvlen = a->kv_lengths;
+  p.climit = a->causal ? causal_offset_of(a) + 1 : a->lk;
   p.page_table = a->page_table; p.page_size = a->page_size; p.pages_per_seq = a->pages_per_seq;
   p.qscale = a->sm_scale * kLog2e / ((float)a->rq * (float)RK);
   auto kern = decode_kernel<D, RK, PAGED>;
@@ -650,6 +653,7 @@ int launch_decode_f32_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   p.part_o = ws; p.part_m = ws + no; p.part_l = ws + no + nm;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.S = S;
   p.kvlen = a->kv_lengths;
+  p.climit = a->causal ? causal_offset_of(a) + 1 : a->lk;
   p.page_table = a->page_table; p.page_size = a->page_size; p.pages_per_seq = a->pages_per_seq;
   p.qscale = a->sm_scale * kLog2e / ((float)a->rq * (float)RK);
   auto kern = decode_f32_kernel<D, RK, PAGED>;
@@ -721,7 +725,7 @@ int tpa_decode_mfma_supported(const TpaFwdArgs* a) {
   if (a->rk != 1 && a->rk != 2 && a->rk != 4 && a->rk != 8 && a->rk != 16 && a->rk != 32) return 0;
   if (a->H % 8 != 0) return 0;
   if (a->lq > 64) return 0;
-  if (a->causal || a->q_segment_ids || a->kv_segment_ids) return 0;
+  if (a->q_segment_ids || a->kv_segment_ids) return 0;
   // rows (token, rank) must be uniformly strided: stride_l == rk * stride_r
   const TpaFactor* fs[4] = {&a->ka, &a->kb, &a->va, &a->vb};
   for (const TpaFactor* f : fs) {
@@ -764,7 +768,7 @@ int tpa_decode_f32_supported(const TpaFwdArgs* a) {
   if (a->dk != a->dv || (a->dk != 64 && a->dk != 128)) return 0;
   if (a->rk != 1 && a->rk != 2 && a->rk != 4 && a->rk != 8 && a->rk != 16 && a->rk != 32) return 0;
   if (a->lq > 64) return 0;
-  if (a->causal || a->q_segment_ids || a->kv_segment_ids) return 0;
+  if (a->q_segment_ids || a->kv_segment_ids) return 0;
   // rows (token, rank) must be uniformly strided: stride_l == rk * stride_r; B rows are read as 16-byte vectors
   const TpaFactor* fs[4] = {&a->ka, &a->kb, &a->va, &a->vb};
   for (const TpaFactor* f : fs)

@@ -185,8 +185,10 @@ def tpa_decode(
     kernel: int = _d.KERNEL_AUTO,
     kv_lengths=None,
     page_table=None,
+    causal: bool = False,
+    causal_offset: int = 0,
 ):
-    """Few query tokens against a long factored KV cache (no mask), split over key ranges.
+    """Few query tokens against a long factored KV cache, split over key ranges.
 
     The reference has no separate entry point for this: it is tpa() with lq = 1
     (block_q = min(128, lq), tpa/tpa.py:485).  Same operands as `tpa_factors`; the cache is
@@ -196,6 +198,9 @@ def tpa_decode(
     `page_table` (int32 [b, pages_per_seq]): the cache arrays are then page pools
     [pages, page_size, rk, x] shared by all sequences, and token t of entry i lives in page
     page_table[i, t // page_size]; the logical cache length is pages_per_seq * page_size.
+    `causal` with `causal_offset` (see `tpa_factors`): query i sees keys up to i + causal_offset,
+    e.g. lq freshly appended tokens that must not see each other's successors
+    (causal_offset = lk - lq); segment ids are not taken here.
     Returns (o[b,lq,h,dv], lse[b,h,lq]).
     """
     device = _pick_device(qa, qb, ka, kb, va, vb)
@@ -227,11 +232,12 @@ def tpa_decode(
         qa=_d.factor(qa), qb=_d.factor(qb), ka=_d.factor(ka), kb=_d.factor(kb), va=_d.factor(va), vb=_d.factor(vb),
         q_segment_ids=None, kv_segment_ids=None, o=o.data_ptr(), lse=lse.data_ptr(),
         B=b, lq=lq, lk=lk, H=h, dk=dk, dv=dv, rq=rq, rk=rk,
-        dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=0, kernel=int(kernel),
+        dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=int(bool(causal)), kernel=int(kernel),
         workspace=workspace.data_ptr(), workspace_bytes=workspace.numel() * workspace.element_size(),
         num_splits=int(num_splits),
         kv_lengths=kvlen.data_ptr() if kvlen is not None else None,
         page_table=pt.data_ptr() if pt is not None else None, page_size=int(page_size), pages_per_seq=int(pages_per_seq),
+        causal_offset=int(causal_offset),
     )
     with torch.cuda.device(device):
         _d.check("tpa_decode", lib.tpa_decode(args, _d.current_stream_ptr(device)))

@@ -917,6 +917,40 @@ def test_causal_offset_rows_equal_the_tail_of_the_full_causal_call(gpu):
     assert torch.equal(lse_tail, lse_full[:, :, t - n :])
 
 
+@pytest.mark.parametrize(
+    "dt,b,lq,lk,h,d,rq,rk,offset,lengths",
+    [
+        (torch.bfloat16, 2, 4, 2048, 16, 128, 6, 2, 2044, None),     # four appended tokens, each sees its predecessors
+        (torch.bfloat16, 2, 8, 1500, 8, 64, 2, 4, 1492, None),
+        (torch.bfloat16, 1, 5, 1200, 8, 128, 2, 2, 0, None),         # top-left: row i sees i + 1 keys
+        (torch.bfloat16, 1, 3, 1100, 8, 128, 2, 2, -2, None),        # rows 0 and 1 see nothing
+        (torch.bfloat16, 3, 4, 2048, 8, 128, 2, 2, 1000, [2048, 1001, 3]),  # together with per-sequence lengths
+        (torch.float32, 2, 4, 1300, 8, 64, 3, 2, 1296, None),        # fp32 cache
+        (torch.float32, 1, 2, 1024, 4, 128, 2, 8, 700, None),
+    ],
+)
+def test_decode_with_a_causal_limit_per_query_row(gpu, dt, b, lq, lk, h, d, rq, rk, offset, lengths):
+    """The split-key kernels give every query row its own key count (row i: i + offset + 1 keys),
+    through tpa_decode and through tpa_fwd's decode route alike (kernel=2: no other kernel may step in)."""
+    from tpa import tpa
+
+    q, k, v = make_factors(150, b, lq, lk, h, d, d, rq, rk, scale_by_rank=dt == torch.bfloat16)
+    tq, tk, tv = (to_gpu(x, dt, gpu) for x in (q, k, v))
+    kvl = None if lengths is None else torch.tensor(lengths, dtype=torch.int32, device=gpu)
+    sm_scale = d**-0.5
+    o, lse = tpa.tpa_decode(*split(tq, tk, tv, h), sm_scale=sm_scale, kernel=2, kv_lengths=kvl, causal=True, causal_offset=offset)
+    fq, fk, fv = as_f64(tq), as_f64(tk), as_f64(tv)
+    if lengths is None:
+        o_ref, l_ref = _offset_reference(fq, fk, fv, h, sm_scale, offset)
+    else:  # padding keys carry segment id 1, everything else 0
+        kvseg = (np.arange(lk)[None, :] >= np.asarray(lengths)[:, None]).astype(np.int32)
+        o_ref, l_ref = _offset_reference(fq, fk, fv, h, sm_scale, offset, np.zeros((b, lq), np.int32), kvseg)
+    tol = F32_TOL if dt == torch.float32 else BF16_TOL
+    check(o, lse, o_ref, l_ref, tol)
+    o2, lse2 = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=sm_scale, causal=True, kernel=2, kv_lengths=kvl, causal_offset=offset)
+    assert torch.equal(torch.nan_to_num(o2.float(), nan=7.0), torch.nan_to_num(o.float(), nan=7.0)) and torch.equal(lse2, lse)
+
+
 # ---------------------------------------------------------------- the ring schedule, one GPU standing in for all shards
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dt,shards", [(torch.float32, 4), (torch.bfloat16, 3)])
