@@ -65,9 +65,14 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
 
   const int S = p.S;
-  const int b = blockIdx.x / S, split = blockIdx.x % S;
-  const int qi = blockIdx.y;
-  const int h0 = blockIdx.z * 32;
+  // workgroup id -> (key range x, query row qi): ids are dealt to the 8 XCDs round-robin, and the
+  // rows of one query token group read the same cache slice, so they get ids that are 8 apart
+  // (same XCD, same L2) and next to each other in launch order (resident together)
+  const int gid = blockIdx.x, grp = gid / (8 * p.lq), rem = gid - grp * 8 * p.lq;
+  const int qi = rem >> 3, x = grp * 8 + (rem & 7);
+  if (x >= p.B * S) return;  // the grid is rounded up to whole groups of 8 ranges
+  const int b = x / S, split = x % S;
+  const int h0 = blockIdx.y * 32;
   const int tid = threadIdx.x;
   const int w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
   const int hl = min(h0 + i, p.H - 1);  // this lane's head (clamped: lanes past H idle along)
@@ -358,9 +363,14 @@ __global__ __launch_bounds__(kWaves * 64) void decode_f32_kernel(DecodeParams p)
   extern __shared__ __attribute__((aligned(16))) float smem_dec_f32[];
 
   const int S = p.S;
-  const int b = blockIdx.x / S, split = blockIdx.x % S;
-  const int qi = blockIdx.y;
-  const int h0 = blockIdx.z * 32;
+  // workgroup id -> (key range x, query row qi): ids are dealt to the 8 XCDs round-robin, and the
+  // rows of one query token group read the same cache slice, so they get ids that are 8 apart
+  // (same XCD, same L2) and next to each other in launch order (resident together)
+  const int gid = blockIdx.x, grp = gid / (8 * p.lq), rem = gid - grp * 8 * p.lq;
+  const int qi = rem >> 3, x = grp * 8 + (rem & 7);
+  if (x >= p.B * S) return;  // the grid is rounded up to whole groups of 8 ranges
+  const int b = x / S, split = x % S;
+  const int h0 = blockIdx.y * 32;
   const int tid = threadIdx.x;
   const int w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
   const int hl = min(h0 + i, p.H - 1);  // this lane's head (clamped: lanes past H idle along)
@@ -636,7 +646,7 @@ int launch_decode_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   auto kern = decode_kernel<D, RK, PAGED>;
   static bool configured[kMaxDevices] = {};
   if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), DecodeLds<D>::kBytes); rc != TPA_OK) return rc;
-  dim3 grid(a->B * S, a->lq, (a->H + 31) / 32);
+  dim3 grid((a->B * S + 7) / 8 * 8 * a->lq, (a->H + 31) / 32);
   hipLaunchKernelGGL(kern, grid, dim3(kWaves * 64), DecodeLds<D>::kBytes, stream, p);
   if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
   hipLaunchKernelGGL((decode_merge_kernel<D, uint16_t>), dim3(a->B * a->lq, a->H), dim3(D), 0, stream, p.part_o, p.part_m, p.part_l,
@@ -659,7 +669,7 @@ int launch_decode_f32_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   auto kern = decode_f32_kernel<D, RK, PAGED>;
   static bool configured[kMaxDevices] = {};
   if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), DecodeF32Lds<D>::kBytes); rc != TPA_OK) return rc;
-  dim3 grid(a->B * S, a->lq, (a->H + 31) / 32);
+  dim3 grid((a->B * S + 7) / 8 * 8 * a->lq, (a->H + 31) / 32);
   hipLaunchKernelGGL(kern, grid, dim3(kWaves * 64), DecodeF32Lds<D>::kBytes, stream, p);
   if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
   hipLaunchKernelGGL((decode_merge_kernel<D, float>), dim3(a->B * a->lq, a->H), dim3(D), 0, stream, p.part_o, p.part_m, p.part_l,
