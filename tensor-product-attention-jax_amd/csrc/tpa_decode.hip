@@ -49,9 +49,11 @@ struct DecodeLds {
   static constexpr int kReduce = 32 * kRedStride * 2 + 128;  // fp32 O^T + m + l, in uint16 units
   static constexpr int kPerWave = kWave > kReduce ? kWave : kReduce;
   static constexpr size_t kBytes = (size_t)kWaves * kPerWave * sizeof(uint16_t);
+  // with NQ > 1 query rows per workgroup: plus their Q fragments (NQ rows x D/16 steps x 64 lanes x 16 bytes)
+  static constexpr size_t bytes(int nq) { return kBytes + (nq > 1 ? (size_t)nq * (D / 16) * 64 * 16 : 0); }
 };
 
-template <int D, int RK, bool PAGED>
+template <int D, int RK, bool PAGED, int NQ>
 __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   constexpr int CPR = D / 8;               // 16-byte chunks per B row
   constexpr int RPI = 64 / CPR;            // B rows per load instruction
@@ -68,8 +70,12 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   // workgroup id -> (key range x, query row qi): ids are dealt to the 8 XCDs round-robin, and the
   // rows of one query token group read the same cache slice, so they get ids that are 8 apart
   // (same XCD, same L2) and next to each other in launch order (resident together)
-  const int gid = blockIdx.x, grp = gid / (8 * p.lq), rem = gid - grp * 8 * p.lq;
-  const int qi = rem >> 3, x = grp * 8 + (rem & 7);
+  // A workgroup serves NQ query rows from one pass over its cache blocks (each staged block is
+  // used NQ times); with an odd row count the last group's second row repeats the first and is
+  // not stored.
+  const int nqg = (p.lq + NQ - 1) / NQ;  // groups of NQ query rows
+  const int gid = blockIdx.x, grp = gid / (8 * nqg), rem = gid - grp * 8 * nqg;
+  const int qi0 = NQ * (rem >> 3), x = grp * 8 + (rem & 7);
   if (x >= p.B * S) return;  // the grid is rounded up to whole groups of 8 ranges
   const int b = x / S, split = x % S;
   const int h0 = blockIdx.y * 32;
@@ -85,19 +91,42 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
 
   // ---- Qm^T fragments (B operand of S'^T = B_k Qm^T): lane (h, g) holds Qm[h][16ks + 8g + 0..7].
   // Called after the first cache loads are in flight so that their latency is not exposed.
-  bf16x8 qf[NKS];
+  // With one query row they stay in registers; with NQ rows wave r builds row r's fragments once
+  // and parks them in LDS behind the waves' staging regions (fragment (r, ks) of lane l at
+  // [(r NKS + ks) 64 + l]), from where every wave reads them as it needs them: the registers go to
+  // the NQ accumulator sets instead.
+  bf16x8 qf[NQ == 1 ? NKS : 1];
+  u32x4* const lds_q = reinterpret_cast<u32x4*>(smem + kWaves * DecodeLds<D>::kPerWave);
   auto build_q = [&]() {
+    const int qi = NQ == 1 ? qi0 : min(qi0 + w, p.lq - 1);
     const uint16_t* ap = static_cast<const uint16_t*>(p.qa.ptr) + b * p.qa.stride_b + (int64_t)qi * p.qa.stride_l + hl;
     const uint16_t* bp = static_cast<const uint16_t*>(p.qb.ptr) + b * p.qb.stride_b + (int64_t)qi * p.qb.stride_l + 8 * g;
-    build_q_fragments<NKS, 6>(ap, p.qa.stride_r, bp, p.qb.stride_r, p.rq, p.qscale, qf);
+    if constexpr (NQ == 1) {
+      build_q_fragments<NKS, 6>(ap, p.qa.stride_r, bp, p.qb.stride_r, p.rq, p.qscale, qf);
+    } else {
+      if (w < NQ) {
+        bf16x8 tmp[NKS];
+        build_q_fragments<NKS, 6>(ap, p.qa.stride_r, bp, p.qb.stride_r, p.rq, p.qscale, tmp);
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) lds_q[(w * NKS + ks) * 64 + l] = __builtin_bit_cast(u32x4, tmp[ks]);
+      }
+      __syncthreads();
+    }
   };
 
   // ---- this wave's blocks: part, part + nparts, part + 2 nparts, ... (dealt round robin, so the
   // waves of the grid, which advance in step, read neighbouring addresses at any one time)
   const int nparts = S * kWaves;
   const int part = split * kWaves + w;
-  // keys of this batch entry that this query row sees
-  const int len_b = max(0, min(p.kvlen ? min(p.kvlen[b], p.lk) : p.lk, qi + p.climit));
+  // keys of this batch entry that each query row sees, and the most any of them sees
+  const int len_all = p.kvlen ? min(p.kvlen[b], p.lk) : p.lk;
+  int row_last[NQ], len_b = 0;
+#pragma unroll
+  for (int r = 0; r < NQ; ++r) {
+    const int len_r = max(0, min(len_all, min(qi0 + r, p.lq - 1) + p.climit));
+    row_last[r] = len_r * RK - 1;
+    len_b = max(len_b, len_r);
+  }
   const int blk_begin = part;
   const int blk_end = (len_b * RK + kRowsPerBlock - 1) / kRowsPerBlock;  // 32-row blocks of its cache
   const int blk_step = nparts;
@@ -118,10 +147,12 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   const int lb_row = l / CPR, lb_c = l % CPR;             // B tiles: row within the instruction, chunk
   const int la_row = l >> 2, la_c = min(l & 3, a_chunks - 1);  // A tiles: 16 rows per instruction
 
-  // two register sets: while one block is staged and consumed, two more are in flight.  The cache
-  // is read exactly once per call, so the loads are marked non-temporal (measured on the whole
-  // call: 5.1 -> 5.75 TB/s)
-  u32x4 rbk[2][NLB], rbv[2][NLB], rak[2][2], rav[2][2];
+  // two register sets: while one block is staged and consumed, two more are in flight (one set
+  // with NQ rows, whose accumulators take the room and whose blocks take NQ times as long to
+  // consume).  The cache is read exactly once per call, so the loads are marked non-temporal
+  // (measured on the whole call: 5.1 -> 5.75 TB/s)
+  constexpr int NSETS = NQ == 1 ? 2 : 1;
+  u32x4 rbk[NSETS][NLB], rbv[NSETS][NLB], rak[NSETS][2], rav[NSETS][2];
   auto issue = [&](auto set_c, int blk) {
     constexpr int set = decltype(set_c)::value;
     const int row0 = blk * kRowsPerBlock;
@@ -166,33 +197,29 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
     }
   };
 
-  f32x16 o[NDB];
+  f32x16 o[NQ][NDB];
+  float m[NQ], lsum[NQ];
 #pragma unroll
-  for (int db = 0; db < NDB; ++db)
+  for (int r = 0; r < NQ; ++r) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
-  float m = -INFINITY, lsum = 0.f;
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[r][db][v] = 0.f;
+    m[r] = -INFINITY;
+    lsum[r] = 0.f;
+  }
 
   const int lp = l & 15, dhalf = (l >> 4) & 1;
 
   using Set0 = std::integral_constant<int, 0>;
   using Set1 = std::integral_constant<int, 1>;
   if (blk_begin < blk_end) issue(Set0{}, blk_begin);
-  if (blk_begin + blk_step < blk_end) issue(Set1{}, blk_begin + blk_step);
+  if constexpr (NSETS == 2) {
+    if (blk_begin + blk_step < blk_end) issue(Set1{}, blk_begin + blk_step);
+  }
   build_q();
 
   auto compute = [&](int blk) {
-    // ---- S'^T[row, h] = sum_d B_k[row, d] Qm[h, d]
-    f32x16 sp;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) sp[v] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) {
-      const int pos = (2 * ks + g) ^ (i & (CPR - 1));
-      const bf16x8 kf = *reinterpret_cast<const bf16x8*>(lds_bk + i * D + 8 * pos);
-      sp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sp, 0, 0, 0);
-    }
-
     // ---- a_k / a_v of this lane's head for its 16 rows (rows 8q + 4g + 0..3, q = 0..3)
     float ak[16], av[16];
 #pragma unroll
@@ -208,125 +235,162 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
         av[4 * q + j] = bf16bits_to_f32((uint16_t)tv[j]);
       }
     }
-
-    // ---- logits per token (log2 domain), masked past the end of the cache
-    // (a token's RK rows are registers v0 .. v0 + NV - 1; from rank 8 on they span both halves of
-    // the wave, which then hold the same tokens and exchange their partial sums)
-    float st[NTOK];
-    float tmax = -INFINITY;
     const int row0 = blk * kRowsPerBlock;
-#pragma unroll
-    for (int t = 0; t < NTOK; ++t) {
-      const int v0 = t * NV;
-      float acc = 0.f;
-#pragma unroll
-      for (int j = 0; j < NV; ++j) acc += ak[v0 + j] * sp[v0 + j];
-      if constexpr (RK >= 8) acc = halves_sum(acc);
-      const int row = RK >= 8 ? row0 + RK * t : row0 + 8 * (v0 >> 2) + 4 * g + (v0 & 3);  // the token's first row
-      if (row > last_row) acc = -INFINITY;
-      st[t] = acc;
-      tmax = fmaxf(tmax, acc);
-    }
-    tmax = halves_max(tmax);
-    const float m_new = fmaxf(m, tmax);  // finite: row0 itself is always inside the cache
-    if (__any(m_new > m)) {
-      const float alpha = __builtin_amdgcn_exp2f(m - m_new);
-      lsum *= alpha;
-#pragma unroll
-      for (int db = 0; db < NDB; ++db)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
-      m = m_new;
-    }
 
-    // ---- P'^T[row, h] = p[h, token(row)] * a_v[row, h], packed as the B operand of the PV product
-    float pp[16];
 #pragma unroll
-    for (int t = 0; t < NTOK; ++t) {
-      const float pt = __builtin_amdgcn_exp2f(st[t] - m);
-      lsum += RK >= 8 ? 0.5f * pt : pt;  // both halves hold the token: each adds half of it
+    for (int r = 0; r < NQ; ++r) {
+      // keep the rows' instruction streams apart: interleaved, their temporaries do not fit the registers
+      if constexpr (NQ > 1) __builtin_amdgcn_sched_barrier(0);
+      // ---- S'^T[row, h] = sum_d B_k[row, d] Qm[h, d]
+      f32x16 sp;
 #pragma unroll
-      for (int j = 0; j < NV; ++j) pp[t * NV + j] = pt * av[t * NV + j];
-    }
-    bf16x8 pf[2];
+      for (int v = 0; v < 16; ++v) sp[v] = 0.f;
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      u32x4 pk;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) pk[j] = pack_bf16(pp[8 * kk + 2 * j], pp[8 * kk + 2 * j + 1]);
-      pf[kk] = __builtin_bit_cast(bf16x8, pk);
-    }
+      for (int ks = 0; ks < NKS; ++ks) {
+        const int pos = (2 * ks + g) ^ (i & (CPR - 1));
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(lds_bk + i * D + 8 * pos);
+        if constexpr (NQ == 1) {
+          sp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sp, 0, 0, 0);
+        } else {
+          const bf16x8 qv = __builtin_bit_cast(bf16x8, lds_q[(r * NKS + ks) * 64 + l]);
+          sp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qv, sp, 0, 0, 0);
+        }
+      }
 
-    // ---- O^T[d, h] += sum_row B_v[row, d] P'^T[row, h]; slot (g, j) = row 16kk + 8(j/4) + 4g + j%4
+      // ---- logits per token (log2 domain), masked past the keys this query row sees
+      // (a token's RK rows are registers v0 .. v0 + NV - 1; from rank 8 on they span both halves of
+      // the wave, which then hold the same tokens and exchange their partial sums)
+      float st[NTOK];
+      float tmax = -INFINITY;
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      const int r_lo = 16 * kk + 4 * g + (lp >> 2);
-      const int r_hi = r_lo + 8;
+      for (int t = 0; t < NTOK; ++t) {
+        const int v0 = t * NV;
+        float acc = 0.f;
 #pragma unroll
-      for (int db = 0; db < NDB; ++db) {
-        const int chunk = 4 * db + 2 * dhalf + ((lp & 3) >> 1);
-        const int sub = 4 * (lp & 1);
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (s16x4 __attribute__((address_space(3)))*)(lds_bv + r_lo * D + 8 * (chunk ^ (r_lo & (CPR - 1))) + sub));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (s16x4 __attribute__((address_space(3)))*)(lds_bv + r_hi * D + 8 * (chunk ^ (r_hi & (CPR - 1))) + sub));
-        const bf16x8 vf = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kk], o[db], 0, 0, 0);
+        for (int j = 0; j < NV; ++j) acc += ak[v0 + j] * sp[v0 + j];
+        if constexpr (RK >= 8) acc = halves_sum(acc);
+        const int row = RK >= 8 ? row0 + RK * t : row0 + 8 * (v0 >> 2) + 4 * g + (v0 & 3);  // the token's first row
+        if (row > row_last[r]) acc = -INFINITY;
+        st[t] = acc;
+        tmax = fmaxf(tmax, acc);
+      }
+      tmax = halves_max(tmax);
+      // finite with one query row (row0 itself is always inside its keys); a row that sees fewer
+      // keys than its neighbour can meet a block with none of its keys, before any or after all
+      const float m_new = fmaxf(m[r], tmax);
+      const float m_use = NQ > 1 && m_new == -INFINITY ? 0.f : m_new;
+      if (__any(m_new > m[r])) {
+        const float alpha = __builtin_amdgcn_exp2f(m[r] - m_use);
+        lsum[r] *= alpha;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) o[r][db][v] *= alpha;
+        m[r] = m_new;
+      }
+
+      // ---- P'^T[row, h] = p[h, token(row)] * a_v[row, h], packed as the B operand of the PV product
+      float pp[16];
+#pragma unroll
+      for (int t = 0; t < NTOK; ++t) {
+        const float pt = __builtin_amdgcn_exp2f(st[t] - m_use);
+        lsum[r] += RK >= 8 ? 0.5f * pt : pt;  // both halves hold the token: each adds half of it
+#pragma unroll
+        for (int j = 0; j < NV; ++j) pp[t * NV + j] = pt * av[t * NV + j];
+      }
+      bf16x8 pf[2];
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        u32x4 pk;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) pk[j] = pack_bf16(pp[8 * kk + 2 * j], pp[8 * kk + 2 * j + 1]);
+        pf[kk] = __builtin_bit_cast(bf16x8, pk);
+      }
+
+      // ---- O^T[d, h] += sum_row B_v[row, d] P'^T[row, h]; slot (g, j) = row 16kk + 8(j/4) + 4g + j%4
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        const int r_lo = 16 * kk + 4 * g + (lp >> 2);
+        const int r_hi = r_lo + 8;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+          const int chunk = 4 * db + 2 * dhalf + ((lp & 3) >> 1);
+          const int sub = 4 * (lp & 1);
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (s16x4 __attribute__((address_space(3)))*)(lds_bv + r_lo * D + 8 * (chunk ^ (r_lo & (CPR - 1))) + sub));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (s16x4 __attribute__((address_space(3)))*)(lds_bv + r_hi * D + 8 * (chunk ^ (r_hi & (CPR - 1))) + sub));
+          const bf16x8 vf = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+          o[r][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kk], o[r][db], 0, 0, 0);
+        }
       }
     }
   };
 
-  for (int blk = blk_begin; blk < blk_end; blk += 2 * blk_step) {
-    stage(Set0{});  // waits for this block's loads only; its registers are then free again
-    if (blk + 2 * blk_step < blk_end) issue(Set0{}, blk + 2 * blk_step);
-    compute(blk);
-    if (blk + blk_step < blk_end) {
-      stage(Set1{});
-      if (blk + 3 * blk_step < blk_end) issue(Set1{}, blk + 3 * blk_step);
-      compute(blk + blk_step);
+  if constexpr (NSETS == 2) {
+    for (int blk = blk_begin; blk < blk_end; blk += 2 * blk_step) {
+      stage(Set0{});  // waits for this block's loads only; its registers are then free again
+      if (blk + 2 * blk_step < blk_end) issue(Set0{}, blk + 2 * blk_step);
+      compute(blk);
+      if (blk + blk_step < blk_end) {
+        stage(Set1{});
+        if (blk + 3 * blk_step < blk_end) issue(Set1{}, blk + 3 * blk_step);
+        compute(blk + blk_step);
+      }
+    }
+  } else {
+    for (int blk = blk_begin; blk < blk_end; blk += blk_step) {
+      stage(Set0{});
+      if (blk + blk_step < blk_end) issue(Set0{}, blk + blk_step);
+      compute(blk);
     }
   }
 
-  // ---- merge the 4 waves through LDS (each wave reuses its own staging region)
+  // ---- merge the 4 waves through LDS (each wave reuses its own staging region), row by row
   constexpr int RS = DecodeLds<D>::kRedStride;
-  const float ltot = halves_sum(lsum);
   float* red_o = reinterpret_cast<float*>(lds);  // [32 heads][RS]
   float* red_m = red_o + 32 * RS;
   float* red_l = red_m + 32;
-#pragma unroll
-  for (int db = 0; db < NDB; ++db)
-#pragma unroll
-    for (int vq = 0; vq < 4; ++vq)
-      *reinterpret_cast<f32x4*>(red_o + i * RS + 32 * db + 8 * vq + 4 * g) =
-          f32x4{o[db][4 * vq], o[db][4 * vq + 1], o[db][4 * vq + 2], o[db][4 * vq + 3]};
-  if (g == 0) {
-    red_m[i] = m;
-    red_l[i] = ltot;
-  }
-  __syncthreads();
-
   const int nh = min(32, p.H - h0);
-  const int64_t pbase = (((int64_t)b * p.lq + qi) * S + split) * p.H + h0;
-  for (int idx = tid; idx < nh * D; idx += kWaves * 64) {
-    const int hh = idx / D, d = idx % D;
-    float mw[kWaves], mmax = -INFINITY;
 #pragma unroll
-    for (int ww = 0; ww < kWaves; ++ww) {
-      mw[ww] = reinterpret_cast<const float*>(smem + ww * DecodeLds<D>::kPerWave)[32 * RS + hh];
-      mmax = fmaxf(mmax, mw[ww]);
-    }
-    float acc = 0.f, lacc = 0.f;
+  for (int r = 0; r < NQ; ++r) {
+    if (qi0 + r >= p.lq) break;  // uniform: the repeated row of an odd count
+    const float ltot = halves_sum(lsum[r]);
+    __syncthreads();  // the staging (or the previous row's merge) has been read by every wave
 #pragma unroll
-    for (int ww = 0; ww < kWaves; ++ww) {
-      const float* ro = reinterpret_cast<const float*>(smem + ww * DecodeLds<D>::kPerWave);
-      const float f = mw[ww] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw[ww] - mmax);
-      acc += f * ro[hh * RS + d];
-      lacc += f * ro[32 * RS + 32 + hh];
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int vq = 0; vq < 4; ++vq)
+        *reinterpret_cast<f32x4*>(red_o + i * RS + 32 * db + 8 * vq + 4 * g) =
+            f32x4{o[r][db][4 * vq], o[r][db][4 * vq + 1], o[r][db][4 * vq + 2], o[r][db][4 * vq + 3]};
+    if (g == 0) {
+      red_m[i] = m[r];
+      red_l[i] = ltot;
     }
-    p.part_o[(pbase + hh) * D + d] = acc;
-    if (d == 0) {
-      p.part_m[pbase + hh] = mmax;
-      p.part_l[pbase + hh] = lacc;
+    __syncthreads();
+
+    const int64_t pbase = (((int64_t)b * p.lq + qi0 + r) * S + split) * p.H + h0;
+    for (int idx = tid; idx < nh * D; idx += kWaves * 64) {
+      const int hh = idx / D, d = idx % D;
+      float mw[kWaves], mmax = -INFINITY;
+#pragma unroll
+      for (int ww = 0; ww < kWaves; ++ww) {
+        mw[ww] = reinterpret_cast<const float*>(smem + ww * DecodeLds<D>::kPerWave)[32 * RS + hh];
+        mmax = fmaxf(mmax, mw[ww]);
+      }
+      float acc = 0.f, lacc = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < kWaves; ++ww) {
+        const float* ro = reinterpret_cast<const float*>(smem + ww * DecodeLds<D>::kPerWave);
+        const float f = mw[ww] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw[ww] - mmax);
+        acc += f * ro[hh * RS + d];
+        lacc += f * ro[32 * RS + 32 + hh];
+      }
+      p.part_o[(pbase + hh) * D + d] = acc;
+      if (d == 0) {
+        p.part_m[pbase + hh] = mmax;
+        p.part_l[pbase + hh] = lacc;
+      }
     }
   }
 }
@@ -630,7 +694,7 @@ size_t workspace_bytes(int B, int lq, int H, int D, int S) {
   return (size_t)B * lq * S * H * (D + 2) * sizeof(float);
 }
 
-template <int D, int RK, bool PAGED>
+template <int D, int RK, bool PAGED, int NQ>
 int launch_decode_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   DecodeParams p{};
   p.qa = a->qa; p.qb = a->qb; p.ka = a->ka; p.kb = a->kb; p.va = a->va; p.vb = a->vb;
@@ -643,11 +707,11 @@ int launch_decode_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   p.climit = a->causal ? causal_offset_of(a) + 1 : a->lk;
   p.page_table = a->page_table; p.page_size = a->page_size; p.pages_per_seq = a->pages_per_seq;
   p.qscale = a->sm_scale * kLog2e / ((float)a->rq * (float)RK);
-  auto kern = decode_kernel<D, RK, PAGED>;
+  auto kern = decode_kernel<D, RK, PAGED, NQ>;
   static bool configured[kMaxDevices] = {};
-  if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), DecodeLds<D>::kBytes); rc != TPA_OK) return rc;
-  dim3 grid((a->B * S + 7) / 8 * 8 * a->lq, (a->H + 31) / 32);
-  hipLaunchKernelGGL(kern, grid, dim3(kWaves * 64), DecodeLds<D>::kBytes, stream, p);
+  if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), DecodeLds<D>::bytes(NQ)); rc != TPA_OK) return rc;
+  dim3 grid((a->B * S + 7) / 8 * 8 * ((a->lq + NQ - 1) / NQ), (a->H + 31) / 32);
+  hipLaunchKernelGGL(kern, grid, dim3(kWaves * 64), DecodeLds<D>::bytes(NQ), stream, p);
   if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
   hipLaunchKernelGGL((decode_merge_kernel<D, uint16_t>), dim3(a->B * a->lq, a->H), dim3(D), 0, stream, p.part_o, p.part_m, p.part_l,
                      static_cast<uint16_t*>(a->o), a->lse, S, a->H, a->lq, 1.f / (float)RK);
@@ -695,9 +759,9 @@ int launch_decode(const TpaFwdArgs* a, int S, hipStream_t stream) {
     if (a->page_size <= 0 || (a->page_size * RK) % kRowsPerBlock != 0 ||
         (int64_t)a->pages_per_seq * a->page_size < a->lk)
       return TPA_ERR_SHAPE;
-    return launch_decode_t<D, RK, true>(a, S, stream);
+    return a->lq >= 2 ? launch_decode_t<D, RK, true, 2>(a, S, stream) : launch_decode_t<D, RK, true, 1>(a, S, stream);
   }
-  return launch_decode_t<D, RK, false>(a, S, stream);
+  return a->lq >= 2 ? launch_decode_t<D, RK, false, 2>(a, S, stream) : launch_decode_t<D, RK, false, 1>(a, S, stream);
 }
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
@@ -705,7 +769,8 @@ bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15)
 int default_splits(int B, int lq, int lk, int H) {
   // one workgroup per CU is resident (the kernel keeps a block of loads in flight in registers),
   // so aim for a whole number of waves of 256 workgroups and at least 4 blocks per wave
-  const int groups = B * lq * ((H + 31) / 32);
+  // (the bf16 kernel serves two query rows per workgroup)
+  const int groups = B * ((lq + 1) / 2) * ((H + 31) / 32);
   int S = (256 + groups - 1) / groups;
   if (groups >= 256) S = 1;
   const int max_s = (lk + 4 * kWaves * 16 - 1) / (4 * kWaves * 16);

@@ -925,6 +925,9 @@ def test_causal_offset_rows_equal_the_tail_of_the_full_causal_call(gpu):
         (torch.bfloat16, 1, 5, 1200, 8, 128, 2, 2, 0, None),         # top-left: row i sees i + 1 keys
         (torch.bfloat16, 1, 3, 1100, 8, 128, 2, 2, -2, None),        # rows 0 and 1 see nothing
         (torch.bfloat16, 3, 4, 2048, 8, 128, 2, 2, 1000, [2048, 1001, 3]),  # together with per-sequence lengths
+        (torch.bfloat16, 1, 2, 1100, 8, 128, 2, 2, -1, None),        # two rows in one workgroup: the first sees nothing
+        (torch.bfloat16, 2, 2, 1100, 8, 128, 2, 2, 1023, None),      # the first row's keys end with a block, the second's go on
+        (torch.bfloat16, 2, 7, 1100, 16, 64, 2, 1, 600, None),       # odd row count: the last workgroup's second row is a repeat
         (torch.float32, 2, 4, 1300, 8, 64, 3, 2, 1296, None),        # fp32 cache
         (torch.float32, 1, 2, 1024, 4, 128, 2, 8, 700, None),
     ],
