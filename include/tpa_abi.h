@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define TPA_ABI_VERSION 4
+#define TPA_ABI_VERSION 5
 
 /* element types of the factor / output arrays */
 enum { TPA_DTYPE_F32 = 0, TPA_DTYPE_BF16 = 1 };
@@ -110,8 +110,7 @@ typedef struct TpaFwdArgs {
      (tpa/tpa.py:377-379); lk - lq aligns the last query with the last key (a chunk of new tokens over a
      cache); a sequence shard passes the distance between its first query and the first key of the key shard
      it meets (tpa/ring_tpa.py:73-79 calls the block function with local indices only).  Rows that see no key
-     end as NaN / -inf like any other empty row.  tpa_fwd and tpa_decode; ignored when causal == 0; the
-     backward does not take it. */
+     end as NaN / -inf like any other empty row.  tpa_fwd and tpa_decode; ignored when causal == 0. */
   int32_t causal_offset;
 } TpaFwdArgs;
 
@@ -178,6 +177,7 @@ typedef struct TpaBwdArgs {
   int32_t kernel;         /* TPA_KERNEL_*: the MFMA kernels take bf16 or fp32 with dk == dv in {64, 128}; d_o must be 16-byte aligned */
   void* workspace;        /* required: at least tpa_bwd_workspace_bytes(...) bytes, 256-byte aligned */
   size_t workspace_bytes;
+  int32_t causal_offset;  /* as in TpaFwdArgs: the value the forward call was made with */
 } TpaBwdArgs;
 
 /*

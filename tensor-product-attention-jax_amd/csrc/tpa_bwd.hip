@@ -152,6 +152,7 @@ struct DenseParams {
   int B, lq, lk, H, dk, dv;
   float sm_scale;
   int causal;
+  int coff;  // with causal: row i sees keys <= i + coff
 };
 
 // ------------------------------------------------------------------------------------ stage 3
@@ -189,7 +190,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_kernel(DenseParams p) {
   const int qseg = (row_ok && p.qseg) ? p.qseg[(int64_t)b * p.lq + row] : 0;
 
   int k_end = p.lk;
-  if (p.causal) k_end = min(p.lk, min(p.lq, (int)(blockIdx.x + 1) * kThreads));
+  if (p.causal) k_end = min(p.lk, min(p.lq, (int)(blockIdx.x + 1) * kThreads) + p.coff);
   for (int k0 = 0; k0 < k_end; k0 += kTile) {
     const int nk = min(kTile, k_end - k0);
     __syncthreads();
@@ -208,7 +209,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dq_kernel(DenseParams p) {
     for (int t = 0; t < nk; ++t) {
       bool keep = true;
       if (p.kvseg) keep = segs[t] == qseg;
-      if (p.causal) keep = keep && (k0 + t <= row);
+      if (p.causal) keep = keep && (k0 + t <= row + p.coff);
       if (!keep) continue;
       float dot = 0.f;
 #pragma unroll
@@ -264,7 +265,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(DenseParams p) {
   const int kseg = (key_ok && p.kvseg) ? p.kvseg[(int64_t)b * p.lk + key] : 0;
 
   // under the causal mask only rows at or after this workgroup's first key can see its keys
-  const int q_begin = p.causal ? min(p.lq, (int)blockIdx.x * kThreads) / kTile * kTile : 0;
+  const int q_begin = p.causal ? min(p.lq, max((int)blockIdx.x * kThreads - p.coff, 0)) / kTile * kTile : 0;
   for (int q0 = q_begin; q0 < p.lq; q0 += kTile) {
     const int nq = min(kTile, p.lq - q0);
     __syncthreads();
@@ -288,7 +289,7 @@ __global__ __launch_bounds__(kThreads) void bwd_dkv_kernel(DenseParams p) {
       const float lse = ls[i];
       bool keep = lse > -INFINITY;
       if (p.qseg) keep = keep && segs[i] == kseg;
-      if (p.causal) keep = keep && (key <= q0 + i);
+      if (p.causal) keep = keep && (key <= q0 + i + p.coff);
       if (!keep) continue;
       float dot = 0.f;
 #pragma unroll
@@ -478,17 +479,17 @@ int tpa_bwd_t(const TpaBwdArgs* a, hipStream_t stream, bool mfma) {
   int rc;
   if (mfma) {
     rc = dense_bwd_mfma_launch(qd, kd, vd, a->d_o, a->lse, delta, a->q_segment_ids, a->kv_segment_ids, dqd, dkd, dvd,
-                               a->B, a->lq, a->lk, a->H, a->dk, a->sm_scale, a->causal, stream);
+                               a->B, a->lq, a->lk, a->H, a->dk, a->sm_scale, a->causal, causal_offset_of(a), stream);
   } else if (mfma32) {
     rc = dense_bwd_f32_launch(qd, kd, vd, static_cast<const float*>(a->d_o), a->lse, delta, a->q_segment_ids, a->kv_segment_ids,
-                              dqd, dkd, dvd, a->B, a->lq, a->lk, a->H, a->dk, a->sm_scale, a->causal, stream);
+                              dqd, dkd, dvd, a->B, a->lq, a->lk, a->H, a->dk, a->sm_scale, a->causal, causal_offset_of(a), stream);
   } else {
     DenseParams p{};
     p.q = qd; p.k = kd; p.v = vd; p.d_o = a->d_o; p.lse = a->lse; p.delta = delta;
     p.qseg = a->q_segment_ids; p.kvseg = a->kv_segment_ids; p.bias = nullptr;
     p.dq = dqd; p.dk_out = dkd; p.dv_out = dvd;
     p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.dk = a->dk; p.dv = a->dv;
-    p.sm_scale = a->sm_scale; p.causal = a->causal;
+    p.sm_scale = a->sm_scale; p.causal = a->causal; p.coff = causal_offset_of(a);
     rc = launch_dense<T>(p, stream);
   }
   if (rc != TPA_OK) return rc;
@@ -516,10 +517,10 @@ int mha_bwd_t(const MhaBwdArgs* a, hipStream_t stream, bool mfma) {
   if (mfma && sizeof(T) == sizeof(float))
     return dense_bwd_f32_launch(static_cast<const float*>(a->q), static_cast<const float*>(a->k), static_cast<const float*>(a->v),
                                 static_cast<const float*>(a->d_o), a->lse, delta, nullptr, nullptr, a->dq, a->dk_out, a->dv_out,
-                                a->B, a->lq, a->lk, a->H, a->dk, a->sm_scale, a->causal, stream);
+                                a->B, a->lq, a->lk, a->H, a->dk, a->sm_scale, a->causal, 0, stream);
   if (mfma)
     return dense_bwd_mfma_launch(a->q, a->k, a->v, a->d_o, a->lse, delta, nullptr, nullptr, a->dq, a->dk_out, a->dv_out,
-                                 a->B, a->lq, a->lk, a->H, a->dk, a->sm_scale, a->causal, stream);
+                                 a->B, a->lq, a->lk, a->H, a->dk, a->sm_scale, a->causal, 0, stream);
   const float *qd, *kd, *vd;
   if constexpr (sizeof(T) == sizeof(float)) {
     qd = static_cast<const float*>(a->q); kd = static_cast<const float*>(a->k); vd = static_cast<const float*>(a->v);

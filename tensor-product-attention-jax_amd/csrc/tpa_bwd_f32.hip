@@ -32,7 +32,7 @@ struct BwdF32Params {
   float *dq, *dk, *dv;
   int B, lq, lk, H;
   float sm_scale;
-  int causal, nblk, npairs;
+  int causal, coff, nblk, npairs;  // coff: with causal, row i sees keys <= i + coff
 };
 
 template <int D>
@@ -161,9 +161,9 @@ __global__ __launch_bounds__(kThreads) void bwd_f32_dq_kernel(BwdF32Params p) {
   const int q0 = blk * kBlock, wrow0 = q0 + 32 * w, qrow = wrow0 + i, qrow_ld = min(qrow, p.lq - 1);
   const int64_t hd = (int64_t)p.H * D;
 
-  const int kend = p.causal ? min(p.lk, q0 + kBlock) : p.lk;
+  const int kend = p.causal ? max(1, min(p.lk, q0 + kBlock + p.coff)) : p.lk;  // at least one (then fully masked) tile
   const int ntiles = (kend + kTile - 1) / kTile;
-  const int wave_last_tile = p.causal ? min(ntiles - 1, (wrow0 + 31) / kTile) : ntiles - 1;
+  const int wave_last_tile = p.causal ? min(ntiles - 1, max(wrow0 + p.coff + 31, 0) / kTile) : ntiles - 1;
 
   float qf[D / 2], gf[D / 2];
   load_own_row<D>(p.q + ((int64_t)b * p.lq + qrow_ld) * hd + (int64_t)h * D, g, p.sm_scale * kLog2e, false, qf);
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(kThreads) void bwd_f32_dq_kernel(BwdF32Params p) {
     f32x16 s[2], dp[2];
     rows_dot<D>(ks, i, g, qf, s[0], s[1]);    // x * log2(e)
     rows_dot<D>(vs, i, g, gf, dp[0], dp[1]);  // dP
-    const int limit = p.causal ? min(qrow, kend - 1) : kend - 1;  // largest visible key index
+    const int limit = p.causal ? min(qrow + p.coff, kend - 1) : kend - 1;  // largest visible key index
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
@@ -256,9 +256,9 @@ __global__ __launch_bounds__(kThreads) void bwd_f32_dkv_kernel(BwdF32Params p) {
   const int64_t hd = (int64_t)p.H * D;
 
   // under the causal mask only rows at or after a key see it
-  const int first_tile = p.causal ? k0 / kTile : 0;
+  const int first_tile = p.causal ? max(k0 - p.coff, 0) / kTile : 0;
   const int ntiles = (p.lq + kTile - 1) / kTile;
-  const int wave_first_tile = p.causal ? wkey0 / kTile : 0;
+  const int wave_first_tile = p.causal ? max(wkey0 - p.coff, 0) / kTile : 0;
 
   float kf[D / 2], vf[D / 2];
   load_own_row<D>(p.k + ((int64_t)b * p.lk + key_ld) * hd + (int64_t)h * D, g, p.sm_scale * kLog2e, false, kf);
@@ -317,7 +317,7 @@ __global__ __launch_bounds__(kThreads) void bwd_f32_dkv_kernel(BwdF32Params p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int v = 4 * vq + e, r = r0 + off + e;
-          bool keep = !p.causal || key <= r;
+          bool keep = !p.causal || key - p.coff <= r;
           if constexpr (SEG) keep = keep && __float_as_int(idf[e]) == kseg;
           const float pt = keep ? __builtin_amdgcn_exp2f(s[mb][v] - lse2[e]) : 0.f;
           s[mb][v] = pt;                                            // p
@@ -384,10 +384,10 @@ int dense_bwd_f32_supported(int dtype, int dk, int dv, int64_t lq, int64_t lk, c
 
 int dense_bwd_f32_launch(const float* q, const float* k, const float* v, const float* d_o, const float* lse, const float* delta,
                          const int32_t* qseg, const int32_t* kvseg, float* dq, float* dk, float* dv, int B, int lq, int lk,
-                         int H, int D, float sm_scale, int causal, hipStream_t stream) {
+                         int H, int D, float sm_scale, int causal, int coff, hipStream_t stream) {
   tpa::BwdF32Params p{};
   p.q = q; p.k = k; p.v = v; p.d_o = d_o; p.lse = lse; p.delta = delta; p.qseg = qseg; p.kvseg = kvseg;
-  p.dq = dq; p.dk = dk; p.dv = dv; p.B = B; p.lq = lq; p.lk = lk; p.H = H; p.sm_scale = sm_scale; p.causal = causal;
+  p.dq = dq; p.dk = dk; p.dv = dv; p.B = B; p.lq = lq; p.lk = lk; p.H = H; p.sm_scale = sm_scale; p.causal = causal; p.coff = causal ? coff : 0;
   if (qseg) return D == 128 ? tpa::launch_pair<128, true>(p, stream) : tpa::launch_pair<64, true>(p, stream);
   return D == 128 ? tpa::launch_pair<128, false>(p, stream) : tpa::launch_pair<64, false>(p, stream);
 }

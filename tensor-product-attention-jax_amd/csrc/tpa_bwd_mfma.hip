@@ -46,6 +46,7 @@ struct BwdParams {
   int B, lq, lk, H;
   float sm_scale;
   int causal;
+  int coff;  // with causal: row i sees keys <= i + coff
   int nblk;    // row blocks (dq) or key blocks (dkv) per (batch, head)
   int npairs;  // nblk * B
 };
@@ -190,7 +191,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(BwdParams p) {
   }
 
   // keys [kpos0, kend) are visited; tiles and key positions below count from kpos0
-  int kpos0 = 0, kend = p.causal ? min(p.lk, min(q0 + kBQ, p.lq)) : p.lk;
+  int kpos0 = 0, kend = p.causal ? max(1, min(p.lk, min(q0 + kBQ, p.lq) + p.coff)) : p.lk;  // at least one (then fully masked) tile
   if constexpr (SEG) {
     int first, lastk;
     id_window<NT>(p.qseg + (int64_t)b * p.lq + q0, min(kBQ, p.lq - q0), p.kvseg + (int64_t)b * p.lk, kend,
@@ -198,7 +199,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(BwdParams p) {
     if (lastk >= 0) { kpos0 = first / kTile * kTile; kend = lastk + 1; }
     else kend = min(kend, kTile);  // nothing visible: one fully masked tile
   }
-  const int lk_r = kend - kpos0, wrow_r = wrow0 - kpos0;
+  const int lk_r = kend - kpos0, wrow_r = wrow0 + p.coff - kpos0;  // rows on the key scale: row r sees keys <= r_r
   const int ntiles = (lk_r + kTile - 1) / kTile, last = ntiles - 1;
   const int wave_last_tile = p.causal ? min(last, max(wrow_r + kWQ - 1, 0) / kTile) : last;
 
@@ -374,7 +375,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
 
   // query tiles tile0 .. : under the causal mask rows before this block's first key see none of
   // its keys; rows from lq_r on are not visited
-  int tile0 = p.causal ? k0 / kTile : 0, lq_r = p.lq;
+  int tile0 = p.causal ? max(k0 - p.coff, 0) / kTile : 0, lq_r = p.lq;
   if constexpr (SEG) {
     int first, lastq;
     const int rbeg = min(tile0 * kTile, p.lq);
@@ -384,7 +385,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
     else lq_r = 0;  // no row can see a key of this block
   }
   const int ntiles = max(0, (lq_r + kTile - 1) / kTile - tile0), last = ntiles - 1;
-  const int wave_first_tile = p.causal ? max(wkey0 / kTile - tile0, 0) : 0;
+  const int wave_first_tile = p.causal ? max(max(wkey0 - p.coff, 0) / kTile - tile0, 0) : 0;
 
   const int lt = tid / CPR, lc = tid % CPR;
   const int64_t tok_stride = (int64_t)p.H * D;
@@ -449,7 +450,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
     const float* nl = lds_nlse + (j & 1) * kTile;
     const float* nd = lds_ndel + (j & 1) * kTile;
     const int r0 = (tile0 + j) * kTile;
-    const bool need_mask = p.causal && (r0 < wkey0 + kWK - 1);  // a row of the tile lies before a key of this wave
+    const bool need_mask = p.causal && (r0 + p.coff < wkey0 + kWK - 1);  // a row of the tile lies before a key of this wave
     static_for<2>([&](auto mb_c) __attribute__((always_inline)) {
       constexpr int mb = decltype(mb_c)::value;
       // accumulator rows of this lane: 32 mb + 8 vq + 4 g + (0..3)
@@ -479,7 +480,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
         if (need_mask) {
-          const int key = wkey0 + 32 * nb + i;
+          const int key = wkey0 + 32 * nb + i - p.coff;  // first row that sees this lane's key
 #pragma unroll
           for (int v = 0; v < 16; ++v)
             if (r0 + 32 * mb + 8 * (v >> 2) + 4 * g + (v & 3) < key) s[nb][v] = -INFINITY;
@@ -615,11 +616,11 @@ int dense_bwd_mfma_supported(int dtype, int dk, int dv, int64_t lq, int64_t lk, 
 
 int dense_bwd_mfma_launch(const void* q, const void* k, const void* v, const void* d_o, const float* lse, const float* delta,
                           const int32_t* qseg, const int32_t* kvseg, float* dq, float* dk, float* dv, int B, int lq, int lk,
-                          int H, int D, float sm_scale, int causal, hipStream_t stream) {
+                          int H, int D, float sm_scale, int causal, int coff, hipStream_t stream) {
   tpa::BwdParams p{};
   p.q = static_cast<const uint16_t*>(q); p.k = static_cast<const uint16_t*>(k); p.v = static_cast<const uint16_t*>(v);
   p.d_o = static_cast<const uint16_t*>(d_o); p.lse = lse; p.delta = delta; p.qseg = qseg; p.kvseg = kvseg;
-  p.dq = dq; p.dk = dk; p.dv = dv; p.B = B; p.lq = lq; p.lk = lk; p.H = H; p.sm_scale = sm_scale; p.causal = causal;
+  p.dq = dq; p.dk = dk; p.dv = dv; p.B = B; p.lq = lq; p.lk = lk; p.H = H; p.sm_scale = sm_scale; p.causal = causal; p.coff = causal ? coff : 0;
   if (D == 128) return tpa::launch_both<128>(p, stream);
   return tpa::launch_both<64>(p, stream);
 }

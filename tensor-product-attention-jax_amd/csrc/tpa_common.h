@@ -130,6 +130,10 @@ inline int causal_offset_of(const TpaFwdArgs* a) {
   if (!a->causal) return 0;
   return a->causal_offset < -a->lq ? -a->lq : (a->causal_offset > a->lk ? a->lk : a->causal_offset);
 }
+inline int causal_offset_of(const TpaBwdArgs* a) {
+  if (!a->causal) return 0;
+  return a->causal_offset < -a->lq ? -a->lq : (a->causal_offset > a->lk ? a->lk : a->causal_offset);
+}
 
 // Raise a kernel's dynamic LDS limit above the 64 KB a kernel gets without asking.  The attribute
 // belongs to one device's copy of the code, so it is set once per device (`done` is the calling
@@ -168,11 +172,11 @@ int mha_bwd_launch(const MhaBwdArgs* a, hipStream_t stream, int mfma);
 int dense_bwd_mfma_supported(int dtype, int dk, int dv, int64_t lq, int64_t lk, int64_t H, float sm_scale, const void* bias);
 int dense_bwd_mfma_launch(const void* q, const void* k, const void* v, const void* d_o, const float* lse, const float* delta,
                           const int32_t* qseg, const int32_t* kvseg, float* dq, float* dk, float* dv, int B, int lq, int lk,
-                          int H, int D, float sm_scale, int causal, hipStream_t stream);
+                          int H, int D, float sm_scale, int causal, int causal_offset, hipStream_t stream);
 int dense_bwd_f32_supported(int dtype, int dk, int dv, int64_t lq, int64_t lk, const void* bias);
 int dense_bwd_f32_launch(const float* q, const float* k, const float* v, const float* d_o, const float* lse, const float* delta,
                          const int32_t* qseg, const int32_t* kvseg, float* dq, float* dk, float* dv, int B, int lq, int lk,
-                         int H, int D, float sm_scale, int causal, hipStream_t stream);
+                         int H, int D, float sm_scale, int causal, int causal_offset, hipStream_t stream);
 size_t tpa_bwd_workspace_size(int64_t B, int64_t lq, int64_t lk, int64_t H, int64_t dk, int64_t dv);
 size_t mha_bwd_workspace_size(int64_t B, int64_t lq, int64_t lk, int64_t H, int64_t dk, int64_t dv, int dtype);
 size_t tpa_prefill_dense_kv_bytes(int64_t B, int64_t lk, int64_t H, int64_t D);

@@ -22,7 +22,7 @@ KERNEL_AUTO = 0
 KERNEL_GENERIC = 1
 KERNEL_MFMA = 2
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 
 class TpaFactor(ctypes.Structure):
@@ -130,6 +130,7 @@ class TpaBwdArgs(ctypes.Structure):
         ("kernel", ctypes.c_int32),
         ("workspace", ctypes.c_void_p),
         ("workspace_bytes", ctypes.c_size_t),
+        ("causal_offset", ctypes.c_int32),
     ]
 
 

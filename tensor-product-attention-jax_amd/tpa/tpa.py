@@ -121,7 +121,7 @@ def tpa_factors(
     `use_workspace=False` withholds the optional scratch memory, which keeps the call on the
     fused prefill kernel whatever the problem.  `kv_lengths` (int32 [b], an addition): batch
     entry i attends to its first kv_lengths[i] keys only; the rest of its k / v rows is padding
-    that is never read.  `causal_offset` (an addition, forward only): with `causal`, query i
+    that is never read.  `causal_offset` (an addition, also taken by `tpa_factors_bwd`): with `causal`, query i
     sees keys up to i + causal_offset; 0 is the reference's top-left alignment
     (tpa/tpa.py:377-379), lk - lq aligns the last query with the last key (new tokens over a
     cache), and a sequence shard of a ring (tpa/ring_tpa.py:73-79) passes the distance from the
@@ -257,13 +257,15 @@ def tpa_factors_bwd(
     grads=None,
     workspace: torch.Tensor | None = None,
     kernel: int = _d.KERNEL_AUTO,
+    causal_offset: int = 0,
 ):
     """Backward pass on the split factor arrays: the operands of the reference's backward kernel
     launch (tpa/tpa.py:872-958) with a leading batch dimension, `lse` as [b, h, lq] fp32.
 
     Returns the six fp32 gradients (dqa, dqb, dka, dkb, dva, dvb), each shaped like its factor.
     `grads` may hold six fp32 tensors (or views, e.g. the two parts of a concatenated
-    dq[b, lq, rq, h+dk]) to be written in place.
+    dq[b, lq, rq, h+dk]) to be written in place.  `causal_offset`: the value the forward call
+    was made with (see `tpa_factors`).
     """
     device = _pick_device(qa, qb, ka, kb, va, vb)
     qa, qb, ka, kb, va, vb, o, lse, do = (_as_device_tensor(x, device) for x in (qa, qb, ka, kb, va, vb, o, lse, do))
@@ -296,6 +298,7 @@ def tpa_factors_bwd(
         B=b, lq=lq, lk=lk, H=h, dk=dk, dv=dv, rq=rq, rk=rk,
         dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=int(bool(causal)), kernel=int(kernel),
         workspace=workspace.data_ptr() + pad, workspace_bytes=workspace.numel() - pad,
+        causal_offset=int(causal_offset),
     )
     with torch.cuda.device(device):
         _d.check("tpa_bwd", lib.tpa_bwd(args, _d.current_stream_ptr(device)))

@@ -282,3 +282,88 @@ def test_backward_bf16_segment_id_patterns(gpu, pattern, causal):
             assert not np.any(g) and not np.any(w), name  # no pair is visible: every gradient is zero
         else:
             assert rel_err(g, w) <= 1.5e-2, name
+
+
+# ---------------------------------------------------------------- causal mask with an offset (key <= query + offset)
+def _offset_backward_reference(q, k, v, h, sm_scale, offset, do, qseg=None, kvseg=None):
+    """Oracle gradients under the bias `key <= query + offset`, composed from the oracle's parts
+    (reconstruction, dense attention backward, projection onto the factors)."""
+    q, k, v, do = (np.asarray(x, dtype=np.float64) for x in (q, k, v, do))
+    b, lq, lk = q.shape[0], q.shape[1], k.shape[1]
+    bias = orc.attention_bias(b, lq, lk, qseg, kvseg, False)
+    bias = bias + np.where(np.tril(np.ones((lq, lk), dtype=bool), k=offset), 0.0, -np.inf)[None]
+    (qa, qb), (ka, kb), (va, vb) = (orc.split_factors(x, h) for x in (q, k, v))
+    dq_, dk_, dv_ = orc.mha_backward(orc.reconstruct(qa, qb), orc.reconstruct(ka, kb), orc.reconstruct(va, vb), bias, sm_scale, do)
+    cat = lambda pair: np.concatenate(pair, axis=-1)
+    return cat(orc.project_to_factors(dq_, qa, qb)), cat(orc.project_to_factors(dk_, ka, kb)), cat(orc.project_to_factors(dv_, va, vb))
+
+
+@pytest.mark.parametrize(
+    "dt,kernel,b,lq,lk,h,d,rq,rk,offset,seg,tol",
+    [
+        (torch.bfloat16, 2, 2, 384, 768, 2, 128, 6, 2, 384, None, 1.5e-2),   # new tokens over a cache
+        (torch.bfloat16, 2, 1, 300, 700, 2, 64, 2, 2, 77, None, 1.5e-2),     # ragged, diagonal off the tile boundaries
+        (torch.bfloat16, 2, 1, 600, 600, 2, 128, 2, 2, -130, None, 1.5e-2),  # the first 130 rows see nothing
+        (torch.bfloat16, 2, 1, 600, 600, 2, 64, 2, 4, -300, None, 1.5e-2),   # a whole query block sees nothing
+        (torch.bfloat16, 2, 2, 512, 768, 2, 128, 2, 2, 256, 200, 1.5e-2),    # with packed documents
+        (torch.bfloat16, 2, 1, 256, 256, 2, 64, 2, 2, 100000, None, 1.5e-2), # nothing masked
+        (torch.float32, 2, 2, 320, 640, 2, 64, 6, 2, 320, None, 2e-4),       # fp32 matrix-core kernels
+        (torch.float32, 2, 1, 400, 400, 2, 128, 2, 2, -97, 150, 2e-4),
+        (torch.float32, 2, 1, 200, 450, 2, 64, 2, 2, 33, None, 2e-4),
+        (torch.float32, 1, 2, 130, 200, 3, 24, 2, 3, 70, None, 2e-4),        # vector-ALU kernels
+        (torch.float32, 1, 1, 130, 200, 3, 24, 2, 3, -40, 50, 2e-4),
+    ],
+)
+def test_backward_with_causal_offset(gpu, dt, kernel, b, lq, lk, h, d, rq, rk, offset, seg, tol):
+    from tpa import tpa
+
+    q, k, v = make_factors(71, b, lq, lk, h, d, d, rq, rk, scale_by_rank=dt == torch.bfloat16)
+    do = np.random.default_rng(72).standard_normal((b, lq, h, d)).astype(np.float32)
+    qseg = segment_ids(lq, seg, b) if seg else None
+    kvseg = segment_ids(lk, seg, b) if seg else None
+    tq, tk, tv, tdo = (torch.from_numpy(x).to(gpu).to(dt) for x in (q, k, v, do))
+    sp = lambda t: (t[..., :h], t[..., h:])
+    tqs = None if qseg is None else torch.from_numpy(qseg).to(gpu)
+    tks = None if kvseg is None else torch.from_numpy(kvseg).to(gpu)
+    o, lse = tpa.tpa_factors(*sp(tq), *sp(tk), *sp(tv), tqs, tks, d**-0.5, True, causal_offset=offset)
+    grads = tpa.tpa_factors_bwd(*sp(tq), *sp(tk), *sp(tv), tqs, tks, o, lse, tdo, d**-0.5, True, kernel=kernel, causal_offset=offset)
+    f64 = lambda t: t.detach().float().cpu().numpy().astype(np.float64)
+    want = _offset_backward_reference(f64(tq), f64(tk), f64(tv), h, d**-0.5, offset, f64(tdo), qseg, kvseg)
+    for n, (name, w) in enumerate(zip("qkv", want)):
+        got = np.concatenate([f64(grads[2 * n]), f64(grads[2 * n + 1])], axis=-1)
+        assert rel_err(got, w) <= tol, name
+
+
+@pytest.mark.parametrize("dt,tol", [(torch.float32, 2e-4), (torch.bfloat16, 1.5e-2)])
+def test_ring_schedule_backward_emulated_on_one_gpu(gpu, dt, tol):
+    """The backward of a sequence-sharded causal call, the devices replaced by a loop: with the
+    global o, lse and do of its rows, every (query shard, key shard) meeting is one backward block
+    call with the shards' distance as causal offset; dq sums over the key shards a query shard
+    meets, dk / dv over the query shards a key shard meets (what tpa/ring_tpa.py rotates around
+    the ring).  The sums equal the gradients of the unsharded call."""
+    from tpa import tpa
+
+    b, h, d, shards, per = 2, 4, 64, 3, 256
+    t = shards * per
+    q, k, v = make_factors(75, b, t, t, h, d, d, 4, 2, scale_by_rank=dt == torch.bfloat16)
+    do = np.random.default_rng(76).standard_normal((b, t, h, d)).astype(np.float32)
+    tq, tk, tv, tdo = (torch.from_numpy(x).to(gpu).to(dt) for x in (q, k, v, do))
+    sp = lambda x: (x[..., :h], x[..., h:])
+    o, lse = tpa.tpa_factors(*sp(tq), *sp(tk), *sp(tv), None, None, d**-0.5, True)
+    full = tpa.tpa_factors_bwd(*sp(tq), *sp(tk), *sp(tv), None, None, o, lse, tdo, d**-0.5, True)
+    acc = [torch.zeros_like(g) for g in full]
+    for s in range(shards):
+        rows = slice(s * per, (s + 1) * per)
+        for j in range(s + 1):  # key shards after the query shard are invisible to it
+            keys = slice(j * per, (j + 1) * per)
+            g = tpa.tpa_factors_bwd(
+                *sp(tq[:, rows]), *sp(tk[:, keys]), *sp(tv[:, keys]), None, None,
+                o[:, rows], lse[:, :, rows], tdo[:, rows], d**-0.5, True, causal_offset=(s - j) * per,
+            )
+            acc[0][:, rows] += g[0]
+            acc[1][:, rows] += g[1]
+            for n in range(2, 6):
+                acc[n][:, keys] += g[n]
+    f64 = lambda x: x.detach().float().cpu().numpy().astype(np.float64)
+    for a, w in zip(acc, full):
+        assert rel_err(f64(a), f64(w)) <= tol
