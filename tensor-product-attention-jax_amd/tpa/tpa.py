@@ -309,14 +309,14 @@ def bwd_workspace_bytes(b: int, lq: int, lk: int, h: int, dk: int, dv: int) -> i
     return int(_d.load_library().tpa_bwd_workspace_bytes(b, lq, lk, h, dk, dv))
 
 
-def _bwd_concat(q, k, v, qseg, kvseg, o, lse_bhl, do, num_heads, sm_scale, causal):
+def _bwd_concat(q, k, v, qseg, kvseg, o, lse_bhl, do, num_heads, sm_scale, causal, causal_offset=0):
     """Gradients in the concatenated layout of q, k, v (fp32), written in place by the kernels."""
     h = num_heads
     dq, dk, dv = (torch.empty(t.shape, dtype=torch.float32, device=t.device) for t in (q, k, v))
     views = (dq[..., :h], dq[..., h:], dk[..., :h], dk[..., h:], dv[..., :h], dv[..., h:])
     tpa_factors_bwd(
         q[..., :h], q[..., h:], k[..., :h], k[..., h:], v[..., :h], v[..., h:],
-        qseg, kvseg, o, lse_bhl, do, sm_scale, causal, grads=views,
+        qseg, kvseg, o, lse_bhl, do, sm_scale, causal, grads=views, causal_offset=causal_offset,
     )
     return dq, dk, dv
 
@@ -325,26 +325,27 @@ class _TpaFunction(torch.autograd.Function):
     """The operator with its vjp, as tpa.defvjp(_tpa_fwd, _tpa_bwd) registers it (tpa/tpa.py:217)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, num_heads, qseg, kvseg, sm_scale, causal, kernel):
+    def forward(ctx, q, k, v, num_heads, qseg, kvseg, sm_scale, causal, kernel, causal_offset=0):
         qa, qb = q[..., :num_heads], q[..., num_heads:]
         ka, kb = k[..., :num_heads], k[..., num_heads:]
         va, vb = v[..., :num_heads], v[..., num_heads:]
-        o, lse = tpa_factors(qa, qb, ka, kb, va, vb, qseg, kvseg, sm_scale, causal, kernel)
+        o, lse = tpa_factors(qa, qb, ka, kb, va, vb, qseg, kvseg, sm_scale, causal, kernel, causal_offset=causal_offset)
         ctx.mark_non_differentiable(lse)
         ctx.save_for_backward(q, k, v, o, lse)
-        ctx.statics = (num_heads, qseg, kvseg, sm_scale, causal)
+        ctx.statics = (num_heads, qseg, kvseg, sm_scale, causal, causal_offset)
         return o, lse
 
     @staticmethod
     def backward(ctx, do, _dlse):
         q, k, v, o, lse = ctx.saved_tensors
-        num_heads, qseg, kvseg, sm_scale, causal = ctx.statics
-        dq, dk, dv = _bwd_concat(q, k, v, qseg, kvseg, o, lse, do, num_heads, sm_scale, causal)
-        return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None, None, None, None, None
+        num_heads, qseg, kvseg, sm_scale, causal, causal_offset = ctx.statics
+        dq, dk, dv = _bwd_concat(q, k, v, qseg, kvseg, o, lse, do, num_heads, sm_scale, causal, causal_offset)
+        return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None, None, None, None, None, None
 
 
 def _tpa_fwd(
-    q, k, v, num_heads, q_segment_ids, kv_segment_ids, sm_scale, causal, block_sizes, nomat, debug, interpret
+    q, k, v, num_heads, q_segment_ids, kv_segment_ids, sm_scale, causal, block_sizes, nomat, debug, interpret,
+    causal_offset: int = 0,
 ):
     """tpa/tpa.py:124-165: returns (o, residuals) with residuals (q, k, v, qseg, kvseg, o, l),
     l[b, lq, h] being the logsumexp in the reference's layout (a transposed view, fp32)."""
@@ -358,7 +359,7 @@ def _tpa_fwd(
     assert tuple(k.shape) == (b, lk, rk, h_dk), k.shape  # tpa/tpa.py:475
     assert 0 < num_heads < h_dk and num_heads < v.shape[-1], (num_heads, q.shape, v.shape)
     kernel = _d.KERNEL_GENERIC if interpret else _d.KERNEL_AUTO
-    o, lse = _TpaFunction.apply(q, k, v, int(num_heads), q_segment_ids, kv_segment_ids, float(sm_scale), bool(causal), kernel)
+    o, lse = _TpaFunction.apply(q, k, v, int(num_heads), q_segment_ids, kv_segment_ids, float(sm_scale), bool(causal), kernel, int(causal_offset))
     l = lse.permute(0, 2, 1)
     return o, (q, k, v, q_segment_ids, kv_segment_ids, o, l)
 
@@ -374,16 +375,19 @@ def tpa(
     nomat: bool = False,
     debug: bool = False,
     interpret: bool = False,
+    causal_offset: int = 0,
 ):
     """Tensor Product Attention (tpa/tpa.py:73-121).
 
     q[b,lq,rq,h+dk], k[b,lk,rk,h+dk], v[b,lk,rk,h+dv]: rank factors concatenated along the
     last dimension, head factor first.  Returns o[b,lq,h,dv] in q's dtype.  numpy inputs give a
-    numpy result.
+    numpy result.  `causal_offset` (an addition, differentiable like the rest): with `causal`,
+    query i sees keys up to i + causal_offset instead of i (see `tpa_factors`).
     """
     was_numpy = not isinstance(q, torch.Tensor)
     o, _ = _tpa_fwd(
-        q, k, v, num_heads, q_segment_ids, kv_segment_ids, sm_scale, causal, block_sizes, nomat, debug, interpret
+        q, k, v, num_heads, q_segment_ids, kv_segment_ids, sm_scale, causal, block_sizes, nomat, debug, interpret,
+        causal_offset=causal_offset,
     )
     return o.cpu().numpy() if was_numpy and o.dtype != torch.bfloat16 else o
 

@@ -367,3 +367,17 @@ def test_ring_schedule_backward_emulated_on_one_gpu(gpu, dt, tol):
     f64 = lambda x: x.detach().float().cpu().numpy().astype(np.float64)
     for a, w in zip(acc, full):
         assert rel_err(f64(a), f64(w)) <= tol
+
+
+def test_causal_offset_through_autograd(gpu):
+    """tpa(..., causal=True, causal_offset=lk - lq): new tokens over a cache, forward and gradients."""
+    from tpa import tpa
+
+    b, lq, lk, h, d = 2, 192, 448, 4, 64
+    q, k, v = make_factors(79, b, lq, lk, h, d, d, 3, 2)
+    tq, tk, tv = (torch.from_numpy(x).to(gpu).requires_grad_() for x in (q, k, v))
+    o = tpa.tpa(tq, tk, tv, num_heads=h, sm_scale=d**-0.5, causal=True, causal_offset=lk - lq)
+    torch.nansum(o).backward()
+    want = _offset_backward_reference(q, k, v, h, d**-0.5, lk - lq, np.ones((b, lq, h, d)))
+    for name, t, w in zip("qkv", (tq, tk, tv), want):
+        assert rel_err(t.grad.cpu().numpy(), w) <= 2e-4, name
