@@ -375,6 +375,7 @@ def tpa(
     nomat: bool = False,
     debug: bool = False,
     interpret: bool = False,
+    *,
     causal_offset: int = 0,
 ):
     """Tensor Product Attention (tpa/tpa.py:73-121).

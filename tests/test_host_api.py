@@ -24,12 +24,14 @@ def test_signature_matches_the_reference():
 
     from tpa import mha, tpa
 
-    params = list(inspect.signature(tpa.tpa).parameters)
-    assert params == [
+    sig = inspect.signature(tpa.tpa)
+    params = list(sig.parameters)
+    assert params[:12] == [
         "q", "k", "v", "num_heads", "q_segment_ids", "kv_segment_ids", "sm_scale", "causal",
         "block_sizes", "nomat", "debug", "interpret",
     ]  # tpa/tpa.py:74-87
-    sig = inspect.signature(tpa.tpa)
+    # additions can only be named, so a positional call of the reference means the same here
+    assert all(sig.parameters[n].kind is inspect.Parameter.KEYWORD_ONLY for n in params[12:])
     assert sig.parameters["sm_scale"].default == 1.0 and sig.parameters["causal"].default is False
     assert list(inspect.signature(mha.mha).parameters)[:5] == ["q", "k", "v", "bias", "sm_scale"]  # tpa/mha.py:11-17
 
