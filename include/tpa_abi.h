@@ -52,6 +52,11 @@ enum {
   TPA_KERNEL_MFMA = 2     /* MFMA kernels only; TPA_ERR_UNSUPPORTED if the problem does not qualify */
 };
 
+/* values of the `causal` fields */
+#define TPA_CAUSAL_NONE 0
+#define TPA_CAUSAL_TOP_LEFT 1     /* the reference's mask (tpa/tpa.py:377-379) */
+#define TPA_CAUSAL_BOTTOM_RIGHT 2 /* an addition: see TpaFwdArgs.causal_offset */
+
 /*
  * One factor array: A factors a[b, l, r, h] or B factors b[b, l, r, d].  The innermost
  * dimension is contiguous; the other three have ELEMENT strides, so both the split arrays
@@ -90,7 +95,8 @@ typedef struct TpaFwdArgs {
   int32_t B, lq, lk, H, dk, dv, rq, rk;
   int32_t dtype;  /* TPA_DTYPE_*: element type of the six factor arrays and of o */
   float sm_scale; /* multiplies the logits after the dot product (tpa/tpa.py:367) */
-  int32_t causal; /* non-zero: key index <= query index, top-left aligned (tpa/tpa.py:377-379) */
+  int32_t causal; /* TPA_CAUSAL_*: 0 none; 1 key index <= query index, top-left aligned (tpa/tpa.py:377-379);
+                     2 the last query aligned with the last key of each batch entry */
   int32_t kernel; /* TPA_KERNEL_* */
   void* workspace;        /* required by tpa_decode (split partials); optional for tpa_fwd (tpa_fwd_workspace_bytes) */
   size_t workspace_bytes; /* size of workspace */
@@ -106,7 +112,10 @@ typedef struct TpaFwdArgs {
   const int32_t* page_table; /* [B, pages_per_seq] or NULL */
   int32_t page_size;         /* tokens per page */
   int32_t pages_per_seq;     /* entries per row of page_table */
-  /* With causal != 0: key index <= query index + causal_offset.  0 is the reference's top-left alignment
+  /* With causal == TPA_CAUSAL_BOTTOM_RIGHT the offset below counts from (keys of the batch entry - lq), the keys of
+     an entry being min(kv_lengths[b], lk): lq freshly appended tokens per sequence of a ragged batch, each masked to
+     its predecessors, need no offset at all.
+     With causal != 0: key index <= query index + causal_offset.  0 is the reference's top-left alignment
      (tpa/tpa.py:377-379); lk - lq aligns the last query with the last key (a chunk of new tokens over a
      cache); a sequence shard passes the distance between its first query and the first key of the key shard
      it meets (tpa/ring_tpa.py:73-79 calls the block function with local indices only).  Rows that see no key

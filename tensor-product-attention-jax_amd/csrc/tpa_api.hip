@@ -17,6 +17,7 @@ int validate_tpa(const TpaFwdArgs* a) {
   if (!a->o) return TPA_ERR_NULL;
   // segment ids come in pairs (tpa/tpa.py:369-371)
   if ((a->q_segment_ids == nullptr) != (a->kv_segment_ids == nullptr)) return TPA_ERR_NULL;
+  if (a->causal < TPA_CAUSAL_NONE || a->causal > TPA_CAUSAL_BOTTOM_RIGHT) return TPA_ERR_UNSUPPORTED;
   if (a->kernel != TPA_KERNEL_AUTO && a->kernel != TPA_KERNEL_GENERIC && a->kernel != TPA_KERNEL_MFMA)
     return TPA_ERR_UNSUPPORTED;
   return TPA_OK;

@@ -126,13 +126,19 @@ __device__ __forceinline__ int xcd_pair_slot(int round, int xcd, int B) {
 // Causal offset of a forward call as the kernels take it: row i sees keys <= i + offset.  Offsets
 // of lk and more mask nothing and offsets of -lq and less mask everything, so the value is clamped
 // to that range (keeps the kernels' index arithmetic far from overflow); 0 without the causal mask.
+// With TPA_CAUSAL_BOTTOM_RIGHT the forward kernels add (keys of the batch entry - lq) themselves, since
+// that differs per entry under kv_lengths; the range is then twice as wide.
+inline int clamp_causal_offset(int offset, int lo, int hi) { return offset < lo ? lo : (offset > hi ? hi : offset); }
 inline int causal_offset_of(const TpaFwdArgs* a) {
   if (!a->causal) return 0;
-  return a->causal_offset < -a->lq ? -a->lq : (a->causal_offset > a->lk ? a->lk : a->causal_offset);
+  if (a->causal == TPA_CAUSAL_BOTTOM_RIGHT) return clamp_causal_offset(a->causal_offset, -a->lq - a->lk, a->lq + a->lk);
+  return clamp_causal_offset(a->causal_offset, -a->lq, a->lk);
 }
+// the backward takes no kv_lengths, so bottom-right alignment is the fixed offset lk - lq
 inline int causal_offset_of(const TpaBwdArgs* a) {
   if (!a->causal) return 0;
-  return a->causal_offset < -a->lq ? -a->lq : (a->causal_offset > a->lk ? a->lk : a->causal_offset);
+  const int base = a->causal == TPA_CAUSAL_BOTTOM_RIGHT ? a->lk - a->lq : 0;
+  return clamp_causal_offset(clamp_causal_offset(a->causal_offset, -a->lq - a->lk, a->lq + a->lk) + base, -a->lq, a->lk);
 }
 
 // Raise a kernel's dynamic LDS limit above the 64 KB a kernel gets without asking.  The attribute

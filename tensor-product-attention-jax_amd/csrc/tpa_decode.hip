@@ -36,6 +36,7 @@ struct DecodeParams {
   int page_size, pages_per_seq;  // tokens per page; table row length
   int B, lq, lk, H, rq;
   int climit;      // query row qi sees its first qi + climit keys (causal: offset + 1; otherwise lk, no limit)
+  int cbr;         // causal, last query aligned with the last key of each batch entry: climit counts from len - lq
   int S;           // key ranges
   float qscale;    // sm_scale * log2(e) / (rq * rk)
 };
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   int row_last[NQ], len_b = 0;
 #pragma unroll
   for (int r = 0; r < NQ; ++r) {
-    const int len_r = max(0, min(len_all, min(qi0 + r, p.lq - 1) + p.climit));
+    const int len_r = max(0, min(len_all, min(qi0 + r, p.lq - 1) + p.climit + (p.cbr ? len_all - p.lq : 0)));
     row_last[r] = len_r * RK - 1;
     len_b = max(len_b, len_r);
   }
@@ -445,7 +446,8 @@ __global__ __launch_bounds__(kWaves * 64) void decode_f32_kernel(DecodeParams p)
 
   const int nparts = S * kWaves;
   const int part = split * kWaves + w;
-  const int len_b = max(0, min(p.kvlen ? min(p.kvlen[b], p.lk) : p.lk, qi + p.climit));
+  const int len_all = p.kvlen ? min(p.kvlen[b], p.lk) : p.lk;
+  const int len_b = max(0, min(len_all, qi + p.climit + (p.cbr ? len_all - p.lq : 0)));
   const int blk_begin = part;
   const int blk_end = (len_b * RK + kRowsPerBlock - 1) / kRowsPerBlock;
   const int blk_step = nparts;
@@ -705,6 +707,7 @@ int launch_decode_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.S = S;
   p.kvlen = a->kv_lengths;
   p.climit = a->causal ? causal_offset_of(a) + 1 : a->lk;
+  p.cbr = a->causal == TPA_CAUSAL_BOTTOM_RIGHT;
   p.page_table = a->page_table; p.page_size = a->page_size; p.pages_per_seq = a->pages_per_seq;
   p.qscale = a->sm_scale * kLog2e / ((float)a->rq * (float)RK);
   auto kern = decode_kernel<D, RK, PAGED, NQ>;
@@ -728,6 +731,7 @@ int launch_decode_f32_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.S = S;
   p.kvlen = a->kv_lengths;
   p.climit = a->causal ? causal_offset_of(a) + 1 : a->lk;
+  p.cbr = a->causal == TPA_CAUSAL_BOTTOM_RIGHT;
   p.page_table = a->page_table; p.page_size = a->page_size; p.pages_per_seq = a->pages_per_seq;
   p.qscale = a->sm_scale * kLog2e / ((float)a->rq * (float)RK);
   auto kern = decode_f32_kernel<D, RK, PAGED>;

@@ -77,9 +77,10 @@ __global__ __launch_bounds__(kRows) void generic_fwd_kernel(GenericParams p) {
 
   // keys this workgroup has to visit
   int k_end = p.kvlen ? max(0, min(p.kvlen[b], p.lk)) : p.lk;
+  const int coff = p.coff + (p.causal == TPA_CAUSAL_BOTTOM_RIGHT ? k_end - p.lq : 0);  // counted from the end of this entry's keys
   if (p.causal) {
     const int last_row = min(p.lq, (int)(blockIdx.x + 1) * kRows) - 1;
-    k_end = min(k_end, last_row + 1 + p.coff);
+    k_end = min(k_end, last_row + 1 + coff);
   }
 
   for (int k0 = 0; k0 < k_end; k0 += kTile) {
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(kRows) void generic_fwd_kernel(GenericParams p) {
         if (p.bias) x += p.bias[((int64_t)b * p.lq + row) * p.lk + k0 + t];
         bool keep = true;
         if (p.kvseg) keep = segs[t] == qseg;
-        if (p.causal) keep = keep && (k0 + t <= row + p.coff);
+        if (p.causal) keep = keep && (k0 + t <= row + coff);
         if (!keep) x = -INFINITY;
       }
       s[t] = x;
@@ -216,7 +217,8 @@ __global__ __launch_bounds__(kFewThreads) void generic_fewrows_kernel(GenericPar
   }
   const int qseg = p.qseg ? p.qseg[(int64_t)b * p.lq + row] : 0;
   int k_end = p.kvlen ? max(0, min(p.kvlen[b], p.lk)) : p.lk;
-  if (p.causal) k_end = min(k_end, row + 1 + p.coff);
+  const int coff = p.coff + (p.causal == TPA_CAUSAL_BOTTOM_RIGHT ? k_end - p.lq : 0);  // counted from the end of this entry's keys
+  if (p.causal) k_end = min(k_end, row + 1 + coff);
   const float inv_rk = 1.f / (float)p.rk;
 
   float m = -INFINITY, l = 0.f, acc = 0.f;  // acc: o[tid] for tid < dv
@@ -371,7 +373,7 @@ int mha_generic_launch(const MhaFwdArgs* a, hipStream_t stream) {
   p.qseg = nullptr; p.kvseg = nullptr; p.bias = a->bias;
   p.o = a->o; p.lse = a->lse;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.dk = a->dk; p.dv = a->dv; p.rq = 1; p.rk = 1;
-  p.sm_scale = a->sm_scale; p.causal = a->causal; p.dense = 1;
+  p.sm_scale = a->sm_scale; p.causal = a->causal ? TPA_CAUSAL_TOP_LEFT : TPA_CAUSAL_NONE; p.dense = 1;
   if (a->B > 65535 || a->H > 65535) return TPA_ERR_SHAPE;
   if (a->dtype == TPA_DTYPE_F32) return tpa::launch_generic<float>(p, stream);
   if (a->dtype == TPA_DTYPE_BF16) return tpa::launch_generic<uint16_t>(p, stream);

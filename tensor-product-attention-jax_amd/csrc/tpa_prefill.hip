@@ -217,7 +217,10 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   // ---- key range [kpos0, kend) this workgroup visits; tiles are counted from kpos0
   int kpos0 = 0;
   const int len_b = p.kvlen ? max(0, min(p.kvlen[b], p.lk)) : p.lk;  // keys of this batch entry
-  int kend = p.causal ? min(len_b, min(q0 + kBQ, p.lq) + p.coff) : len_b;
+  // causal offset of this batch entry: counted from the end of its keys where the caller aligns the last
+  // query with the last key
+  const int coff = p.coff + (p.causal == TPA_CAUSAL_BOTTOM_RIGHT ? len_b - p.lq : 0);
+  int kend = p.causal ? min(len_b, min(q0 + kBQ, p.lq) + coff) : len_b;
   if (kend <= 0) {  // no key at all: the rows end as NaN / -inf (tpa/tpa.py:437-439)
     if (qrow < p.lq) {
       uint16_t* op = p.o + (((int64_t)b * p.lq + qrow) * p.H + h) * D;
@@ -287,8 +290,8 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   const int lk_r = kend - kpos0;          // keys counted from kpos0
   // this wave's first row and this lane's row on that scale, shifted by the causal offset: row r
   // sees keys up to r_r, which is negative for a row that sees none
-  const int wrow_r = wrow0 + p.coff - kpos0;
-  const int qrow_r = qrow + p.coff - kpos0;
+  const int wrow_r = wrow0 + coff - kpos0;
+  const int qrow_r = qrow + coff - kpos0;
   const int ntiles = (lk_r + kTK - 1) / kTK;
   const int last = ntiles - 1;
   // last tile this wave needs under the causal mask (its rows: wrow0 .. wrow0 + 31)
@@ -1010,7 +1013,7 @@ int mha_prefill_mfma_launch(const MhaFwdArgs* a, hipStream_t stream) {
   p.qa = p.ka = p.va = TpaFactor{nullptr, 0, 0, 0};
   p.o = static_cast<uint16_t*>(a->o); p.lse = a->lse;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = 1; p.rk = 1;
-  p.sm_scale = a->sm_scale; p.causal = a->causal; p.coff = 0;
+  p.sm_scale = a->sm_scale; p.causal = a->causal ? TPA_CAUSAL_TOP_LEFT : TPA_CAUSAL_NONE; p.coff = 0;
   p.nqb = (a->lq + kBQ - 1) / kBQ;
   p.npairs = p.nqb * a->B;
   if (a->dk == 128) return launch_prefill<128, LOAD_DENSE>(p, stream);

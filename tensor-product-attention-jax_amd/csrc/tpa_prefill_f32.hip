@@ -89,7 +89,8 @@ __global__ __launch_bounds__(kNW * 64) void prefill_f32_kernel(F32Params pp) {
 
   // ---- key range
   const int len_b = p.kvlen ? max(0, min(p.kvlen[b], p.lk)) : p.lk;
-  const int kend = p.causal ? min(len_b, min(q0 + kBQ, p.lq) + p.coff) : len_b;
+  const int coff = p.coff + (p.causal == TPA_CAUSAL_BOTTOM_RIGHT ? len_b - p.lq : 0);  // bottom-right alignment counts from the end of this entry's keys
+  const int kend = p.causal ? min(len_b, min(q0 + kBQ, p.lq) + coff) : len_b;
   float* const orow = p.o + (((int64_t)b * p.lq + qrow) * p.H + h) * D;
   if (kend <= 0) {  // no key at all: the rows end as NaN / -inf (tpa/tpa.py:437-439)
     if (qrow < p.lq) {
@@ -101,7 +102,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_f32_kernel(F32Params pp) {
     return;
   }
   const int ntiles = (kend + kTK - 1) / kTK;
-  const int wave_last_tile = p.causal ? min(ntiles - 1, max(wrow0 + p.coff + 31, 0) / kTK) : ntiles - 1;
+  const int wave_last_tile = p.causal ? min(ntiles - 1, max(wrow0 + coff + 31, 0) / kTK) : ntiles - 1;
 
   // ---- Q (B operand of S^T = K Q^T), scaled: qf[4m + e] = c * Q[qrow][8m + 4g + e]
   float qf[NQ];
@@ -186,9 +187,9 @@ __global__ __launch_bounds__(kNW * 64) void prefill_f32_kernel(F32Params pp) {
       }
     }
     // register v of block mb, wave half g  <->  key k0 + 32 mb + 8 (v / 4) + 4 g + v % 4
-    const bool need_mask = (k0 + kTK > kend) || (p.causal && (k0 + kTK - 1 > wrow0 + p.coff));
+    const bool need_mask = (k0 + kTK > kend) || (p.causal && (k0 + kTK - 1 > wrow0 + coff));
     if (need_mask) {
-      const int limit = p.causal ? min(qrow + p.coff, kend - 1) : kend - 1;  // largest visible key index
+      const int limit = p.causal ? min(qrow + coff, kend - 1) : kend - 1;  // largest visible key index
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
@@ -341,7 +342,7 @@ int mha_prefill_f32_launch(const MhaFwdArgs* a, hipStream_t stream) {
   p.qa = p.ka = p.va = TpaFactor{nullptr, 0, 0, 0};
   p.o = static_cast<float*>(a->o); p.lse = a->lse;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = 1; p.rk = 1;
-  p.sm_scale = a->sm_scale; p.causal = a->causal;
+  p.sm_scale = a->sm_scale; p.causal = a->causal ? TPA_CAUSAL_TOP_LEFT : TPA_CAUSAL_NONE;
   p.nqb = (a->lq + kBQ - 1) / kBQ;
   p.npairs = p.nqb * a->B;
   return launch_any(p, a->dk, stream);

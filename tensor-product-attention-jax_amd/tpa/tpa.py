@@ -63,6 +63,22 @@ def _lse_accum(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     return torch.where(torch.isneginf(hi), hi, lse)
 
 
+CAUSAL_BOTTOM_RIGHT = 2  # value of `causal`: the last query aligned with the last key of each batch entry
+
+
+def _causal_code(causal) -> int:
+    """False / True as in the reference (tpa/tpa.py:82; True = top-left aligned mask), or
+    CAUSAL_BOTTOM_RIGHT (an addition): the mask counted from the end of each batch entry's keys
+    (`kv_lengths[b]` where given), so that the last query sees every key, the one before it all
+    but the last, ... - freshly appended tokens over caches of different lengths."""
+    if causal is True or causal is False:
+        return int(causal)
+    code = int(causal)
+    if code not in (0, 1, CAUSAL_BOTTOM_RIGHT):
+        raise ValueError(f"causal must be False, True or CAUSAL_BOTTOM_RIGHT, got {causal!r}")
+    return code
+
+
 def _as_device_tensor(x, device):
     """torch GPU tensors pass through; numpy arrays / CPU tensors are copied to `device`."""
     if isinstance(x, torch.Tensor):
@@ -167,7 +183,7 @@ def tpa_factors(
         kv_segment_ids=kvseg.data_ptr() if kvseg is not None else None,
         o=o.data_ptr(), lse=lse.data_ptr() if lse is not None else None,
         B=b, lq=lq, lk=lk, H=h, dk=dk, dv=dv, rq=rq, rk=rk,
-        dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=int(bool(causal)), kernel=int(kernel),
+        dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=_causal_code(causal), kernel=int(kernel),
         workspace=ws_ptr, workspace_bytes=ws_bytes, num_splits=0,
         kv_lengths=kvlen.data_ptr() if kvlen is not None else None,
         causal_offset=int(causal_offset),
@@ -232,7 +248,7 @@ def tpa_decode(
         qa=_d.factor(qa), qb=_d.factor(qb), ka=_d.factor(ka), kb=_d.factor(kb), va=_d.factor(va), vb=_d.factor(vb),
         q_segment_ids=None, kv_segment_ids=None, o=o.data_ptr(), lse=lse.data_ptr(),
         B=b, lq=lq, lk=lk, H=h, dk=dk, dv=dv, rq=rq, rk=rk,
-        dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=int(bool(causal)), kernel=int(kernel),
+        dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=_causal_code(causal), kernel=int(kernel),
         workspace=workspace.data_ptr(), workspace_bytes=workspace.numel() * workspace.element_size(),
         num_splits=int(num_splits),
         kv_lengths=kvlen.data_ptr() if kvlen is not None else None,
@@ -296,7 +312,7 @@ def tpa_factors_bwd(
         dqa=_d.grad(grads[0]), dqb=_d.grad(grads[1]), dka=_d.grad(grads[2]), dkb=_d.grad(grads[3]),
         dva=_d.grad(grads[4]), dvb=_d.grad(grads[5]),
         B=b, lq=lq, lk=lk, H=h, dk=dk, dv=dv, rq=rq, rk=rk,
-        dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=int(bool(causal)), kernel=int(kernel),
+        dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=_causal_code(causal), kernel=int(kernel),
         workspace=workspace.data_ptr() + pad, workspace_bytes=workspace.numel() - pad,
         causal_offset=int(causal_offset),
     )
@@ -359,7 +375,7 @@ def _tpa_fwd(
     assert tuple(k.shape) == (b, lk, rk, h_dk), k.shape  # tpa/tpa.py:475
     assert 0 < num_heads < h_dk and num_heads < v.shape[-1], (num_heads, q.shape, v.shape)
     kernel = _d.KERNEL_GENERIC if interpret else _d.KERNEL_AUTO
-    o, lse = _TpaFunction.apply(q, k, v, int(num_heads), q_segment_ids, kv_segment_ids, float(sm_scale), bool(causal), kernel, int(causal_offset))
+    o, lse = _TpaFunction.apply(q, k, v, int(num_heads), q_segment_ids, kv_segment_ids, float(sm_scale), _causal_code(causal), kernel, int(causal_offset))
     l = lse.permute(0, 2, 1)
     return o, (q, k, v, q_segment_ids, kv_segment_ids, o, l)
 
@@ -412,7 +428,7 @@ def _tpa_bwd(num_heads, sm_scale, causal, block_sizes, nomat, debug, interpret, 
     q, k, v, q_segment_ids, kv_segment_ids, o, l = residuals
     device = _pick_device(q, k, v)
     q, k, v, o, l, do = (_as_device_tensor(x, device) for x in (q, k, v, o, l, do))
-    dq, dk, dv = _bwd_concat(q, k, v, q_segment_ids, kv_segment_ids, o, l.permute(0, 2, 1), do, int(num_heads), float(sm_scale), bool(causal))
+    dq, dk, dv = _bwd_concat(q, k, v, q_segment_ids, kv_segment_ids, o, l.permute(0, 2, 1), do, int(num_heads), float(sm_scale), _causal_code(causal))
     return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None
 
 

@@ -381,3 +381,22 @@ def test_causal_offset_through_autograd(gpu):
     want = _offset_backward_reference(q, k, v, h, d**-0.5, lk - lq, np.ones((b, lq, h, d)))
     for name, t, w in zip("qkv", (tq, tk, tv), want):
         assert rel_err(t.grad.cpu().numpy(), w) <= 2e-4, name
+
+
+def test_backward_bottom_right_alignment_is_the_offset_lk_minus_lq(gpu):
+    """Without per-sequence lengths (which the backward does not take) CAUSAL_BOTTOM_RIGHT is the
+    fixed offset lk - lq, forward and backward: the same launches, equal bits."""
+    from tpa import tpa
+
+    b, lq, lk, h, d = 2, 200, 456, 2, 64
+    q, k, v = make_factors(81, b, lq, lk, h, d, d, 3, 2)
+    do = np.random.default_rng(82).standard_normal((b, lq, h, d)).astype(np.float32)
+    tq, tk, tv, tdo = (torch.from_numpy(x).to(gpu) for x in (q, k, v, do))
+    sp = lambda t: (t[..., :h], t[..., h:])
+    outs = []
+    for causal, off in ((tpa.CAUSAL_BOTTOM_RIGHT, 0), (True, lk - lq)):
+        o, lse = tpa.tpa_factors(*sp(tq), *sp(tk), *sp(tv), None, None, d**-0.5, causal, causal_offset=off)
+        g = tpa.tpa_factors_bwd(*sp(tq), *sp(tk), *sp(tv), None, None, o, lse, tdo, d**-0.5, causal, causal_offset=off)
+        outs.append((o, lse) + tuple(g))
+    for x, y in zip(*outs):
+        assert torch.equal(x, y)

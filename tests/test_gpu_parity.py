@@ -954,6 +954,68 @@ def test_decode_with_a_causal_limit_per_query_row(gpu, dt, b, lq, lk, h, d, rq, 
     assert torch.equal(torch.nan_to_num(o2.float(), nan=7.0), torch.nan_to_num(o.float(), nan=7.0)) and torch.equal(lse2, lse)
 
 
+def _bottom_right_reference(q, k, v, lengths, h, sm_scale, extra=0):
+    """Per batch entry: the oracle on its first lengths[b] keys with the diagonal through (last query, last key)."""
+    lq = q.shape[1]
+    os_, ls_ = [], []
+    for bi, n in enumerate(lengths):
+        if n == 0:
+            os_.append(np.full((1, lq, h, v.shape[-1] - h), np.nan))
+            ls_.append(np.full((1, lq, h), -np.inf))
+            continue
+        o, l_ = _offset_reference(q[bi : bi + 1], k[bi : bi + 1, :n], v[bi : bi + 1, :n], h, sm_scale, n - lq + extra)
+        os_.append(o)
+        ls_.append(l_)
+    return np.concatenate(os_), np.concatenate(ls_)
+
+
+@pytest.mark.parametrize(
+    "dt,kernel,lq,lk,h,d,rq,rk,lengths,extra",
+    [
+        (torch.bfloat16, 2, 4, 2048, 16, 128, 6, 2, [2048, 1001, 3], 0),   # split-key decode: appended tokens, ragged caches
+        (torch.bfloat16, 2, 7, 1536, 8, 64, 2, 4, [1536, 9, 700], 0),
+        (torch.float32, 2, 3, 1200, 8, 64, 2, 2, [1200, 640, 2], 0),
+        (torch.bfloat16, 2, 300, 700, 2, 128, 6, 2, [700, 450, 301], 0),    # prefill: a chunk of new tokens per sequence
+        (torch.bfloat16, 2, 300, 700, 2, 128, 2, 2, [700, 450, 120], -5),   # shorter than the chunk: its first rows see nothing
+        (torch.bfloat16, 2, 320, 640, 2, 64, 2, 4, [640, 333, 500], 0),     # through dense K and V
+        (torch.float32, 2, 260, 520, 2, 128, 2, 2, [520, 300, 261], 3),
+        (torch.float32, 1, 130, 200, 3, 24, 2, 3, [200, 131, 7], 0),        # vector-ALU kernel
+        (torch.float32, 1, 3, 1500, 2, 40, 2, 2, [1500, 900, 1], 0),        # few-rows vector kernel
+    ],
+)
+def test_causal_mask_aligned_with_the_end_of_each_sequence(gpu, dt, kernel, lq, lk, h, d, rq, rk, lengths, extra):
+    from tpa import tpa
+
+    b = len(lengths)
+    q, k, v = make_factors(160, b, lq, lk, h, d, d, rq, rk, scale_by_rank=dt == torch.bfloat16)
+    tq, tk, tv = (to_gpu(x, dt, gpu) for x in (q, k, v))
+    kvl = torch.tensor(lengths, dtype=torch.int32, device=gpu)
+    sm_scale = d**-0.5
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=sm_scale, causal=tpa.CAUSAL_BOTTOM_RIGHT, kernel=kernel,
+                             kv_lengths=kvl, causal_offset=extra)
+    o_ref, l_ref = _bottom_right_reference(as_f64(tq), as_f64(tk), as_f64(tv), lengths, h, sm_scale, extra)
+    check(o, lse, o_ref, l_ref, F32_TOL if dt == torch.float32 else BF16_TOL)
+    if lq <= 16 and kernel == 2:  # the same through tpa_decode, contiguous and as a pool of shuffled pages
+        o2, lse2 = tpa.tpa_decode(*split(tq, tk, tv, h), sm_scale=sm_scale, kernel=2, kv_lengths=kvl,
+                                  causal=tpa.CAUSAL_BOTTOM_RIGHT, causal_offset=extra)
+        same = lambda x, y: torch.equal(torch.nan_to_num(x.float(), nan=7.0), torch.nan_to_num(y.float(), nan=7.0))
+        assert same(o2, o) and torch.equal(lse2, lse)
+        page_size = 16
+        assert lk % page_size == 0
+        pages_per_seq = lk // page_size
+        perm = torch.from_numpy(np.random.default_rng(161).permutation(2 * b * pages_per_seq)[: b * pages_per_seq].astype(np.int32)).reshape(b, pages_per_seq)
+        pool_k = torch.full((2 * b * pages_per_seq, page_size, rk, h + d), float("nan"), dtype=dt, device=gpu)
+        pool_v = torch.full_like(pool_k, float("nan"))
+        for bi in range(b):
+            for pg in range(pages_per_seq):
+                pool_k[perm[bi, pg]] = tk[bi, pg * page_size : (pg + 1) * page_size]
+                pool_v[perm[bi, pg]] = tv[bi, pg * page_size : (pg + 1) * page_size]
+        o3, lse3 = tpa.tpa_decode(tq[..., :h].contiguous(), tq[..., h:].contiguous(), pool_k[..., :h].contiguous(), pool_k[..., h:].contiguous(),
+                                  pool_v[..., :h].contiguous(), pool_v[..., h:].contiguous(), sm_scale=sm_scale, kernel=2, kv_lengths=kvl,
+                                  page_table=perm, causal=tpa.CAUSAL_BOTTOM_RIGHT, causal_offset=extra)
+        assert same(o3, o) and torch.equal(lse3, lse)
+
+
 # ---------------------------------------------------------------- the ring schedule, one GPU standing in for all shards
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dt,shards", [(torch.float32, 4), (torch.bfloat16, 3)])
