@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c4pg|c5|c2f|c3f|c2fb|c4f|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|copy] [--no-cpu] [--no-decode] [--no-backward]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c4pg|c4s|c5|c2f|c3f|c2fb|c4f|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|copy] [--no-cpu] [--no-decode] [--no-backward]
 
 A step is one forward pass over one batch of synthetic, seeded inputs that are resident in HBM
 before the timed region starts.  The default workload is the prefill configuration the headline
@@ -35,6 +35,7 @@ WORKLOADS = {
     "c5": ("prefill", 8, 2048, 2048, 64, 64, 16, 8, False),
     "c4": ("decode", 64, 1, 8192, 32, 128, 6, 2, False),
     "c4pg": ("decode", 64, 1, 8192, 32, 128, 6, 2, False),  # the c4 cache as a pool of shuffled 64-token pages
+    "c4s": ("decode", 64, 4, 8192, 32, 128, 6, 2, True),  # four appended tokens per sequence, each masked to its predecessors
     # dense flash attention (tpa/mha.py) at the prefill shapes: the same-shape baseline
     "c2m": ("dense", 4, 4096, 4096, 16, 128, 0, 0, True),
     "c3m": ("dense", 1, 32768, 32768, 32, 128, 0, 0, True),
@@ -191,7 +192,8 @@ def run_backward(torch, tpa, device, name, steps, warmup):
 
 
 def run_decode(torch, tpa, device, name, steps, warmup):
-    _, B, lq, lk, H, D, rq, rk, _ = WORKLOADS[name]
+    _, B, lq, lk, H, D, rq, rk, causal = WORKLOADS[name]
+    causal = tpa.CAUSAL_BOTTOM_RIGHT if causal else False
     # two distinct caches, alternated, so that no launch finds its cache in the 256 MB last-level cache
     f32 = name in F32_WORKLOADS
     xs = [make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed=s, dtype=torch.float32 if f32 else None) for s in (0, 1)]
@@ -208,7 +210,7 @@ def run_decode(torch, tpa, device, name, steps, warmup):
         xs = [x[:2] + tuple(t.reshape(B * lk // page, page, rk, t.shape[-1]) for t in x[2:]) for x in xs]
 
     def step(i):
-        out["o"], out["lse"] = tpa.tpa_decode(*xs[i & 1], sm_scale=scale, workspace=ws, kernel=2, page_table=table)
+        out["o"], out["lse"] = tpa.tpa_decode(*xs[i & 1], sm_scale=scale, workspace=ws, kernel=2, page_table=table, causal=causal)
 
     wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
     nbytes = decode_bytes(B, lq, lk, H, D, rq, rk, elem=4 if f32 else 2)
