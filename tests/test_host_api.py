@@ -91,3 +91,15 @@ def test_product_package_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cc", "Makefile")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert not pat.search(text), os.path.join(dirpath, f)
+
+
+def test_causal_argument_values():
+    """False / True as in the reference (tpa/tpa.py:82), CAUSAL_BOTTOM_RIGHT as the one addition; anything else raises."""
+    from tpa import tpa
+
+    assert tpa._causal_code(False) == 0 and tpa._causal_code(True) == 1
+    assert tpa._causal_code(np.bool_(True)) == 1 and tpa._causal_code(0) == 0
+    assert tpa._causal_code(tpa.CAUSAL_BOTTOM_RIGHT) == 2
+    for bad in (3, -1):
+        with pytest.raises(ValueError):
+            tpa._causal_code(bad)
