@@ -400,3 +400,39 @@ def test_backward_bottom_right_alignment_is_the_offset_lk_minus_lq(gpu):
         outs.append((o, lse) + tuple(g))
     for x, y in zip(*outs):
         assert torch.equal(x, y)
+
+
+@pytest.mark.parametrize("rank_q", [1, 6])
+@pytest.mark.parametrize("rank_k", [1, 4])
+@pytest.mark.parametrize("batch_size,lq,lk,h,dim_k,dim_v", [(1, 8, 8, 1, 4, 6), (2, 1024, 128, 2, 3, 5), (2, 128, 1024, 2, 3, 5), (1, 1024, 1024, 2, 3, 5)])
+def test_ring_schedule_backward_on_the_references_ring_grid(gpu, batch_size, rank_q, rank_k, lq, lk, h, dim_k, dim_v):
+    """The grid of the reference's ring backward test (tpa/ring_tpa_test.py:141-233: eight sequence
+    shards, uniform inputs, segment ids position // 42, d nansum(o), atol 1e-3 / rtol 1e-2), the
+    devices replaced by a loop: a block backward per (query shard, key shard) meeting with the
+    global o and lse of the rows, dq summed over key shards, dk / dv over query shards."""
+    from tpa import tpa
+
+    shards = 8
+    q, k, v = make_factors(190, batch_size, lq, lk, h, dim_k, dim_v, rank_q, rank_k, dist="uniform")
+    qseg, kvseg = segment_ids(lq, 42, batch_size), segment_ids(lk, 42, batch_size)
+    tq, tk, tv = (torch.from_numpy(x).to(gpu) for x in (q, k, v))
+    tqs, tks = torch.from_numpy(qseg).to(gpu), torch.from_numpy(kvseg).to(gpu)
+    sp = lambda t: (t[..., :h], t[..., h:])
+    o, lse = tpa.tpa_factors(*sp(tq), *sp(tk), *sp(tv), tqs, tks, 1.0, False)
+    do = torch.ones_like(o)  # d nansum(o) / d o; rows that are NaN take no gradient
+    acc = [torch.zeros(t.shape, dtype=torch.float32, device=gpu) for x in (tq, tk, tv) for t in sp(x)]
+    pq, pk = lq // shards, lk // shards
+    for s in range(shards):
+        rows = slice(s * pq, (s + 1) * pq)
+        for j in range(shards):
+            keys = slice(j * pk, (j + 1) * pk)
+            g = tpa.tpa_factors_bwd(*sp(tq[:, rows]), *sp(tk[:, keys]), *sp(tv[:, keys]), tqs[:, rows], tks[:, keys],
+                                    o[:, rows], lse[:, :, rows], do[:, rows], 1.0, False)
+            acc[0][:, rows] += g[0]
+            acc[1][:, rows] += g[1]
+            for n in range(2, 6):
+                acc[n][:, keys] += g[n]
+    want = orc.tpa_backward(q, k, v, qseg, kvseg, h, np.ones((batch_size, lq, h, dim_v)), sm_scale=1.0, causal=False)
+    for n, w in enumerate(want):
+        got = torch.cat([acc[2 * n], acc[2 * n + 1]], dim=-1).cpu().numpy()
+        np.testing.assert_allclose(got, w, atol=1e-3, rtol=1e-2)

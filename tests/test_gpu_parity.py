@@ -1061,3 +1061,39 @@ def test_ring_schedule_emulated_on_one_gpu(gpu, dt, shards, causal):
     assert (torch.nan_to_num(o_ring) - torch.nan_to_num(o_full.float())).abs().max().item() <= tol
     o_ref, _ = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), seg, seg, h, sm_scale=d**-0.5, causal=causal)
     assert np.nanmax(np.abs(as_f64(o_ring) - o_ref)) <= tol
+
+
+@pytest.mark.parametrize("rank_q", [1, 6])
+@pytest.mark.parametrize("rank_k", [1, 4])
+@pytest.mark.parametrize("batch_size,lq,lk,h,dk,dv", [(1, 16, 16, 1, 4, 6), (2, 1024, 128, 4, 32, 8), (2, 128, 1024, 4, 32, 8)])
+def test_ring_schedule_on_the_references_ring_grid(gpu, batch_size, rank_q, rank_k, lq, lk, h, dk, dv):
+    """The grid of the reference's ring test (tpa/ring_tpa_test.py:60-140: eight sequence shards,
+    uniform inputs, segment ids position // 42, sm_scale 1, no causal mask, tolerance 1e-3; run
+    here at 1e-4), with the eight devices replaced by a loop over the schedule."""
+    from tpa import tpa
+
+    shards = 8
+    q, k, v = make_factors(180, batch_size, lq, lk, h, dk, dv, rank_q, rank_k, dist="uniform")
+    qseg, kvseg = segment_ids(lq, 42, batch_size), segment_ids(lk, 42, batch_size)
+    tq, tk, tv = (to_gpu(x, torch.float32, gpu) for x in (q, k, v))
+    tqs, tks = torch.from_numpy(qseg).to(gpu), torch.from_numpy(kvseg).to(gpu)
+    pq, pk = lq // shards, lk // shards
+    outs = []
+    for s in range(shards):
+        qs, qsid = tq[:, s * pq : (s + 1) * pq], tqs[:, s * pq : (s + 1) * pq]
+        o = torch.zeros((batch_size, pq, h, dv), dtype=torch.float32, device=gpu)
+        l = torch.full((batch_size, pq, h), float("-inf"), dtype=torch.float32, device=gpu)
+        for i in range(shards):
+            j = (s - i) % shards
+            sl = slice(j * pk, (j + 1) * pk)
+            o_, res = tpa._tpa_fwd(qs, tk[:, sl], tv[:, sl], h, qsid, tks[:, sl], 1.0, False, None, False, False, False)
+            l_ = res[-1]
+            l_next = tpa._lse_accum(l, l_)
+            o = torch.nan_to_num(o * torch.exp(l - l_next)[..., None], nan=0.0)
+            o = o + torch.nan_to_num(o_ * torch.exp(l_ - l_next)[..., None], nan=0.0)
+            l = l_next
+        outs.append(torch.where(torch.isneginf(l)[..., None], torch.full_like(o, float("nan")), o))
+    o_ring = as_f64(torch.cat(outs, dim=1))
+    o_ref, _ = orc.tpa_reference(q, k, v, qseg, kvseg, h, sm_scale=1.0)
+    np.testing.assert_array_equal(np.isnan(o_ring), np.isnan(o_ref))
+    assert np.nanmax(np.abs(o_ring - o_ref), initial=0.0) <= F32_TOL
