@@ -401,6 +401,16 @@ def test_abi_error_codes(gpu):
     with pytest.raises(d.TpaError) as e:
         tpa.tpa_factors(x[..., :4], x[..., 4:], x[..., :4], x[..., 4:], x[..., :4], x[..., 4:], kernel=d.KERNEL_MFMA)
     assert e.value.code == -6
+    # a value of `causal` the library does not know (the Python layer refuses it first, so straight through the ABI)
+    o = torch.empty((1, 8, 4, 3), device=gpu)
+    args = d.TpaFwdArgs(
+        qa=d.factor(x[..., :4]), qb=d.factor(x[..., 4:]), ka=d.factor(x[..., :4]), kb=d.factor(x[..., 4:]),
+        va=d.factor(x[..., :4]), vb=d.factor(x[..., 4:]), o=o.data_ptr(), B=1, lq=8, lk=8, H=4, dk=3, dv=3, rq=1, rk=1,
+        dtype=d.dtype_code(torch.float32), sm_scale=1.0, causal=3, kernel=d.KERNEL_AUTO,
+    )
+    assert d.load_library().tpa_fwd(args, d.current_stream_ptr(gpu)) == -6
+    with pytest.raises(ValueError):
+        tpa.tpa_factors(x[..., :4], x[..., 4:], x[..., :4], x[..., 4:], x[..., :4], x[..., 4:], causal=3)
 
 
 # ---------------------------------------------------------------- dense decode (split over keys)
