@@ -770,11 +770,13 @@ int launch_decode(const TpaFwdArgs* a, int S, hipStream_t stream) {
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
 
-int default_splits(int B, int lq, int lk, int H) {
+int default_splits(int B, int lq, int lk, int H, int rows_per_group = 2) {
   // one workgroup per CU is resident (the kernel keeps a block of loads in flight in registers),
-  // so aim for a whole number of waves of 256 workgroups and at least 4 blocks per wave
-  // (the bf16 kernel serves two query rows per workgroup)
-  const int groups = B * ((lq + 1) / 2) * ((H + 31) / 32);
+  // so aim for a whole number of waves of 256 workgroups and at least 4 blocks per wave.
+  // The bf16 kernel serves two query rows per workgroup, which is what callers are told to size
+  // the workspace for; the fp32 kernel serves one, launches twice the workgroups per range and so
+  // asks for at most as many ranges (and never more workspace).
+  const int groups = B * ((lq + rows_per_group - 1) / rows_per_group) * ((H + 31) / 32);
   int S = (256 + groups - 1) / groups;
   if (groups >= 256) S = 1;
   const int max_s = (lk + 4 * kWaves * 16 - 1) / (4 * kWaves * 16);
@@ -860,7 +862,7 @@ int tpa_decode_f32_supported(const TpaFwdArgs* a) {
 
 int tpa_decode_f32_launch(const TpaFwdArgs* a, hipStream_t stream) {
   using namespace tpa;
-  const int S = a->num_splits > 0 ? a->num_splits : default_splits(a->B, a->lq, a->lk, a->H);
+  const int S = a->num_splits > 0 ? a->num_splits : default_splits(a->B, a->lq, a->lk, a->H, 1);
   if (S > 65535 || (int64_t)a->B * S > 2147483647LL) return TPA_ERR_SHAPE;
   if (!a->workspace || a->workspace_bytes < workspace_bytes(a->B, a->lq, a->H, a->dv, S)) return TPA_ERR_WORKSPACE;
   if (!aligned16(a->workspace)) return TPA_ERR_ALIGN;
