@@ -15,7 +15,9 @@
  *     work enqueued on `stream` has completed;
  *   - calls only enqueue work on `stream` (a hipStream_t passed as void*; NULL = the null
  *     stream); they never synchronise, allocate or free device memory, throw or abort;
- *   - return 0 on success or a negative TPA_ERR_* code, with nothing enqueued on error;
+ *   - return 0 on success or a negative TPA_ERR_* code; an argument that fails validation is
+ *     reported before anything is enqueued (TPA_ERR_LAUNCH, the runtime refusing one launch of a
+ *     call that makes several, can leave the earlier ones enqueued);
  *   - re-entrant: may be called concurrently from several host threads.
  */
 #ifndef TPA_ABI_H_
@@ -253,7 +255,9 @@ int tpa_decode(const TpaFwdArgs* args, void* stream);
 /* Bytes of workspace tpa_decode needs for this problem (num_splits = 0: the default choice). */
 size_t tpa_decode_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dv, int32_t num_splits);
 
-/* Number of key ranges tpa_decode uses when args->num_splits == 0. */
+/* Number of key ranges tpa_decode_workspace_bytes sizes the workspace for when num_splits == 0: what
+   the bf16 kernel uses, and an upper bound on what the fp32 kernel uses (it serves one query row per
+   workgroup and so asks for at most as many ranges). */
 int32_t tpa_decode_default_splits(int32_t B, int32_t lq, int32_t lk, int32_t H);
 
 /* Dense attention forward with the layouts of tpa/mha.py:11-17 (see MhaFwdArgs). */

@@ -5,7 +5,9 @@ namespace {
 
 int check_factor(const TpaFactor& f) { return f.ptr == nullptr ? TPA_ERR_NULL : TPA_OK; }
 
-int validate_tpa(const TpaFwdArgs* a) {
+}  // namespace
+
+int tpa_validate_fwd_args(const TpaFwdArgs* a) {
   if (!a) return TPA_ERR_NULL;
   if (a->dtype != TPA_DTYPE_F32 && a->dtype != TPA_DTYPE_BF16) return TPA_ERR_DTYPE;
   if (a->B <= 0 || a->lq <= 0 || a->lk <= 0 || a->H <= 0 || a->dk <= 0 || a->dv <= 0 || a->rq <= 0 || a->rk <= 0)
@@ -23,12 +25,15 @@ int validate_tpa(const TpaFwdArgs* a) {
   return TPA_OK;
 }
 
+namespace {
+
 int validate_mha(const MhaFwdArgs* a) {
   if (!a) return TPA_ERR_NULL;
   if (a->dtype != TPA_DTYPE_F32 && a->dtype != TPA_DTYPE_BF16) return TPA_ERR_DTYPE;
   if (a->B <= 0 || a->lq <= 0 || a->lk <= 0 || a->H <= 0 || a->dk <= 0 || a->dv <= 0) return TPA_ERR_SHAPE;
   if (a->dk > 256 || a->dv > 256) return TPA_ERR_SHAPE;
   if (!a->q || !a->k || !a->v || !a->o) return TPA_ERR_NULL;
+  if (a->causal != 0 && a->causal != 1) return TPA_ERR_UNSUPPORTED;  // dense attention knows the top-left mask only
   if (a->kernel != TPA_KERNEL_AUTO && a->kernel != TPA_KERNEL_GENERIC && a->kernel != TPA_KERNEL_MFMA)
     return TPA_ERR_UNSUPPORTED;
   return TPA_OK;
@@ -55,7 +60,7 @@ const char* tpa_strerror(int code) {
 }
 
 int tpa_fwd(const TpaFwdArgs* a, void* stream) {
-  const int rc = validate_tpa(a);
+  const int rc = tpa_validate_fwd_args(a);
   if (rc != TPA_OK) return rc;
   if (a->page_table) return TPA_ERR_UNSUPPORTED;  // paged caches are read by tpa_decode only
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -86,7 +91,7 @@ size_t tpa_fwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int
 }
 
 int tpa_decode(const TpaFwdArgs* a, void* stream) {
-  const int rc = validate_tpa(a);
+  const int rc = tpa_validate_fwd_args(a);
   if (rc != TPA_OK) return rc;
   if (a->q_segment_ids) return TPA_ERR_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -124,6 +129,7 @@ int tpa_bwd(const TpaBwdArgs* a, void* stream) {
     if (!g->ptr) return TPA_ERR_NULL;
   if (!a->o || !a->lse || !a->d_o) return TPA_ERR_NULL;
   if ((a->q_segment_ids == nullptr) != (a->kv_segment_ids == nullptr)) return TPA_ERR_NULL;
+  if (a->causal < TPA_CAUSAL_NONE || a->causal > TPA_CAUSAL_BOTTOM_RIGHT) return TPA_ERR_UNSUPPORTED;
   if (a->kernel != TPA_KERNEL_AUTO && a->kernel != TPA_KERNEL_GENERIC && a->kernel != TPA_KERNEL_MFMA)
     return TPA_ERR_UNSUPPORTED;
   // matrix-core kernels: bf16 ones for bf16 inputs, fp32 ones for fp32 inputs; both read do with 16-byte loads
@@ -149,6 +155,7 @@ int mha_bwd(const MhaBwdArgs* a, void* stream) {
   if (a->B <= 0 || a->lq <= 0 || a->lk <= 0 || a->H <= 0 || a->dk <= 0 || a->dv <= 0) return TPA_ERR_SHAPE;
   if (a->dk > 256 || a->dv > 256) return TPA_ERR_SHAPE;
   if (!a->q || !a->k || !a->v || !a->o || !a->lse || !a->d_o || !a->dq || !a->dk_out || !a->dv_out) return TPA_ERR_NULL;
+  if (a->causal != 0 && a->causal != 1) return TPA_ERR_UNSUPPORTED;  // dense attention knows the top-left mask only
   if (a->kernel != TPA_KERNEL_AUTO && a->kernel != TPA_KERNEL_GENERIC && a->kernel != TPA_KERNEL_MFMA)
     return TPA_ERR_UNSUPPORTED;
   const int mfma = a->kernel != TPA_KERNEL_GENERIC &&

@@ -157,6 +157,7 @@ inline int raise_lds_limit(bool (&done)[kMaxDevices], const void* kern, size_t b
 }  // namespace tpa
 
 // host-side entry points of the individual kernel files (launchers return TPA_* codes)
+int tpa_validate_fwd_args(const TpaFwdArgs* a);  // the checks every forward entry point makes first
 int tpa_generic_launch(const TpaFwdArgs* a, hipStream_t stream);
 int mha_generic_launch(const MhaFwdArgs* a, hipStream_t stream);
 int tpa_prefill_mfma_supported(const TpaFwdArgs* a);

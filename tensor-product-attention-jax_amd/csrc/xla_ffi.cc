@@ -5,6 +5,8 @@
 // k[b,lk,rk,h+dk], v[b,lk,rk,h+dv], read in place through strides.
 //
 // Not part of `make`: it needs the XLA FFI headers (python -c "import jax; print(jax.ffi.include_dir())").
+// SOURCE ONLY: no XLA headers exist where this library is built and tested, so this file has never
+// been through a compiler; every tested path binds the C ABI directly.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -50,6 +52,14 @@ ffi::Error fill(TpaFwdArgs* a, const ffi::AnyBuffer& q, const ffi::AnyBuffer& k,
   if (kd[0] != qd[0] || vd[0] != qd[0] || kd[1] != vd[1] || kd[2] != vd[2] || kd[3] != qd[3] || num_heads <= 0 ||
       qd[3] <= num_heads || vd[3] <= num_heads)
     return ffi::Error::InvalidArgument("inconsistent q / k / v shapes");
+  // results: o[b, lq, h, dv] in the input type, lse[b, h, lq] fp32 (NOT the reference's l[b, lq, h] in
+  // the input type, tpa/tpa.py:530: a caller that declares that shape for bf16 would be written past)
+  const auto od = o->dimensions(), ld = lse->dimensions();
+  if (o->element_type() != q.element_type() || od.size() != 4 || od[0] != qd[0] || od[1] != qd[1] || od[2] != num_heads ||
+      od[3] != vd[3] - num_heads)
+    return ffi::Error::InvalidArgument("o must be [b, lq, h, dv] in the type of q");
+  if (lse->element_type() != ffi::DataType::F32 || ld.size() != 3 || ld[0] != qd[0] || ld[1] != num_heads || ld[2] != qd[1])
+    return ffi::Error::InvalidArgument("lse must be f32 [b, h, lq]");
   *a = TpaFwdArgs{};
   split(q, num_heads, code, &a->qa, &a->qb);
   split(k, num_heads, code, &a->ka, &a->kb);
@@ -63,21 +73,41 @@ ffi::Error fill(TpaFwdArgs* a, const ffi::AnyBuffer& q, const ffi::AnyBuffer& k,
   return ffi::Error::Success();
 }
 
+// workspace: an extra u8 result of max(tpa_fwd_workspace_bytes(...), 1) bytes allocated by XLA (256-byte aligned,
+// as XLA's buffers are), with which tpa_fwd picks the split-key decode kernel or the dense-K/V route where
+// they are faster; a one-byte buffer keeps every call on the fused prefill kernel
+void attach_workspace(TpaFwdArgs* a, ffi::Result<ffi::AnyBuffer>& workspace) {
+  const size_t need = tpa_fwd_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dk, a->dv, a->rq, a->rk);
+  if (need && workspace->size_bytes() >= need) {
+    a->workspace = workspace->untyped_data();
+    a->workspace_bytes = workspace->size_bytes();
+  }
+}
+
+bool seg_ok(const ffi::Buffer<ffi::DataType::S32>& ids, int64_t b, int64_t l) {
+  const auto d = ids.dimensions();
+  return d.size() == 2 && d[0] == b && d[1] == l;
+}
+
 ffi::Error TpaFwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v,
-                      ffi::Result<ffi::AnyBuffer> o, ffi::Result<ffi::AnyBuffer> lse, int32_t num_heads,
-                      float sm_scale, bool causal) {
+                      ffi::Result<ffi::AnyBuffer> o, ffi::Result<ffi::AnyBuffer> lse,
+                      ffi::Result<ffi::AnyBuffer> workspace, int32_t num_heads, float sm_scale, bool causal) {
   TpaFwdArgs a;
   if (ffi::Error e = fill(&a, q, k, v, o, lse, num_heads, sm_scale, causal); e.failure()) return e;
+  attach_workspace(&a, workspace);
   const int rc = tpa_fwd(&a, stream);
   return rc == TPA_OK ? ffi::Error::Success() : fail(rc);
 }
 
 ffi::Error TpaFwdSegImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v,
                          ffi::Buffer<ffi::DataType::S32> q_segment_ids, ffi::Buffer<ffi::DataType::S32> kv_segment_ids,
-                         ffi::Result<ffi::AnyBuffer> o, ffi::Result<ffi::AnyBuffer> lse, int32_t num_heads,
-                         float sm_scale, bool causal) {
+                         ffi::Result<ffi::AnyBuffer> o, ffi::Result<ffi::AnyBuffer> lse,
+                         ffi::Result<ffi::AnyBuffer> workspace, int32_t num_heads, float sm_scale, bool causal) {
   TpaFwdArgs a;
   if (ffi::Error e = fill(&a, q, k, v, o, lse, num_heads, sm_scale, causal); e.failure()) return e;
+  if (!seg_ok(q_segment_ids, a.B, a.lq) || !seg_ok(kv_segment_ids, a.B, a.lk))
+    return ffi::Error::InvalidArgument("segment ids must be s32 [b, lq] and [b, lk]");
+  attach_workspace(&a, workspace);
   a.q_segment_ids = q_segment_ids.typed_data();
   a.kv_segment_ids = kv_segment_ids.typed_data();
   const int rc = tpa_fwd(&a, stream);
@@ -102,6 +132,12 @@ ffi::Error MhaFwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ff
                       ffi::Result<ffi::AnyBuffer> workspace, float sm_scale, bool causal) {
   const auto qd = q.dimensions(), kd = k.dimensions(), vd = v.dimensions();
   if (qd.size() != 4 || kd.size() != 4 || vd.size() != 4) return ffi::Error::InvalidArgument("q, k, v must be [b, l, h, d]");
+  const auto od = o->dimensions(), ld = lse->dimensions();
+  if (k.element_type() != q.element_type() || v.element_type() != q.element_type() || o->element_type() != q.element_type() ||
+      od.size() != 4 || od[0] != qd[0] || od[1] != qd[1] || od[2] != qd[2] || od[3] != vd[3])
+    return ffi::Error::InvalidArgument("q, k, v, o must share one type; o is [b, lq, h, dv]");
+  if (lse->element_type() != ffi::DataType::F32 || ld.size() != 3 || ld[0] != qd[0] || ld[1] != qd[2] || ld[2] != qd[1])
+    return ffi::Error::InvalidArgument("lse must be f32 [b, h, lq]");
   MhaFwdArgs a{};
   a.q = q.untyped_data(); a.k = k.untyped_data(); a.v = v.untyped_data();
   a.o = o->untyped_data(); a.lse = static_cast<float*>(lse->untyped_data());
@@ -140,6 +176,10 @@ ffi::Error TpaBwdCommon(hipStream_t stream, const ffi::AnyBuffer& q, const ffi::
   if (lse.element_type() != ffi::DataType::F32 || dq->element_type() != ffi::DataType::F32 ||
       dk->element_type() != ffi::DataType::F32 || dv->element_type() != ffi::DataType::F32)
     return ffi::Error::InvalidArgument("lse and the gradients are f32");
+  const auto ld = lse.dimensions();
+  if (ld.size() != 3 || ld[0] != qd[0] || ld[1] != num_heads || ld[2] != qd[1]) return ffi::Error::InvalidArgument("lse must be [b, h, lq]");
+  if (dq->dimensions() != qd || dk->dimensions() != kd || dv->dimensions() != vd || o.dimensions() != d_o.dimensions())
+    return ffi::Error::InvalidArgument("gradients are shaped like q, k, v; do like o");
   TpaBwdArgs a{};
   split(q, num_heads, code, &a.qa, &a.qb);
   split(k, num_heads, code, &a.ka, &a.kb);
@@ -170,6 +210,9 @@ ffi::Error TpaBwdSegImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k,
                          ffi::AnyBuffer o, ffi::AnyBuffer lse, ffi::AnyBuffer d_o, ffi::Result<ffi::AnyBuffer> dq,
                          ffi::Result<ffi::AnyBuffer> dk, ffi::Result<ffi::AnyBuffer> dv,
                          ffi::Result<ffi::AnyBuffer> workspace, int32_t num_heads, float sm_scale, bool causal) {
+  const auto qd = q.dimensions(), kd = k.dimensions();
+  if (qd.size() != 4 || kd.size() != 4 || !seg_ok(q_segment_ids, qd[0], qd[1]) || !seg_ok(kv_segment_ids, kd[0], kd[1]))
+    return ffi::Error::InvalidArgument("segment ids must be s32 [b, lq] and [b, lk]");
   return TpaBwdCommon(stream, q, k, v, q_segment_ids.typed_data(), kv_segment_ids.typed_data(), o, lse, d_o, dq, dk, dv,
                       workspace, num_heads, sm_scale, causal);
 }
@@ -197,7 +240,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(TpaFwd, TpaFwdImpl,
                               ffi::Ffi::Bind()
                                   .Ctx<ffi::PlatformStream<hipStream_t>>()
                                   .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
-                                  .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
+                                  .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
                                   .Attr<int32_t>("num_heads").Attr<float>("sm_scale").Attr<bool>("causal"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(TpaFwdSeg, TpaFwdSegImpl,
@@ -205,7 +248,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(TpaFwdSeg, TpaFwdSegImpl,
                                   .Ctx<ffi::PlatformStream<hipStream_t>>()
                                   .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
                                   .Arg<ffi::Buffer<ffi::DataType::S32>>().Arg<ffi::Buffer<ffi::DataType::S32>>()
-                                  .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
+                                  .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
                                   .Attr<int32_t>("num_heads").Attr<float>("sm_scale").Attr<bool>("causal"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(TpaDecode, TpaDecodeImpl,

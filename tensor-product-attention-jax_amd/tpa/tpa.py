@@ -281,7 +281,9 @@ def tpa_factors_bwd(
     Returns the six fp32 gradients (dqa, dqb, dka, dkb, dva, dvb), each shaped like its factor.
     `grads` may hold six fp32 tensors (or views, e.g. the two parts of a concatenated
     dq[b, lq, rq, h+dk]) to be written in place.  `causal_offset`: the value the forward call
-    was made with (see `tpa_factors`).
+    was made with (see `tpa_factors`).  There is no `kv_lengths` here: the backward reads all lk
+    keys, so the gradients of a forward that was made with `kv_lengths` are not available (slice
+    the batch entries to their lengths instead).
     """
     device = _pick_device(qa, qb, ka, kb, va, vb)
     qa, qb, ka, kb, va, vb, o, lse, do = (_as_device_tensor(x, device) for x in (qa, qb, ka, kb, va, vb, o, lse, do))
@@ -421,14 +423,17 @@ def _fwd(
     return o[0], res[-1][0]
 
 
-def _tpa_bwd(num_heads, sm_scale, causal, block_sizes, nomat, debug, interpret, residuals, do):
+def _tpa_bwd(num_heads, sm_scale, causal, block_sizes, nomat, debug, interpret, residuals, do, *, causal_offset: int = 0):
     """tpa/tpa.py:168-214: (dq, dk, dv, None, None) from the residuals `_tpa_fwd` returned, in the
-    dtype and the concatenated layout of q, k, v."""
+    dtype and the concatenated layout of q, k, v.  The residuals carry no causal offset (they have
+    the reference's seven entries), so a forward made with `causal_offset != 0` must hand the same
+    value to this call."""
     del block_sizes, nomat, debug, interpret
     q, k, v, q_segment_ids, kv_segment_ids, o, l = residuals
     device = _pick_device(q, k, v)
     q, k, v, o, l, do = (_as_device_tensor(x, device) for x in (q, k, v, o, l, do))
-    dq, dk, dv = _bwd_concat(q, k, v, q_segment_ids, kv_segment_ids, o, l.permute(0, 2, 1), do, int(num_heads), float(sm_scale), _causal_code(causal))
+    dq, dk, dv = _bwd_concat(q, k, v, q_segment_ids, kv_segment_ids, o, l.permute(0, 2, 1), do, int(num_heads), float(sm_scale), _causal_code(causal),
+                             int(causal_offset))
     return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None
 
 

@@ -114,6 +114,32 @@ def test_null_and_shape_errors_are_reported_before_any_launch():
     assert lib.mha_bwd(None, None) == -1
 
 
+def test_unknown_causal_values_are_refused_by_every_entry_point():
+    """`causal` outside the declared values is an error in the forward and in the backward calls
+    (checked before the workspace and before any launch; the pointers below are never read)."""
+    from tpa import _dispatch as d
+
+    lib = d.load_library()
+    fake = d.TpaFactor(256, 0, 0, 0)
+    fwd = d.TpaFwdArgs(qa=fake, qb=fake, ka=fake, kb=fake, va=fake, vb=fake, o=256, B=1, lq=1, lk=1, H=1, dk=1, dv=1, rq=1, rk=1,
+                       dtype=d.TPA_DTYPE_F32, causal=3)
+    assert lib.tpa_fwd(ctypes.byref(fwd), None) == -6
+    assert lib.tpa_decode(ctypes.byref(fwd), None) == -6
+    g = d.TpaGrad(256, 0, 0, 0)
+    for bad in (3, -1):
+        bwd = d.TpaBwdArgs(qa=fake, qb=fake, ka=fake, kb=fake, va=fake, vb=fake, o=256, lse=256, d_o=256,
+                           dqa=g, dqb=g, dka=g, dkb=g, dva=g, dvb=g, B=1, lq=1, lk=1, H=1, dk=1, dv=1, rq=1, rk=1,
+                           dtype=d.TPA_DTYPE_F32, causal=bad)
+        assert lib.tpa_bwd(ctypes.byref(bwd), None) == -6
+    bwd.causal = 2  # a known value passes this check and stops at the missing workspace
+    assert lib.tpa_bwd(ctypes.byref(bwd), None) == -5
+    mf = d.MhaFwdArgs(q=256, k=256, v=256, o=256, B=1, lq=1, lk=1, H=1, dk=1, dv=1, dtype=d.TPA_DTYPE_F32, causal=2)
+    assert lib.mha_fwd(ctypes.byref(mf), None) == -6
+    mb = d.MhaBwdArgs(q=256, k=256, v=256, o=256, lse=256, d_o=256, dq=256, dk_out=256, dv_out=256,
+                      B=1, lq=1, lk=1, H=1, dk=1, dv=1, dtype=d.TPA_DTYPE_F32, causal=2)
+    assert lib.mha_bwd(ctypes.byref(mb), None) == -6
+
+
 def test_missing_library_fails_loudly(tmp_path):
     from tpa import _dispatch
 

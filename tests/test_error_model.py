@@ -1,0 +1,50 @@
+"""The bf16 error model (tests/error_model.py) against a numpy emulation of the bf16 prefill
+kernel's rounding points: the bound holds, is not vacuous, and on benchmark-like inputs the
+emulated errors stay inside the absolute gates stated for the benchmark configurations."""
+
+import numpy as np
+import torch
+
+from conftest import bf16_round, make_factors
+from error_model import emulate_bf16_prefill, round_bf16, tpa_bounds
+from oracle import tpa_oracle as orc
+
+
+def test_round_bf16_matches_torch():
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(4096) * 10.0 ** rng.integers(-6, 6, 4096), [0.0, 1.0, 1.00390625, 1.01171875, -3.0]])
+    want = torch.from_numpy(x.astype(np.float32)).to(torch.bfloat16).to(torch.float64).numpy()
+    np.testing.assert_array_equal(round_bf16(x), want)
+
+
+def _errors(seed, b, lq, lk, h, d, rq, rk, scaled, causal):
+    q, k, v = (bf16_round(x) for x in make_factors(seed, b, lq, lk, h, d, d, rq, rk, scale_by_rank=scaled))
+    scale = d**-0.5
+    o_ref, l_ref = orc.tpa_reference(q, k, v, None, None, h, sm_scale=scale, causal=causal)
+    o, l = emulate_bf16_prefill(q, k, v, h, scale, causal)
+    lse_b, o_b = tpa_bounds(q, k, v, h, scale)
+    return np.abs(o - o_ref).max(-1), np.abs(l - l_ref), o_b, lse_b
+
+
+def test_bound_holds_and_is_not_vacuous_on_sharp_inputs():
+    # unscaled N(0,1) factors, query rank one: logits of order ten
+    eo, el, o_b, lse_b = _errors(1, 2, 96, 160, 4, 128, 1, 2, False, True)
+    assert (eo <= o_b).all() and (el <= lse_b).all()
+    assert el.max() > 2e-3, "this distribution is the one where the absolute 1e-3 does not hold"
+    # the worst row comes within a factor of 40 of its bound (the bound is a sum of absolute
+    # values, the error a sum of signed terms: sqrt(D) apart at best)
+    assert (el / lse_b).max() > 1 / 40 and (eo / o_b).max() > 1 / 40
+
+
+def test_bound_stays_inside_the_absolute_gates_on_benchmark_like_inputs():
+    # N(0,1)/sqrt(R) factors, ranks 6/2, D = 128: the distribution of the benchmark configurations
+    eo, el, o_b, lse_b = _errors(2, 1, 128, 256, 4, 128, 6, 2, True, True)
+    assert (eo <= o_b).all() and (el <= lse_b).all()
+    # the worst-case bound (sums of absolute values) is a few 1e-3 here; the errors themselves
+    # (signed sums) stay inside the absolute gates stated for the benchmark configurations
+    assert lse_b.max() <= 5e-3 and o_b.max() <= 5e-2
+    assert el.max() <= 1e-3 and eo.max() <= 2e-2
+    # the factored form (decode kernels) bounds the materialised one
+    q, k, v = (bf16_round(x) for x in make_factors(2, 1, 128, 256, 4, 128, 128, 6, 2, scale_by_rank=True))
+    lse_f, o_f = tpa_bounds(q, k, v, 4, 128**-0.5, form="factored")
+    assert (lse_f >= lse_b).all() and (o_f >= o_b).all()

@@ -383,6 +383,22 @@ def test_causal_offset_through_autograd(gpu):
         assert rel_err(t.grad.cpu().numpy(), w) <= 2e-4, name
 
 
+def test_causal_offset_through_the_residual_interface(gpu):
+    """_tpa_fwd(..., causal_offset=) followed by _tpa_bwd(residuals, do, causal_offset=): the residuals
+    hold the reference's seven entries and no offset, so the backward call is given the same value."""
+    from tpa import tpa
+
+    b, lq, lk, h, d = 2, 192, 448, 4, 64
+    q, k, v = make_factors(80, b, lq, lk, h, d, d, 3, 2)
+    tq, tk, tv = (torch.from_numpy(x).to(gpu) for x in (q, k, v))
+    o, res = tpa._tpa_fwd(tq, tk, tv, h, None, None, d**-0.5, True, None, False, False, False, causal_offset=lk - lq)
+    do = torch.ones_like(o)
+    got = tpa._tpa_bwd(h, d**-0.5, True, None, False, False, False, res, do, causal_offset=lk - lq)
+    want = _offset_backward_reference(q, k, v, h, d**-0.5, lk - lq, np.ones((b, lq, h, d)))
+    for name, t, w in zip("qkv", got[:3], want):
+        assert rel_err(t.cpu().numpy(), w) <= 2e-4, name
+
+
 def test_backward_bottom_right_alignment_is_the_offset_lk_minus_lq(gpu):
     """Without per-sequence lengths (which the backward does not take) CAUSAL_BOTTOM_RIGHT is the
     fixed offset lk - lq, forward and backward: the same launches, equal bits."""

@@ -55,8 +55,11 @@ def test_backward_signatures_and_delta():
     from tpa import tpa
 
     # tpa/tpa.py:168-178 and tpa/tpa.py:823-839
-    assert list(inspect.signature(tpa._tpa_bwd).parameters) == [
-        "num_heads", "sm_scale", "causal", "block_sizes", "nomat", "debug", "interpret", "residuals", "do"]
+    # (the reference's positional parameters, then the keyword-only addition for the causal offset)
+    params = inspect.signature(tpa._tpa_bwd).parameters
+    assert list(params) == [
+        "num_heads", "sm_scale", "causal", "block_sizes", "nomat", "debug", "interpret", "residuals", "do", "causal_offset"]
+    assert params["causal_offset"].kind is inspect.Parameter.KEYWORD_ONLY and params["causal_offset"].default == 0
     assert list(inspect.signature(tpa._bwd).parameters) == [
         "q", "k", "v", "q_segment_ids", "kv_segment_ids", "o", "l", "do", "num_heads", "sm_scale", "causal",
         "block_sizes", "nomat", "debug", "interpret"]
