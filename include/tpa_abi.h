@@ -252,6 +252,22 @@ size_t tpa_fwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int
  */
 int tpa_decode(const TpaFwdArgs* args, void* stream);
 
+/*
+ * tpa_decode without a caller workspace.  No counterpart in the reference: it exists for callers
+ * that cannot allocate device memory (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  Same arguments, kernels and results as tpa_decode, but args->workspace
+ * and args->workspace_bytes are ignored: the split partials go to a fixed device array of
+ * TPA_DECODE_NOALLOC_SCRATCH_BYTES inside the library, one copy per GPU, held until the process
+ * ends.  Problems whose partials (tpa_decode_workspace_bytes) exceed that size return
+ * TPA_ERR_WORKSPACE; problems the split-key kernels do not take return TPA_ERR_UNSUPPORTED (there is
+ * no fallback to the vector-ALU kernel here).  The call allocates and frees nothing; the first call
+ * on a device looks up the array's device address (make that call outside a graph capture).  All
+ * calls on one GPU share the array: calls that overlap in time on one GPU (different streams, or
+ * several host threads) race on it and must be serialised by the caller.
+ */
+#define TPA_DECODE_NOALLOC_SCRATCH_BYTES (8u << 20)
+int tpa_decode_noalloc(const TpaFwdArgs* args, void* stream);
+
 /* Bytes of workspace tpa_decode needs for this problem (num_splits = 0: the default choice). */
 size_t tpa_decode_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dv, int32_t num_splits);
 

@@ -15,6 +15,7 @@
 // online softmax (tpa/tpa.py:389-424).  The waves are merged through LDS, the key ranges
 // through a workspace and a small second kernel, both with the rule of _lse_accum
 // (tpa/tpa.py:228-242).
+#include <mutex>
 #include <type_traits>
 
 #include "tpa_common.h"
@@ -884,4 +885,57 @@ int tpa_decode_f32_launch(const TpaFwdArgs* a, hipStream_t stream) {
     case 16: return launch_decode_f32<64, 16>(a, S, stream);
     default: return launch_decode_f32<64, 32>(a, S, stream);
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// tpa_decode for callers that cannot allocate device memory (code under HIP graph capture, tight
+// serving loops): the split partials go to a fixed array in this code object instead of a caller
+// workspace.  Every device the library runs on holds its own copy of the array until the process
+// ends.  Host code must not use the array's name as an address (in host code the name is a
+// stand-in for the symbol, not device memory); the device address is looked up once per device
+// and kept.
+namespace tpa {
+namespace {
+
+static __device__ __align__(256) unsigned char scratch[TPA_DECODE_NOALLOC_SCRATCH_BYTES];
+
+void* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int scratch_of_current_device(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return TPA_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return TPA_ERR_LAUNCH;
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return TPA_OK;
+}
+
+}  // namespace
+}  // namespace tpa
+
+extern "C" int tpa_decode_noalloc(const TpaFwdArgs* a, void* stream) {
+  using namespace tpa;
+  const int rc = tpa_validate_fwd_args(a);
+  if (rc != TPA_OK) return rc;
+  if (a->q_segment_ids) return TPA_ERR_UNSUPPORTED;
+  const bool bf16 = tpa_decode_mfma_supported(a), f32 = !bf16 && tpa_decode_f32_supported(a);
+  if (a->kernel == TPA_KERNEL_GENERIC || (!bf16 && !f32)) return TPA_ERR_UNSUPPORTED;  // the split-key kernels only
+  const int S = a->num_splits > 0 ? a->num_splits : default_splits(a->B, a->lq, a->lk, a->H, bf16 ? 2 : 1);
+  if (S > 65535 || (int64_t)a->B * S > 2147483647LL) return TPA_ERR_SHAPE;
+  if (workspace_bytes(a->B, a->lq, a->H, a->dv, S) > (size_t)TPA_DECODE_NOALLOC_SCRATCH_BYTES) return TPA_ERR_WORKSPACE;  // partials exceed the fixed array
+  void* ptr = nullptr;
+  if (int rc2 = scratch_of_current_device(&ptr); rc2 != TPA_OK) return rc2;
+  // every (batch entry, query row, key range, head) slot that the merge kernel reads is written by
+  // the decode kernel of the same call, so nothing of the previous call's contents has to be cleared
+  TpaFwdArgs b = *a;
+  b.workspace = ptr;
+  b.workspace_bytes = TPA_DECODE_NOALLOC_SCRATCH_BYTES;
+  b.num_splits = S;
+  return bf16 ? tpa_decode_mfma_launch(&b, static_cast<hipStream_t>(stream)) : tpa_decode_f32_launch(&b, static_cast<hipStream_t>(stream));
 }

@@ -190,7 +190,7 @@ def load_library(path: str | None = None) -> ctypes.CDLL:
         lib.tpa_abi_version.argtypes = []
         lib.tpa_strerror.restype = ctypes.c_char_p
         lib.tpa_strerror.argtypes = [ctypes.c_int]
-        for name in ("tpa_fwd", "tpa_decode"):
+        for name in ("tpa_fwd", "tpa_decode", "tpa_decode_noalloc"):
             fn = getattr(lib, name)
             fn.restype = ctypes.c_int
             fn.argtypes = [ctypes.POINTER(TpaFwdArgs), ctypes.c_void_p]

@@ -112,6 +112,8 @@ def test_null_and_shape_errors_are_reported_before_any_launch():
     mb = d.MhaBwdArgs()
     assert lib.mha_bwd(ctypes.byref(mb), None) == -2
     assert lib.mha_bwd(None, None) == -1
+    assert lib.tpa_decode_noalloc(None, None) == -1
+    assert lib.tpa_decode_noalloc(ctypes.byref(d.TpaFwdArgs()), None) == -2
 
 
 def test_unknown_causal_values_are_refused_by_every_entry_point():
@@ -125,6 +127,7 @@ def test_unknown_causal_values_are_refused_by_every_entry_point():
                        dtype=d.TPA_DTYPE_F32, causal=3)
     assert lib.tpa_fwd(ctypes.byref(fwd), None) == -6
     assert lib.tpa_decode(ctypes.byref(fwd), None) == -6
+    assert lib.tpa_decode_noalloc(ctypes.byref(fwd), None) == -6
     g = d.TpaGrad(256, 0, 0, 0)
     for bad in (3, -1):
         bwd = d.TpaBwdArgs(qa=fake, qb=fake, ka=fake, kb=fake, va=fake, vb=fake, o=256, lse=256, d_o=256,
