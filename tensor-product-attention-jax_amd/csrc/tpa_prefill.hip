@@ -1,7 +1,12 @@
 // Flash-style prefill for gfx950: bf16 MFMA contractions, fp32 online softmax.
 //
-// One workgroup = one (batch, head, block of 256 query rows) and has eight waves, two per SIMD,
-// each owning 32 query rows.  Per tile of 64 keys the workgroup rebuilds the head's K and V
+// One workgroup = one (batch, head, block of 256 query rows), i.e. eight blocks of 32 rows, held
+// either by eight waves (two per SIMD) of one row block each (RB = 1) or by four waves (one per
+// SIMD, 512 registers) of two row blocks each (RB = 2): a wave then feeds every K / V fragment it
+// reads from LDS to two MFMAs, which halves the LDS traffic per MFMA - with one row block per wave
+// the LDS read port (128 B/clk, 76 for transposed reads) is as busy as the matrix pipe.  A wave's
+// two row blocks are w and 7 - w, so that the waves do equal work on the causal diagonal.
+// Per tile of 64 keys the workgroup rebuilds the head's K and V
 // tile from the rank factors (K = (1/R) sum_r a_r (x) b_r, tpa/tpa.py:364,417) straight out of
 // coalesced 16-byte factor loads and stores it once, as bf16, in LDS.  Each wave then computes
 //     S^T = K Q^T        (v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = Q kept in registers,
@@ -22,6 +27,8 @@
 // waves of a SIMD that are both in a vector-only or both in a matrix-only phase just queue up;
 // the dot instruction is the exception: it occupies the matrix pipe.)
 // The dense flash baseline (tpa/mha.py:23-37) is the same kernel with a plain K/V loader.
+#include <stdlib.h>
+
 #include <type_traits>
 #include <utility>
 
@@ -31,8 +38,7 @@ namespace tpa {
 namespace {
 
 constexpr int kTK = 64;   // keys per tile
-constexpr int kNW = 8;    // waves per workgroup
-constexpr int kBQ = 256;  // query rows per workgroup (32 per wave)
+constexpr int kBQ = 256;  // query rows per workgroup: 8 blocks of 32, RB of them per wave
 
 enum { LOAD_TPA_R2 = 0, LOAD_TPA_ANY = 1, LOAD_DENSE = 2 };
 
@@ -52,7 +58,11 @@ struct PrefillParams {
   int q_factors;  // dense K/V loader only: 1 = Q is still given by its rank factors qa, qb
 };
 
-template <int D>
+// LDS: two buffers each of a K tile, a V tile, a slot of head factors and a slot of key segment
+// ids.  With one row block per wave the layout is [K0][K1][V0][V1][A0][A1][seg0][seg1]; with two
+// (RB = 2) it is two sets [K][V][A][seg] that lie 64 KiB apart, so that the hand-written loop
+// flips every address between the sets with one xor.  Offsets are in uint16 units.
+template <int D, int RB>
 struct Lds {
   static constexpr int KS = D + 8;   // K row stride (elements): 16-byte reads of 16 rows hit distinct banks
   static constexpr int VS = D + 32;  // V row stride: 4 consecutive rows of a transposed read hit distinct banks
@@ -60,7 +70,12 @@ struct Lds {
   static constexpr int kV = kTK * VS;  // elements of one V buffer
   static constexpr int kA = 2 * kTK * 2;  // one slot of head factors: [K|V][token][rank 0|1]
   static constexpr int kSeg = 2 * kTK;    // one slot of key segment ids (int32), in uint16 units
-  static constexpr size_t kBytes = (2 * (kK + kV) + 2 * kA + 2 * kSeg) * sizeof(uint16_t);
+  static constexpr int kSet = 32768;      // RB = 2: distance between the two sets
+  static constexpr int k_off(int buf) { return RB == 2 ? buf * kSet : buf * kK; }
+  static constexpr int v_off(int buf) { return RB == 2 ? buf * kSet + kK : 2 * kK + buf * kV; }
+  static constexpr int a_off(int buf) { return RB == 2 ? buf * kSet + kK + kV : 2 * (kK + kV) + buf * kA; }
+  static constexpr int seg_off(int buf) { return RB == 2 ? buf * kSet + kK + kV + kA : 2 * (kK + kV) + 2 * kA + buf * kSeg; }
+  static constexpr size_t kBytes = (RB == 2 ? kSet + kK + kV + kA + kSeg : 2 * (kK + kV) + 2 * kA + 2 * kSeg) * sizeof(uint16_t);
 };
 
 // a0*b0 + a1*b1 on packed bf16 pairs, fp32 result.  Through the builtin on purpose: the dot
@@ -87,11 +102,49 @@ template <int N, typename F>
 __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
+template <int V>
+using IC = std::integral_constant<int, V>;
 
-template <int D, int LOADER, bool SEG>
-__global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
+// Matrix instructions with the register file of every operand chosen by hand, for the kernel
+// with two row blocks per wave: its O^T accumulators (128 registers at D = 128) and Q fragments
+// (64) only ever meet matrix instructions, so they live in the accumulation registers (AGPRs) and
+// leave the 256 architectural registers to the logits, the factor loads and the vector work.
+// (C and D of a matrix instruction share one register file; A and B choose theirs freely.)
+// The compiler inserts no hazard wait states around inline assembly.  A matrix instruction may
+// read a register two wait states after a vector instruction (v_accvgpr_write included) wrote it:
+// each wrapper starts with them, since the compiler is free to put such a write right in front.
+// A vector instruction may read the result of an 8-pass matrix instruction 11 wait states after
+// its issue at the earliest (mfma_result_guard where the instruction stream does not already
+// guarantee it).  These wrappers serve the plain iterations; the interleaved loop is generated.
+__device__ __forceinline__ void mfma_qk_first(f32x16& d, const bf16x8& k, const bf16x8& q, const f32x16& c) {
+  asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(k), "a"(q), "v"(c));
+}
+__device__ __forceinline__ void mfma_qk_next(f32x16& d, const bf16x8& k, const bf16x8& q) {
+  asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(k), "a"(q));
+}
+__device__ __forceinline__ void mfma_pv(f32x16& acc, const bf16x8& v, const bf16x8& pfrag) {
+  asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(v), "v"(pfrag));
+}
+// acc *= alpha for an accumulator tuple that lives in AGPRs, register by register through one
+// temporary, so that the tuple never has to move to the architectural registers
+__device__ __forceinline__ void scale_agpr_tuple(f32x16& acc, float alpha) {
+  float t;
+#define TPA_SCALE1(i) \
+  asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1" : "+a"(acc[i]), "=&v"(t) : "v"(alpha));
+  TPA_SCALE1(0) TPA_SCALE1(1) TPA_SCALE1(2) TPA_SCALE1(3) TPA_SCALE1(4) TPA_SCALE1(5) TPA_SCALE1(6) TPA_SCALE1(7)
+  TPA_SCALE1(8) TPA_SCALE1(9) TPA_SCALE1(10) TPA_SCALE1(11) TPA_SCALE1(12) TPA_SCALE1(13) TPA_SCALE1(14) TPA_SCALE1(15)
+#undef TPA_SCALE1
+}
+__device__ __forceinline__ void pin_vgpr_tuple(f32x16& x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void mfma_result_guard() { asm volatile("s_nop 7\n\ts_nop 3" ::: "memory"); }
+
+template <int D, int LOADER, bool SEG, int RB>
+__global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp) {
+  static_assert(RB == 1 || RB == 2, "row blocks per wave");
+  constexpr int kNW = 8 / RB;  // waves per workgroup
   constexpr int NT = kNW * 64;
-  constexpr int KS = Lds<D>::KS, VS = Lds<D>::VS;
+  using L = Lds<D, RB>;
+  constexpr int KS = L::KS, VS = L::VS;
   constexpr int CPR = D / 8;             // 16-byte chunks per row
   constexpr int TPP = NT / CPR;          // tokens per loader pass
   constexpr int NPASS = kTK / TPP;       // loader passes per tile and matrix
@@ -108,10 +161,10 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
       pp.sm_scale, pp.causal, pp.causal ? pp.coff : 0, pp.nqb, pp.npairs, pp.q_factors};
 
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-  uint16_t* const lds_k = smem;                                  // [2][kTK][KS]
-  uint16_t* const lds_v = smem + 2 * Lds<D>::kK;                 // [2][kTK][VS]
-  uint16_t* const lds_a = smem + 2 * (Lds<D>::kK + Lds<D>::kV);  // [2][K|V][kTK][2]
-  int32_t* const lds_seg = reinterpret_cast<int32_t*>(lds_a + 2 * Lds<D>::kA);  // [2][kTK] key segment ids
+  auto lds_k = [&](int buf) __attribute__((always_inline)) { return smem + L::k_off(buf); };    // [kTK][KS]
+  auto lds_v = [&](int buf) __attribute__((always_inline)) { return smem + L::v_off(buf); };    // [kTK][VS]
+  auto lds_a = [&](int buf) __attribute__((always_inline)) { return smem + L::a_off(buf); };    // [K|V][kTK][2]
+  auto lds_seg = [&](int buf) __attribute__((always_inline)) { return reinterpret_cast<int32_t*>(smem + L::seg_off(buf)); };  // [kTK]
 
   // ---- which (query block, batch, head): heads of one (block, batch) pair sit on one XCD
   // (workgroup ids are dealt round-robin to the 8 XCDs) so they share the B-factor tiles in
@@ -128,27 +181,36 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   const int tid = threadIdx.x;
   const int w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
   const int q0 = qblk * kBQ;
-  const int wrow0 = q0 + 32 * w;  // first query row of this wave
-  const int qrow = wrow0 + i;
-  const int qrow_ld = min(qrow, p.lq - 1);
+  // row block r of this wave within the workgroup's eight: w, and (RB = 2) 7 - w
+  int rblk[RB], wrow0[RB], qrow[RB], qrow_ld[RB];
+#pragma unroll
+  for (int r = 0; r < RB; ++r) {
+    rblk[r] = r == 0 ? w : 7 - w;
+    wrow0[r] = q0 + 32 * rblk[r];  // first query row of the block
+    qrow[r] = wrow0[r] + i;        // this lane's row in it
+    qrow_ld[r] = min(qrow[r], p.lq - 1);
+  }
   const float c = p.sm_scale * kLog2e;
 
   // ---- Q fragments (B operand of S^T = K Q^T), scaled by c: lane (i, g) holds
-  // c * Q[qrow][16ks + 8g + 0..7]
-  bf16x8 qf[NKS];
+  // c * Q[qrow[r]][16ks + 8g + 0..7]
+  bf16x8 qf[RB][NKS];
   auto build_q = [&]() __attribute__((always_inline)) {
     // the dense loader serves dense attention (Q dense too) and factored attention whose K and V
     // were reconstructed beforehand (Q still in factors)
     const bool dense_q = LOADER == LOAD_DENSE && !p.q_factors;
     if (dense_q) {
-      const uint16_t* qp = p.qb.ptr + b * p.qb.stride_b + (int64_t)qrow_ld * p.qb.stride_l + (int64_t)h * D;
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) {
-        const u32x4 raw = *reinterpret_cast<const u32x4*>(qp + 16 * ks + 8 * g);
-        u32x4 sc;
+      for (int r = 0; r < RB; ++r) {
+        const uint16_t* qp = p.qb.ptr + b * p.qb.stride_b + (int64_t)qrow_ld[r] * p.qb.stride_l + (int64_t)h * D;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) sc[j] = pack_bf16(bf16lo_to_f32(raw[j]) * c, bf16hi_to_f32(raw[j]) * c);
-        qf[ks] = __builtin_bit_cast(bf16x8, sc);
+        for (int ks = 0; ks < NKS; ++ks) {
+          const u32x4 raw = *reinterpret_cast<const u32x4*>(qp + 16 * ks + 8 * g);
+          u32x4 sc;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) sc[j] = pack_bf16(bf16lo_to_f32(raw[j]) * c, bf16hi_to_f32(raw[j]) * c);
+          qf[r][ks] = __builtin_bit_cast(bf16x8, sc);
+        }
       }
     } else {
       // One rank at a time through LDS: the workgroup copies the 256 x D slab qb[q0.., r, :] with
@@ -158,7 +220,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
       constexpr int CH = kBQ * CPR / NT;         // 16-byte chunks per thread and rank
       uint16_t* const qs = smem;                 // [kBQ][QS]
       uint16_t* const qas = smem + kBQ * QS;     // [kBQ] head factors of this rank
-      static_assert((kBQ * QS + kBQ) * sizeof(uint16_t) <= Lds<D>::kBytes, "Q staging fits the K/V buffers");
+      static_assert((kBQ * QS + kBQ) * sizeof(uint16_t) <= L::kBytes, "Q staging fits the K/V buffers");
       const uint16_t* qb_b = p.qb.ptr + b * p.qb.stride_b;
       const uint16_t* qa_b = p.qa.ptr + b * p.qa.stride_b + h;
       u32x4 nxt[CH];
@@ -172,11 +234,13 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
         }
         if (tid < kBQ) a_nxt = qa_b[(int64_t)min(q0 + tid, p.lq - 1) * p.qa.stride_l + r * p.qa.stride_r];
       };
-      float acc[NKS][8];
+      float acc[RB][NKS][8];
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks)
+      for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[ks][j] = 0.f;
+        for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) acc[rb][ks][j] = 0.f;
       load_rank(0);
       for (int r = 0; r < p.rq; ++r) {
 #pragma unroll
@@ -189,28 +253,34 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
         lds_barrier();
         // a * b[d] for a packed pair (b[d], b[d+1]) is one dot instruction with (a, 0) or (0, a):
         // no unpacking, and the dot unit is idle here anyway
-        const uint32_t a_lo = qas[32 * w + i], a_hi = a_lo << 16;
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) {
-          const u32x4 bv = *reinterpret_cast<const u32x4*>(qs + (32 * w + i) * QS + 16 * ks + 8 * g);
+        for (int rb = 0; rb < RB; ++rb) {
+          const int row = 32 * rblk[rb] + i;
+          const uint32_t a_lo = qas[row], a_hi = a_lo << 16;
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            uint32_t pair = bv[j];
-            asm volatile("" : "+v"(pair));  // keeps the compiler from taking element 0 of the vector for every j
-            acc[ks][2 * j] = dot2_bf16_acc(pair, a_lo, acc[ks][2 * j]);
-            acc[ks][2 * j + 1] = dot2_bf16_acc(pair, a_hi, acc[ks][2 * j + 1]);
+          for (int ks = 0; ks < NKS; ++ks) {
+            const u32x4 bv = *reinterpret_cast<const u32x4*>(qs + row * QS + 16 * ks + 8 * g);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              uint32_t pair = bv[j];
+              asm volatile("" : "+v"(pair));  // keeps the compiler from taking element 0 of the vector for every j
+              acc[rb][ks][2 * j] = dot2_bf16_acc(pair, a_lo, acc[rb][ks][2 * j]);
+              acc[rb][ks][2 * j + 1] = dot2_bf16_acc(pair, a_hi, acc[rb][ks][2 * j + 1]);
+            }
           }
         }
         lds_barrier();  // everyone has read this rank before the next one overwrites it
       }
       const float scale = c / (float)p.rq;
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) {
-        u32x4 packed;
+      for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) packed[j] = pack_bf16(acc[ks][2 * j] * scale, acc[ks][2 * j + 1] * scale);
-        qf[ks] = __builtin_bit_cast(bf16x8, packed);
-      }
+        for (int ks = 0; ks < NKS; ++ks) {
+          u32x4 packed;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) packed[j] = pack_bf16(acc[rb][ks][2 * j] * scale, acc[rb][ks][2 * j + 1] * scale);
+          qf[rb][ks] = __builtin_bit_cast(bf16x8, packed);
+        }
     }
   };
 
@@ -222,13 +292,15 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   const int coff = p.coff + (p.causal == TPA_CAUSAL_BOTTOM_RIGHT ? len_b - p.lq : 0);
   int kend = p.causal ? min(len_b, min(q0 + kBQ, p.lq) + coff) : len_b;
   if (kend <= 0) {  // no key at all: the rows end as NaN / -inf (tpa/tpa.py:437-439)
-    if (qrow < p.lq) {
-      uint16_t* op = p.o + (((int64_t)b * p.lq + qrow) * p.H + h) * D;
-      const u32x4 nan4 = {0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u};
 #pragma unroll
-      for (int cch = 0; cch < D / 16; ++cch) *reinterpret_cast<u32x4*>(op + 16 * cch + 8 * g) = nan4;
-      if (p.lse && g == 0) p.lse[((int64_t)b * p.H + h) * p.lq + qrow] = -INFINITY;
-    }
+    for (int r = 0; r < RB; ++r)
+      if (qrow[r] < p.lq) {
+        uint16_t* op = p.o + (((int64_t)b * p.lq + qrow[r]) * p.H + h) * D;
+        const u32x4 nan4 = {0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u};
+#pragma unroll
+        for (int cch = 0; cch < D / 16; ++cch) *reinterpret_cast<u32x4*>(op + 16 * cch + 8 * g) = nan4;
+        if (p.lse && g == 0) p.lse[((int64_t)b * p.H + h) * p.lq + qrow[r]] = -INFINITY;
+      }
     return;
   }
   bool seg_pure = false;  // every visited key from the second tile on carries the rows' one segment id
@@ -288,14 +360,18 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     }
   }
   const int lk_r = kend - kpos0;          // keys counted from kpos0
-  // this wave's first row and this lane's row on that scale, shifted by the causal offset: row r
-  // sees keys up to r_r, which is negative for a row that sees none
-  const int wrow_r = wrow0 + coff - kpos0;
-  const int qrow_r = qrow + coff - kpos0;
   const int ntiles = (lk_r + kTK - 1) / kTK;
   const int last = ntiles - 1;
-  // last tile this wave needs under the causal mask (its rows: wrow0 .. wrow0 + 31)
-  const int wave_last_tile = p.causal ? min(last, max(wrow_r + 31, 0) / kTK) : last;
+  // first row of each of this wave's row blocks and this lane's row in it on that scale, shifted by
+  // the causal offset: row x sees keys up to x_r, which is negative for a row that sees none;
+  // last tile the block needs under the causal mask (its rows: wrow0 .. wrow0 + 31)
+  int wrow_r[RB], qrow_r[RB], wave_last_tile[RB];
+#pragma unroll
+  for (int r = 0; r < RB; ++r) {
+    wrow_r[r] = wrow0[r] + coff - kpos0;
+    qrow_r[r] = qrow[r] + coff - kpos0;
+    wave_last_tile[r] = p.causal ? min(last, max(wrow_r[r] + 31, 0) / kTK) : last;
+  }
 
   // ---- loader: this thread rebuilds chunk lc (8 elements) of token lt (+ TPP per pass).
   // Addresses are a uniform (scalar) tile base plus a per-thread 32-bit element offset.
@@ -357,25 +433,29 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   auto store_a = [&](int slot_idx) __attribute__((always_inline)) {
     if constexpr (LOADER != LOAD_TPA_R2) return;
     // stored halved (exact in bf16): the 1/R of the reconstruction with R = 2
-    if (tid < 4 * kTK) lds_a[slot_idx * Lds<D>::kA + tid] = (uint16_t)(pack_bf16(bf16lo_to_f32(a_pending) * 0.5f, 0.f));
+    if (tid < 4 * kTK) lds_a(slot_idx)[tid] = (uint16_t)(pack_bf16(bf16lo_to_f32(a_pending) * 0.5f, 0.f));
   };
 
-  // Key segment ids (packed sequences, tpa/tpa.py:369-375): threads 256..319 fetch one id of a tile
-  // each, park it in a register and store it into an LDS slot one iteration later, like the head
-  // factors; slot j&1 holds the ids of tile j during iteration j.
+  // Key segment ids (packed sequences, tpa/tpa.py:369-375): the threads of one wave (wave 4 where
+  // there are eight, else wave 0) fetch one id of a tile each, park it in a register and store it
+  // into an LDS slot one iteration later, like the head factors; slot j&1 holds the ids of tile j
+  // during iteration j.
   constexpr bool has_seg = SEG;  // a kernel of its own: the mask code slows the others down even when skipped
+  constexpr int kSegWave = kNW > 4 ? 4 : 0;
   int32_t seg_pending = 0;
   auto issue_seg = [&](int tile) __attribute__((always_inline)) {
     if constexpr (has_seg)
-      if (tid >= 4 * kTK && tid < 5 * kTK)
-        seg_pending = p.kvseg[(int64_t)b * p.lk + kpos0 + min(tile * kTK + tid - 4 * kTK, lk_r - 1)];
+      if (w == kSegWave) seg_pending = p.kvseg[(int64_t)b * p.lk + kpos0 + min(tile * kTK + l, lk_r - 1)];
   };
   auto store_seg = [&](int slot_idx) __attribute__((always_inline)) {
     if constexpr (has_seg)
-      if (tid >= 4 * kTK && tid < 5 * kTK) lds_seg[slot_idx * kTK + tid - 4 * kTK] = seg_pending;
+      if (w == kSegWave) lds_seg(slot_idx)[l] = seg_pending;
   };
-  int32_t qseg = 0;
-  if constexpr (has_seg) qseg = p.qseg[(int64_t)b * p.lq + qrow_ld];
+  int32_t qseg[RB] = {};
+  if constexpr (has_seg) {
+#pragma unroll
+    for (int r = 0; r < RB; ++r) qseg[r] = p.qseg[(int64_t)b * p.lq + qrow_ld[r]];
+  }
 
   // (a0/2)*b0[d] + (a1/2)*b1[d] for 8 consecutive d; aa = packed (a0/2, a1/2): fetch_aa hands out
   // halved head factors.
@@ -480,7 +560,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     const uint16_t* ab = is_v ? va_b : ka_b;
     const int b_sl = is_v ? p.vb.stride_l : p.kb.stride_l, b_sr = is_v ? p.vb.stride_r : p.kb.stride_r;
     const int a_sl = is_v ? p.va.stride_l : p.ka.stride_l, a_sr = is_v ? p.va.stride_r : p.ka.stride_r;
-    uint16_t* dst = is_v ? lds_v + (tile & 1) * Lds<D>::kV : lds_k + (tile & 1) * Lds<D>::kK;
+    uint16_t* dst = is_v ? lds_v(tile & 1) : lds_k(tile & 1);
     constexpr int row_stride = is_v ? VS : KS;
 #pragma unroll
     for (int ps = 0; ps < NPASS; ++ps) {
@@ -499,105 +579,120 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     }
   };
 
-  // ---- per-wave state
-  f32x16 o[NDB];
+  // ---- per-wave state, one set per row block r (always indexed with compile-time constants)
+  f32x16 o[RB][NDB];
 #pragma unroll
-  for (int db = 0; db < NDB; ++db)
+  for (int r = 0; r < RB; ++r)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
-  f32x16 s[2];          // exponents x*c - mref of the tile in flight: two 32-key blocks
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[r][db][v] = 0.f;
+  f32x16 s[RB][2];      // exponents x*c - mref of the tile in flight: two 32-key blocks per row block
   // P^T of the tile (packed bf16 pairs, the B operands of the four 16-key steps of O^T) is kept
-  // in the registers of the logits it was made from: fragment k = s[k / 2][4 (k % 2) .. + 3]
-  auto pf_set = [&](auto mb_c, auto idx_c, uint32_t bits) __attribute__((always_inline)) {
-    s[decltype(mb_c)::value][decltype(idx_c)::value] = __uint_as_float(bits);
+  // in the registers of the logits it was made from: fragment k = s[r][k / 2][4 (k % 2) .. + 3]
+  auto pf_set = [&](auto r_c, auto mb_c, auto idx_c, uint32_t bits) __attribute__((always_inline)) {
+    s[decltype(r_c)::value][decltype(mb_c)::value][decltype(idx_c)::value] = __uint_as_float(bits);
   };
-  auto pf_get = [&](auto kk_c) __attribute__((always_inline)) -> bf16x8 {
-    constexpr int kk = decltype(kk_c)::value, mb = kk / 2, h4 = 4 * (kk % 2);
-    const u32x4 w4 = {__float_as_uint(s[mb][h4]), __float_as_uint(s[mb][h4 + 1]), __float_as_uint(s[mb][h4 + 2]), __float_as_uint(s[mb][h4 + 3])};
+  auto pf_get = [&](auto r_c, auto kk_c) __attribute__((always_inline)) -> bf16x8 {
+    constexpr int r = decltype(r_c)::value, kk = decltype(kk_c)::value, mb = kk / 2, h4 = 4 * (kk % 2);
+    const u32x4 w4 = {__float_as_uint(s[r][mb][h4]), __float_as_uint(s[r][mb][h4 + 1]), __float_as_uint(s[r][mb][h4 + 2]), __float_as_uint(s[r][mb][h4 + 3])};
     return __builtin_bit_cast(bf16x8, w4);
   };
-  float mref = 0.f;     // reference (log2 domain, includes c) of row qrow
+  float mref[RB];       // reference (log2 domain, includes c) of row qrow[r]
   // -mref in all 16 registers of an accumulator tuple: the addend of the first S^T MFMA of a
   // block, so the contraction lands on x*c - mref.  Rewritten only when the reference moves.
-  f32x16 nmref;
+  f32x16 nmref[RB];
+  float lsum[RB];       // this lane's share of sum exp2(x*c - mref)
+  bool seen[RB];        // the row has met a visible key (its reference is set)
 #pragma unroll
-  for (int v = 0; v < 16; ++v) nmref[v] = 0.f;
-  auto refresh_nmref = [&]() __attribute__((always_inline)) {
+  for (int r = 0; r < RB; ++r) {
+    mref[r] = 0.f;
+    lsum[r] = 0.f;
+    seen[r] = false;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) nmref[v] = -mref;
+    for (int v = 0; v < 16; ++v) nmref[r][v] = 0.f;
+  }
+  auto refresh_nmref = [&](auto r_c) __attribute__((always_inline)) {
+    constexpr int r = decltype(r_c)::value;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) nmref[r][v] = -mref[r];
   };
-  float lsum = 0.f;     // this lane's share of sum exp2(x*c - mref)
   const int lp = l & 15, dhalf = (l >> 4) & 1;
 
-  // masks + online softmax of tile `tile` (32 of the 64 logits of row qrow live in this lane)
-  bool seen = false;  // this row has met a visible key (its reference is set)
-  auto do_softmax = [&](int tile) __attribute__((always_inline)) {
+  // masks + online softmax of tile `tile` for row block r (32 of the 64 logits of row qrow[r] live in this lane)
+  auto do_softmax = [&](int tile, auto r_c) __attribute__((always_inline)) {
+    constexpr int r = decltype(r_c)::value;
     const int k0 = tile * kTK;
     // keys beyond lk, and keys after the query under the causal mask
-    const bool need_mask = (k0 + kTK > lk_r) || (p.causal && (k0 + kTK - 1 > wrow_r));
+    const bool need_mask = (k0 + kTK > lk_r) || (p.causal && (k0 + kTK - 1 > wrow_r[r]));
     if (need_mask) {
-      const int limit = p.causal ? min(qrow_r, lk_r - 1) : lk_r - 1;  // largest visible key index
+      const int limit = p.causal ? min(qrow_r[r], lk_r - 1) : lk_r - 1;  // largest visible key index
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int t = k0 + 32 * mb + 8 * (v >> 2) + 4 * g + (v & 3);
-          if (t > limit) s[mb][v] = -INFINITY;
+          if (t > limit) s[r][mb][v] = -INFINITY;
         }
     }
     if constexpr (has_seg) {  // keys of another segment (tpa/tpa.py:369-375)
-      const int32_t* slot = lds_seg + (tile & 1) * kTK;
+      const int32_t* slot = lds_seg(tile & 1);
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
         for (int vq = 0; vq < 4; ++vq) {
           const int4 ids = *reinterpret_cast<const int4*>(slot + 32 * mb + 8 * vq + 4 * g);
-          if (ids.x != qseg) s[mb][4 * vq] = -INFINITY;
-          if (ids.y != qseg) s[mb][4 * vq + 1] = -INFINITY;
-          if (ids.z != qseg) s[mb][4 * vq + 2] = -INFINITY;
-          if (ids.w != qseg) s[mb][4 * vq + 3] = -INFINITY;
+          if (ids.x != qseg[r]) s[r][mb][4 * vq] = -INFINITY;
+          if (ids.y != qseg[r]) s[r][mb][4 * vq + 1] = -INFINITY;
+          if (ids.z != qseg[r]) s[r][mb][4 * vq + 2] = -INFINITY;
+          if (ids.w != qseg[r]) s[r][mb][4 * vq + 3] = -INFINITY;
         }
     }
-    float tmax = s[0][0];
+    float tmax = s[r][0][0];
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) tmax = fmaxf(tmax, s[mb][v]);
+      for (int v = 0; v < 16; ++v) tmax = fmaxf(tmax, s[r][mb][v]);
     tmax = halves_max(tmax);
-    const bool first = !seen && tmax > -INFINITY;  // first tile with a visible key for this row
-    const bool up = seen && tmax > kSlack;         // rare: the row's max left the slack
+    const bool first = !seen[r] && tmax > -INFINITY;  // first tile with a visible key for this row
+    const bool up = seen[r] && tmax > kSlack;         // rare: the row's max left the slack
     if (__any(first || up)) {
       // a first tile sets the reference (nothing accumulated yet, so nothing to rescale); later
       // the references move up and O and the row sums are rescaled
       const float delta = first ? tmax : (up ? tmax : 0.f);
       const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);
-      mref += delta;
-      refresh_nmref();
-      lsum *= alpha;
+      mref[r] += delta;
+      refresh_nmref(r_c);
+      lsum[r] *= alpha;
       if (__any(up)) {
 #pragma unroll
-        for (int db = 0; db < NDB; ++db)
+        for (int db = 0; db < NDB; ++db) {
+          if constexpr (RB == 2) {
+            scale_agpr_tuple(o[r][db], alpha);
+          } else {
 #pragma unroll
-          for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+            for (int v = 0; v < 16; ++v) o[r][db][v] *= alpha;
+          }
+        }
       }
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) s[mb][v] -= delta;
-      seen = seen || first;
+        for (int v = 0; v < 16; ++v) s[r][mb][v] -= delta;
+      seen[r] = seen[r] || first;
     }
     static_for<4>([&](auto k_c) __attribute__((always_inline)) {
       constexpr int k = decltype(k_c)::value, mb = k / 2, half = k % 2;
       u32x4 pk;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const float p0 = __builtin_amdgcn_exp2f(s[mb][8 * half + 2 * j]);
-        const float p1 = __builtin_amdgcn_exp2f(s[mb][8 * half + 2 * j + 1]);
-        lsum += p0 + p1;
+        const float p0 = __builtin_amdgcn_exp2f(s[r][mb][8 * half + 2 * j]);
+        const float p1 = __builtin_amdgcn_exp2f(s[r][mb][8 * half + 2 * j + 1]);
+        lsum[r] += p0 + p1;
         pk[j] = pack_bf16(p0, p1);
       }
       static_for<4>([&](auto j_c) __attribute__((always_inline)) {
-        pf_set(std::integral_constant<int, mb>{}, std::integral_constant<int, 4 * half + decltype(j_c)::value>{}, pk[decltype(j_c)::value]);
+        pf_set(r_c, IC<mb>{}, IC<4 * half + decltype(j_c)::value>{}, pk[decltype(j_c)::value]);
       });
     });
   };
@@ -609,9 +704,9 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
   // An iteration computes S^T = K Q^T, the softmax and O^T += V^T P^T of tile j, rebuilds tile
   // j+1 into the other buffers and refills the registers with tile j+2; one barrier ends it.
   constexpr int N_QK = 2 * NKS, N_PV = 4 * NDB, N_MFMA = N_QK + N_PV;
-  // operand fragment of MFMA step n from LDS: steps 0..N_QK-1 are S^T (32-key block mb = n / NKS),
-  // the rest O^T (k-step kk covers keys 16kk .. 16kk+15 of the tile in the slot order the S^T
-  // accumulator already has: slot (g, j) = key 16kk + 8(j/4) + 4g + j%4)
+  // operand fragment n from LDS, shared by the wave's row blocks: fragments 0..N_QK-1 are rows of K
+  // (32-key block mb = n / NKS), the rest columns of V (k-step kk covers keys 16kk .. 16kk+15 of the
+  // tile in the slot order the S^T accumulator already has: slot (g, j) = key 16kk + 8(j/4) + 4g + j%4)
   auto load_frag = [&](auto n_c, const uint16_t* ks, const uint16_t* vs) __attribute__((always_inline)) -> bf16x8 {
     constexpr int n = decltype(n_c)::value;
     if constexpr (n < N_QK) {
@@ -625,81 +720,103 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
       return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
     }
   };
-  auto mfma_with = [&](auto n_c, const bf16x8& f) __attribute__((always_inline)) {
-    constexpr int n = decltype(n_c)::value;
+  // the MFMA of fragment n for row block r
+  auto mfma_with = [&](auto n_c, auto r_c, const bf16x8& f) __attribute__((always_inline)) {
+    constexpr int n = decltype(n_c)::value, r = decltype(r_c)::value;
     if constexpr (n < N_QK) {
       constexpr int mb = n / NKS, kk = n % NKS;
-      if constexpr (kk == 0) s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, qf[kk], nmref, 0, 0, 0);
-      else s[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, qf[kk], s[mb], 0, 0, 0);
+      if constexpr (RB == 2) {
+        if constexpr (kk == 0) mfma_qk_first(s[r][mb], f, qf[r][kk], nmref[r]);
+        else mfma_qk_next(s[r][mb], f, qf[r][kk]);
+      } else {
+        if constexpr (kk == 0) s[r][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, qf[r][kk], nmref[r], 0, 0, 0);
+        else s[r][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, qf[r][kk], s[r][mb], 0, 0, 0);
+      }
     } else {
       constexpr int m = n - N_QK, kk = m / NDB, db = m % NDB;
-      o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, pf_get(std::integral_constant<int, kk>{}), o[db], 0, 0, 0);
+      if constexpr (RB == 2) mfma_pv(o[r][db], f, pf_get(r_c, IC<kk>{}));
+      else o[r][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, pf_get(r_c, IC<kk>{}), o[r][db], 0, 0, 0);
     }
+  };
+  // The logits of block (r, mb) may be read from here on: pins the vector code that follows behind
+  // the matrix instructions issued so far (it would otherwise be free to move up to the one that
+  // wrote them, inside its 11 wait states).
+  auto logits_ready = [&](auto r_c, auto mb_c) __attribute__((always_inline)) {
+    if constexpr (RB == 2) pin_vgpr_tuple(s[decltype(r_c)::value][decltype(mb_c)::value]);
   };
   // ---- pieces of the softmax of one 32-key block, for the interleaved (unmasked) path
   // Move the reference up where this block's row max left the slack (rare).  delta is a whole
   // number, so the scale factors are exact powers of two.  `pf_done` = number of already packed
-  // P fragments of this tile, which are rescaled too; s[1] is adjusted with s[0] because its
+  // P fragments of this tile, which are rescaled too; s[r][1] is adjusted with s[r][0] because its
   // accumulation (still running when block 0 is inspected) started from the old reference.
-  auto move_reference = [&](float tmax, int pf_done) __attribute__((always_inline)) {
+  auto move_reference = [&](auto r_c, float tmax, int pf_done) __attribute__((always_inline)) {
+    constexpr int r = decltype(r_c)::value;
     const float delta = tmax > 0.f ? __builtin_ceilf(tmax) : 0.f;
     const float alpha = __builtin_amdgcn_exp2f(-delta);
-    mref += delta;
-    refresh_nmref();
-    lsum *= alpha;
+    if constexpr (RB == 2) mfma_result_guard();  // O^T and the other block's logits may have been written just now
+    mref[r] += delta;
+    refresh_nmref(r_c);
+    lsum[r] *= alpha;
 #pragma unroll
-    for (int db = 0; db < NDB; ++db)
+    for (int db = 0; db < NDB; ++db) {
+      if constexpr (RB == 2) {
+        scale_agpr_tuple(o[r][db], alpha);
+      } else {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+        for (int v = 0; v < 16; ++v) o[r][db][v] *= alpha;
+      }
+    }
     // pf_done = 0: block 0 is being inspected, nothing of this tile is packed yet, both blocks move;
-    // pf_done = 2: block 0 has become fragments 0 and 1 (s[0][0..7]), block 1 moves
+    // pf_done = 2: block 0 has become fragments 0 and 1 (s[r][0][0..7]), block 1 moves
     if (pf_done == 0) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) s[0][v] -= delta;
+      for (int v = 0; v < 16; ++v) s[r][0][v] -= delta;
     } else {
 #pragma unroll
       for (int v = 0; v < 8; ++v) {
-        const uint32_t w1 = __float_as_uint(s[0][v]);
-        s[0][v] = __uint_as_float(pack_bf16(bf16lo_to_f32(w1) * alpha, bf16hi_to_f32(w1) * alpha));
+        const uint32_t w1 = __float_as_uint(s[r][0][v]);
+        s[r][0][v] = __uint_as_float(pack_bf16(bf16lo_to_f32(w1) * alpha, bf16hi_to_f32(w1) * alpha));
       }
     }
 #pragma unroll
-    for (int v = 0; v < 16; ++v) s[1][v] -= delta;
+    for (int v = 0; v < 16; ++v) s[r][1][v] -= delta;
   };
-  auto sm_max = [&](auto mb_c) __attribute__((always_inline)) {
-    constexpr int mb = decltype(mb_c)::value;
-    float t = s[mb][0];
+  auto sm_max = [&](auto r_c, auto mb_c) __attribute__((always_inline)) {
+    constexpr int r = decltype(r_c)::value, mb = decltype(mb_c)::value;
+    logits_ready(r_c, mb_c);
+    float t = s[r][mb][0];
 #pragma unroll
-    for (int v = 1; v < 16; ++v) t = fmaxf(t, s[mb][v]);
+    for (int v = 1; v < 16; ++v) t = fmaxf(t, s[r][mb][v]);
     t = halves_max(t);
-    if (__any(t > kSlack)) move_reference(t, 2 * mb);
+    if (__any(t > kSlack)) move_reference(r_c, t, 2 * mb);
   };
-  auto sm_exp = [&](auto mb_c, auto q_c) __attribute__((always_inline)) {  // 4 of the block's 16 logits
-    constexpr int mb = decltype(mb_c)::value, q = decltype(q_c)::value;
-    const float p0 = __builtin_amdgcn_exp2f(s[mb][4 * q]);
-    const float p1 = __builtin_amdgcn_exp2f(s[mb][4 * q + 1]);
-    const float p2 = __builtin_amdgcn_exp2f(s[mb][4 * q + 2]);
-    const float p3 = __builtin_amdgcn_exp2f(s[mb][4 * q + 3]);
-    lsum += (p0 + p1) + (p2 + p3);
-    pf_set(mb_c, std::integral_constant<int, 2 * q>{}, pack_bf16(p0, p1));
-    pf_set(mb_c, std::integral_constant<int, 2 * q + 1>{}, pack_bf16(p2, p3));
+  auto sm_exp = [&](auto r_c, auto mb_c, auto q_c) __attribute__((always_inline)) {  // 4 of the block's 16 logits
+    constexpr int r = decltype(r_c)::value, mb = decltype(mb_c)::value, q = decltype(q_c)::value;
+    const float p0 = __builtin_amdgcn_exp2f(s[r][mb][4 * q]);
+    const float p1 = __builtin_amdgcn_exp2f(s[r][mb][4 * q + 1]);
+    const float p2 = __builtin_amdgcn_exp2f(s[r][mb][4 * q + 2]);
+    const float p3 = __builtin_amdgcn_exp2f(s[r][mb][4 * q + 3]);
+    lsum[r] += (p0 + p1) + (p2 + p3);
+    pf_set(r_c, mb_c, IC<2 * q>{}, pack_bf16(p0, p1));
+    pf_set(r_c, mb_c, IC<2 * q + 1>{}, pack_bf16(p2, p3));
   };
 
   // ---- interleaved iteration (tiles that need no mask, with a next tile to rebuild): every
   // MFMA is followed by a short slice of independent vector work of the same wave, so that the
-  // vector ALU runs in the shadow of the matrix pipe:
+  // vector ALU runs in the shadow of the matrix pipe.  A fragment read from LDS feeds one MFMA
+  // per row block; with G = fragments per group:
   //   S^T block 0   | rebuild K tile j+1, refill kreg
-  //   S^T block 1   | softmax of block 0
-  //   O^T, keys 0-31  | softmax of block 1 (its max is taken before these MFMAs start)
+  //   S^T block 1   | softmax of block 0 (all row blocks)
+  //   O^T, keys 0-31  | softmax of block 1
   //   O^T, keys 32-63 | rebuild V tile j+1, refill vreg
-  // LDS operands are read LA steps ahead of the MFMA that consumes them.
+  // LDS operands are read LA fragments ahead of the MFMAs that consume them.
   auto hot_iteration = [&](int j) __attribute__((always_inline)) {
     constexpr int LA = 2;
-    const uint16_t* ks = lds_k + (j & 1) * Lds<D>::kK;
-    const uint16_t* vs = lds_v + (j & 1) * Lds<D>::kV;
-    const uint16_t* a_slot = lds_a + (j & 1) * Lds<D>::kA;
-    uint16_t* k_dst = lds_k + ((j + 1) & 1) * Lds<D>::kK;
-    uint16_t* v_dst = lds_v + ((j + 1) & 1) * Lds<D>::kV;
+    const uint16_t* ks = lds_k(j & 1);
+    const uint16_t* vs = lds_v(j & 1);
+    const uint16_t* a_slot = lds_a(j & 1);
+    uint16_t* k_dst = lds_k((j + 1) & 1);
+    uint16_t* v_dst = lds_v((j + 1) & 1);
     uint32_t aa_k[NPASS], aa_v[NPASS];
     fetch_aa(IsK{}, j + 1, a_slot, aa_k);
     fetch_aa(IsV{}, j + 1, a_slot, aa_v);
@@ -726,28 +843,39 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
       }
     };
     constexpr int NP = 3 * NPASS;       // rebuild pieces per matrix
-    constexpr int G1 = NKS, G2 = NKS, G3 = 2 * NDB, G4 = 2 * NDB;  // MFMAs per group
+    // slots (one per MFMA) of the four groups; slot = fragment * RB + row block
+    constexpr int G1 = NKS * RB, G2 = NKS * RB, G3 = 2 * NDB * RB, G4 = 2 * NDB * RB;
     static_assert(G1 > NP && G4 >= 1, "slices fit their groups");
+    // the softmax of 32-key block mb as items: with one row block {max (block 0 only), exp 0..3},
+    // with two {max r0, max r1, exp (r0, 0), exp (r1, 0), ..., exp (r1, 3)}; item k of NI goes
+    // behind MFMA slot k * G / NI of its group.  (With one row block the maximum of block 1 is
+    // taken before the group starts, see below.)
+    auto softmax_items = [&](auto mb_c, auto q_c, auto g_c) __attribute__((always_inline)) {
+      constexpr int mb = decltype(mb_c)::value, q = decltype(q_c)::value, G = decltype(g_c)::value;
+      constexpr int NMAX = (RB == 1 && mb == 1) ? 0 : RB, NI = NMAX + 4 * RB;
+      static_for<NI>([&](auto k_c) __attribute__((always_inline)) {
+        constexpr int k = decltype(k_c)::value;
+        if constexpr (k * G / NI == q) {
+          if constexpr (k < NMAX) sm_max(IC<k>{}, mb_c);
+          else sm_exp(IC<(k - NMAX) % RB>{}, mb_c, IC<(k - NMAX) / RB>{});
+        }
+      });
+    };
     auto slice = [&](auto n_c) __attribute__((always_inline)) {
       constexpr int n = decltype(n_c)::value;
       if constexpr (n < G1) {
-        if constexpr (n < NP) piece(IsK{}, n_c);
-        if constexpr (n == NP) issue(IsK{}, min(j + 2, last));
-      } else if constexpr (n < G1 + G2) {
-        constexpr int q = n - G1;  // items 0..4 = max, exp 0..3; item k sits in slot k*G2/5
-        static_for<5>([&](auto k_c) __attribute__((always_inline)) {
+        constexpr int NI = NP + 1;  // items: NP rebuild pieces of K, refill kreg
+        static_for<NI>([&](auto k_c) __attribute__((always_inline)) {
           constexpr int k = decltype(k_c)::value;
-          if constexpr (k * G2 / 5 == q) {
-            if constexpr (k == 0) sm_max(std::integral_constant<int, 0>{});
-            else sm_exp(std::integral_constant<int, 0>{}, std::integral_constant<int, k - 1>{});
+          if constexpr (k * G1 / NI == n) {
+            if constexpr (k < NP) piece(IsK{}, k_c);
+            else issue(IsK{}, min(j + 2, last));
           }
         });
+      } else if constexpr (n < G1 + G2) {
+        softmax_items(IC<0>{}, IC<n - G1>{}, IC<G2>{});
       } else if constexpr (n < G1 + G2 + G3) {
-        constexpr int q = n - G1 - G2;  // exp 0..3 of block 1; item k sits in slot k*G3/4
-        static_for<4>([&](auto k_c) __attribute__((always_inline)) {
-          constexpr int k = decltype(k_c)::value;
-          if constexpr (k * G3 / 4 == q) sm_exp(std::integral_constant<int, 1>{}, k_c);
-        });
+        softmax_items(IC<1>{}, IC<n - G1 - G2>{}, IC<G3>{});
       } else {
         constexpr int q = n - G1 - G2 - G3;  // items: NP rebuild pieces of V, refill vreg
         constexpr int NI = NP + 1;
@@ -755,7 +883,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
           constexpr int k = decltype(k_c)::value;
           if constexpr (k * G4 / NI == q) {
             if constexpr (k < NP) piece(IsV{}, k_c);
-            else if constexpr (k == NP) issue(IsV{}, min(j + 2, last));
+            else issue(IsV{}, min(j + 2, last));
           }
         });
       }
@@ -764,40 +892,62 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     static_for<LA>([&](auto n_c) __attribute__((always_inline)) { fr[decltype(n_c)::value] = load_frag(n_c, ks, vs); });
     static_for<N_MFMA>([&](auto n_c) __attribute__((always_inline)) {
       constexpr int n = decltype(n_c)::value;
-      if constexpr (n == G1 + G2) {
-        sm_max(std::integral_constant<int, 1>{});  // before any O^T MFMA of this tile is issued
+      if constexpr (RB == 1 && n == N_QK) {
+        sm_max(IC<0>{}, IC<1>{});  // before any O^T MFMA of this tile is issued
         __builtin_amdgcn_sched_barrier(0);
       }
-      if constexpr (n + LA < N_MFMA) fr[n + LA] = load_frag(std::integral_constant<int, n + LA>{}, ks, vs);
-      mfma_with(n_c, fr[n]);
-      slice(n_c);
+      if constexpr (n + LA < N_MFMA) fr[n + LA] = load_frag(IC<n + LA>{}, ks, vs);
+      static_for<RB>([&](auto r_c) __attribute__((always_inline)) {
+        mfma_with(n_c, r_c, fr[n]);
+        slice(IC<n * RB + decltype(r_c)::value>{});
+      });
     });
   };
 
-  // ---- plain iteration: first tile, masked tiles, tiles a wave skips, last tile
+  // ---- plain iteration: first tile, masked tiles, tiles a row block skips, last tile.
+  // `mask_c` = the row blocks of this wave that take part (bit r).
+  auto cold_compute = [&](int j, auto mask_c) __attribute__((always_inline)) {
+    constexpr int M = decltype(mask_c)::value;
+    const uint16_t* ks = lds_k(j & 1);
+    const uint16_t* vs = lds_v(j & 1);
+    // operands are read three fragments ahead here too (the V fragments of the first O^T steps
+    // while the softmax runs); not with the any-rank loader, whose kernel got slower with it
+    constexpr int LA = LOADER == LOAD_TPA_ANY ? 0 : 3;
+    bf16x8 fr[N_MFMA];
+    static_for<LA>([&](auto n_c) __attribute__((always_inline)) { fr[decltype(n_c)::value] = load_frag(n_c, ks, vs); });
+    static_for<N_QK>([&](auto n_c) __attribute__((always_inline)) {
+      constexpr int n = decltype(n_c)::value;
+      if constexpr (n + LA < N_MFMA) fr[n + LA] = load_frag(IC<n + LA>{}, ks, vs);
+      static_for<RB>([&](auto r_c) __attribute__((always_inline)) {
+        if constexpr ((M >> decltype(r_c)::value) & 1) mfma_with(n_c, r_c, fr[n]);
+      });
+    });
+    if constexpr (RB == 2) mfma_result_guard();
+    static_for<RB>([&](auto r_c) __attribute__((always_inline)) {
+      if constexpr ((M >> decltype(r_c)::value) & 1) {
+        logits_ready(r_c, IC<0>{});
+        logits_ready(r_c, IC<1>{});
+        do_softmax(j, r_c);
+      }
+    });
+    static_for<N_PV>([&](auto n_c) __attribute__((always_inline)) {
+      constexpr int n = N_QK + decltype(n_c)::value;
+      if constexpr (n + LA < N_MFMA) fr[n + LA] = load_frag(IC<n + LA>{}, ks, vs);
+      static_for<RB>([&](auto r_c) __attribute__((always_inline)) {
+        if constexpr ((M >> decltype(r_c)::value) & 1) mfma_with(IC<n>{}, r_c, fr[n]);
+      });
+    });
+  };
   auto cold_iteration = [&](int j) __attribute__((always_inline)) {
-    if (j <= wave_last_tile) {
-      const uint16_t* ks = lds_k + (j & 1) * Lds<D>::kK;
-      const uint16_t* vs = lds_v + (j & 1) * Lds<D>::kV;
-      // operands are read three MFMAs ahead here too (the V fragments of the first O^T steps
-      // while the softmax runs); not with the any-rank loader, whose kernel got slower with it
-      constexpr int LA = LOADER == LOAD_TPA_ANY ? 0 : 3;
-      bf16x8 fr[N_MFMA];
-      static_for<LA>([&](auto n_c) __attribute__((always_inline)) { fr[decltype(n_c)::value] = load_frag(n_c, ks, vs); });
-      static_for<N_QK>([&](auto n_c) __attribute__((always_inline)) {
-        constexpr int n = decltype(n_c)::value;
-        if constexpr (n + LA < N_MFMA) fr[n + LA] = load_frag(std::integral_constant<int, n + LA>{}, ks, vs);
-        mfma_with(n_c, fr[n]);
-      });
-      do_softmax(j);
-      static_for<N_PV>([&](auto n_c) __attribute__((always_inline)) {
-        constexpr int n = N_QK + decltype(n_c)::value;
-        if constexpr (n + LA < N_MFMA) fr[n + LA] = load_frag(std::integral_constant<int, n + LA>{}, ks, vs);
-        mfma_with(std::integral_constant<int, n>{}, fr[n]);
-      });
+    if constexpr (RB == 1) {
+      if (j <= wave_last_tile[0]) cold_compute(j, IC<1>{});
+    } else {
+      // block 1 lies below block 0 in the sequence, so it needs every tile that block 0 needs
+      if (j <= wave_last_tile[0]) cold_compute(j, IC<3>{});
+      else if (j <= wave_last_tile[1]) cold_compute(j, IC<2>{});
     }
     if (j + 1 < ntiles) {
-      const uint16_t* a_slot = LOADER == LOAD_TPA_R2 ? lds_a + (j & 1) * Lds<D>::kA : nullptr;
+      const uint16_t* a_slot = LOADER == LOAD_TPA_R2 ? lds_a(j & 1) : nullptr;
       uint32_t aa_k[NPASS], aa_v[NPASS];
       fetch_aa(IsK{}, j + 1, a_slot, aa_k);
       fetch_aa(IsV{}, j + 1, a_slot, aa_v);
@@ -837,44 +987,137 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     if (w < 4) {  // head factors: publish those of tile j+2, fetch those of tile j+3
       store_a((j + 1) & 1);
       issue_a(min(j + 3, last), min(j + 3, last));
-    } else {      // key segment ids: publish those of tile j+1, fetch those of tile j+2
-      store_seg((j + 1) & 1);
-      issue_seg(min(j + 2, last));
     }
+    // key segment ids (one wave): publish those of tile j+1, fetch those of tile j+2
+    store_seg((j + 1) & 1);
+    issue_seg(min(j + 2, last));
     lds_barrier();
   };
   int hot_end = 1;
   if constexpr (LOADER != LOAD_TPA_ANY) {
     int first_masked = lk_r / kTK;                                   // ragged last tile
-    if (p.causal) first_masked = min(first_masked, max(wrow_r + 1, 0) / kTK);  // first tile with a key past row wrow0
-    hot_end = max(1, min(min(ntiles - 1, first_masked), wave_last_tile + 1));
+    int needed = last;                                               // last tile every row block of the wave needs
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      if (p.causal) first_masked = min(first_masked, max(wrow_r[r] + 1, 0) / kTK);  // first tile with a key past the block's first row
+      needed = min(needed, wave_last_tile[r]);
+    }
+    hot_end = max(1, min(min(ntiles - 1, first_masked), needed + 1));
     // segment masks are applied by the plain iteration only: the interleaved one runs where no
     // key of another segment can turn up (tile 0, which may start before the run, is plain anyway)
     if constexpr (has_seg) if (!seg_pure) hot_end = 1;
   }
   int j = 0;
   for (; j < 1; ++j) { cold_iteration(j); tail(j); }
-  if constexpr (LOADER != LOAD_TPA_ANY) {
+  if constexpr (LOADER != LOAD_TPA_ANY && RB == 1) {
     for (; j < hot_end; ++j) { hot_iteration(j); tail(j); }
+  }
+  if constexpr (LOADER != LOAD_TPA_ANY && RB == 2) {
+    // The interleaved iterations 1 .. hot_end - 1 as one block of assembly with every register
+    // named (gen_prefill_loop.py writes it and documents the register map): the state goes in and
+    // comes back in operands pinned to those registers.
+    static_assert(D == 128 && !SEG, "the generated loop exists for D = 128 without segment ids");
+    if (hot_end > 1) {
+      auto cat4 = [](const u32x4& a0, const u32x4& a1, const u32x4& a2, const u32x4& a3) __attribute__((always_inline)) -> f32x16 {
+        const u32x8 lo = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+        const u32x8 hi = __builtin_shufflevector(a2, a3, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(f32x16, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
+      };
+      auto quarter = [](const f32x16& t, auto k_c) __attribute__((always_inline)) -> u32x4 {
+        constexpr int k = 4 * decltype(k_c)::value;
+        const u32x16 u = __builtin_bit_cast(u32x16, t);
+        return __builtin_shufflevector(u, u, k, k + 1, k + 2, k + 3);
+      };
+      auto qv = [&](int r, int ks) __attribute__((always_inline)) { return __builtin_bit_cast(u32x4, qf[r][ks]); };
+      const f32x16 qp0 = cat4(qv(0, 0), qv(0, 1), qv(0, 2), qv(0, 3)), qp1 = cat4(qv(0, 4), qv(0, 5), qv(0, 6), qv(0, 7));
+      const f32x16 qp2 = cat4(qv(1, 0), qv(1, 1), qv(1, 2), qv(1, 3)), qp3 = cat4(qv(1, 4), qv(1, 5), qv(1, 6), qv(1, 7));
+      constexpr bool two = LOADER == LOAD_TPA_R2;  // factor registers of the second rank exist
+      const u32x4 z4 = {0, 0, 0, 0};
+      f32x16 kv0 = cat4(kreg[0][0], two ? kreg[0][1] : z4, kreg[1][0], two ? kreg[1][1] : z4);
+      f32x16 kv1 = cat4(kreg[2][0], two ? kreg[2][1] : z4, kreg[3][0], two ? kreg[3][1] : z4);
+      f32x16 kv2 = cat4(vreg[0][0], two ? vreg[0][1] : z4, vreg[1][0], two ? vreg[1][1] : z4);
+      f32x16 kv3 = cat4(vreg[2][0], two ? vreg[2][1] : z4, vreg[3][0], two ? vreg[3][1] : z4);
+      f32x8 st8 = {mref[0], mref[1], lsum[0], lsum[1], __uint_as_float(a_pending), 0.f, 0.f, 0.f};
+      // LDS byte addresses of this lane in set 0 (the loop flips them between the sets)
+      const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t*)smem;
+      u32x16 ad16 = {};
+      ad16[0] = lds0 + 2 * (L::k_off(0) + i * KS + 8 * g);                                                   // K fragment rows
+      ad16[1] = lds0 + 2 * (L::v_off(0) + (4 * g + (lp >> 2)) * VS + 16 * dhalf + 4 * (lp & 3));             // V fragment columns
+      ad16[2] = lds0 + 2 * (L::k_off(0) + lt * KS + 8 * lc);                                                 // rebuilt K chunk
+      ad16[3] = lds0 + 2 * (L::v_off(0) + lt * VS + 8 * lc);                                                 // rebuilt V chunk
+      ad16[4] = lds0 + 2 * (L::a_off(0) + 2 * lt);                                                           // head-factor pairs of this lane's tokens
+      ad16[5] = lds0 + 2 * (L::a_off(0) + tid);                                                              // head factor this thread publishes
+      ad16[6] = kvoff; ad16[7] = vvoff; ad16[8] = a_mat == 0 ? ka_voff : va_voff;
+      auto uni = [](uint32_t x) __attribute__((always_inline)) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); };
+      u32x16 sc16 = {};
+      sc16[0] = uni(j); sc16[1] = uni(hot_end); sc16[2] = uni(last);
+      sc16[3] = uni(kTK * p.kb.stride_l * 2); sc16[4] = uni(kTK * p.vb.stride_l * 2);
+      sc16[5] = uni(kTK * (w < 2 ? p.ka.stride_l : p.va.stride_l) * 2);
+      sc16[6] = uni(TPP * p.kb.stride_l * 2); sc16[7] = uni(p.kb.stride_r * 2);
+      sc16[8] = uni(TPP * p.vb.stride_l * 2); sc16[9] = uni(p.vb.stride_r * 2);
+      sc16[10] = 0x05040100u; sc16[11] = 0x07060302u;
+      auto rsrc_words = [&](const uint16_t* base, int bytes) __attribute__((always_inline)) -> u32x4 {
+        const uint64_t a64 = reinterpret_cast<uint64_t>(base);
+        return u32x4{uni((uint32_t)a64), uni((uint32_t)(a64 >> 32) & 0xffffu), uni((uint32_t)bytes), (uint32_t)kRsrcFlags};
+      };
+      const u32x4 kbr = rsrc_words(kb_b, k_rows_bytes), vbr = rsrc_words(vb_b, v_rows_bytes);
+      const u32x4 abr = LOADER == LOAD_TPA_R2 ? rsrc_words(w < 2 ? ka_b : va_b, w < 2 ? ka_bytes : va_bytes) : z4;  // waves 0, 1 fetch K's head factors, waves 2, 3 V's
+#define TPA_PF_LOOP_OPERANDS                                                                                           \
+  : "+{a[0:15]}"(o[0][0]), "+{a[16:31]}"(o[0][1]), "+{a[32:47]}"(o[0][2]), "+{a[48:63]}"(o[0][3]),                   \
+    "+{a[64:79]}"(o[1][0]), "+{a[80:95]}"(o[1][1]), "+{a[96:111]}"(o[1][2]), "+{a[112:127]}"(o[1][3]),               \
+    "+{v[64:79]}"(nmref[0]), "+{v[80:95]}"(nmref[1]),                                                                \
+    "+{v[96:111]}"(kv0), "+{v[112:127]}"(kv1), "+{v[128:143]}"(kv2), "+{v[144:159]}"(kv3),                            \
+    "+{v[188:195]}"(st8), "+{v[196:211]}"(ad16), "+{s[32:47]}"(sc16)                                                 \
+  : "{a[128:143]}"(qp0), "{a[144:159]}"(qp1), "{a[160:175]}"(qp2), "{a[176:191]}"(qp3),                              \
+    "{s[48:51]}"(kbr), "{s[52:55]}"(vbr), "{s[56:59]}"(abr)                                                          \
+  :
+      if constexpr (LOADER == LOAD_TPA_R2) {
+        asm volatile(
+#include "gen/prefill_loop_128_r2.inc"
+            TPA_PF_LOOP_OPERANDS
+#include "gen/prefill_loop_128_r2_clobbers.inc"
+        );
+      } else {
+        asm volatile(
+#include "gen/prefill_loop_128_dense.inc"
+            TPA_PF_LOOP_OPERANDS
+#include "gen/prefill_loop_128_dense_clobbers.inc"
+        );
+      }
+#undef TPA_PF_LOOP_OPERANDS
+      kreg[0][0] = quarter(kv0, IC<0>{}); kreg[1][0] = quarter(kv0, IC<2>{}); kreg[2][0] = quarter(kv1, IC<0>{}); kreg[3][0] = quarter(kv1, IC<2>{});
+      vreg[0][0] = quarter(kv2, IC<0>{}); vreg[1][0] = quarter(kv2, IC<2>{}); vreg[2][0] = quarter(kv3, IC<0>{}); vreg[3][0] = quarter(kv3, IC<2>{});
+      if constexpr (two) {
+        kreg[0][1] = quarter(kv0, IC<1>{}); kreg[1][1] = quarter(kv0, IC<3>{}); kreg[2][1] = quarter(kv1, IC<1>{}); kreg[3][1] = quarter(kv1, IC<3>{});
+        vreg[0][1] = quarter(kv2, IC<1>{}); vreg[1][1] = quarter(kv2, IC<3>{}); vreg[2][1] = quarter(kv3, IC<1>{}); vreg[3][1] = quarter(kv3, IC<3>{});
+      }
+      mref[0] = st8[0]; mref[1] = st8[1]; lsum[0] = st8[2]; lsum[1] = st8[3];
+      a_pending = __float_as_uint(st8[4]);
+      j = hot_end;
+    }
   }
   for (; j < ntiles; ++j) { cold_iteration(j); tail(j); }
 
   // ---- epilogue: normalise, store O[b, qrow, h, :] and LSE[b, h, qrow]
-  const float ltot = halves_sum(lsum);
-  const float inv = 1.f / ltot;
-  // The wave's 32 output rows go through its own slice of LDS (free after the last barrier), so
-  // that they leave as whole 16-byte chunks of whole rows instead of 8-byte pieces of 32 rows.
-  {
+  // A row block's 32 output rows go through the wave's own slice of LDS (free after the last
+  // barrier), so that they leave as whole 16-byte chunks of whole rows instead of 8-byte pieces
+  // of 32 rows.  (LDS operations of one wave complete in order: the next row block's writes
+  // cannot overtake the reads of this one.)
+  if constexpr (RB == 2) mfma_result_guard();
+  static_for<RB>([&](auto r_c) __attribute__((always_inline)) {
+    constexpr int r = decltype(r_c)::value;
+    const float ltot = halves_sum(lsum[r]);
+    const float inv = 1.f / ltot;
     constexpr int OS = D + 8;  // row stride (elements)
     uint16_t* const ot = smem + w * 32 * OS;
-    static_assert(kNW * 32 * OS * sizeof(uint16_t) <= Lds<D>::kBytes, "output staging fits");
+    static_assert(kNW * 32 * OS * sizeof(uint16_t) <= L::kBytes, "output staging fits");
 #pragma unroll
     for (int db = 0; db < NDB; ++db)
 #pragma unroll
       for (int vq = 0; vq < 4; ++vq) {
         u32x2 pk;
-        pk[0] = pack_bf16(o[db][4 * vq] * inv, o[db][4 * vq + 1] * inv);
-        pk[1] = pack_bf16(o[db][4 * vq + 2] * inv, o[db][4 * vq + 3] * inv);
+        pk[0] = pack_bf16(o[r][db][4 * vq] * inv, o[r][db][4 * vq + 1] * inv);
+        pk[1] = pack_bf16(o[r][db][4 * vq + 2] * inv, o[r][db][4 * vq + 3] * inv);
         *reinterpret_cast<u32x2*>(ot + i * OS + 32 * db + 8 * vq + 4 * g) = pk;
       }
     __builtin_amdgcn_wave_barrier();
@@ -882,24 +1125,49 @@ __global__ __launch_bounds__(kNW * 64) void prefill_kernel(PrefillParams pp) {
     const int orow_l = l / CPRO, ochunk = l % CPRO;
 #pragma unroll
     for (int n = 0; n < 32 / RPI; ++n) {
-      const int r = n * RPI + orow_l;
-      const u32x4 val = *reinterpret_cast<const u32x4*>(ot + r * OS + 8 * ochunk);
-      if (wrow0 + r < p.lq)
-        *reinterpret_cast<u32x4*>(p.o + (((int64_t)b * p.lq + wrow0 + r) * p.H + h) * D + 8 * ochunk) = val;
+      const int rr = n * RPI + orow_l;
+      const u32x4 val = *reinterpret_cast<const u32x4*>(ot + rr * OS + 8 * ochunk);
+      if (wrow0[r] + rr < p.lq)
+        *reinterpret_cast<u32x4*>(p.o + (((int64_t)b * p.lq + wrow0[r] + rr) * p.H + h) * D + 8 * ochunk) = val;
     }
-  }
-  if (qrow < p.lq && p.lse && g == 0) p.lse[((int64_t)b * p.H + h) * p.lq + qrow] = (mref + __builtin_amdgcn_logf(ltot)) * kLn2;
+    __builtin_amdgcn_wave_barrier();
+    if (qrow[r] < p.lq && p.lse && g == 0)
+      p.lse[((int64_t)b * p.H + h) * p.lq + qrow[r]] = (mref[r] + __builtin_amdgcn_logf(ltot)) * kLn2;
+  });
+}
+
+template <int D, int LOADER, bool SEG, int RB>
+int launch_prefill_rb(const PrefillParams& p, hipStream_t stream) {
+  auto kern = prefill_kernel<D, LOADER, SEG, RB>;
+  constexpr size_t lds_bytes = Lds<D, RB>::kBytes;
+  static bool configured[kMaxDevices] = {};
+  if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), lds_bytes); rc != TPA_OK) return rc;
+  const int groups = (p.npairs + 7) / 8;
+  dim3 grid(groups * 8 * p.H);
+  hipLaunchKernelGGL(kern, grid, dim3((8 / RB) * 64), lds_bytes, stream, p);
+  return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
+}
+
+// Rows per wave.  Eight waves of 32 rows is what every problem runs on.  Four waves of 64 rows
+// (head size 128, rank-2 or dense loader, no segment ids: the hand-scheduled loop exists for
+// exactly that) halves the LDS reads per MFMA but leaves each SIMD with a single wave, which
+// issues one vector instruction per ~6 cycles whatever it does: measured 4 % slower at 32768
+// rows and 40 % slower at 4096, so it is only selected by TPA_PREFILL_ROW_BLOCKS=2 in the
+// environment (a measuring aid, read once per process).
+bool two_row_blocks_requested() {
+  static const bool v = [] {
+    const char* e = getenv("TPA_PREFILL_ROW_BLOCKS");
+    return e && e[0] == '2';
+  }();
+  return v;
 }
 
 template <int D, int LOADER, bool SEG = false>
 int launch_prefill(const PrefillParams& p, hipStream_t stream) {
-  auto kern = prefill_kernel<D, LOADER, SEG>;
-  static bool configured[kMaxDevices] = {};
-  if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), Lds<D>::kBytes); rc != TPA_OK) return rc;
-  const int groups = (p.npairs + 7) / 8;
-  dim3 grid(groups * 8 * p.H);
-  hipLaunchKernelGGL(kern, grid, dim3(kNW * 64), Lds<D>::kBytes, stream, p);
-  return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
+  if constexpr (D == 128 && !SEG && LOADER != LOAD_TPA_ANY) {
+    if (two_row_blocks_requested()) return launch_prefill_rb<D, LOADER, SEG, 2>(p, stream);
+  }
+  return launch_prefill_rb<D, LOADER, SEG, 1>(p, stream);
 }
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
