@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define TPA_ABI_VERSION 5
+#define TPA_ABI_VERSION 6
 
 /* element types of the factor / output arrays */
 enum { TPA_DTYPE_F32 = 0, TPA_DTYPE_BF16 = 1 };
@@ -215,6 +215,48 @@ typedef struct MhaBwdArgs {
   void* workspace;        /* required: at least mha_bwd_workspace_bytes(...) bytes, 256-byte aligned */
   size_t workspace_bytes;
 } MhaBwdArgs;
+
+/*
+ * tpa_cache_append arguments: the producer step of a TPA layer for n new tokens per sequence.  No
+ * counterpart in the reference, which takes the factors as given (tpa/tpa.py:74-77); this is the
+ * step that makes them (arXiv 2501.06425, section 3: the factors are linear in the hidden state and
+ * rotary position embedding is applied to the B factors of Q and K) and appends the K / V factors
+ * to the cache that tpa_decode and tpa_fwd read:
+ *   y[b, i, :] = W x[b, i, :]                      W[n_out, d_model] row-major (out, in), columns of y in
+ *                                                  the order qa[rq*H] qb[rq*D] ka[rk*H] kb[rk*D] va[rk*H] vb[rk*D]
+ *   qb, kb: each rank row rotated pairwise, (y[2j], y[2j+1]) by the angle of position pos and
+ *           frequency j:  y'[2j] = y[2j] c - y[2j+1] s,  y'[2j+1] = y[2j+1] c + y[2j] s,
+ *           c = rope_cos[pos, j], s = rope_sin[pos, j]
+ *   pos = positions[b, i] if given, else kv_lengths[b] + i (0 + i without kv_lengths)
+ *   qa, qb are written to the q arrays at token i; ka, kb, va, vb at token kv_lengths[b] + i of batch
+ *   entry b's cache (contiguous, or paged exactly as in TpaFwdArgs).  Tokens that would land at or
+ *   beyond cache_len are dropped.  new_kv_lengths[b] = min(kv_lengths[b] + n, cache_len) if given.
+ * The 1/R of the reconstruction is not applied here (tpa_fwd / tpa_decode apply it).
+ */
+typedef struct TpaAppendArgs {
+  const void* x;          /* [B, n, d_model] contiguous, element type = dtype */
+  const void* w;          /* [rq*(H+D) + 2*rk*(H+D), d_model] contiguous, element type = dtype */
+  const float* rope_cos;  /* [rope_len, D/2] fp32 */
+  const float* rope_sin;  /* [rope_len, D/2] fp32 */
+  const int32_t* positions;   /* [B, n] or NULL */
+  const int32_t* kv_lengths;  /* [B] tokens already in each cache, or NULL (= 0) */
+  int32_t* new_kv_lengths;    /* [B] or NULL; must not alias kv_lengths */
+  TpaFactor qa, qb;           /* outputs [B, n, rq, H], [B, n, rq, D] (ptr is written through) */
+  TpaFactor ka, kb, va, vb;   /* the cache, [B, cache_len, rk, H|D] or page pools (ptr is written through) */
+  const int32_t* page_table;  /* as in TpaFwdArgs, or NULL */
+  int32_t page_size, pages_per_seq;
+  int32_t B, n, d_model, H, D, rq, rk;
+  int32_t cache_len;          /* token capacity of one sequence (paged: pages_per_seq * page_size) */
+  int32_t rope_len;           /* rows of the rotary tables: positions are clamped to rope_len - 1 */
+  int32_t dtype;              /* TPA_DTYPE_*: element type of x, w, the q outputs and the cache */
+  int32_t kernel;             /* TPA_KERNEL_*: the MFMA kernel takes bf16 with d_model % 64 == 0, H % 8 == 0, D % 8 == 0 */
+} TpaAppendArgs;
+
+/*
+ * Projections to the rank factors, rotary embedding and append to the factored cache (see
+ * TpaAppendArgs).  Enqueues one kernel on `stream`; needs no workspace.
+ */
+int tpa_cache_append(const TpaAppendArgs* args, void* stream);
 
 /* ABI version of the loaded library (TPA_ABI_VERSION it was built with). */
 int tpa_abi_version(void);

@@ -29,6 +29,15 @@ Backward (the gradients of the same functions):
   dense attention, central finite differences on a tiny case, and the literal gradients the
   reference holds (tpa/mha_test.py:87-118: dq = dk = 0, dv = [[1,1],[0,0],[1,1]]).
 
+Producer step (no counterpart in the reference, which takes the factors as given; arXiv 2501.06425,
+section 3, is what is restated):
+  * `rope_rotate`          - rotary position embedding on adjacent pairs (y[2j], y[2j+1])
+  * `tpa_append_reference` - the six factors of new tokens as linear maps of the hidden state, with
+                             the B factors of Q and K rotated
+  pinned by tests/test_oracle.py: float64 loops over every output element on a tiny case, and the
+  closed forms of a rotation (position 0 is the identity, pair norms are preserved, angles add,
+  the dot product of a rotated query and key depends on the distance of their positions only).
+
 How this oracle is pinned (tests/test_oracle.py): brute-force float64 loops on tiny shapes,
 torch's scaled_dot_product_attention and scipy's softmax/logsumexp as independent library
 routines, closed forms (zero queries -> running mean of V and LSE = ln(count); lk = 1), rank
@@ -54,6 +63,8 @@ __all__ = [
     "mha_backward",
     "project_to_factors",
     "tpa_backward",
+    "rope_rotate",
+    "tpa_append_reference",
 ]
 
 
@@ -234,3 +245,39 @@ def tpa_backward(q, k, v, q_segment_ids, kv_segment_ids, num_heads, do, sm_scale
     dq_, dk_, dv_ = mha_backward(reconstruct(qa, qb), reconstruct(ka, kb), reconstruct(va, vb), bias, sm_scale, do)
     cat = lambda pair: np.concatenate(pair, axis=-1)
     return cat(project_to_factors(dq_, qa, qb)), cat(project_to_factors(dk_, ka, kb)), cat(project_to_factors(dv_, va, vb))
+
+
+def rope_rotate(y, cos, sin):
+    """Rotate adjacent pairs: y[..., 2j] c - y[..., 2j+1] s, y[..., 2j+1] c + y[..., 2j] s with
+    c = cos[..., j], s = sin[..., j] (cos / sin broadcast against y's leading dimensions)."""
+    y = np.asarray(y, dtype=np.float64)
+    even, odd = y[..., 0::2], y[..., 1::2]
+    out = np.empty_like(y)
+    out[..., 0::2] = even * cos - odd * sin
+    out[..., 1::2] = odd * cos + even * sin
+    return out
+
+
+def tpa_append_reference(x, w, rope_cos, rope_sin, positions, num_heads, head_dim, rank_q, rank_k):
+    """Factors of new tokens: y = x w^T with w[n_out, d_model], y's columns in the order
+    qa[rq*h] qb[rq*d] ka[rk*h] kb[rk*d] va[rk*h] vb[rk*d]; qb and kb rotated at `positions[b, i]`.
+
+    x[b, n, d_model], rope_cos / rope_sin[rope_len, d/2], positions[b, n] ->
+    dict of float64 arrays qa[b,n,rq,h], qb[b,n,rq,d], ka[b,n,rk,h], kb[b,n,rk,d], va, vb."""
+    x = np.asarray(x, dtype=np.float64)
+    w = np.asarray(w, dtype=np.float64)
+    b, n, _ = x.shape
+    h, d = num_heads, head_dim
+    y = x @ w.T
+    widths = [rank_q * h, rank_q * d, rank_k * h, rank_k * d, rank_k * h, rank_k * d]
+    assert w.shape[0] == sum(widths), (w.shape, widths)
+    out, c0 = {}, 0
+    for name, width, r, inner in zip(("qa", "qb", "ka", "kb", "va", "vb"), widths, (rank_q,) * 2 + (rank_k,) * 4, (h, d) * 3):
+        out[name] = y[..., c0 : c0 + width].reshape(b, n, r, inner)
+        c0 += width
+    pos = np.asarray(positions)
+    c = np.asarray(rope_cos, dtype=np.float64)[pos][:, :, None, :]  # [b, n, 1, d/2]
+    s_ = np.asarray(rope_sin, dtype=np.float64)[pos][:, :, None, :]
+    out["qb"] = rope_rotate(out["qb"], c, s_)
+    out["kb"] = rope_rotate(out["kb"], c, s_)
+    return out

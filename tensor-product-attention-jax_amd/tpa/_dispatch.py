@@ -22,7 +22,7 @@ KERNEL_AUTO = 0
 KERNEL_GENERIC = 1
 KERNEL_MFMA = 2
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 
 class TpaFactor(ctypes.Structure):
@@ -161,6 +161,38 @@ class MhaBwdArgs(ctypes.Structure):
     ]
 
 
+class TpaAppendArgs(ctypes.Structure):
+    _fields_ = [
+        ("x", ctypes.c_void_p),
+        ("w", ctypes.c_void_p),
+        ("rope_cos", ctypes.c_void_p),
+        ("rope_sin", ctypes.c_void_p),
+        ("positions", ctypes.c_void_p),
+        ("kv_lengths", ctypes.c_void_p),
+        ("new_kv_lengths", ctypes.c_void_p),
+        ("qa", TpaFactor),
+        ("qb", TpaFactor),
+        ("ka", TpaFactor),
+        ("kb", TpaFactor),
+        ("va", TpaFactor),
+        ("vb", TpaFactor),
+        ("page_table", ctypes.c_void_p),
+        ("page_size", ctypes.c_int32),
+        ("pages_per_seq", ctypes.c_int32),
+        ("B", ctypes.c_int32),
+        ("n", ctypes.c_int32),
+        ("d_model", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("D", ctypes.c_int32),
+        ("rq", ctypes.c_int32),
+        ("rk", ctypes.c_int32),
+        ("cache_len", ctypes.c_int32),
+        ("rope_len", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("kernel", ctypes.c_int32),
+    ]
+
+
 class TpaError(RuntimeError):
     """A non-zero return code of the C ABI."""
 
@@ -196,6 +228,8 @@ def load_library(path: str | None = None) -> ctypes.CDLL:
             fn.argtypes = [ctypes.POINTER(TpaFwdArgs), ctypes.c_void_p]
         lib.mha_fwd.restype = ctypes.c_int
         lib.mha_fwd.argtypes = [ctypes.POINTER(MhaFwdArgs), ctypes.c_void_p]
+        lib.tpa_cache_append.restype = ctypes.c_int
+        lib.tpa_cache_append.argtypes = [ctypes.POINTER(TpaAppendArgs), ctypes.c_void_p]
         lib.tpa_decode_workspace_bytes.restype = ctypes.c_size_t
         lib.tpa_decode_workspace_bytes.argtypes = [ctypes.c_int32] * 6
         lib.tpa_decode_default_splits.restype = ctypes.c_int32

@@ -30,7 +30,7 @@ import torch
 from . import _dispatch as _d
 
 __all__ = [
-    "BlockSizes", "tpa", "tpa_factors", "tpa_decode", "tpa_factors_bwd", "_tpa_fwd", "_tpa_bwd", "_fwd", "_bwd",
+    "BlockSizes", "tpa", "tpa_factors", "tpa_decode", "tpa_cache_append", "tpa_factors_bwd", "_tpa_fwd", "_tpa_bwd", "_fwd", "_bwd",
     "_precompute_delta", "_lse", "_lse_accum",
 ]
 
@@ -258,6 +258,72 @@ def tpa_decode(
     with torch.cuda.device(device):
         _d.check("tpa_decode", lib.tpa_decode(args, _d.current_stream_ptr(device)))
     return o, lse
+
+
+def tpa_cache_append(
+    x, w, rope_cos, rope_sin, ka, kb, va, vb,
+    kv_lengths=None,
+    *,
+    rank_q: int,
+    positions=None,
+    page_table=None,
+    kernel: int = _d.KERNEL_AUTO,
+):
+    """The producer step for `n` new tokens per sequence (an addition: the reference takes the
+    factors as given): y = x w^T gives the six rank factors of every token, the B factors of Q and
+    K are rotated by the rotary tables at the token's position, and the K / V factors are written
+    into the cache `ka, kb, va, vb` at token `kv_lengths[b] + i` - the arrays `tpa_decode` reads.
+
+    x[b, n, d_model]; w[rq*(h+d) + 2*rk*(h+d), d_model] (rows in the order qa, qb, ka, kb, va, vb,
+    as torch.nn.Linear keeps its weight); rope_cos, rope_sin[rope_len, d/2] fp32; the cache arrays
+    [b, cache_len, rk, h|d], or page pools [pages, page_size, rk, h|d] with `page_table`
+    [b, pages_per_seq]; `positions` [b, n] defaults to kv_lengths[b] + i.
+    Returns (qa[b, n, rq, h], qb[b, n, rq, d], new_kv_lengths[b])."""
+    device = _pick_device(x, w, ka, kb, va, vb)
+    x, w, ka, kb, va, vb = (_as_device_tensor(t, device) for t in (x, w, ka, kb, va, vb))
+    dtype = x.dtype
+    for name, t in (("w", w), ("ka", ka), ("kb", kb), ("va", va), ("vb", vb)):
+        if t.dtype != dtype:
+            raise TypeError(f"{name} has dtype {t.dtype}, expected {dtype}")
+    b, n, d_model = x.shape
+    rk, h = ka.shape[2], ka.shape[3]
+    d = kb.shape[3]
+    rq = int(rank_q)
+    assert tuple(w.shape) == (rq * (h + d) + 2 * rk * (h + d), d_model), w.shape
+    assert kb.shape[:3] == ka.shape[:3] and va.shape == ka.shape and vb.shape == kb.shape, (ka.shape, kb.shape, va.shape, vb.shape)
+    cos = _as_device_tensor(rope_cos, device).to(torch.float32).contiguous()
+    sin = _as_device_tensor(rope_sin, device).to(torch.float32).contiguous()
+    assert cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] == d // 2, (cos.shape, d)
+    pt, page_size, pages_per_seq = None, 0, 0
+    if page_table is None:
+        assert ka.shape[0] == b, ka.shape
+        cache_len = ka.shape[1]
+    else:
+        pt = _as_device_tensor(page_table, device).to(torch.int32).contiguous()
+        assert pt.dim() == 2 and pt.shape[0] == b, pt.shape
+        page_size, pages_per_seq = ka.shape[1], pt.shape[1]
+        cache_len = pages_per_seq * page_size
+    kvlen = _lengths(kv_lengths, b, device)
+    pos = None
+    if positions is not None:
+        pos = _as_device_tensor(positions, device).to(torch.int32).contiguous()
+        assert tuple(pos.shape) == (b, n), pos.shape
+    x, w = x.contiguous(), w.contiguous()
+    qa = torch.empty((b, n, rq, h), dtype=dtype, device=device)
+    qb = torch.empty((b, n, rq, d), dtype=dtype, device=device)
+    new_len = torch.empty((b,), dtype=torch.int32, device=device)
+    args = _d.TpaAppendArgs(
+        x=x.data_ptr(), w=w.data_ptr(), rope_cos=cos.data_ptr(), rope_sin=sin.data_ptr(),
+        positions=None if pos is None else pos.data_ptr(), kv_lengths=None if kvlen is None else kvlen.data_ptr(),
+        new_kv_lengths=new_len.data_ptr(),
+        qa=_d.factor(qa), qb=_d.factor(qb), ka=_d.factor(ka), kb=_d.factor(kb), va=_d.factor(va), vb=_d.factor(vb),
+        page_table=None if pt is None else pt.data_ptr(), page_size=int(page_size), pages_per_seq=int(pages_per_seq),
+        B=b, n=n, d_model=d_model, H=h, D=d, rq=rq, rk=rk, cache_len=int(cache_len), rope_len=int(cos.shape[0]),
+        dtype=_d.dtype_code(dtype), kernel=int(kernel),
+    )
+    with torch.cuda.device(device):
+        _d.check("tpa_cache_append", _d.load_library().tpa_cache_append(args, _d.current_stream_ptr(device)))
+    return qa, qb, new_len
 
 
 def decode_workspace_bytes(b: int, lq: int, lk: int, h: int, dv: int, num_splits: int = 0) -> int:

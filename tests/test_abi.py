@@ -43,7 +43,8 @@ def test_struct_layout_matches_the_c_compiler(tmp_path):
     from tpa import _dispatch as d
 
     fields = {"TpaFactor": d.TpaFactor, "TpaFwdArgs": d.TpaFwdArgs, "MhaFwdArgs": d.MhaFwdArgs,
-              "TpaGrad": d.TpaGrad, "TpaBwdArgs": d.TpaBwdArgs, "MhaBwdArgs": d.MhaBwdArgs}
+              "TpaGrad": d.TpaGrad, "TpaBwdArgs": d.TpaBwdArgs, "MhaBwdArgs": d.MhaBwdArgs,
+              "TpaAppendArgs": d.TpaAppendArgs}
     lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "tpa_abi.h"', "int main(void) {"]
     for sname, cls in fields.items():
         lines.append(f'printf("{sname} %zu\\n", sizeof({sname}));')
@@ -112,6 +113,17 @@ def test_null_and_shape_errors_are_reported_before_any_launch():
     mb = d.MhaBwdArgs()
     assert lib.mha_bwd(ctypes.byref(mb), None) == -2
     assert lib.mha_bwd(None, None) == -1
+    assert lib.tpa_cache_append(None, None) == -1
+    ap = d.TpaAppendArgs()
+    ap.dtype = 7
+    assert lib.tpa_cache_append(ctypes.byref(ap), None) == -3
+    ap.dtype = d.TPA_DTYPE_BF16
+    assert lib.tpa_cache_append(ctypes.byref(ap), None) == -2  # all dimensions are zero
+    ap.B = ap.n = ap.d_model = ap.rq = ap.rk = ap.cache_len = ap.rope_len = 1
+    ap.H, ap.D = 8, 12
+    assert lib.tpa_cache_append(ctypes.byref(ap), None) == -2  # head size not a multiple of 8
+    ap.D = 16
+    assert lib.tpa_cache_append(ctypes.byref(ap), None) == -1  # pointers are NULL
     assert lib.tpa_decode_noalloc(None, None) == -1
     assert lib.tpa_decode_noalloc(ctypes.byref(d.TpaFwdArgs()), None) == -2
 

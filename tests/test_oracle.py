@@ -303,3 +303,59 @@ def test_mha_backward_with_finite_bias_against_autograd():
         got = orc.mha_backward(q, k, v, bias, scale, do)
         for g, w in zip(got, (tq.grad, tk.grad, tv.grad)):
             np.testing.assert_allclose(g, w.numpy(), rtol=1e-10, atol=1e-12)
+
+
+# ---------------------------------------------------------------- the producer step (projections + rotary embedding)
+def _rope_tables(rope_len, d, base=10000.0):
+    inv = base ** (-np.arange(0, d, 2, dtype=np.float64) / d)
+    ang = np.arange(rope_len, dtype=np.float64)[:, None] * inv[None, :]
+    return np.cos(ang), np.sin(ang)
+
+
+def test_append_reference_against_loops():
+    rng = np.random.default_rng(5)
+    b, n, dm, h, d, rq, rk = 2, 3, 7, 2, 4, 2, 3
+    x = rng.standard_normal((b, n, dm))
+    w = rng.standard_normal((rq * (h + d) + 2 * rk * (h + d), dm))
+    cos, sin = _rope_tables(16, d)
+    pos = rng.integers(0, 16, (b, n))
+    got = orc.tpa_append_reference(x, w, cos, sin, pos, h, d, rq, rk)
+    row = 0
+    for name, r_, inner in (("qa", rq, h), ("qb", rq, d), ("ka", rk, h), ("kb", rk, d), ("va", rk, h), ("vb", rk, d)):
+        want = np.zeros((b, n, r_, inner))
+        for bi in range(b):
+            for i in range(n):
+                for r in range(r_):
+                    for e in range(inner):
+                        want[bi, i, r, e] = sum(x[bi, i, k] * w[row + r * inner + e, k] for k in range(dm))
+                    if name in ("qb", "kb"):
+                        y = want[bi, i, r].copy()
+                        for j in range(inner // 2):
+                            c, s_ = cos[pos[bi, i], j], sin[pos[bi, i], j]
+                            want[bi, i, r, 2 * j] = y[2 * j] * c - y[2 * j + 1] * s_
+                            want[bi, i, r, 2 * j + 1] = y[2 * j + 1] * c + y[2 * j] * s_
+        row += r_ * inner
+        np.testing.assert_allclose(got[name], want, rtol=1e-12, atol=1e-12, err_msg=name)
+
+
+def test_rope_closed_forms():
+    rng = np.random.default_rng(6)
+    d = 8
+    cos, sin = _rope_tables(64, d)
+    y = rng.standard_normal((5, d))
+    # position 0 is the identity
+    np.testing.assert_allclose(orc.rope_rotate(y, cos[0], sin[0]), y, atol=1e-15)
+    # a rotation: the norm of every pair is preserved
+    r = orc.rope_rotate(y, cos[17], sin[17])
+    np.testing.assert_allclose(r[:, 0::2] ** 2 + r[:, 1::2] ** 2, y[:, 0::2] ** 2 + y[:, 1::2] ** 2, rtol=1e-12)
+    # angles add: rotating by position 5 and then by position 9 is rotating by position 14
+    np.testing.assert_allclose(orc.rope_rotate(orc.rope_rotate(y, cos[5], sin[5]), cos[9], sin[9]), orc.rope_rotate(y, cos[14], sin[14]), atol=1e-12)
+    # the dot product of a rotated query and key depends on the distance of their positions only
+    q, k = rng.standard_normal(d), rng.standard_normal(d)
+    dots = [orc.rope_rotate(q, cos[m], sin[m]) @ orc.rope_rotate(k, cos[m - 7], sin[m - 7]) for m in (7, 20, 63)]
+    np.testing.assert_allclose(dots, dots[0], rtol=1e-12)
+    # ... and it is not the unrotated one (a sign slip in the rotation would pass the norm test)
+    assert abs(dots[0] - q @ k) > 1e-3
+    # direction: the first pair of (1, 0) at position p is (cos p, sin p) for frequency 1
+    e = np.zeros(d); e[0] = 1.0
+    np.testing.assert_allclose(orc.rope_rotate(e, cos[3], sin[3])[:2], [np.cos(3.0), np.sin(3.0)], atol=1e-12)
