@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c4pg|c4s|c5|c2f|c3f|c2fb|c4f|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|copy] [--no-cpu] [--no-decode] [--no-backward]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c3u|c4|c4pg|c4s|c5|c5u|c2n|c5n|c2f|c3f|c2fb|c4f|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|ap1|ap2|copy] [--no-cpu] [--no-decode] [--no-backward]
 
 A step is one forward pass over one batch of synthetic, seeded inputs that are resident in HBM
 before the timed region starts.  The default workload is the prefill configuration the headline
@@ -33,6 +33,13 @@ WORKLOADS = {
     "c2": ("prefill", 4, 4096, 4096, 16, 128, 6, 2, True),
     "c3": ("prefill", 1, 32768, 32768, 32, 128, 6, 2, True),
     "c5": ("prefill", 8, 2048, 2048, 64, 64, 16, 8, False),
+    # the same two without the optional workspace: the fused kernel that rebuilds every K/V tile from the
+    # rank factors inside the flash loop (with the workspace these shapes reconstruct dense K, V once)
+    "c3u": ("prefill", 1, 32768, 32768, 32, 128, 6, 2, True),
+    "c5u": ("prefill", 8, 2048, 2048, 64, 64, 16, 8, False),
+    # nomat=True (tpa/tpa.py:250): the order of operations that never forms K or V, at the c2 and c5 shapes
+    "c2n": ("prefill", 4, 4096, 4096, 16, 128, 6, 2, True),
+    "c5n": ("prefill", 8, 2048, 2048, 64, 64, 16, 8, False),
     "c4": ("decode", 64, 1, 8192, 32, 128, 6, 2, False),
     "c4pg": ("decode", 64, 1, 8192, 32, 128, 6, 2, False),  # the c4 cache as a pool of shuffled 64-token pages
     "c4s": ("decode", 64, 4, 8192, 32, 128, 6, 2, True),  # four appended tokens per sequence, each masked to its predecessors
@@ -52,17 +59,37 @@ WORKLOADS = {
     "c3f": ("prefill", 1, 16384, 16384, 32, 128, 6, 2, True),
     "c2fb": ("backward", 4, 4096, 4096, 16, 128, 6, 2, True),
     "c4f": ("decode", 64, 1, 8192, 32, 128, 6, 2, False),
+    # the producer step (tpa_cache_append): (kind, B, new tokens, cache length, H, D, rq, rk, -) with d_model = H * D:
+    # one decode step of the c4 batch, and a prefill chunk of 4096 tokens for four sequences
+    "ap1": ("append", 64, 1, 8192, 32, 128, 6, 2, False),
+    "ap2": ("append", 4, 4096, 8192, 32, 128, 6, 2, False),
 }
 F32_WORKLOADS = ("c2f", "c3f", "c2fb", "c4f")
 COPY_BYTES = 1 << 30  # --workload copy: bytes read (and bytes written) by each plain copy launch
 
-# HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counters (profiles/), each scaled by what
-# the same counter reads for the 1 GiB copy of `--workload copy`; None where no counter run exists.
-# FETCH_SIZE reads 0.5 KiB per KiB the copy fetches (scale 2.0), WRITE_SIZE 1.0 per KiB (scale 1.0).
-MEASURED_TRAFFIC = {
-    "c2": (2.0 * 56386.7 + 1.0 * 66560.0) * 1024,                     # prefill_kernel<128,0,false>
-    "c4": (2.0 * (328100.3 + 2135.5) + 1.0 * (4160.0 + 520.0)) * 1024,  # decode_kernel + decode_merge_kernel
-}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "prefill_c2_decode_c4_hbm_bytes.txt")
+
+
+def measured_traffic(workload):
+    """HBM bytes per launch of the workload's kernels, read from the committed rocprofv3 counter summary
+    (FETCH_SIZE / WRITE_SIZE in KiB per dispatch, one table row per kernel), each counter scaled by what it
+    reads for the 1 GiB device copy in the same table.  None where the summary has no row for the kernels."""
+    kernels = {"c2": ["prefill_kernel<128, 0, false"], "c4": ["decode_kernel<128, 2, false, 1", "decode_merge_kernel<128, bf16"]}.get(workload)
+    if not kernels or not os.path.exists(TRAFFIC_PROFILE):
+        return None
+    rows = {}
+    for line in open(TRAFFIC_PROFILE):
+        parts = line.split()
+        for k in kernels + ["__amd_rocclr_copyBuffer"]:
+            if line.strip().startswith(k):
+                nums = [float(x) for x in parts if x.replace(".", "", 1).isdigit() and "." in x]
+                if len(nums) >= 2:
+                    rows[k] = nums[:2]
+    if "__amd_rocclr_copyBuffer" not in rows or any(k not in rows for k in kernels):
+        return None
+    kib = COPY_BYTES / 1024
+    fetch_scale, write_scale = kib / rows["__amd_rocclr_copyBuffer"][0], kib / rows["__amd_rocclr_copyBuffer"][1]
+    return sum(fetch_scale * rows[k][0] + write_scale * rows[k][1] for k in kernels) * 1024
 
 
 def log(*a):
@@ -127,8 +154,11 @@ def run_prefill(torch, tpa, device, name, steps, warmup):
     if doc:
         seg = (torch.arange(lq, device=device, dtype=torch.int32) // doc).repeat(B, 1).contiguous()
 
+    use_ws = not name.endswith("u")
+    nomat = name.endswith("n")
+
     def step(i):
-        out["o"], out["lse"] = tpa.tpa_factors(*x, seg, seg, sm_scale=scale, causal=causal, kernel=2)
+        out["o"], out["lse"] = tpa.tpa_factors(*x, seg, seg, sm_scale=scale, causal=causal, kernel=2, use_workspace=use_ws, nomat=nomat)
 
     wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
     # packed: only pairs inside a document count
@@ -219,6 +249,31 @@ def run_decode(torch, tpa, device, name, steps, warmup):
         gbs_wall=nbytes / wall_ms / 1e6, gbs_kernel=nbytes / ev_ms / 1e6,
         shape=dict(B=B, lq=lq, lk=lk, H=H, D=D, rank_q=rq, rank_k=rk), inputs=xs[0], out=out,
     )
+
+
+def run_append(torch, tpa, device, name, steps, warmup):
+    """One step = one tpa_cache_append call: y = x W^T (M = B * n tokens, d_model = H * D inputs,
+    rq (H + D) + 2 rk (H + D) outputs), rotary embedding, rows appended to a bf16 factored cache."""
+    _, B, n, cache_len, H, D, rq, rk, _ = WORKLOADS[name]
+    dm = H * D
+    n_out = rq * (H + D) + 2 * rk * (H + D)
+    g = torch.Generator(device=device)
+    g.manual_seed(9)
+    x = torch.randn((B, n, dm), generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    w = (torch.randn((n_out, dm), generator=g, device=device, dtype=torch.float32) / dm**0.5).to(torch.bfloat16)
+    ang = torch.arange(cache_len, device=device, dtype=torch.float32)[:, None] * (10000.0 ** (-torch.arange(0, D, 2, device=device, dtype=torch.float32) / D))[None]
+    cos, sin = torch.cos(ang), torch.sin(ang)
+    caches = [torch.zeros((B, cache_len, rk, inner), dtype=torch.bfloat16, device=device) for inner in (H, D, H, D)]
+    lengths = torch.full((B,), cache_len - n - 1, dtype=torch.int32, device=device)
+
+    def step(i):
+        tpa.tpa_cache_append(x, w, cos, sin, *caches, lengths, rank_q=rq, kernel=2)
+
+    wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
+    fl = 2.0 * B * n * dm * n_out
+    nbytes = (B * n * dm + n_out * dm + B * n * n_out) * 2
+    return dict(wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, flops=fl, bytes=nbytes,
+                shape=dict(B=B, new_tokens=n, d_model=dm, H=H, D=D, rank_q=rq, rank_k=rk, outputs=n_out))
 
 
 def run_dense_decode(torch, mha, device, name, steps, warmup):
@@ -324,10 +379,11 @@ def main():
             metric="TPA causal prefill forward throughput" if r["shape"]["causal"] else "TPA prefill forward throughput",
             value=r["tflops_wall"], unit="TFLOP/s", ms_per_step=r["wall_ms"],
             roofline=dict(bound="mfma", achieved=r["tflops_kernel"], peak=peak, unit="TFLOP/s",
-                          frac=r["tflops_kernel"] / peak, traffic=MEASURED_TRAFFIC.get(args.workload),
-                          kernel="prefill_f32_kernel" if f32 else "prefill_kernel", ms_per_launch=r["kernel_ms"],
+                          frac=r["tflops_kernel"] / peak, traffic=measured_traffic(args.workload),
+                          kernel="prefill_f32_kernel" if f32 else ("decode_kernel + decode_merge_kernel per 64 query rows" if args.workload.endswith("n") else "prefill_kernel"),
+                          ms_per_launch=r["kernel_ms"],
                           ms_per_launch_min=r["kernel_ms_min"], algorithmic_flops_per_launch=r["flops"]),
-            config=dict(workload=f"{args.workload}: TPA prefill" + (", fp32 inputs" if f32 else ""), **r["shape"]),
+            config=dict(workload=f"{args.workload}: TPA prefill" + (", fp32 inputs" if f32 else "") + (", nomat" if args.workload.endswith("n") else ""), **r["shape"]),
         )
         if not args.no_decode and not f32:
             log("[bench] decode c4")
@@ -336,7 +392,7 @@ def main():
             result["decode"] = dict(
                 metric="TPA decode effective HBM bandwidth", value=d["gbs_wall"], unit="GB/s", ms_per_step=d["wall_ms"],
                 roofline=dict(bound="hbm", achieved=d["gbs_kernel"], peak=PEAK_HBM_GBS, unit="GB/s",
-                              frac=d["gbs_kernel"] / PEAK_HBM_GBS, traffic=MEASURED_TRAFFIC.get("c4"),
+                              frac=d["gbs_kernel"] / PEAK_HBM_GBS, traffic=measured_traffic("c4"),
                               kernel="decode_kernel + decode_merge_kernel",
                               ms_per_launch=d["kernel_ms"], ms_per_launch_min=d["kernel_ms_min"],
                               algorithmic_bytes_per_launch=d["bytes"]),
@@ -385,6 +441,22 @@ def main():
                           algorithmic_flops_per_launch=r["flops"]),
             config=dict(workload=f"{args.workload}: dense flash attention (tpa/mha.py) at the prefill shape", **r["shape"]),
         )
+    elif kind == "append":
+        log(f"[bench] cache append {args.workload}: warmup {args.warmup}, steps {args.steps}")
+        r = run_append(torch, tpa, device, args.workload, args.steps, args.warmup)
+        # few tokens: the weights are read once (HBM); many: the product is bound by the matrix cores
+        hbm = r["shape"]["new_tokens"] * r["shape"]["B"] <= 256
+        ach = r["bytes"] / r["kernel_ms"] / 1e6 if hbm else r["flops"] / r["kernel_ms"] / 1e9
+        log(f"[bench] {r['kernel_ms']*1e3:.1f} us/launch, {ach:.1f} {'GB/s' if hbm else 'TFLOP/s'}")
+        result.update(
+            metric="TPA cache append (factor projections + rotary embedding) throughput", value=(r["bytes"] / r["wall_ms"] / 1e6 if hbm else r["flops"] / r["wall_ms"] / 1e9),
+            unit="GB/s" if hbm else "TFLOP/s", ms_per_step=r["wall_ms"],
+            roofline=dict(bound="hbm" if hbm else "mfma", achieved=ach, peak=PEAK_HBM_GBS if hbm else PEAK_BF16_TFLOPS,
+                          unit="GB/s" if hbm else "TFLOP/s", frac=ach / (PEAK_HBM_GBS if hbm else PEAK_BF16_TFLOPS), traffic=None,
+                          kernel="append_mfma_kernel", ms_per_launch=r["kernel_ms"], ms_per_launch_min=r["kernel_ms_min"],
+                          algorithmic_flops_per_launch=r["flops"], algorithmic_bytes_per_launch=r["bytes"]),
+            config=dict(workload=f"{args.workload}: TPA cache append", **r["shape"]),
+        )
     elif kind == "backward":
         log(f"[bench] backward {args.workload}: warmup {args.warmup}, steps {args.steps}")
         r = run_backward(torch, tpa, device, args.workload, args.steps, args.warmup)
@@ -408,7 +480,7 @@ def main():
         result.update(
             metric="TPA decode effective HBM bandwidth", value=d["gbs_wall"], unit="GB/s", ms_per_step=d["wall_ms"],
             roofline=dict(bound="hbm", achieved=d["gbs_kernel"], peak=PEAK_HBM_GBS, unit="GB/s",
-                          frac=d["gbs_kernel"] / PEAK_HBM_GBS, traffic=MEASURED_TRAFFIC.get(args.workload),
+                          frac=d["gbs_kernel"] / PEAK_HBM_GBS, traffic=measured_traffic(args.workload),
                           kernel=("decode_f32_kernel" if args.workload in F32_WORKLOADS else "decode_kernel") + " + decode_merge_kernel",
                           ms_per_launch=d["kernel_ms"], ms_per_launch_min=d["kernel_ms_min"],
                           algorithmic_bytes_per_launch=d["bytes"]),

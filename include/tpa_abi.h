@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define TPA_ABI_VERSION 6
+#define TPA_ABI_VERSION 7
 
 /* element types of the factor / output arrays */
 enum { TPA_DTYPE_F32 = 0, TPA_DTYPE_BF16 = 1 };
@@ -123,6 +123,18 @@ typedef struct TpaFwdArgs {
      it meets (tpa/ring_tpa.py:73-79 calls the block function with local indices only).  Rows that see no key
      end as NaN / -inf like any other empty row.  tpa_fwd and tpa_decode; ignored when causal == 0. */
   int32_t causal_offset;
+  /* tpa_fwd only; replaces the static `nomat` of the reference kernel (tpa/tpa.py:250, 333-359, 398-413).  Non-zero:
+     never form K or V.  The logits come from the rank-space identity x = (sm_scale / (rq rk)) sum_{r,s}
+     (qa_r . ka_s restricted to the head)(qb_r . kb_s), whose (qb_r . kb_s) table is shared by every head, and
+     o = (1/rk) sum_s (sum_k p_k va_s[k]) vb_s likewise.  Query rows are served in windows of at most 64 by the
+     split-key kernels of tpa_decode, which need args.workspace >= tpa_fwd_nomat_workspace_bytes(...) (else
+     TPA_ERR_WORKSPACE) and the shapes those kernels take (dk == dv in {64, 128}, rk a power of two <= 32, no
+     segment ids; bf16 also H % 8 == 0 and 16-byte aligned factors); any other problem runs the generic kernel
+     (TPA_ERR_UNSUPPORTED with kernel == TPA_KERNEL_MFMA).  The result is the same function of the inputs as with
+     nomat == 0 (tpa/tpa_test.py:122-190 runs one grid over both), in another order of operations.  Never chosen
+     by the library itself: on matrix cores it is the faster route only for a few query rows over a long
+     cache, which is what tpa_decode is. */
+  int32_t nomat;
 } TpaFwdArgs;
 
 /*
@@ -283,6 +295,13 @@ int tpa_fwd(const TpaFwdArgs* args, void* stream);
  * query block) and the flash kernel runs with its plain tile loader.
  */
 size_t tpa_fwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dk, int32_t dv, int32_t rq, int32_t rk);
+
+/*
+ * Bytes of workspace (256-byte aligned) tpa_fwd needs with args.nomat != 0 for the split-key kernels to serve
+ * the problem, 0 if its head sizes or rank are not theirs (then the generic kernel runs and needs none).  The
+ * same workspace serves every window of query rows in turn.
+ */
+size_t tpa_fwd_nomat_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dk, int32_t dv, int32_t rq, int32_t rk);
 
 /*
  * Forward pass for few query tokens over a long factored cache (the reference reaches this as

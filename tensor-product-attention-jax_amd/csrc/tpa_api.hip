@@ -59,11 +59,61 @@ const char* tpa_strerror(int code) {
   }
 }
 
+namespace {
+
+constexpr int kNomatWindow = 64;  // query rows one pass of the split-key kernels serves
+
+bool nomat_rank_and_heads(int dk, int dv, int rk) {
+  return dk == dv && (dk == 64 || dk == 128) && rk >= 1 && rk <= 32 && (rk & (rk - 1)) == 0;
+}
+
+// tpa_fwd with nomat: the split-key kernels, which never form K or V, over windows of query rows.  Every window
+// shares the workspace; they run one after the other on the stream.
+int tpa_fwd_nomat(const TpaFwdArgs* a, hipStream_t s) {
+  TpaFwdArgs w = *a;
+  w.lq = a->lq < kNomatWindow ? a->lq : kNomatWindow;
+  w.nomat = 0;
+  const bool bf16 = a->kernel != TPA_KERNEL_GENERIC && tpa_decode_mfma_supported(&w);
+  const bool f32 = a->kernel != TPA_KERNEL_GENERIC && !bf16 && tpa_decode_f32_supported(&w);
+  if (!bf16 && !f32) {
+    if (a->kernel == TPA_KERNEL_MFMA) return TPA_ERR_UNSUPPORTED;
+    return tpa_generic_launch(a, s);
+  }
+  const size_t need = a->num_splits > 0 ? tpa_decode_workspace_bytes(a->B, w.lq, a->lk, a->H, a->dv, a->num_splits)
+                                        : tpa_fwd_nomat_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dk, a->dv, a->rq, a->rk);
+  if (!a->workspace || a->workspace_bytes < need) return TPA_ERR_WORKSPACE;
+  const size_t esz = a->dtype == TPA_DTYPE_BF16 ? 2 : 4;
+  for (int row0 = 0; row0 < a->lq; row0 += kNomatWindow) {
+    w.lq = a->lq - row0 < kNomatWindow ? a->lq - row0 : kNomatWindow;
+    w.qa.ptr = static_cast<const char*>(a->qa.ptr) + (size_t)row0 * a->qa.stride_l * esz;
+    w.qb.ptr = static_cast<const char*>(a->qb.ptr) + (size_t)row0 * a->qb.stride_l * esz;
+    const int rc = bf16 ? tpa_decode_mfma_launch_rows(&w, s, row0, a->lq) : tpa_decode_f32_launch_rows(&w, s, row0, a->lq);
+    if (rc != TPA_OK) return rc;
+  }
+  return TPA_OK;
+}
+
+}  // namespace
+
+size_t tpa_fwd_nomat_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dk, int32_t dv, int32_t rq, int32_t rk) {
+  (void)rq;
+  if (B <= 0 || lq <= 0 || lk <= 0 || H <= 0 || !nomat_rank_and_heads(dk, dv, rk)) return 0;
+  // full windows and the last, shorter one choose their own number of key ranges
+  const int full = lq < kNomatWindow ? lq : kNomatWindow, tail = lq % kNomatWindow;
+  size_t need = tpa_decode_workspace_bytes(B, full, lk, H, dv, 0);
+  if (lq > kNomatWindow && tail) {
+    const size_t t = tpa_decode_workspace_bytes(B, tail, lk, H, dv, 0);
+    if (t > need) need = t;
+  }
+  return need;
+}
+
 int tpa_fwd(const TpaFwdArgs* a, void* stream) {
   const int rc = tpa_validate_fwd_args(a);
   if (rc != TPA_OK) return rc;
   if (a->page_table) return TPA_ERR_UNSUPPORTED;  // paged caches are read by tpa_decode only
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (a->nomat) return tpa_fwd_nomat(a, s);
   // few query tokens over a long cache (the reference's decode is this same call with lq = 1,
   // tpa/tpa.py:485): split over keys, if the caller brought the workspace for it
   if (a->kernel != TPA_KERNEL_GENERIC && a->workspace && a->lq <= 16 && a->lk >= 1024 &&

@@ -175,6 +175,10 @@ int tpa_decode_mfma_supported(const TpaFwdArgs* a);
 int tpa_decode_mfma_launch(const TpaFwdArgs* a, hipStream_t stream);
 int tpa_decode_f32_supported(const TpaFwdArgs* a);
 int tpa_decode_f32_launch(const TpaFwdArgs* a, hipStream_t stream);
+// the same for a->lq query rows that are rows row0 .. row0 + a->lq - 1 of lq_total: a->qa / a->qb point at row row0,
+// a->o / a->lse at row 0 of the full arrays, the causal mask counts rows from row0
+int tpa_decode_mfma_launch_rows(const TpaFwdArgs* a, hipStream_t stream, int row0, int lq_total);
+int tpa_decode_f32_launch_rows(const TpaFwdArgs* a, hipStream_t stream, int row0, int lq_total);
 int mha_decode_supported(const MhaFwdArgs* a);
 int mha_decode_launch(const MhaFwdArgs* a, hipStream_t stream);
 int tpa_bwd_launch(const TpaBwdArgs* a, hipStream_t stream, int mfma);

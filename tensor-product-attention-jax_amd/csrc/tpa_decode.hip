@@ -37,7 +37,9 @@ struct DecodeParams {
   int page_size, pages_per_seq;  // tokens per page; table row length
   int B, lq, lk, H, rq;
   int climit;      // query row qi sees its first qi + climit keys (causal: offset + 1; otherwise lk, no limit)
-  int cbr;         // causal, last query aligned with the last key of each batch entry: climit counts from len - lq
+  int cbr;         // causal, last query aligned with the last key of each batch entry: climit counts from len - lq_total
+  int row0;        // this call serves query rows row0 .. row0 + lq - 1 of lq_total (outputs are indexed with them)
+  int lq_total;
   int S;           // key ranges
   float qscale;    // sm_scale * log2(e) / (rq * rk)
 };
@@ -125,7 +127,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
   int row_last[NQ], len_b = 0;
 #pragma unroll
   for (int r = 0; r < NQ; ++r) {
-    const int len_r = max(0, min(len_all, min(qi0 + r, p.lq - 1) + p.climit + (p.cbr ? len_all - p.lq : 0)));
+    const int len_r = max(0, min(len_all, min(qi0 + r, p.lq - 1) + p.climit + (p.cbr ? len_all - p.lq_total : 0)));
     row_last[r] = len_r * RK - 1;
     len_b = max(len_b, len_r);
   }
@@ -448,7 +450,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_f32_kernel(DecodeParams p)
   const int nparts = S * kWaves;
   const int part = split * kWaves + w;
   const int len_all = p.kvlen ? min(p.kvlen[b], p.lk) : p.lk;
-  const int len_b = max(0, min(len_all, qi + p.climit + (p.cbr ? len_all - p.lq : 0)));
+  const int len_b = max(0, min(len_all, qi + p.climit + (p.cbr ? len_all - p.lq_total : 0)));
   const int blk_begin = part;
   const int blk_end = (len_b * RK + kRowsPerBlock - 1) / kRowsPerBlock;
   const int blk_step = nparts;
@@ -655,7 +657,7 @@ __global__ __launch_bounds__(kWaves * 64) void decode_f32_kernel(DecodeParams p)
 // Merge the key ranges: o = sum_s f_s O_s / (Rk sum_s f_s l_s), f_s = 2^(m_s - max m); lse = ln of the total.
 template <int D, typename TO>
 __global__ __launch_bounds__(D) void decode_merge_kernel(const float* part_o, const float* part_m, const float* part_l,
-                                                         TO* o, float* lse, int S, int H, int lq, float inv_rk) {
+                                                         TO* o, float* lse, int S, int H, int lq, float inv_rk, int row0, int lq_total) {
   const int bq = blockIdx.x;  // b * lq + qi
   const int h = blockIdx.y;
   const int d = threadIdx.x;
@@ -686,19 +688,22 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(const float* part_o, co
     }
     mmax = gmax;
   }
-  store_from_f32(o + ((int64_t)bq * H + h) * D + d, acc * inv_rk / lacc);
-  if (lse && d == 0) {
-    const int b = bq / lq, qi = bq % lq;
-    lse[((int64_t)b * H + h) * lq + qi] = (mmax + __builtin_amdgcn_logf(lacc)) * kLn2;
-  }
+  // this call's rows are row0 .. row0 + lq - 1 of the lq_total rows of o and lse
+  const int b = bq / lq, qi = bq % lq;
+  store_from_f32(o + (((int64_t)b * lq_total + row0 + qi) * H + h) * D + d, acc * inv_rk / lacc);
+  if (lse && d == 0) lse[((int64_t)b * H + h) * lq_total + row0 + qi] = (mmax + __builtin_amdgcn_logf(lacc)) * kLn2;
 }
 
 size_t workspace_bytes(int B, int lq, int H, int D, int S) {
   return (size_t)B * lq * S * H * (D + 2) * sizeof(float);
 }
 
+// `rows` = {row0, lq_total}: the call serves a->lq query rows that are rows row0 .. of lq_total (a->qa / a->qb point at
+// row row0; a->o and a->lse at row 0); a plain call has {0, a->lq}
+struct RowWindow { int row0, lq_total; };
+
 template <int D, int RK, bool PAGED, int NQ>
-int launch_decode_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
+int launch_decode_t(const TpaFwdArgs* a, int S, hipStream_t stream, RowWindow rows) {
   DecodeParams p{};
   p.qa = a->qa; p.qb = a->qb; p.ka = a->ka; p.kb = a->kb; p.va = a->va; p.vb = a->vb;
   float* ws = static_cast<float*>(a->workspace);
@@ -707,8 +712,9 @@ int launch_decode_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   p.part_o = ws; p.part_m = ws + no; p.part_l = ws + no + nm;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.S = S;
   p.kvlen = a->kv_lengths;
-  p.climit = a->causal ? causal_offset_of(a) + 1 : a->lk;
+  p.climit = a->causal ? causal_offset_of(a) + 1 + rows.row0 : a->lk;
   p.cbr = a->causal == TPA_CAUSAL_BOTTOM_RIGHT;
+  p.row0 = rows.row0; p.lq_total = rows.lq_total;
   p.page_table = a->page_table; p.page_size = a->page_size; p.pages_per_seq = a->pages_per_seq;
   p.qscale = a->sm_scale * kLog2e / ((float)a->rq * (float)RK);
   auto kern = decode_kernel<D, RK, PAGED, NQ>;
@@ -718,12 +724,12 @@ int launch_decode_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   hipLaunchKernelGGL(kern, grid, dim3(kWaves * 64), DecodeLds<D>::bytes(NQ), stream, p);
   if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
   hipLaunchKernelGGL((decode_merge_kernel<D, uint16_t>), dim3(a->B * a->lq, a->H), dim3(D), 0, stream, p.part_o, p.part_m, p.part_l,
-                     static_cast<uint16_t*>(a->o), a->lse, S, a->H, a->lq, 1.f / (float)RK);
+                     static_cast<uint16_t*>(a->o), a->lse, S, a->H, a->lq, 1.f / (float)RK, rows.row0, rows.lq_total);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
 }
 
 template <int D, int RK, bool PAGED>
-int launch_decode_f32_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
+int launch_decode_f32_t(const TpaFwdArgs* a, int S, hipStream_t stream, RowWindow rows) {
   DecodeParams p{};
   p.qa = a->qa; p.qb = a->qb; p.ka = a->ka; p.kb = a->kb; p.va = a->va; p.vb = a->vb;
   float* ws = static_cast<float*>(a->workspace);
@@ -731,8 +737,9 @@ int launch_decode_f32_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   p.part_o = ws; p.part_m = ws + no; p.part_l = ws + no + nm;
   p.B = a->B; p.lq = a->lq; p.lk = a->lk; p.H = a->H; p.rq = a->rq; p.S = S;
   p.kvlen = a->kv_lengths;
-  p.climit = a->causal ? causal_offset_of(a) + 1 : a->lk;
+  p.climit = a->causal ? causal_offset_of(a) + 1 + rows.row0 : a->lk;
   p.cbr = a->causal == TPA_CAUSAL_BOTTOM_RIGHT;
+  p.row0 = rows.row0; p.lq_total = rows.lq_total;
   p.page_table = a->page_table; p.page_size = a->page_size; p.pages_per_seq = a->pages_per_seq;
   p.qscale = a->sm_scale * kLog2e / ((float)a->rq * (float)RK);
   auto kern = decode_f32_kernel<D, RK, PAGED>;
@@ -742,31 +749,31 @@ int launch_decode_f32_t(const TpaFwdArgs* a, int S, hipStream_t stream) {
   hipLaunchKernelGGL(kern, grid, dim3(kWaves * 64), DecodeF32Lds<D>::kBytes, stream, p);
   if (hipGetLastError() != hipSuccess) return TPA_ERR_LAUNCH;
   hipLaunchKernelGGL((decode_merge_kernel<D, float>), dim3(a->B * a->lq, a->H), dim3(D), 0, stream, p.part_o, p.part_m, p.part_l,
-                     static_cast<float*>(a->o), a->lse, S, a->H, a->lq, 1.f / (float)RK);
+                     static_cast<float*>(a->o), a->lse, S, a->H, a->lq, 1.f / (float)RK, rows.row0, rows.lq_total);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
 }
 
 template <int D, int RK>
-int launch_decode_f32(const TpaFwdArgs* a, int S, hipStream_t stream) {
+int launch_decode_f32(const TpaFwdArgs* a, int S, hipStream_t stream, RowWindow rows) {
   if (a->page_table) {
     if (a->page_size <= 0 || (a->page_size * RK) % kRowsPerBlock != 0 ||
         (int64_t)a->pages_per_seq * a->page_size < a->lk)
       return TPA_ERR_SHAPE;
-    return launch_decode_f32_t<D, RK, true>(a, S, stream);
+    return launch_decode_f32_t<D, RK, true>(a, S, stream, rows);
   }
-  return launch_decode_f32_t<D, RK, false>(a, S, stream);
+  return launch_decode_f32_t<D, RK, false>(a, S, stream, rows);
 }
 
 template <int D, int RK>
-int launch_decode(const TpaFwdArgs* a, int S, hipStream_t stream) {
+int launch_decode(const TpaFwdArgs* a, int S, hipStream_t stream, RowWindow rows) {
   if (a->page_table) {
     // a block of 32 (token, rank) rows must not straddle pages, and the table must cover lk
     if (a->page_size <= 0 || (a->page_size * RK) % kRowsPerBlock != 0 ||
         (int64_t)a->pages_per_seq * a->page_size < a->lk)
       return TPA_ERR_SHAPE;
-    return a->lq >= 2 ? launch_decode_t<D, RK, true, 2>(a, S, stream) : launch_decode_t<D, RK, true, 1>(a, S, stream);
+    return a->lq >= 2 ? launch_decode_t<D, RK, true, 2>(a, S, stream, rows) : launch_decode_t<D, RK, true, 1>(a, S, stream, rows);
   }
-  return a->lq >= 2 ? launch_decode_t<D, RK, false, 2>(a, S, stream) : launch_decode_t<D, RK, false, 1>(a, S, stream);
+  return a->lq >= 2 ? launch_decode_t<D, RK, false, 2>(a, S, stream, rows) : launch_decode_t<D, RK, false, 1>(a, S, stream, rows);
 }
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
@@ -818,29 +825,32 @@ int tpa_decode_mfma_supported(const TpaFwdArgs* a) {
   return 1;
 }
 
-int tpa_decode_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
+int tpa_decode_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) { return tpa_decode_mfma_launch_rows(a, stream, 0, a->lq); }
+
+int tpa_decode_mfma_launch_rows(const TpaFwdArgs* a, hipStream_t stream, int row0, int lq_total) {
   using namespace tpa;
+  const RowWindow rows{row0, lq_total};
   const int S = a->num_splits > 0 ? a->num_splits : default_splits(a->B, a->lq, a->lk, a->H);
   if (S > 65535 || (int64_t)a->B * S > 2147483647LL) return TPA_ERR_SHAPE;
   if (!a->workspace || a->workspace_bytes < workspace_bytes(a->B, a->lq, a->H, a->dv, S)) return TPA_ERR_WORKSPACE;
   if (!aligned16(a->workspace)) return TPA_ERR_ALIGN;
   if (a->dk == 128) {
     switch (a->rk) {
-      case 1: return launch_decode<128, 1>(a, S, stream);
-      case 2: return launch_decode<128, 2>(a, S, stream);
-      case 4: return launch_decode<128, 4>(a, S, stream);
-      case 8: return launch_decode<128, 8>(a, S, stream);
-      case 16: return launch_decode<128, 16>(a, S, stream);
-      default: return launch_decode<128, 32>(a, S, stream);
+      case 1: return launch_decode<128, 1>(a, S, stream, rows);
+      case 2: return launch_decode<128, 2>(a, S, stream, rows);
+      case 4: return launch_decode<128, 4>(a, S, stream, rows);
+      case 8: return launch_decode<128, 8>(a, S, stream, rows);
+      case 16: return launch_decode<128, 16>(a, S, stream, rows);
+      default: return launch_decode<128, 32>(a, S, stream, rows);
     }
   }
   switch (a->rk) {
-    case 1: return launch_decode<64, 1>(a, S, stream);
-    case 2: return launch_decode<64, 2>(a, S, stream);
-    case 4: return launch_decode<64, 4>(a, S, stream);
-    case 8: return launch_decode<64, 8>(a, S, stream);
-    case 16: return launch_decode<64, 16>(a, S, stream);
-    default: return launch_decode<64, 32>(a, S, stream);
+    case 1: return launch_decode<64, 1>(a, S, stream, rows);
+    case 2: return launch_decode<64, 2>(a, S, stream, rows);
+    case 4: return launch_decode<64, 4>(a, S, stream, rows);
+    case 8: return launch_decode<64, 8>(a, S, stream, rows);
+    case 16: return launch_decode<64, 16>(a, S, stream, rows);
+    default: return launch_decode<64, 32>(a, S, stream, rows);
   }
 }
 
@@ -861,29 +871,32 @@ int tpa_decode_f32_supported(const TpaFwdArgs* a) {
   return 1;
 }
 
-int tpa_decode_f32_launch(const TpaFwdArgs* a, hipStream_t stream) {
+int tpa_decode_f32_launch(const TpaFwdArgs* a, hipStream_t stream) { return tpa_decode_f32_launch_rows(a, stream, 0, a->lq); }
+
+int tpa_decode_f32_launch_rows(const TpaFwdArgs* a, hipStream_t stream, int row0, int lq_total) {
   using namespace tpa;
+  const RowWindow rows{row0, lq_total};
   const int S = a->num_splits > 0 ? a->num_splits : default_splits(a->B, a->lq, a->lk, a->H, 1);
   if (S > 65535 || (int64_t)a->B * S > 2147483647LL) return TPA_ERR_SHAPE;
   if (!a->workspace || a->workspace_bytes < workspace_bytes(a->B, a->lq, a->H, a->dv, S)) return TPA_ERR_WORKSPACE;
   if (!aligned16(a->workspace)) return TPA_ERR_ALIGN;
   if (a->dk == 128) {
     switch (a->rk) {
-      case 1: return launch_decode_f32<128, 1>(a, S, stream);
-      case 2: return launch_decode_f32<128, 2>(a, S, stream);
-      case 4: return launch_decode_f32<128, 4>(a, S, stream);
-      case 8: return launch_decode_f32<128, 8>(a, S, stream);
-      case 16: return launch_decode_f32<128, 16>(a, S, stream);
-      default: return launch_decode_f32<128, 32>(a, S, stream);
+      case 1: return launch_decode_f32<128, 1>(a, S, stream, rows);
+      case 2: return launch_decode_f32<128, 2>(a, S, stream, rows);
+      case 4: return launch_decode_f32<128, 4>(a, S, stream, rows);
+      case 8: return launch_decode_f32<128, 8>(a, S, stream, rows);
+      case 16: return launch_decode_f32<128, 16>(a, S, stream, rows);
+      default: return launch_decode_f32<128, 32>(a, S, stream, rows);
     }
   }
   switch (a->rk) {
-    case 1: return launch_decode_f32<64, 1>(a, S, stream);
-    case 2: return launch_decode_f32<64, 2>(a, S, stream);
-    case 4: return launch_decode_f32<64, 4>(a, S, stream);
-    case 8: return launch_decode_f32<64, 8>(a, S, stream);
-    case 16: return launch_decode_f32<64, 16>(a, S, stream);
-    default: return launch_decode_f32<64, 32>(a, S, stream);
+    case 1: return launch_decode_f32<64, 1>(a, S, stream, rows);
+    case 2: return launch_decode_f32<64, 2>(a, S, stream, rows);
+    case 4: return launch_decode_f32<64, 4>(a, S, stream, rows);
+    case 8: return launch_decode_f32<64, 8>(a, S, stream, rows);
+    case 16: return launch_decode_f32<64, 16>(a, S, stream, rows);
+    default: return launch_decode_f32<64, 32>(a, S, stream, rows);
   }
 }
 

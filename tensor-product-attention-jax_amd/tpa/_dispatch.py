@@ -22,7 +22,7 @@ KERNEL_AUTO = 0
 KERNEL_GENERIC = 1
 KERNEL_MFMA = 2
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 
 class TpaFactor(ctypes.Structure):
@@ -66,6 +66,7 @@ class TpaFwdArgs(ctypes.Structure):
         ("page_size", ctypes.c_int32),
         ("pages_per_seq", ctypes.c_int32),
         ("causal_offset", ctypes.c_int32),
+        ("nomat", ctypes.c_int32),
     ]
 
 
@@ -238,6 +239,8 @@ def load_library(path: str | None = None) -> ctypes.CDLL:
         lib.mha_fwd_workspace_bytes.argtypes = [ctypes.c_int32] * 6
         lib.tpa_fwd_workspace_bytes.restype = ctypes.c_size_t
         lib.tpa_fwd_workspace_bytes.argtypes = [ctypes.c_int32] * 8
+        lib.tpa_fwd_nomat_workspace_bytes.restype = ctypes.c_size_t
+        lib.tpa_fwd_nomat_workspace_bytes.argtypes = [ctypes.c_int32] * 8
         lib.tpa_bwd.restype = ctypes.c_int
         lib.tpa_bwd.argtypes = [ctypes.POINTER(TpaBwdArgs), ctypes.c_void_p]
         lib.mha_bwd.restype = ctypes.c_int

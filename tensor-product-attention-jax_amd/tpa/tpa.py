@@ -9,9 +9,11 @@ reference, all on purpose:
   * the logsumexp residual is fp32 (the reference keeps it in the input dtype, tpa/tpa.py:530);
   * sequence lengths need not be multiples of the block sizes (tpa/tpa.py:489-490 asserts that);
     `block_sizes` is accepted and ignored because the kernels fix their own tiles;
-  * `nomat` does not change results in the reference (it picks an evaluation order,
-    tpa/tpa.py:333-359) and is ignored here: prefill rebuilds K/V tiles in LDS, decode uses the
-    non-materialising form;
+  * `nomat` picks an evaluation order, as in the reference (tpa/tpa.py:333-359,398-413), and
+    changes no result: `nomat=True` runs the kernels that never form K or V (the split-key
+    decode kernels, over windows of 64 query rows) wherever they take the problem, and the
+    plain kernel elsewhere; the default rebuilds K/V tiles in LDS, which is the faster order on
+    matrix cores except for a few query rows over a long cache (`tpa_decode`);
   * `interpret=True` (the Pallas CPU interpreter upstream) selects the plain fp32-arithmetic
     kernel instead of the MFMA kernels; `debug` is ignored;
   * the backward pass (tpa/tpa.py:168-214,546-995) goes through dense Q, K, V and dense gradients
@@ -126,6 +128,7 @@ def tpa_factors(
     use_workspace: bool = True,
     kv_lengths=None,
     causal_offset: int = 0,
+    nomat: bool = False,
 ):
     """Forward pass on the six split factor arrays, the operands of the reference's kernel
     launch (tpa/tpa.py:246-251,543) with a leading batch dimension:
@@ -141,7 +144,8 @@ def tpa_factors(
     sees keys up to i + causal_offset; 0 is the reference's top-left alignment
     (tpa/tpa.py:377-379), lk - lq aligns the last query with the last key (new tokens over a
     cache), and a sequence shard of a ring (tpa/ring_tpa.py:73-79) passes the distance from the
-    first key of the shard it meets to its own first query.
+    first key of the shard it meets to its own first query.  `nomat` (tpa/tpa.py:250): never
+    form K or V - same results, the rank-space order of operations (see the module docstring).
     """
     device = _pick_device(qa, qb, ka, kb, va, vb)
     qa, qb, ka, kb, va, vb = (_as_device_tensor(x, device) for x in (qa, qb, ka, kb, va, vb))
@@ -171,7 +175,14 @@ def tpa_factors(
     # the problem qualifies
     ws, ws_ptr, ws_bytes = None, None, 0
     # (fp32 inputs: only the split-key decode kernel takes a workspace)
-    if use_workspace and kernel != _d.KERNEL_GENERIC and (dtype == torch.bfloat16 or lq <= 16):
+    if nomat:
+        # the split partials of the non-materialising kernels: required, not optional
+        need = lib.tpa_fwd_nomat_workspace_bytes(b, lq, lk, h, dk, dv, rq, rk) if kernel != _d.KERNEL_GENERIC else 0
+        if need:
+            ws = torch.empty(need + 256, dtype=torch.uint8, device=device)
+            pad = (-ws.data_ptr()) % 256
+            ws_ptr, ws_bytes = ws.data_ptr() + pad, need
+    elif use_workspace and kernel != _d.KERNEL_GENERIC and (dtype == torch.bfloat16 or lq <= 16):
         need = lib.tpa_fwd_workspace_bytes(b, lq, lk, h, dk, dv, rq, rk)
         if need:
             ws = torch.empty(need + 256, dtype=torch.uint8, device=device)
@@ -186,7 +197,7 @@ def tpa_factors(
         dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=_causal_code(causal), kernel=int(kernel),
         workspace=ws_ptr, workspace_bytes=ws_bytes, num_splits=0,
         kv_lengths=kvlen.data_ptr() if kvlen is not None else None,
-        causal_offset=int(causal_offset),
+        causal_offset=int(causal_offset), nomat=int(bool(nomat)),
     )
     with torch.cuda.device(device):
         _d.check("tpa_fwd", lib.tpa_fwd(args, _d.current_stream_ptr(device)))
@@ -409,11 +420,11 @@ class _TpaFunction(torch.autograd.Function):
     """The operator with its vjp, as tpa.defvjp(_tpa_fwd, _tpa_bwd) registers it (tpa/tpa.py:217)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, num_heads, qseg, kvseg, sm_scale, causal, kernel, causal_offset=0):
+    def forward(ctx, q, k, v, num_heads, qseg, kvseg, sm_scale, causal, kernel, causal_offset=0, nomat=False):
         qa, qb = q[..., :num_heads], q[..., num_heads:]
         ka, kb = k[..., :num_heads], k[..., num_heads:]
         va, vb = v[..., :num_heads], v[..., num_heads:]
-        o, lse = tpa_factors(qa, qb, ka, kb, va, vb, qseg, kvseg, sm_scale, causal, kernel, causal_offset=causal_offset)
+        o, lse = tpa_factors(qa, qb, ka, kb, va, vb, qseg, kvseg, sm_scale, causal, kernel, causal_offset=causal_offset, nomat=nomat)
         ctx.mark_non_differentiable(lse)
         ctx.save_for_backward(q, k, v, o, lse)
         ctx.statics = (num_heads, qseg, kvseg, sm_scale, causal, causal_offset)
@@ -424,7 +435,7 @@ class _TpaFunction(torch.autograd.Function):
         q, k, v, o, lse = ctx.saved_tensors
         num_heads, qseg, kvseg, sm_scale, causal, causal_offset = ctx.statics
         dq, dk, dv = _bwd_concat(q, k, v, qseg, kvseg, o, lse, do, num_heads, sm_scale, causal, causal_offset)
-        return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None, None, None, None, None, None
+        return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None, None, None, None, None, None, None
 
 
 def _tpa_fwd(
@@ -433,7 +444,7 @@ def _tpa_fwd(
 ):
     """tpa/tpa.py:124-165: returns (o, residuals) with residuals (q, k, v, qseg, kvseg, o, l),
     l[b, lq, h] being the logsumexp in the reference's layout (a transposed view, fp32)."""
-    del block_sizes, nomat, debug
+    del block_sizes, debug
     device = _pick_device(q, k, v)
     q, k, v = (_as_device_tensor(x, device) for x in (q, k, v))
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
@@ -443,7 +454,7 @@ def _tpa_fwd(
     assert tuple(k.shape) == (b, lk, rk, h_dk), k.shape  # tpa/tpa.py:475
     assert 0 < num_heads < h_dk and num_heads < v.shape[-1], (num_heads, q.shape, v.shape)
     kernel = _d.KERNEL_GENERIC if interpret else _d.KERNEL_AUTO
-    o, lse = _TpaFunction.apply(q, k, v, int(num_heads), q_segment_ids, kv_segment_ids, float(sm_scale), _causal_code(causal), kernel, int(causal_offset))
+    o, lse = _TpaFunction.apply(q, k, v, int(num_heads), q_segment_ids, kv_segment_ids, float(sm_scale), _causal_code(causal), kernel, int(causal_offset), bool(nomat))
     l = lse.permute(0, 2, 1)
     return o, (q, k, v, q_segment_ids, kv_segment_ids, o, l)
 

@@ -1,0 +1,25 @@
+"""bench.py's `roofline.traffic` comes from the committed rocprofv3 counter summary, not from constants
+in the script: the summary parses, and what it yields is consistent with the workloads' algorithmic bytes."""
+
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+
+
+def test_traffic_is_read_from_the_committed_counter_summary():
+    import bench
+
+    assert os.path.exists(bench.TRAFFIC_PROFILE)
+    c2, c4 = bench.measured_traffic("c2"), bench.measured_traffic("c4")
+    assert c2 is not None and c4 is not None
+    # prefill c2 moves at least its inputs and outputs: factors 47.2 MB in, O + LSE 68.2 MB out
+    _, B, lq, lk, H, D, rq, rk, _ = bench.WORKLOADS["c2"]
+    algorithmic = (B * lq * rq * (H + D) + 2 * B * lk * rk * (H + D) + B * lq * H * D) * 2 + B * H * lq * 4
+    assert algorithmic <= c2 <= 3 * algorithmic
+    # decode c4 reads its cache once: within 5 % of the algorithmic bytes
+    _, B, lq, lk, H, D, rq, rk, _ = bench.WORKLOADS["c4"]
+    assert 1.0 <= c4 / bench.decode_bytes(B, lq, lk, H, D, rq, rk) <= 1.05
+    # a workload without a counter run reports none
+    assert bench.measured_traffic("c5") is None
