@@ -58,11 +58,10 @@ struct PrefillParams {
   int q_factors;  // dense K/V loader only: 1 = Q is still given by its rank factors qa, qb
 };
 
-// LDS: two buffers each of a K tile, a V tile, a slot of head factors and a slot of key segment
-// ids.  With one row block per wave the layout is [K0][K1][V0][V1][A0][A1][seg0][seg1]; with two
-// (RB = 2) it is two sets [K][V][A][seg] that lie 64 KiB apart, so that the hand-written loop
-// flips every address between the sets with one xor.  Offsets are in uint16 units.
-template <int D, int RB>
+// LDS: three buffers of a K tile (tile j is read while tile j+1 is already there for waves that run
+// a tile ahead with their logits, and tile j+2 is being written), two of a V tile, two slots of head
+// factors and two of key segment ids: [K0][K1][K2][V0][V1][A0][A1][seg0][seg1], offsets in uint16 units.
+template <int D>
 struct Lds {
   static constexpr int KS = D + 8;   // K row stride (elements): 16-byte reads of 16 rows hit distinct banks
   static constexpr int VS = D + 32;  // V row stride: 4 consecutive rows of a transposed read hit distinct banks
@@ -70,12 +69,11 @@ struct Lds {
   static constexpr int kV = kTK * VS;  // elements of one V buffer
   static constexpr int kA = 2 * kTK * 2;  // one slot of head factors: [K|V][token][rank 0|1]
   static constexpr int kSeg = 2 * kTK;    // one slot of key segment ids (int32), in uint16 units
-  static constexpr int kSet = 32768;      // RB = 2: distance between the two sets
-  static constexpr int k_off(int buf) { return RB == 2 ? buf * kSet : buf * kK; }
-  static constexpr int v_off(int buf) { return RB == 2 ? buf * kSet + kK : 2 * kK + buf * kV; }
-  static constexpr int a_off(int buf) { return RB == 2 ? buf * kSet + kK + kV : 2 * (kK + kV) + buf * kA; }
-  static constexpr int seg_off(int buf) { return RB == 2 ? buf * kSet + kK + kV + kA : 2 * (kK + kV) + 2 * kA + buf * kSeg; }
-  static constexpr size_t kBytes = (RB == 2 ? kSet + kK + kV + kA + kSeg : 2 * (kK + kV) + 2 * kA + 2 * kSeg) * sizeof(uint16_t);
+  static constexpr int k_off(int buf) { return buf * kK; }
+  static constexpr int v_off(int buf) { return 3 * kK + buf * kV; }
+  static constexpr int a_off(int buf) { return 3 * kK + 2 * kV + buf * kA; }
+  static constexpr int seg_off(int buf) { return 3 * kK + 2 * kV + 2 * kA + buf * kSeg; }
+  static constexpr size_t kBytes = (3 * kK + 2 * (kV + kA + kSeg)) * sizeof(uint16_t);
 };
 
 // a0*b0 + a1*b1 on packed bf16 pairs, fp32 result.  Through the builtin on purpose: the dot
@@ -105,45 +103,12 @@ __device__ __forceinline__ void static_for(F&& f) {
 template <int V>
 using IC = std::integral_constant<int, V>;
 
-// Matrix instructions with the register file of every operand chosen by hand, for the kernel
-// with two row blocks per wave: its O^T accumulators (128 registers at D = 128) and Q fragments
-// (64) only ever meet matrix instructions, so they live in the accumulation registers (AGPRs) and
-// leave the 256 architectural registers to the logits, the factor loads and the vector work.
-// (C and D of a matrix instruction share one register file; A and B choose theirs freely.)
-// The compiler inserts no hazard wait states around inline assembly.  A matrix instruction may
-// read a register two wait states after a vector instruction (v_accvgpr_write included) wrote it:
-// each wrapper starts with them, since the compiler is free to put such a write right in front.
-// A vector instruction may read the result of an 8-pass matrix instruction 11 wait states after
-// its issue at the earliest (mfma_result_guard where the instruction stream does not already
-// guarantee it).  These wrappers serve the plain iterations; the interleaved loop is generated.
-__device__ __forceinline__ void mfma_qk_first(f32x16& d, const bf16x8& k, const bf16x8& q, const f32x16& c) {
-  asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(k), "a"(q), "v"(c));
-}
-__device__ __forceinline__ void mfma_qk_next(f32x16& d, const bf16x8& k, const bf16x8& q) {
-  asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(k), "a"(q));
-}
-__device__ __forceinline__ void mfma_pv(f32x16& acc, const bf16x8& v, const bf16x8& pfrag) {
-  asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(v), "v"(pfrag));
-}
-// acc *= alpha for an accumulator tuple that lives in AGPRs, register by register through one
-// temporary, so that the tuple never has to move to the architectural registers
-__device__ __forceinline__ void scale_agpr_tuple(f32x16& acc, float alpha) {
-  float t;
-#define TPA_SCALE1(i) \
-  asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1" : "+a"(acc[i]), "=&v"(t) : "v"(alpha));
-  TPA_SCALE1(0) TPA_SCALE1(1) TPA_SCALE1(2) TPA_SCALE1(3) TPA_SCALE1(4) TPA_SCALE1(5) TPA_SCALE1(6) TPA_SCALE1(7)
-  TPA_SCALE1(8) TPA_SCALE1(9) TPA_SCALE1(10) TPA_SCALE1(11) TPA_SCALE1(12) TPA_SCALE1(13) TPA_SCALE1(14) TPA_SCALE1(15)
-#undef TPA_SCALE1
-}
-__device__ __forceinline__ void pin_vgpr_tuple(f32x16& x) { asm volatile("" : "+v"(x)); }
-__device__ __forceinline__ void mfma_result_guard() { asm volatile("s_nop 7\n\ts_nop 3" ::: "memory"); }
-
 template <int D, int LOADER, bool SEG, int RB>
 __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp) {
-  static_assert(RB == 1 || RB == 2, "row blocks per wave");
+  static_assert(RB == 1, "one block of 32 query rows per wave");
   constexpr int kNW = 8 / RB;  // waves per workgroup
   constexpr int NT = kNW * 64;
-  using L = Lds<D, RB>;
+  using L = Lds<D>;
   constexpr int KS = L::KS, VS = L::VS;
   constexpr int CPR = D / 8;             // 16-byte chunks per row
   constexpr int TPP = NT / CPR;          // tokens per loader pass
@@ -395,21 +360,19 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   const __amdgpu_buffer_rsrc_t kb_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(kb_b), 0, k_rows_bytes, kRsrcFlags);
   const __amdgpu_buffer_rsrc_t vb_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(vb_b), 0, v_rows_bytes, kRsrcFlags);
   const int kvoff = (lt * p.kb.stride_l + 8 * lc) * 2, vvoff = (lt * p.vb.stride_l + 8 * lc) * 2;
-  auto issue = [&](auto is_v_c, int tile) __attribute__((always_inline)) {
+  auto issue_into = [&](u32x4 (&regs)[NPASS][2], auto is_v_c, int tile) __attribute__((always_inline)) {
     constexpr bool is_v = decltype(is_v_c)::value;
     if constexpr (LOADER == LOAD_TPA_ANY) return;
     const int sl = is_v ? p.vb.stride_l : p.kb.stride_l, sr = is_v ? p.vb.stride_r : p.kb.stride_r;
 #pragma unroll
     for (int ps = 0; ps < NPASS; ++ps) {
       const int soff = (tile * kTK + ps * TPP) * sl * 2;  // uniform
-      if constexpr (is_v) {
-        vreg[ps][0] = __builtin_amdgcn_raw_buffer_load_b128(vb_rs, vvoff, soff, 0);
-        if constexpr (LOADER == LOAD_TPA_R2) vreg[ps][1] = __builtin_amdgcn_raw_buffer_load_b128(vb_rs, vvoff, soff + 2 * sr, 0);
-      } else {
-        kreg[ps][0] = __builtin_amdgcn_raw_buffer_load_b128(kb_rs, kvoff, soff, 0);
-        if constexpr (LOADER == LOAD_TPA_R2) kreg[ps][1] = __builtin_amdgcn_raw_buffer_load_b128(kb_rs, kvoff, soff + 2 * sr, 0);
-      }
+      regs[ps][0] = __builtin_amdgcn_raw_buffer_load_b128(is_v ? vb_rs : kb_rs, is_v ? vvoff : kvoff, soff, 0);
+      if constexpr (LOADER == LOAD_TPA_R2) regs[ps][1] = __builtin_amdgcn_raw_buffer_load_b128(is_v ? vb_rs : kb_rs, is_v ? vvoff : kvoff, soff + 2 * sr, 0);
     }
+  };
+  auto issue = [&](auto is_v_c, int tile) __attribute__((always_inline)) {
+    if constexpr (decltype(is_v_c)::value) issue_into(vreg, is_v_c, tile); else issue_into(kreg, is_v_c, tile);
   };
   using IsK = std::integral_constant<bool, false>;
   using IsV = std::integral_constant<bool, true>;
@@ -554,29 +517,31 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   };
 
   // Rebuild one matrix of tile `tile` from the registers `issue` filled and store it in LDS.
-  auto commit = [&](auto is_v_c, int tile, const uint32_t (&aa)[NPASS]) __attribute__((always_inline)) {
+  auto commit_from = [&](const u32x4 (&regs)[NPASS][2], auto is_v_c, int tile, const uint32_t (&aa)[NPASS]) __attribute__((always_inline)) {
     constexpr bool is_v = decltype(is_v_c)::value;
     const uint16_t* bb = is_v ? vb_b : kb_b;
     const uint16_t* ab = is_v ? va_b : ka_b;
     const int b_sl = is_v ? p.vb.stride_l : p.kb.stride_l, b_sr = is_v ? p.vb.stride_r : p.kb.stride_r;
     const int a_sl = is_v ? p.va.stride_l : p.ka.stride_l, a_sr = is_v ? p.va.stride_r : p.ka.stride_r;
-    uint16_t* dst = is_v ? lds_v(tile & 1) : lds_k(tile & 1);
+    uint16_t* dst = is_v ? lds_v(tile & 1) : lds_k(tile % 3);
     constexpr int row_stride = is_v ? VS : KS;
 #pragma unroll
     for (int ps = 0; ps < NPASS; ++ps) {
       const int t = ps * TPP + lt;
       u32x4 val;
       if constexpr (LOADER == LOAD_TPA_R2) {
-        if constexpr (is_v) val = rebuild_r2(vreg[ps][0], vreg[ps][1], aa[ps]);
-        else val = rebuild_r2(kreg[ps][0], kreg[ps][1], aa[ps]);
+        val = rebuild_r2(regs[ps][0], regs[ps][1], aa[ps]);
       } else if constexpr (LOADER == LOAD_TPA_ANY) {
         const int tok = min(tile * kTK + t, lk_r - 1);
         val = rebuild_any(bb + (int64_t)tok * b_sl + 8 * lc, ab + (int64_t)tok * a_sl, b_sr, a_sr);
       } else {
-        if constexpr (is_v) val = vreg[ps][0]; else val = kreg[ps][0];
+        val = regs[ps][0];
       }
       *reinterpret_cast<u32x4*>(dst + t * row_stride + 8 * lc) = val;
     }
+  };
+  auto commit = [&](auto is_v_c, int tile, const uint32_t (&aa)[NPASS]) __attribute__((always_inline)) {
+    if constexpr (decltype(is_v_c)::value) commit_from(vreg, is_v_c, tile, aa); else commit_from(kreg, is_v_c, tile, aa);
   };
 
   // ---- per-wave state, one set per row block r (always indexed with compile-time constants)
@@ -667,12 +632,8 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
       if (__any(up)) {
 #pragma unroll
         for (int db = 0; db < NDB; ++db) {
-          if constexpr (RB == 2) {
-            scale_agpr_tuple(o[r][db], alpha);
-          } else {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) o[r][db][v] *= alpha;
-          }
+          for (int v = 0; v < 16; ++v) o[r][db][v] *= alpha;
         }
       }
 #pragma unroll
@@ -698,11 +659,14 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   };
 
   // ---------------------------------------------------------------------------------------
-  // Main loop.  Invariant at entry of iteration j: K tile j and V tile j are in LDS buffers j&1;
-  // kreg / vreg hold the B factors of tile j+1; head-factor slot j&1 holds those of tile j+1 and
-  // a_pending (waves 0-3) those of tile j+2 (tile indices clamped to the last tile).
-  // An iteration computes S^T = K Q^T, the softmax and O^T += V^T P^T of tile j, rebuilds tile
-  // j+1 into the other buffers and refills the registers with tile j+2; one barrier ends it.
+  // Main loop.  K runs one tile ahead of V, so that a wave may compute the logits of tile j+1
+  // while it is still busy with the softmax of tile j.  Invariant at entry of iteration j: K tiles
+  // j and j+1 are in LDS buffers j%3 and (j+1)%3, V tile j in buffer j&1; kreg holds the B factors
+  // of K tile j+2 and vreg those of V tile j+1; head-factor slot j&1 holds those of K tile j+2 and
+  // V tile j+1, a_pending (waves 0-3) those of K tile j+3 / V tile j+2 (tile indices clamped to
+  // the last tile).  An iteration computes S^T = K Q^T, the softmax and O^T += V^T P^T of tile j,
+  // rebuilds K tile j+2 and V tile j+1 into the free buffers and refills the registers with K
+  // tile j+3 and V tile j+2; one barrier ends it.
   constexpr int N_QK = 2 * NKS, N_PV = 4 * NDB, N_MFMA = N_QK + N_PV;
   // operand fragment n from LDS, shared by the wave's row blocks: fragments 0..N_QK-1 are rows of K
   // (32-key block mb = n / NKS), the rest columns of V (k-step kk covers keys 16kk .. 16kk+15 of the
@@ -725,24 +689,12 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
     constexpr int n = decltype(n_c)::value, r = decltype(r_c)::value;
     if constexpr (n < N_QK) {
       constexpr int mb = n / NKS, kk = n % NKS;
-      if constexpr (RB == 2) {
-        if constexpr (kk == 0) mfma_qk_first(s[r][mb], f, qf[r][kk], nmref[r]);
-        else mfma_qk_next(s[r][mb], f, qf[r][kk]);
-      } else {
-        if constexpr (kk == 0) s[r][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, qf[r][kk], nmref[r], 0, 0, 0);
-        else s[r][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, qf[r][kk], s[r][mb], 0, 0, 0);
-      }
+      if constexpr (kk == 0) s[r][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, qf[r][kk], nmref[r], 0, 0, 0);
+      else s[r][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, qf[r][kk], s[r][mb], 0, 0, 0);
     } else {
       constexpr int m = n - N_QK, kk = m / NDB, db = m % NDB;
-      if constexpr (RB == 2) mfma_pv(o[r][db], f, pf_get(r_c, IC<kk>{}));
-      else o[r][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, pf_get(r_c, IC<kk>{}), o[r][db], 0, 0, 0);
+      o[r][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f, pf_get(r_c, IC<kk>{}), o[r][db], 0, 0, 0);
     }
-  };
-  // The logits of block (r, mb) may be read from here on: pins the vector code that follows behind
-  // the matrix instructions issued so far (it would otherwise be free to move up to the one that
-  // wrote them, inside its 11 wait states).
-  auto logits_ready = [&](auto r_c, auto mb_c) __attribute__((always_inline)) {
-    if constexpr (RB == 2) pin_vgpr_tuple(s[decltype(r_c)::value][decltype(mb_c)::value]);
   };
   // ---- pieces of the softmax of one 32-key block, for the interleaved (unmasked) path
   // Move the reference up where this block's row max left the slack (rare).  delta is a whole
@@ -753,18 +705,13 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
     constexpr int r = decltype(r_c)::value;
     const float delta = tmax > 0.f ? __builtin_ceilf(tmax) : 0.f;
     const float alpha = __builtin_amdgcn_exp2f(-delta);
-    if constexpr (RB == 2) mfma_result_guard();  // O^T and the other block's logits may have been written just now
     mref[r] += delta;
     refresh_nmref(r_c);
     lsum[r] *= alpha;
 #pragma unroll
     for (int db = 0; db < NDB; ++db) {
-      if constexpr (RB == 2) {
-        scale_agpr_tuple(o[r][db], alpha);
-      } else {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) o[r][db][v] *= alpha;
-      }
+      for (int v = 0; v < 16; ++v) o[r][db][v] *= alpha;
     }
     // pf_done = 0: block 0 is being inspected, nothing of this tile is packed yet, both blocks move;
     // pf_done = 2: block 0 has become fragments 0 and 1 (s[r][0][0..7]), block 1 moves
@@ -783,7 +730,6 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   };
   auto sm_max = [&](auto r_c, auto mb_c) __attribute__((always_inline)) {
     constexpr int r = decltype(r_c)::value, mb = decltype(mb_c)::value;
-    logits_ready(r_c, mb_c);
     float t = s[r][mb][0];
 #pragma unroll
     for (int v = 1; v < 16; ++v) t = fmaxf(t, s[r][mb][v]);
@@ -805,20 +751,20 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   // MFMA is followed by a short slice of independent vector work of the same wave, so that the
   // vector ALU runs in the shadow of the matrix pipe.  A fragment read from LDS feeds one MFMA
   // per row block; with G = fragments per group:
-  //   S^T block 0   | rebuild K tile j+1, refill kreg
+  //   S^T block 0   | rebuild K tile j+2, refill kreg
   //   S^T block 1   | softmax of block 0 (all row blocks)
   //   O^T, keys 0-31  | softmax of block 1
   //   O^T, keys 32-63 | rebuild V tile j+1, refill vreg
   // LDS operands are read LA fragments ahead of the MFMAs that consume them.
   auto hot_iteration = [&](int j) __attribute__((always_inline)) {
     constexpr int LA = 2;
-    const uint16_t* ks = lds_k(j & 1);
+    const uint16_t* ks = lds_k(j % 3);
     const uint16_t* vs = lds_v(j & 1);
     const uint16_t* a_slot = lds_a(j & 1);
-    uint16_t* k_dst = lds_k((j + 1) & 1);
+    uint16_t* k_dst = lds_k((j + 2) % 3);
     uint16_t* v_dst = lds_v((j + 1) & 1);
     uint32_t aa_k[NPASS], aa_v[NPASS];
-    fetch_aa(IsK{}, j + 1, a_slot, aa_k);
+    fetch_aa(IsK{}, j + 2, a_slot, aa_k);
     fetch_aa(IsV{}, j + 1, a_slot, aa_v);
     Chunk ch;
     // one rebuild piece: 3 per loader pass (pair up the ranks, dot with the head factors, pack + store)
@@ -869,7 +815,7 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
           constexpr int k = decltype(k_c)::value;
           if constexpr (k * G1 / NI == n) {
             if constexpr (k < NP) piece(IsK{}, k_c);
-            else issue(IsK{}, min(j + 2, last));
+            else issue(IsK{}, min(j + 3, last));
           }
         });
       } else if constexpr (n < G1 + G2) {
@@ -908,7 +854,7 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   // `mask_c` = the row blocks of this wave that take part (bit r).
   auto cold_compute = [&](int j, auto mask_c) __attribute__((always_inline)) {
     constexpr int M = decltype(mask_c)::value;
-    const uint16_t* ks = lds_k(j & 1);
+    const uint16_t* ks = lds_k(j % 3);
     const uint16_t* vs = lds_v(j & 1);
     // operands are read three fragments ahead here too (the V fragments of the first O^T steps
     // while the softmax runs); not with the any-rank loader, whose kernel got slower with it
@@ -922,13 +868,8 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
         if constexpr ((M >> decltype(r_c)::value) & 1) mfma_with(n_c, r_c, fr[n]);
       });
     });
-    if constexpr (RB == 2) mfma_result_guard();
     static_for<RB>([&](auto r_c) __attribute__((always_inline)) {
-      if constexpr ((M >> decltype(r_c)::value) & 1) {
-        logits_ready(r_c, IC<0>{});
-        logits_ready(r_c, IC<1>{});
-        do_softmax(j, r_c);
-      }
+      if constexpr ((M >> decltype(r_c)::value) & 1) do_softmax(j, r_c);
     });
     static_for<N_PV>([&](auto n_c) __attribute__((always_inline)) {
       constexpr int n = N_QK + decltype(n_c)::value;
@@ -938,43 +879,51 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
       });
     });
   };
-  auto cold_iteration = [&](int j) __attribute__((always_inline)) {
-    if constexpr (RB == 1) {
-      if (j <= wave_last_tile[0]) cold_compute(j, IC<1>{});
-    } else {
-      // block 1 lies below block 0 in the sequence, so it needs every tile that block 0 needs
-      if (j <= wave_last_tile[0]) cold_compute(j, IC<3>{});
-      else if (j <= wave_last_tile[1]) cold_compute(j, IC<2>{});
+  // the loader's share of iteration j: K tile j+2 and V tile j+1 into LDS, K tile j+3 and V tile j+2 on their way
+  auto advance_tiles = [&](int j) __attribute__((always_inline)) {
+    const uint16_t* a_slot = LOADER == LOAD_TPA_R2 ? lds_a(j & 1) : nullptr;
+    if (j + 2 < ntiles) {
+      uint32_t aa_k[NPASS];
+      fetch_aa(IsK{}, j + 2, a_slot, aa_k);
+      commit(IsK{}, j + 2, aa_k);
+      issue(IsK{}, min(j + 3, last));
     }
     if (j + 1 < ntiles) {
-      const uint16_t* a_slot = LOADER == LOAD_TPA_R2 ? lds_a(j & 1) : nullptr;
-      uint32_t aa_k[NPASS], aa_v[NPASS];
-      fetch_aa(IsK{}, j + 1, a_slot, aa_k);
+      uint32_t aa_v[NPASS];
       fetch_aa(IsV{}, j + 1, a_slot, aa_v);
-      commit(IsK{}, j + 1, aa_k);
       commit(IsV{}, j + 1, aa_v);
-      issue(IsK{}, min(j + 2, last));
       issue(IsV{}, min(j + 2, last));
     }
   };
+  auto cold_iteration = [&](int j) __attribute__((always_inline)) {
+    if (j <= wave_last_tile[0]) cold_compute(j, IC<1>{});
+    advance_tiles(j);
+  };
 
-  // ---- prologue: tile 0 into LDS (head factors straight from global memory), the head factors
-  // of tile 1 in slot 0, those of tile 2 pending, the B factors of tile 1 in registers
-  issue(IsK{}, 0);
-  issue(IsV{}, 0);
-  issue_a(min(1, last), min(1, last));
-  build_q();
+  // ---- prologue: K tiles 0 and 1 and V tile 0 into LDS (head factors straight from global memory),
+  // the head factors of K tile 2 / V tile 1 in slot 0, those of K tile 3 / V tile 2 pending, the B
+  // factors of K tile 2 and V tile 1 in registers
   {
-    uint32_t aa0[NPASS], aa1[NPASS];
+    u32x4 kreg1[NPASS][2];  // K tile 1, on its way during the Q build like tile 0
+    issue(IsK{}, 0);
+    issue(IsV{}, 0);
+    issue_into(kreg1, IsK{}, min(1, last));
+    issue_a(min(2, last), min(1, last));
+    build_q();
+    uint32_t aa0[NPASS], aa1[NPASS], aa2[NPASS];
     fetch_aa(IsK{}, 0, nullptr, aa0);
     fetch_aa(IsV{}, 0, nullptr, aa1);
     commit(IsK{}, 0, aa0);
     commit(IsV{}, 0, aa1);
+    if (last >= 1) {
+      fetch_aa(IsK{}, 1, nullptr, aa2);
+      commit_from(kreg1, IsK{}, 1, aa2);
+    }
   }
-  issue(IsK{}, min(1, last));
+  issue(IsK{}, min(2, last));
   issue(IsV{}, min(1, last));
   store_a(0);
-  issue_a(min(2, last), min(2, last));
+  issue_a(min(3, last), min(2, last));
   issue_seg(0);
   store_seg(0);
   issue_seg(min(1, last));
@@ -984,9 +933,9 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   // tiles, tiles past this wave's causal range, the last tile).  Three separate loops rather than
   // a branch inside one: every wave passes the same number of barriers either way.
   auto tail = [&](int j) __attribute__((always_inline)) {
-    if (w < 4) {  // head factors: publish those of tile j+2, fetch those of tile j+3
+    if (w < 4) {  // head factors: publish those of K tile j+3 / V tile j+2, fetch those of K tile j+4 / V tile j+3
       store_a((j + 1) & 1);
-      issue_a(min(j + 3, last), min(j + 3, last));
+      issue_a(min(j + 4, last), min(j + 3, last));
     }
     // key segment ids (one wave): publish those of tile j+1, fetch those of tile j+2
     store_seg((j + 1) & 1);
@@ -1012,90 +961,6 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   if constexpr (LOADER != LOAD_TPA_ANY && RB == 1) {
     for (; j < hot_end; ++j) { hot_iteration(j); tail(j); }
   }
-  if constexpr (LOADER != LOAD_TPA_ANY && RB == 2) {
-    // The interleaved iterations 1 .. hot_end - 1 as one block of assembly with every register
-    // named (gen_prefill_loop.py writes it and documents the register map): the state goes in and
-    // comes back in operands pinned to those registers.
-    static_assert(D == 128 && !SEG, "the generated loop exists for D = 128 without segment ids");
-    if (hot_end > 1) {
-      auto cat4 = [](const u32x4& a0, const u32x4& a1, const u32x4& a2, const u32x4& a3) __attribute__((always_inline)) -> f32x16 {
-        const u32x8 lo = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
-        const u32x8 hi = __builtin_shufflevector(a2, a3, 0, 1, 2, 3, 4, 5, 6, 7);
-        return __builtin_bit_cast(f32x16, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
-      };
-      auto quarter = [](const f32x16& t, auto k_c) __attribute__((always_inline)) -> u32x4 {
-        constexpr int k = 4 * decltype(k_c)::value;
-        const u32x16 u = __builtin_bit_cast(u32x16, t);
-        return __builtin_shufflevector(u, u, k, k + 1, k + 2, k + 3);
-      };
-      auto qv = [&](int r, int ks) __attribute__((always_inline)) { return __builtin_bit_cast(u32x4, qf[r][ks]); };
-      const f32x16 qp0 = cat4(qv(0, 0), qv(0, 1), qv(0, 2), qv(0, 3)), qp1 = cat4(qv(0, 4), qv(0, 5), qv(0, 6), qv(0, 7));
-      const f32x16 qp2 = cat4(qv(1, 0), qv(1, 1), qv(1, 2), qv(1, 3)), qp3 = cat4(qv(1, 4), qv(1, 5), qv(1, 6), qv(1, 7));
-      constexpr bool two = LOADER == LOAD_TPA_R2;  // factor registers of the second rank exist
-      const u32x4 z4 = {0, 0, 0, 0};
-      f32x16 kv0 = cat4(kreg[0][0], two ? kreg[0][1] : z4, kreg[1][0], two ? kreg[1][1] : z4);
-      f32x16 kv1 = cat4(kreg[2][0], two ? kreg[2][1] : z4, kreg[3][0], two ? kreg[3][1] : z4);
-      f32x16 kv2 = cat4(vreg[0][0], two ? vreg[0][1] : z4, vreg[1][0], two ? vreg[1][1] : z4);
-      f32x16 kv3 = cat4(vreg[2][0], two ? vreg[2][1] : z4, vreg[3][0], two ? vreg[3][1] : z4);
-      f32x8 st8 = {mref[0], mref[1], lsum[0], lsum[1], __uint_as_float(a_pending), 0.f, 0.f, 0.f};
-      // LDS byte addresses of this lane in set 0 (the loop flips them between the sets)
-      const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t*)smem;
-      u32x16 ad16 = {};
-      ad16[0] = lds0 + 2 * (L::k_off(0) + i * KS + 8 * g);                                                   // K fragment rows
-      ad16[1] = lds0 + 2 * (L::v_off(0) + (4 * g + (lp >> 2)) * VS + 16 * dhalf + 4 * (lp & 3));             // V fragment columns
-      ad16[2] = lds0 + 2 * (L::k_off(0) + lt * KS + 8 * lc);                                                 // rebuilt K chunk
-      ad16[3] = lds0 + 2 * (L::v_off(0) + lt * VS + 8 * lc);                                                 // rebuilt V chunk
-      ad16[4] = lds0 + 2 * (L::a_off(0) + 2 * lt);                                                           // head-factor pairs of this lane's tokens
-      ad16[5] = lds0 + 2 * (L::a_off(0) + tid);                                                              // head factor this thread publishes
-      ad16[6] = kvoff; ad16[7] = vvoff; ad16[8] = a_mat == 0 ? ka_voff : va_voff;
-      auto uni = [](uint32_t x) __attribute__((always_inline)) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); };
-      u32x16 sc16 = {};
-      sc16[0] = uni(j); sc16[1] = uni(hot_end); sc16[2] = uni(last);
-      sc16[3] = uni(kTK * p.kb.stride_l * 2); sc16[4] = uni(kTK * p.vb.stride_l * 2);
-      sc16[5] = uni(kTK * (w < 2 ? p.ka.stride_l : p.va.stride_l) * 2);
-      sc16[6] = uni(TPP * p.kb.stride_l * 2); sc16[7] = uni(p.kb.stride_r * 2);
-      sc16[8] = uni(TPP * p.vb.stride_l * 2); sc16[9] = uni(p.vb.stride_r * 2);
-      sc16[10] = 0x05040100u; sc16[11] = 0x07060302u;
-      auto rsrc_words = [&](const uint16_t* base, int bytes) __attribute__((always_inline)) -> u32x4 {
-        const uint64_t a64 = reinterpret_cast<uint64_t>(base);
-        return u32x4{uni((uint32_t)a64), uni((uint32_t)(a64 >> 32) & 0xffffu), uni((uint32_t)bytes), (uint32_t)kRsrcFlags};
-      };
-      const u32x4 kbr = rsrc_words(kb_b, k_rows_bytes), vbr = rsrc_words(vb_b, v_rows_bytes);
-      const u32x4 abr = LOADER == LOAD_TPA_R2 ? rsrc_words(w < 2 ? ka_b : va_b, w < 2 ? ka_bytes : va_bytes) : z4;  // waves 0, 1 fetch K's head factors, waves 2, 3 V's
-#define TPA_PF_LOOP_OPERANDS                                                                                           \
-  : "+{a[0:15]}"(o[0][0]), "+{a[16:31]}"(o[0][1]), "+{a[32:47]}"(o[0][2]), "+{a[48:63]}"(o[0][3]),                   \
-    "+{a[64:79]}"(o[1][0]), "+{a[80:95]}"(o[1][1]), "+{a[96:111]}"(o[1][2]), "+{a[112:127]}"(o[1][3]),               \
-    "+{v[64:79]}"(nmref[0]), "+{v[80:95]}"(nmref[1]),                                                                \
-    "+{v[96:111]}"(kv0), "+{v[112:127]}"(kv1), "+{v[128:143]}"(kv2), "+{v[144:159]}"(kv3),                            \
-    "+{v[188:195]}"(st8), "+{v[196:211]}"(ad16), "+{s[32:47]}"(sc16)                                                 \
-  : "{a[128:143]}"(qp0), "{a[144:159]}"(qp1), "{a[160:175]}"(qp2), "{a[176:191]}"(qp3),                              \
-    "{s[48:51]}"(kbr), "{s[52:55]}"(vbr), "{s[56:59]}"(abr)                                                          \
-  :
-      if constexpr (LOADER == LOAD_TPA_R2) {
-        asm volatile(
-#include "gen/prefill_loop_128_r2.inc"
-            TPA_PF_LOOP_OPERANDS
-#include "gen/prefill_loop_128_r2_clobbers.inc"
-        );
-      } else {
-        asm volatile(
-#include "gen/prefill_loop_128_dense.inc"
-            TPA_PF_LOOP_OPERANDS
-#include "gen/prefill_loop_128_dense_clobbers.inc"
-        );
-      }
-#undef TPA_PF_LOOP_OPERANDS
-      kreg[0][0] = quarter(kv0, IC<0>{}); kreg[1][0] = quarter(kv0, IC<2>{}); kreg[2][0] = quarter(kv1, IC<0>{}); kreg[3][0] = quarter(kv1, IC<2>{});
-      vreg[0][0] = quarter(kv2, IC<0>{}); vreg[1][0] = quarter(kv2, IC<2>{}); vreg[2][0] = quarter(kv3, IC<0>{}); vreg[3][0] = quarter(kv3, IC<2>{});
-      if constexpr (two) {
-        kreg[0][1] = quarter(kv0, IC<1>{}); kreg[1][1] = quarter(kv0, IC<3>{}); kreg[2][1] = quarter(kv1, IC<1>{}); kreg[3][1] = quarter(kv1, IC<3>{});
-        vreg[0][1] = quarter(kv2, IC<1>{}); vreg[1][1] = quarter(kv2, IC<3>{}); vreg[2][1] = quarter(kv3, IC<1>{}); vreg[3][1] = quarter(kv3, IC<3>{});
-      }
-      mref[0] = st8[0]; mref[1] = st8[1]; lsum[0] = st8[2]; lsum[1] = st8[3];
-      a_pending = __float_as_uint(st8[4]);
-      j = hot_end;
-    }
-  }
   for (; j < ntiles; ++j) { cold_iteration(j); tail(j); }
 
   // ---- epilogue: normalise, store O[b, qrow, h, :] and LSE[b, h, qrow]
@@ -1103,7 +968,6 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   // barrier), so that they leave as whole 16-byte chunks of whole rows instead of 8-byte pieces
   // of 32 rows.  (LDS operations of one wave complete in order: the next row block's writes
   // cannot overtake the reads of this one.)
-  if constexpr (RB == 2) mfma_result_guard();
   static_for<RB>([&](auto r_c) __attribute__((always_inline)) {
     constexpr int r = decltype(r_c)::value;
     const float ltot = halves_sum(lsum[r]);
@@ -1136,38 +1000,16 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   });
 }
 
-template <int D, int LOADER, bool SEG, int RB>
-int launch_prefill_rb(const PrefillParams& p, hipStream_t stream) {
-  auto kern = prefill_kernel<D, LOADER, SEG, RB>;
-  constexpr size_t lds_bytes = Lds<D, RB>::kBytes;
+template <int D, int LOADER, bool SEG = false>
+int launch_prefill(const PrefillParams& p, hipStream_t stream) {
+  auto kern = prefill_kernel<D, LOADER, SEG, 1>;
+  constexpr size_t lds_bytes = Lds<D>::kBytes;
   static bool configured[kMaxDevices] = {};
   if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), lds_bytes); rc != TPA_OK) return rc;
   const int groups = (p.npairs + 7) / 8;
   dim3 grid(groups * 8 * p.H);
-  hipLaunchKernelGGL(kern, grid, dim3((8 / RB) * 64), lds_bytes, stream, p);
+  hipLaunchKernelGGL(kern, grid, dim3(512), lds_bytes, stream, p);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
-}
-
-// Rows per wave.  Eight waves of 32 rows is what every problem runs on.  Four waves of 64 rows
-// (head size 128, rank-2 or dense loader, no segment ids: the hand-scheduled loop exists for
-// exactly that) halves the LDS reads per MFMA but leaves each SIMD with a single wave, which
-// issues one vector instruction per ~6 cycles whatever it does: measured 4 % slower at 32768
-// rows and 40 % slower at 4096, so it is only selected by TPA_PREFILL_ROW_BLOCKS=2 in the
-// environment (a measuring aid, read once per process).
-bool two_row_blocks_requested() {
-  static const bool v = [] {
-    const char* e = getenv("TPA_PREFILL_ROW_BLOCKS");
-    return e && e[0] == '2';
-  }();
-  return v;
-}
-
-template <int D, int LOADER, bool SEG = false>
-int launch_prefill(const PrefillParams& p, hipStream_t stream) {
-  if constexpr (D == 128 && !SEG && LOADER != LOAD_TPA_ANY) {
-    if (two_row_blocks_requested()) return launch_prefill_rb<D, LOADER, SEG, 2>(p, stream);
-  }
-  return launch_prefill_rb<D, LOADER, SEG, 1>(p, stream);
 }
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }

@@ -171,20 +171,6 @@ def test_prefill_bf16_sharp_softmax(gpu, causal):
     assert rel < 2e-2
 
 
-def test_prefill_four_wave_variant_in_a_child_process(gpu):
-    """TPA_PREFILL_ROW_BLOCKS=2 (a measuring aid, read once per process) selects the prefill kernel
-    with four waves of 64 query rows and the generated tile loop: tests/prefill_row_blocks_case.py
-    holds it to the same bounds, in a process of its own."""
-    import os
-    import subprocess
-    import sys
-
-    env = dict(os.environ, TPA_PREFILL_ROW_BLOCKS="2")
-    case = os.path.join(os.path.dirname(os.path.abspath(__file__)), "prefill_row_blocks_case.py")
-    r = subprocess.run([sys.executable, case], env=env, capture_output=True, text=True, timeout=300)
-    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stdout[-2000:] + r.stderr[-4000:]
-
-
 def test_prefill_concatenated_layout_in_place(gpu):
     """tpa() reads the A and B factors in place from the concatenated tensors (strided views)."""
     from tpa import tpa
