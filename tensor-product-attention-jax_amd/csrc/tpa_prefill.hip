@@ -851,33 +851,42 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   };
 
   // ---- plain iteration: first tile, masked tiles, tiles a row block skips, last tile.
-  // `mask_c` = the row blocks of this wave that take part (bit r).
-  auto cold_compute = [&](int j, auto mask_c) __attribute__((always_inline)) {
-    constexpr int M = decltype(mask_c)::value;
+  // `mask_c` = the row blocks of this wave that take part (bit r); `part_c` = 0: the whole tile, 1: its
+  // logits only (they stay in s), 2: the rest of a tile whose logits are in s already.
+  auto cold_compute = [&](int j, auto mask_c, auto part_c) __attribute__((always_inline)) {
+    constexpr int M = decltype(mask_c)::value, PART = decltype(part_c)::value;
     const uint16_t* ks = lds_k(j % 3);
     const uint16_t* vs = lds_v(j & 1);
     // operands are read three fragments ahead here too (the V fragments of the first O^T steps
     // while the softmax runs); not with the any-rank loader, whose kernel got slower with it
     constexpr int LA = LOADER == LOAD_TPA_ANY ? 0 : 3;
     bf16x8 fr[N_MFMA];
-    static_for<LA>([&](auto n_c) __attribute__((always_inline)) { fr[decltype(n_c)::value] = load_frag(n_c, ks, vs); });
-    static_for<N_QK>([&](auto n_c) __attribute__((always_inline)) {
-      constexpr int n = decltype(n_c)::value;
-      if constexpr (n + LA < N_MFMA) fr[n + LA] = load_frag(IC<n + LA>{}, ks, vs);
-      static_for<RB>([&](auto r_c) __attribute__((always_inline)) {
-        if constexpr ((M >> decltype(r_c)::value) & 1) mfma_with(n_c, r_c, fr[n]);
+    constexpr int FIRST = PART == 2 ? N_QK : 0, END = PART == 1 ? N_QK : N_MFMA;  // fragments this call uses
+    static_for<LA>([&](auto n_c) __attribute__((always_inline)) {
+      constexpr int n = FIRST + decltype(n_c)::value;
+      if constexpr (n < END) fr[n] = load_frag(IC<n>{}, ks, vs);
+    });
+    if constexpr (PART != 2) {
+      static_for<N_QK>([&](auto n_c) __attribute__((always_inline)) {
+        constexpr int n = decltype(n_c)::value;
+        if constexpr (n + LA < END) fr[n + LA] = load_frag(IC<n + LA>{}, ks, vs);
+        static_for<RB>([&](auto r_c) __attribute__((always_inline)) {
+          if constexpr ((M >> decltype(r_c)::value) & 1) mfma_with(n_c, r_c, fr[n]);
+        });
       });
-    });
-    static_for<RB>([&](auto r_c) __attribute__((always_inline)) {
-      if constexpr ((M >> decltype(r_c)::value) & 1) do_softmax(j, r_c);
-    });
-    static_for<N_PV>([&](auto n_c) __attribute__((always_inline)) {
-      constexpr int n = N_QK + decltype(n_c)::value;
-      if constexpr (n + LA < N_MFMA) fr[n + LA] = load_frag(IC<n + LA>{}, ks, vs);
+    }
+    if constexpr (PART != 1) {
       static_for<RB>([&](auto r_c) __attribute__((always_inline)) {
-        if constexpr ((M >> decltype(r_c)::value) & 1) mfma_with(IC<n>{}, r_c, fr[n]);
+        if constexpr ((M >> decltype(r_c)::value) & 1) do_softmax(j, r_c);
       });
-    });
+      static_for<N_PV>([&](auto n_c) __attribute__((always_inline)) {
+        constexpr int n = N_QK + decltype(n_c)::value;
+        if constexpr (n + LA < END) fr[n + LA] = load_frag(IC<n + LA>{}, ks, vs);
+        static_for<RB>([&](auto r_c) __attribute__((always_inline)) {
+          if constexpr ((M >> decltype(r_c)::value) & 1) mfma_with(IC<n>{}, r_c, fr[n]);
+        });
+      });
+    }
   };
   // the loader's share of iteration j: K tile j+2 and V tile j+1 into LDS, K tile j+3 and V tile j+2 on their way
   auto advance_tiles = [&](int j) __attribute__((always_inline)) {
@@ -896,7 +905,7 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
     }
   };
   auto cold_iteration = [&](int j) __attribute__((always_inline)) {
-    if (j <= wave_last_tile[0]) cold_compute(j, IC<1>{});
+    if (j <= wave_last_tile[0]) cold_compute(j, IC<1>{}, IC<0>{});
     advance_tiles(j);
   };
 
@@ -958,7 +967,83 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   }
   int j = 0;
   for (; j < 1; ++j) { cold_iteration(j); tail(j); }
-  if constexpr (LOADER != LOAD_TPA_ANY && RB == 1) {
+  if constexpr (LOADER == LOAD_DENSE && !SEG) {
+    // Unmasked tiles 1 .. hot_end - 1 pipelined: tile j's softmax and O^T run beside the logits of
+    // tile j+1 (K is a tile ahead in LDS for this).  The logits of tile 1 are computed here, the
+    // loop (generated by gen_prefill_loop.py, which documents the register assignment) then runs
+    // iterations 1 .. hot_end - 2 and leaves the logits of tile hot_end - 1, which is finished
+    // here.  The state goes in and comes back in operands pinned to the loop's registers.
+    if (hot_end >= 3) {
+      cold_compute(1, IC<1>{}, IC<1>{});
+      auto cat4 = [](const u32x4& a0, const u32x4& a1, const u32x4& a2, const u32x4& a3) __attribute__((always_inline)) -> f32x16 {
+        const u32x8 lo = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+        const u32x8 hi = __builtin_shufflevector(a2, a3, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(f32x16, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
+      };
+      auto qv = [&](int ks) __attribute__((always_inline)) { return __builtin_bit_cast(u32x4, qf[0][ks]); };
+      const u32x4 z4 = {0, 0, 0, 0};
+      const f32x16 qp0 = cat4(qv(0), qv(1), qv(2), qv(3));
+      const f32x16 qp1 = NKS > 4 ? cat4(qv(NKS > 4 ? 4 : 0), qv(NKS > 4 ? 5 : 0), qv(NKS > 4 ? 6 : 0), qv(NKS > 4 ? 7 : 0)) : qp0;
+      u32x8 kv_k = __builtin_shufflevector(kreg[0][0], NPASS > 1 ? kreg[NPASS - 1][0] : z4, 0, 1, 2, 3, 4, 5, 6, 7);
+      u32x8 kv_v = __builtin_shufflevector(vreg[0][0], NPASS > 1 ? vreg[NPASS - 1][0] : z4, 0, 1, 2, 3, 4, 5, 6, 7);
+      f32x16 sa0 = {}, sa1 = {}, sb0 = s[0][0], sb1 = s[0][1];  // tile 1 is odd: its logits sit in the second set
+      const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t*)smem;
+      u32x16 st16 = {};
+      st16[0] = __float_as_uint(mref[0]); st16[1] = __float_as_uint(lsum[0]);
+      st16[2] = lds0 + 2 * (L::k_off(0) + i * KS + 8 * g);                                                   // K fragment rows
+      st16[3] = lds0 + 2 * (L::v_off(0) + (4 * g + (lp >> 2)) * VS + 16 * dhalf + 4 * (lp & 3));             // V fragment columns
+      st16[4] = lds0 + 2 * (L::k_off(0) + lt * KS + 8 * lc);                                                 // this thread's chunk of a K tile
+      st16[5] = lds0 + 2 * (L::v_off(0) + lt * VS + 8 * lc);                                                 // ... of a V tile
+      st16[6] = kvoff; st16[7] = vvoff;
+      auto uni = [](uint32_t x) __attribute__((always_inline)) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); };
+      u32x16 sc16 = {};
+      sc16[0] = 1; sc16[1] = uni(hot_end - 1); sc16[2] = uni(last);
+      sc16[3] = uni(kTK * p.kb.stride_l * 2); sc16[4] = uni(kTK * p.vb.stride_l * 2);
+      sc16[5] = uni(TPP * p.kb.stride_l * 2); sc16[6] = uni(TPP * p.vb.stride_l * 2);
+      sc16[7] = 2 * L::kK * 2; sc16[8] = 0;  // K buffers: iteration 1 reads tile 2 in buffer 2 and writes tile 3 into buffer 0
+      auto rsrc_words = [&](const uint16_t* base, int bytes) __attribute__((always_inline)) -> u32x4 {
+        const uint64_t a64 = reinterpret_cast<uint64_t>(base);
+        return u32x4{uni((uint32_t)a64), uni((uint32_t)(a64 >> 32) & 0xffffu), uni((uint32_t)bytes), (uint32_t)kRsrcFlags};
+      };
+      const u32x4 kbr = rsrc_words(kb_b, k_rows_bytes), vbr = rsrc_words(vb_b, v_rows_bytes);
+      if constexpr (D == 128) {
+        asm volatile(
+#include "gen/prefill_loop_128_dense.inc"
+            : "+{v[0:15]}"(sa0), "+{v[16:31]}"(sa1), "+{v[32:47]}"(sb0), "+{v[48:63]}"(sb1), "+{v[64:79]}"(nmref[0]),
+              "+{v[80:95]}"(o[0][0]), "+{v[96:111]}"(o[0][1]), "+{v[112:127]}"(o[0][NDB > 2 ? 2 : 0]), "+{v[128:143]}"(o[0][NDB > 2 ? 3 : 0]),
+              "+{v[176:183]}"(kv_k), "+{v[184:191]}"(kv_v), "+{v[204:219]}"(st16), "+{s[32:47]}"(sc16)
+            : "{v[144:159]}"(qp0), "{v[160:175]}"(qp1), "{s[48:51]}"(kbr), "{s[52:55]}"(vbr)
+            :
+#include "gen/prefill_loop_128_dense_clobbers.inc"
+        );
+      } else {
+        asm volatile(
+#include "gen/prefill_loop_64_dense.inc"
+            : "+{v[0:15]}"(sa0), "+{v[16:31]}"(sa1), "+{v[32:47]}"(sb0), "+{v[48:63]}"(sb1), "+{v[64:79]}"(nmref[0]),
+              "+{v[80:95]}"(o[0][0]), "+{v[96:111]}"(o[0][1]),
+              "+{v[176:183]}"(kv_k), "+{v[184:191]}"(kv_v), "+{v[204:219]}"(st16), "+{s[32:47]}"(sc16)
+            : "{v[144:159]}"(qp0), "{s[48:51]}"(kbr), "{s[52:55]}"(vbr)
+            :
+#include "gen/prefill_loop_64_dense_clobbers.inc"
+        );
+      }
+      kreg[0][0] = __builtin_shufflevector(kv_k, kv_k, 0, 1, 2, 3);
+      vreg[0][0] = __builtin_shufflevector(kv_v, kv_v, 0, 1, 2, 3);
+      if constexpr (NPASS > 1) {
+        kreg[NPASS - 1][0] = __builtin_shufflevector(kv_k, kv_k, 4, 5, 6, 7);
+        vreg[NPASS - 1][0] = __builtin_shufflevector(kv_v, kv_v, 4, 5, 6, 7);
+      }
+      mref[0] = __uint_as_float(st16[0]); lsum[0] = __uint_as_float(st16[1]);
+      j = hot_end - 1;
+      const bool odd = j & 1;  // uniform
+      s[0][0] = odd ? sb0 : sa0;
+      s[0][1] = odd ? sb1 : sa1;
+      cold_compute(j, IC<1>{}, IC<2>{});
+      advance_tiles(j);
+      tail(j);
+      ++j;
+    }
+  } else if constexpr (LOADER != LOAD_TPA_ANY) {
     for (; j < hot_end; ++j) { hot_iteration(j); tail(j); }
   }
   for (; j < ntiles; ++j) { cold_iteration(j); tail(j); }
