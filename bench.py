@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c3u|c4|c4pg|c4s|c5|c5u|c2n|c5n|c2f|c3f|c2fb|c4f|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|ap1|ap2|copy] [--no-cpu] [--no-decode] [--no-backward]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2u|c3|c3u|c4|c4pg|c4s|c5|c5u|c2n|c5n|c2f|c3f|c2fb|c4f|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|ap1|ap2|copy] [--no-cpu] [--no-decode] [--no-backward]
 
 A step is one forward pass over one batch of synthetic, seeded inputs that are resident in HBM
 before the timed region starts.  The default workload is the prefill configuration the headline
@@ -35,6 +35,7 @@ WORKLOADS = {
     "c5": ("prefill", 8, 2048, 2048, 64, 64, 16, 8, False),
     # the same two without the optional workspace: the fused kernel that rebuilds every K/V tile from the
     # rank factors inside the flash loop (with the workspace these shapes reconstruct dense K, V once)
+    "c2u": ("prefill", 4, 4096, 4096, 16, 128, 6, 2, True),
     "c3u": ("prefill", 1, 32768, 32768, 32, 128, 6, 2, True),
     "c5u": ("prefill", 8, 2048, 2048, 64, 64, 16, 8, False),
     # nomat=True (tpa/tpa.py:250): the order of operations that never forms K or V, at the c2 and c5 shapes

@@ -332,6 +332,10 @@ def sm_exp(e, p, mb, q):
     T0, T1 = ((T0A, T1A), (T0B, T1B))[mb]   # the two blocks' instructions interleave: a pair of temporaries each
     for k in range(4):
         e.ins("v_mov_b32" if "exp" in KO else "v_exp_f32", f"v{s + 4 * q + k}", f"v{s + 4 * q + k}")
+    if "lsum" in KO:
+        e.ins("v_cvt_pk_bf16_f32", f"v{s + 2 * q}", f"v{s + 4 * q}", f"v{s + 4 * q + 1}")
+        e.ins("v_cvt_pk_bf16_f32", f"v{s + 2 * q + 1}", f"v{s + 4 * q + 2}", f"v{s + 4 * q + 3}")
+        return
     e.ins("v_add_f32", f"v{T0}", f"v{s + 4 * q}", f"v{s + 4 * q + 1}")
     e.ins("v_add_f32", f"v{T1}", f"v{s + 4 * q + 2}", f"v{s + 4 * q + 3}")
     e.ins("v_cvt_pk_bf16_f32", f"v{s + 2 * q}", f"v{s + 4 * q}", f"v{s + 4 * q + 1}")

@@ -133,8 +133,8 @@ size_t tpa_fwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int
   if (dk != dv || (dk != 64 && dk != 128)) return 0;  // the kernels that use a workspace take these head sizes only
   size_t need = 0;
   if (lq <= 16 && lk >= 1024) need = tpa_decode_workspace_bytes(B, lq, lk, H, dv, 0);
-  if (tpa_prefill_wants_dense_kv(lq, rk)) {
-    const size_t dense = tpa_prefill_dense_kv_bytes(B, lk, H, dk);
+  if (tpa_prefill_wants_dense(lq, rk)) {
+    const size_t dense = tpa_prefill_dense_bytes(B, lq, lk, H, dk);
     if (dense > need) need = dense;
   }
   return need;

@@ -45,11 +45,11 @@ __global__ void recon_kernel(TpaFactor fa, TpaFactor fb, TO* out, int L, int H, 
 // once, so that several independent load chains are in flight (one token per workgroup left the
 // kernel waiting for one small load after the other).  Needs D % 8 == 0 and 16-byte aligned b rows.
 constexpr int kReconTokens = 4;
-__global__ __launch_bounds__(256) void recon_bf16_kernel(TpaFactor fa, TpaFactor fb, uint16_t* out, int L, int H, int D, int R) {
+__global__ __launch_bounds__(256) void recon_bf16_kernel(TpaFactor fa, TpaFactor fb, uint16_t* out, int L, int H, int D, int R, float scale) {
   const int t0 = blockIdx.x * kReconTokens, b = blockIdx.y;
   const uint16_t* ap = static_cast<const uint16_t*>(fa.ptr) + b * fa.stride_b;
   const uint16_t* bp = static_cast<const uint16_t*>(fb.ptr) + b * fb.stride_b;
-  const float inv = 1.f / (float)R;
+  const float inv = scale / (float)R;
   const int cpr = D / 8;
   for (int idx = threadIdx.x; idx < H * cpr; idx += blockDim.x) {
     const int h = idx / cpr, cc = idx - h * cpr;
@@ -83,6 +83,54 @@ __global__ __launch_bounds__(256) void recon_bf16_kernel(TpaFactor fa, TpaFactor
       for (int j = 0; j < 4; ++j) pk[j] = pack_bf16(acc[u][2 * j] * inv, acc[u][2 * j + 1] * inv);
       *reinterpret_cast<u32x4*>(out + (((int64_t)b * L + t0 + u) * H + h) * D + 8 * cc) = pk;
     }
+  }
+}
+
+// The same for head counts that are multiples of 8 with 16-byte aligned a rows: a thread owns one
+// (token, 16-byte piece of D, group of 8 heads) and reads, per rank, one 16-byte piece of b and
+// the 8 head factors as one 16-byte piece of a - 64 multiply-adds per two loads.  Pieces are the
+// fastest thread index, so the 16 threads of a (token, head group) store whole rows of D.
+__global__ __launch_bounds__(256) void recon_bf16_h8_kernel(TpaFactor fa, TpaFactor fb, uint16_t* out, int L, int H, int D, int R, float scale) {
+  const int cpr = D / 8, hg = H / 8;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int cc = (int)(idx % cpr);
+  const int g = (int)(idx / cpr % hg);
+  const int64_t t = idx / ((int64_t)cpr * hg);
+  const int b = blockIdx.y;
+  if (t >= L) return;
+  const uint16_t* ap = static_cast<const uint16_t*>(fa.ptr) + b * fa.stride_b + t * fa.stride_l + 8 * g;
+  const uint16_t* bp = static_cast<const uint16_t*>(fb.ptr) + b * fb.stride_b + t * fb.stride_l + 8 * cc;
+  float acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = 0.f;
+  u32x4 av = *reinterpret_cast<const u32x4*>(ap), bv = *reinterpret_cast<const u32x4*>(bp);
+  for (int r = 0; r < R; ++r) {
+    const u32x4 a_cur = av, b_cur = bv;
+    if (r + 1 < R) {  // the next rank's pieces are on their way during this rank's arithmetic
+      av = *reinterpret_cast<const u32x4*>(ap + (int64_t)(r + 1) * fa.stride_r);
+      bv = *reinterpret_cast<const u32x4*>(bp + (int64_t)(r + 1) * fb.stride_r);
+    }
+    float af[8], bf[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      af[2 * j] = bf16lo_to_f32(a_cur[j]); af[2 * j + 1] = bf16hi_to_f32(a_cur[j]);
+      bf[2 * j] = bf16lo_to_f32(b_cur[j]); bf[2 * j + 1] = bf16hi_to_f32(b_cur[j]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[i][j] += af[i] * bf[j];
+  }
+  const float inv = scale / (float)R;
+  uint16_t* op = out + (((int64_t)b * L + t) * H + 8 * g) * D + 8 * cc;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    u32x4 pk;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) pk[j] = pack_bf16(acc[i][2 * j] * inv, acc[i][2 * j + 1] * inv);
+    *reinterpret_cast<u32x4*>(op + (int64_t)i * D) = pk;
   }
 }
 
@@ -457,7 +505,7 @@ int tpa_bwd_t(const TpaBwdArgs* a, hipStream_t stream, bool mfma) {
       const bool vec = sizeof(T) == 2 && !(reinterpret_cast<uintptr_t>(fb.ptr) & 15) && fb.stride_b % 8 == 0 && fb.stride_l % 8 == 0 &&
                        fb.stride_r % 8 == 0;
       if (vec)
-        hipLaunchKernelGGL(recon_bf16_kernel, dim3((L + kReconTokens - 1) / kReconTokens, a->B), dim3(threads), 0, stream, fa, fb, out, L, a->H, D, R);
+        hipLaunchKernelGGL(recon_bf16_kernel, dim3((L + kReconTokens - 1) / kReconTokens, a->B), dim3(threads), 0, stream, fa, fb, out, L, a->H, D, R, 1.f);
       else
         hipLaunchKernelGGL((recon_kernel<T, uint16_t>), dim3(L, a->B), dim3(threads), 0, stream, fa, fb, out, L, a->H, D, R);
     };
@@ -545,12 +593,19 @@ int mha_bwd_t(const MhaBwdArgs* a, hipStream_t stream, bool mfma) {
 }  // namespace
 }  // namespace tpa
 
-int tpa_recon_dense_bf16(const TpaFactor* fa, const TpaFactor* fb, uint16_t* out, int B, int L, int H, int D, int R, hipStream_t stream) {
+int tpa_recon_dense_bf16(const TpaFactor* fa, const TpaFactor* fb, uint16_t* out, int B, int L, int H, int D, int R, float scale, hipStream_t stream) {
   if (B > 65535) return TPA_ERR_SHAPE;
   const bool vec = D % 8 == 0 && !(reinterpret_cast<uintptr_t>(fb->ptr) & 15) && fb->stride_b % 8 == 0 && fb->stride_l % 8 == 0 &&
                    fb->stride_r % 8 == 0;
-  if (vec)
-    hipLaunchKernelGGL(tpa::recon_bf16_kernel, dim3((L + tpa::kReconTokens - 1) / tpa::kReconTokens, B), dim3(256), 0, stream, *fa, *fb, out, L, H, D, R);
+  const bool vec_a = vec && H % 8 == 0 && !(reinterpret_cast<uintptr_t>(fa->ptr) & 15) && fa->stride_b % 8 == 0 && fa->stride_l % 8 == 0 &&
+                     fa->stride_r % 8 == 0;
+  const int64_t threads = (int64_t)L * (D / 8) * (H / 8);
+  if (vec_a && (threads + 255) / 256 <= 2147483647LL)
+    hipLaunchKernelGGL(tpa::recon_bf16_h8_kernel, dim3((unsigned)((threads + 255) / 256), B), dim3(256), 0, stream, *fa, *fb, out, L, H, D, R, scale);
+  else if (vec)
+    hipLaunchKernelGGL(tpa::recon_bf16_kernel, dim3((L + tpa::kReconTokens - 1) / tpa::kReconTokens, B), dim3(256), 0, stream, *fa, *fb, out, L, H, D, R, scale);
+  else if (scale != 1.f)
+    return TPA_ERR_ALIGN;  // the scaled form exists for 16-byte aligned factors only
   else
     hipLaunchKernelGGL((tpa::recon_kernel<uint16_t, uint16_t>), dim3(L, B), dim3(256), 0, stream, *fa, *fb, out, L, H, D, R);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;

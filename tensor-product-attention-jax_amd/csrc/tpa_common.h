@@ -193,7 +193,7 @@ int dense_bwd_f32_launch(const float* q, const float* k, const float* v, const f
                          int H, int D, float sm_scale, int causal, int causal_offset, hipStream_t stream);
 size_t tpa_bwd_workspace_size(int64_t B, int64_t lq, int64_t lk, int64_t H, int64_t dk, int64_t dv);
 size_t mha_bwd_workspace_size(int64_t B, int64_t lq, int64_t lk, int64_t H, int64_t dk, int64_t dv, int dtype);
-size_t tpa_prefill_dense_kv_bytes(int64_t B, int64_t lk, int64_t H, int64_t D);
-int tpa_prefill_wants_dense_kv(int64_t lq, int64_t rk);
-// dense bf16 X[B, L, H, D] = (1/R) sum_r a_r (x) b_r from bf16 factors
-int tpa_recon_dense_bf16(const TpaFactor* fa, const TpaFactor* fb, uint16_t* out, int B, int L, int H, int D, int R, hipStream_t stream);
+size_t tpa_prefill_dense_bytes(int64_t B, int64_t lq, int64_t lk, int64_t H, int64_t D);
+int tpa_prefill_wants_dense(int64_t lq, int64_t rk);
+// dense bf16 X[B, L, H, D] = (scale/R) sum_r a_r (x) b_r from bf16 factors
+int tpa_recon_dense_bf16(const TpaFactor* fa, const TpaFactor* fb, uint16_t* out, int B, int L, int H, int D, int R, float scale, hipStream_t stream);

@@ -55,7 +55,7 @@ struct PrefillParams {
   int coff;         // with causal: row i sees keys <= i + coff (0 = top-left aligned)
   int nqb;     // query blocks per (batch, head)
   int npairs;  // nqb * B
-  int q_factors;  // dense K/V loader only: 1 = Q is still given by its rank factors qa, qb
+  int q_scaled;   // dense loader only: 1 = q already holds sm_scale * log2(e) * Q (it was reconstructed with that factor)
 };
 
 // LDS: three buffers of a K tile (tile j is read while tile j+1 is already there for waves that run
@@ -121,9 +121,9 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   // scalars out of the argument block (never take the address of the block itself)
   struct Fac { const uint16_t* ptr; int64_t stride_b; int stride_l, stride_r; };
   auto fac = [](const TpaFactor& f) { return Fac{static_cast<const uint16_t*>(f.ptr), f.stride_b, (int)f.stride_l, (int)f.stride_r}; };
-  struct { Fac qa, qb, ka, kb, va, vb; const int32_t* qseg; const int32_t* kvseg; const int32_t* kvlen; uint16_t* o; float* lse; int B, lq, lk, H, rq, rk; float sm_scale; int causal, coff, nqb, npairs, q_factors; } const p = {
+  struct { Fac qa, qb, ka, kb, va, vb; const int32_t* qseg; const int32_t* kvseg; const int32_t* kvlen; uint16_t* o; float* lse; int B, lq, lk, H, rq, rk; float sm_scale; int causal, coff, nqb, npairs, q_scaled; } const p = {
       fac(pp.qa), fac(pp.qb), fac(pp.ka), fac(pp.kb), fac(pp.va), fac(pp.vb), pp.qseg, pp.kvseg, pp.kvlen, pp.o, pp.lse, pp.B, pp.lq, pp.lk, pp.H, pp.rq, pp.rk,
-      pp.sm_scale, pp.causal, pp.causal ? pp.coff : 0, pp.nqb, pp.npairs, pp.q_factors};
+      pp.sm_scale, pp.causal, pp.causal ? pp.coff : 0, pp.nqb, pp.npairs, pp.q_scaled};
 
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   auto lds_k = [&](int buf) __attribute__((always_inline)) { return smem + L::k_off(buf); };    // [kTK][KS]
@@ -136,12 +136,27 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   // that XCD's L2; pairs are ordered heaviest (last causal block) first.
   const int id = blockIdx.x;
   const int xcd = id & 7, slot = id >> 3;
-  const int round = slot / p.H;
-  const int pair = round * 8 + xcd_pair_slot(round, xcd, p.B);
-  const int h = slot % p.H;
-  if (pair >= p.npairs) return;
-  const int qblk = p.nqb - 1 - pair / p.B;
-  const int b = pair % p.B;
+  int h, b, qblk;
+  if constexpr (LOADER == LOAD_DENSE) {
+    // Dense K and V belong to one (batch, head): what workgroups can share is the K/V stream of
+    // their head.  An XCD therefore owns whole (batch, head) pairs and runs their query blocks
+    // heaviest first, the same block of all its pairs side by side: the 32 workgroups that are
+    // resident together are neighbouring query blocks of a few pairs, which walk the same tiles
+    // at about the same time and find them in that XCD's L2.
+    const int per_xcd = (p.B * p.H + 7) / 8;
+    const int bh = (slot % per_xcd) * 8 + xcd;
+    if (bh >= p.B * p.H) return;
+    qblk = p.nqb - 1 - slot / per_xcd;
+    b = bh / p.H;
+    h = bh % p.H;
+  } else {
+    const int round = slot / p.H;
+    const int pair = round * 8 + xcd_pair_slot(round, xcd, p.B);
+    h = slot % p.H;
+    if (pair >= p.npairs) return;
+    qblk = p.nqb - 1 - pair / p.B;
+    b = pair % p.B;
+  }
 
   const int tid = threadIdx.x;
   const int w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
@@ -155,16 +170,15 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
     qrow[r] = wrow0[r] + i;        // this lane's row in it
     qrow_ld[r] = min(qrow[r], p.lq - 1);
   }
-  const float c = p.sm_scale * kLog2e;
+  const float c = (LOADER == LOAD_DENSE && p.q_scaled) ? 1.f : p.sm_scale * kLog2e;
 
   // ---- Q fragments (B operand of S^T = K Q^T), scaled by c: lane (i, g) holds
   // c * Q[qrow[r]][16ks + 8g + 0..7]
   bf16x8 qf[RB][NKS];
   auto build_q = [&]() __attribute__((always_inline)) {
-    // the dense loader serves dense attention (Q dense too) and factored attention whose K and V
-    // were reconstructed beforehand (Q still in factors)
-    const bool dense_q = LOADER == LOAD_DENSE && !p.q_factors;
-    if (dense_q) {
+    // the dense loader serves dense attention and factored attention whose Q, K and V were
+    // reconstructed beforehand (Q with its scale factor, so that it is rounded to bf16 once)
+    if constexpr (LOADER == LOAD_DENSE) {
 #pragma unroll
       for (int r = 0; r < RB; ++r) {
         const uint16_t* qp = p.qb.ptr + b * p.qb.stride_b + (int64_t)qrow_ld[r] * p.qb.stride_l + (int64_t)h * D;
@@ -1091,8 +1105,10 @@ int launch_prefill(const PrefillParams& p, hipStream_t stream) {
   constexpr size_t lds_bytes = Lds<D>::kBytes;
   static bool configured[kMaxDevices] = {};
   if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), lds_bytes); rc != TPA_OK) return rc;
-  const int groups = (p.npairs + 7) / 8;
-  dim3 grid(groups * 8 * p.H);
+  // one workgroup per (query block, batch, head): see the kernel for how ids map to them
+  const int64_t n = LOADER == LOAD_DENSE ? (int64_t)((p.B * p.H + 7) / 8) * 8 * p.nqb : (int64_t)((p.npairs + 7) / 8) * 8 * p.H;
+  if (n > 2147483647LL) return TPA_ERR_SHAPE;
+  dim3 grid((unsigned)n);
   hipLaunchKernelGGL(kern, grid, dim3(512), lds_bytes, stream, p);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
 }
@@ -1124,20 +1140,21 @@ int tpa_prefill_mfma_supported(const TpaFwdArgs* a) {
   return 1;
 }
 
-// bytes of workspace that let the prefill kernel run on dense K and V (both bf16 [B, lk, H, D]);
-// 0 if a batch entry would not fit the kernel's 32-bit tile offsets
-size_t tpa_prefill_dense_kv_bytes(int64_t B, int64_t lk, int64_t H, int64_t D) {
+// bytes of workspace that let the prefill kernel run on dense Q [B, lq, H, D], K and V [B, lk, H, D]
+// (bf16, each rounded up to 256 bytes); 0 if a batch entry would not fit the kernel's 32-bit tile offsets
+size_t tpa_prefill_dense_bytes(int64_t B, int64_t lq, int64_t lk, int64_t H, int64_t D) {
   if (lk * H * D * 2 >= (int64_t(1) << 31)) return 0;
-  return (size_t)(2 * ((B * lk * H * D * 2 + 255) / 256 * 256));
+  const auto slot = [](int64_t n) { return (size_t)((n * 2 + 255) / 256 * 256); };
+  return slot(B * lq * H * D) + 2 * slot(B * lk * H * D);
 }
 
-// Whether reconstructing dense K and V once (two HBM-bound launches) and running the plain tile
-// loader beats rebuilding every tile in the flash loop.  Ranks other than 2: from the second
-// query block on (the loop over ranks has no tuned rebuild).  Rank 2: the tuned rebuild costs the
-// loop about 9 % and the reconstruction grows with the length only, so it pays for long sequences.
-int tpa_prefill_wants_dense_kv(int64_t lq, int64_t rk) {
-  if (rk != 2) return lq > tpa::kBQ;
-  return lq >= 16384;
+// Whether reconstructing dense Q, K and V once (three HBM-bound launches) and running the plain
+// tile loader beats rebuilding every tile in the flash loop: from the second query block on.  The
+// loop over dense tiles overlaps the logits of one tile with the softmax of the one before and
+// has no rebuild in it; the reconstruction grows with the length only.
+int tpa_prefill_wants_dense(int64_t lq, int64_t rk) {
+  (void)rk;
+  return lq > tpa::kBQ;
 }
 
 int tpa_prefill_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
@@ -1150,21 +1167,25 @@ int tpa_prefill_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
   p.sm_scale = a->sm_scale; p.causal = a->causal; p.coff = tpa::causal_offset_of(a);
   p.nqb = (a->lq + kBQ - 1) / kBQ;
   p.npairs = p.nqb * a->B;
-  // Ranks other than 2: every workgroup of the fused kernel would rebuild the K/V tiles of its
-  // head from all ranks again (once per 256 query rows).  With a workspace the dense K and V are
-  // built once and the kernel runs with its plain tile loader, Q still coming from its factors.
-  const size_t dense_bytes = tpa_prefill_dense_kv_bytes(a->B, a->lk, a->H, a->dk);
-  if (tpa_prefill_wants_dense_kv(a->lq, a->rk) && a->workspace && dense_bytes && a->workspace_bytes >= dense_bytes &&
+  // With a workspace Q (times sm_scale * log2 e), K and V are reconstructed once as dense bf16 and
+  // the kernel runs with its plain tile loader: no workgroup rebuilds tiles from the rank factors
+  // (the fused kernel does that once per 256 query rows and head).
+  const size_t dense_bytes = tpa_prefill_dense_bytes(a->B, a->lq, a->lk, a->H, a->dk);
+  if (tpa_prefill_wants_dense(a->lq, a->rk) && a->workspace && dense_bytes && a->workspace_bytes >= dense_bytes &&
       !(reinterpret_cast<uintptr_t>(a->workspace) & 255)) {
-    uint16_t* kd = static_cast<uint16_t*>(a->workspace);
-    uint16_t* vd = kd + dense_bytes / 4;
-    int rc = tpa_recon_dense_bf16(&a->ka, &a->kb, kd, a->B, a->lk, a->H, a->dk, a->rk, stream);
-    if (rc == TPA_OK) rc = tpa_recon_dense_bf16(&a->va, &a->vb, vd, a->B, a->lk, a->H, a->dv, a->rk, stream);
-    if (rc != TPA_OK) return rc;
     const int64_t hd = (int64_t)a->H * a->dk;
+    const size_t kv_slot = ((size_t)a->B * a->lk * hd * 2 + 255) / 256 * 256;
+    uint16_t* kd = static_cast<uint16_t*>(a->workspace);
+    uint16_t* vd = kd + kv_slot / 2;
+    uint16_t* qd = vd + kv_slot / 2;
+    int rc = tpa_recon_dense_bf16(&a->ka, &a->kb, kd, a->B, a->lk, a->H, a->dk, a->rk, 1.f, stream);
+    if (rc == TPA_OK) rc = tpa_recon_dense_bf16(&a->va, &a->vb, vd, a->B, a->lk, a->H, a->dv, a->rk, 1.f, stream);
+    if (rc == TPA_OK) rc = tpa_recon_dense_bf16(&a->qa, &a->qb, qd, a->B, a->lq, a->H, a->dk, a->rq, a->sm_scale * kLog2e, stream);
+    if (rc != TPA_OK) return rc;
+    p.qb = TpaFactor{qd, a->lq * hd, hd, 0};
     p.kb = TpaFactor{kd, a->lk * hd, hd, 0};
     p.vb = TpaFactor{vd, a->lk * hd, hd, 0};
-    p.q_factors = 1;
+    p.q_scaled = 1;
     if (p.kvseg) {
       if (a->dk == 128) return launch_prefill<128, LOAD_DENSE, true>(p, stream);
       return launch_prefill<64, LOAD_DENSE, true>(p, stream);

@@ -37,6 +37,11 @@ __all__ = [
 ]
 
 
+# Whether forward calls bring the optional workspace with which the library reconstructs dense Q, K, V
+# once and runs its fastest prefill loop (`tpa_factors(use_workspace=...)` overrides it per call).
+USE_WORKSPACE = True
+
+
 @dataclasses.dataclass
 class BlockSizes:
     """Tile configuration of the reference kernels (tpa/tpa.py:35-70).  Kept for signature
@@ -125,7 +130,7 @@ def tpa_factors(
     causal: bool = False,
     kernel: int = _d.KERNEL_AUTO,
     return_lse: bool = True,
-    use_workspace: bool = True,
+    use_workspace: bool | None = None,
     kv_lengths=None,
     causal_offset: int = 0,
     nomat: bool = False,
@@ -138,7 +143,7 @@ def tpa_factors(
     Returns (o[b,lq,h,dv] in the input dtype, lse[b,h,lq] fp32 or None).  The arrays may be
     views (e.g. slices of the concatenated tensors); only the last dimension must be contiguous.
     `use_workspace=False` withholds the optional scratch memory, which keeps the call on the
-    fused prefill kernel whatever the problem.  `kv_lengths` (int32 [b], an addition): batch
+    fused prefill kernel whatever the problem (None: the module's `USE_WORKSPACE`, True unless changed).  `kv_lengths` (int32 [b], an addition): batch
     entry i attends to its first kv_lengths[i] keys only; the rest of its k / v rows is padding
     that is never read.  `causal_offset` (an addition, also taken by `tpa_factors_bwd`): with `causal`, query i
     sees keys up to i + causal_offset; 0 is the reference's top-left alignment
@@ -147,6 +152,8 @@ def tpa_factors(
     first key of the shard it meets to its own first query.  `nomat` (tpa/tpa.py:250): never
     form K or V - same results, the rank-space order of operations (see the module docstring).
     """
+    if use_workspace is None:
+        use_workspace = USE_WORKSPACE
     device = _pick_device(qa, qb, ka, kb, va, vb)
     qa, qb, ka, kb, va, vb = (_as_device_tensor(x, device) for x in (qa, qb, ka, kb, va, vb))
     dtype = qa.dtype

@@ -18,6 +18,18 @@ from oracle import tpa_oracle as orc
 
 pytestmark = pytest.mark.gpu
 
+
+@pytest.fixture(params=["dense", "fused"], autouse=True)
+def prefill_route(request, monkeypatch):
+    """Every test of this file runs twice: with the optional workspace (bf16 prefills longer than one query
+    block then go through dense Q, K, V and the pipelined loop) and without it (the fused kernels that rebuild
+    K/V tiles from the rank factors).  Calls that name `use_workspace` themselves are not affected."""
+    from tpa import tpa
+
+    monkeypatch.setattr(tpa, "USE_WORKSPACE", request.param == "dense")
+    return request.param
+
+
 F32_TOL = 1e-4
 BF16_TOL = 2e-2
 LSE_TOL = 1e-3
@@ -126,7 +138,7 @@ def split(tq, tk, tv, h):
     return tuple(t.contiguous() for x in (tq, tk, tv) for t in (x[..., :h], x[..., h:]))
 
 
-def run_bf16(gpu, q, k, v, h, sm_scale, causal, kernel=2, use_workspace=True):
+def run_bf16(gpu, q, k, v, h, sm_scale, causal, kernel=2, use_workspace=None):
     from tpa import tpa
 
     tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
@@ -186,7 +198,7 @@ def test_prefill_concatenated_layout_in_place(gpu):
     assert np.abs(as_f64(o_gen) - o_ref).max() <= BF16_TOL
 
 
-def sampled_rows_check(gpu, b, t, h, d, rq, rk, causal, rows, batches, seed=0, use_workspace=True):
+def sampled_rows_check(gpu, b, t, h, d, rq, rk, causal, rows, batches, seed=0, use_workspace=None):
     q, k, v = make_factors(seed, b, t, t, h, d, d, rq, rk, scale_by_rank=True)
     scale = d**-0.5
     (tq, tk, tv), o, lse = run_bf16(gpu, q, k, v, h, scale, causal, use_workspace=use_workspace)
@@ -225,21 +237,19 @@ def test_config2_full_size_sampled_rows_and_prefix(gpu):
     assert torch.equal(o2, o) and torch.equal(lse2, lse)
 
 
-@pytest.mark.parametrize("use_workspace", [True, False])
-def test_config3_long_context_sampled_rows(gpu, use_workspace):
+def test_config3_long_context_sampled_rows(gpu):
     """B=1, T=32768, H=32, D=128, causal: sampled rows.  With the workspace the call reconstructs
     dense K and V once and runs the plain tile loader; without it the fused kernel rebuilds every
     K/V tile from the rank factors inside the flash loop."""
     rows = np.array([0, 255, 256, 4097, 16383, 32767])
-    sampled_rows_check(gpu, 1, 32768, 32, 128, 6, 2, True, rows, batches=[0], use_workspace=use_workspace)
+    sampled_rows_check(gpu, 1, 32768, 32, 128, 6, 2, True, rows, batches=[0])
 
 
-@pytest.mark.parametrize("use_workspace", [True, False])
-def test_config5_high_rank_noncausal_sampled_rows(gpu, use_workspace):
+def test_config5_high_rank_noncausal_sampled_rows(gpu):
     """B=8, T=2048, H=64, D=64, Rq=16, Rk=Rv=8, non-causal; through dense K/V (workspace) and
     through the fused any-rank tile rebuild (no workspace)."""
     rows = np.array([0, 100, 1023, 2047])
-    sampled_rows_check(gpu, 8, 2048, 64, 64, 16, 8, False, rows, batches=[0, 7], use_workspace=use_workspace)
+    sampled_rows_check(gpu, 8, 2048, 64, 64, 16, 8, False, rows, batches=[0, 7])
 
 
 # ---------------------------------------------------------------- decode over the factored cache
@@ -553,11 +563,14 @@ def test_prefill_bf16_segment_ids(gpu, b, lq, lk, h, d, rk, seg, causal):
         assert np.isnan(o_ref).any()  # the case really has empty rows
 
 
-def test_tpa_entry_point_serves_decode_with_the_split_key_kernel(gpu):
+def test_tpa_entry_point_serves_decode_with_the_split_key_kernel(gpu, prefill_route):
     """tpa(q[b, 1, ...], k, v) - how the reference itself expresses decode - gives the result of
     tpa_decode (bit for bit: it is the same kernel) and matches the oracle, reading the
-    concatenated cache in place."""
+    concatenated cache in place.  (The split partials need the workspace.)"""
     from tpa import tpa
+
+    if prefill_route != "dense":
+        pytest.skip("without the workspace tpa() cannot reach the split-key kernel")
 
     b, lk, h, d = 3, 4096, 32, 128
     q, k, v = make_factors(61, b, 1, lk, h, d, d, 6, 2, scale_by_rank=True)
@@ -936,11 +949,12 @@ def test_causal_offset(gpu, dt, kernel, b, lq, lk, h, d, rq, rk, offset, seg):
 
 
 def test_causal_offset_rows_equal_the_tail_of_the_full_causal_call(gpu):
-    """The last 256 rows of a causal call over 1024 tokens, and those 256 rows alone as queries with
-    causal_offset = 768 over the same keys: the same launch-level arithmetic, equal results."""
+    """The last 512 rows of a causal call over 1024 tokens, and those 512 rows alone as queries with
+    causal_offset = 512 over the same keys: the same launch-level arithmetic, equal results - on the
+    route through dense Q, K, V (with the workspace) and on the fused kernel (without)."""
     from tpa import tpa
 
-    b, t, h, d, n = 2, 1024, 4, 128, 256
+    b, t, h, d, n = 2, 1024, 4, 128, 512
     q, k, v = make_factors(141, b, t, t, h, d, d, 6, 2, scale_by_rank=True)
     tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
     o_full, lse_full = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=d**-0.5, causal=True)
@@ -982,7 +996,8 @@ def test_decode_with_a_causal_limit_per_query_row(gpu, dt, b, lq, lk, h, d, rq, 
         o_ref, l_ref = _offset_reference(fq, fk, fv, h, sm_scale, offset, np.zeros((b, lq), np.int32), kvseg)
     tol = F32_TOL if dt == torch.float32 else BF16_TOL
     check(o, lse, o_ref, l_ref, tol, bf16_bounds(tq, tk, tv, h, sm_scale, form="factored"))
-    o2, lse2 = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=sm_scale, causal=True, kernel=2, kv_lengths=kvl, causal_offset=offset)
+    o2, lse2 = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=sm_scale, causal=True, kernel=2, kv_lengths=kvl, causal_offset=offset,
+                               use_workspace=True)  # with it this entry point reaches the same split-key kernel
     assert torch.equal(torch.nan_to_num(o2.float(), nan=7.0), torch.nan_to_num(o.float(), nan=7.0)) and torch.equal(lse2, lse)
 
 
@@ -1024,7 +1039,7 @@ def test_causal_mask_aligned_with_the_end_of_each_sequence(gpu, dt, kernel, lq, 
     kvl = torch.tensor(lengths, dtype=torch.int32, device=gpu)
     sm_scale = d**-0.5
     o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=sm_scale, causal=tpa.CAUSAL_BOTTOM_RIGHT, kernel=kernel,
-                             kv_lengths=kvl, causal_offset=extra)
+                             kv_lengths=kvl, causal_offset=extra, use_workspace=True if lq <= 16 else None)
     o_ref, l_ref = _bottom_right_reference(as_f64(tq), as_f64(tk), as_f64(tv), lengths, h, sm_scale, extra)
     check(o, lse, o_ref, l_ref, F32_TOL if dt == torch.float32 else BF16_TOL, bf16_bounds(tq, tk, tv, h, sm_scale))
     if lq <= 16 and kernel == 2:  # the same through tpa_decode, contiguous and as a pool of shuffled pages
