@@ -90,7 +90,15 @@ __global__ __launch_bounds__(256) void recon_bf16_kernel(TpaFactor fa, TpaFactor
 // (token, 16-byte piece of D, group of 8 heads) and reads, per rank, one 16-byte piece of b and
 // the 8 head factors as one 16-byte piece of a - 64 multiply-adds per two loads.  Pieces are the
 // fastest thread index, so the 16 threads of a (token, head group) store whole rows of D.
-__global__ __launch_bounds__(256) void recon_bf16_h8_kernel(TpaFactor fa, TpaFactor fb, uint16_t* out, int L, int H, int D, int R, float scale) {
+struct ReconJob { TpaFactor fa, fb; uint16_t* out; int L, R; float scale; };
+struct ReconJobs { ReconJob job[3]; };  // blockIdx.z picks one: several arrays in one launch
+__global__ __launch_bounds__(256) void recon_bf16_h8_kernel(ReconJobs jobs, int H, int D) {
+  const TpaFactor fa = blockIdx.z == 0 ? jobs.job[0].fa : blockIdx.z == 1 ? jobs.job[1].fa : jobs.job[2].fa;
+  const TpaFactor fb = blockIdx.z == 0 ? jobs.job[0].fb : blockIdx.z == 1 ? jobs.job[1].fb : jobs.job[2].fb;
+  uint16_t* const out = blockIdx.z == 0 ? jobs.job[0].out : blockIdx.z == 1 ? jobs.job[1].out : jobs.job[2].out;
+  const int L = blockIdx.z == 0 ? jobs.job[0].L : blockIdx.z == 1 ? jobs.job[1].L : jobs.job[2].L;
+  const int R = blockIdx.z == 0 ? jobs.job[0].R : blockIdx.z == 1 ? jobs.job[1].R : jobs.job[2].R;
+  const float scale = blockIdx.z == 0 ? jobs.job[0].scale : blockIdx.z == 1 ? jobs.job[1].scale : jobs.job[2].scale;
   const int cpr = D / 8, hg = H / 8;
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int cc = (int)(idx % cpr);
@@ -600,14 +608,34 @@ int tpa_recon_dense_bf16(const TpaFactor* fa, const TpaFactor* fb, uint16_t* out
   const bool vec_a = vec && H % 8 == 0 && !(reinterpret_cast<uintptr_t>(fa->ptr) & 15) && fa->stride_b % 8 == 0 && fa->stride_l % 8 == 0 &&
                      fa->stride_r % 8 == 0;
   const int64_t threads = (int64_t)L * (D / 8) * (H / 8);
-  if (vec_a && (threads + 255) / 256 <= 2147483647LL)
-    hipLaunchKernelGGL(tpa::recon_bf16_h8_kernel, dim3((unsigned)((threads + 255) / 256), B), dim3(256), 0, stream, *fa, *fb, out, L, H, D, R, scale);
-  else if (vec)
+  if (vec_a && (threads + 255) / 256 <= 2147483647LL) {
+    tpa::ReconJobs jobs{};
+    jobs.job[0] = tpa::ReconJob{*fa, *fb, out, L, R, scale};
+    hipLaunchKernelGGL(tpa::recon_bf16_h8_kernel, dim3((unsigned)((threads + 255) / 256), B, 1), dim3(256), 0, stream, jobs, H, D);
+  } else if (vec)
     hipLaunchKernelGGL(tpa::recon_bf16_kernel, dim3((L + tpa::kReconTokens - 1) / tpa::kReconTokens, B), dim3(256), 0, stream, *fa, *fb, out, L, H, D, R, scale);
   else if (scale != 1.f)
     return TPA_ERR_ALIGN;  // the scaled form exists for 16-byte aligned factors only
   else
     hipLaunchKernelGGL((tpa::recon_kernel<uint16_t, uint16_t>), dim3(L, B), dim3(256), 0, stream, *fa, *fb, out, L, H, D, R);
+  return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
+}
+
+// Q (with its scale), K and V in one launch where every factor is 16-byte aligned and H % 8 == 0;
+// TPA_ERR_UNSUPPORTED otherwise (the caller then reconstructs them one by one).
+int tpa_recon_dense_qkv_bf16(const TpaFwdArgs* a, uint16_t* qd, uint16_t* kd, uint16_t* vd, float q_scale, hipStream_t stream) {
+  if (a->B > 65535 || a->H % 8 != 0 || a->dk % 8 != 0 || a->dk != a->dv) return TPA_ERR_UNSUPPORTED;
+  const TpaFactor* fs[6] = {&a->qa, &a->qb, &a->ka, &a->kb, &a->va, &a->vb};
+  for (const TpaFactor* f : fs)
+    if ((reinterpret_cast<uintptr_t>(f->ptr) & 15) || f->stride_b % 8 != 0 || f->stride_l % 8 != 0 || f->stride_r % 8 != 0) return TPA_ERR_UNSUPPORTED;
+  const int lmax = a->lq > a->lk ? a->lq : a->lk;
+  const int64_t blocks = ((int64_t)lmax * (a->dk / 8) * (a->H / 8) + 255) / 256;
+  if (blocks > 2147483647LL) return TPA_ERR_UNSUPPORTED;
+  tpa::ReconJobs jobs{};
+  jobs.job[0] = tpa::ReconJob{a->qa, a->qb, qd, a->lq, a->rq, q_scale};
+  jobs.job[1] = tpa::ReconJob{a->ka, a->kb, kd, a->lk, a->rk, 1.f};
+  jobs.job[2] = tpa::ReconJob{a->va, a->vb, vd, a->lk, a->rk, 1.f};
+  hipLaunchKernelGGL(tpa::recon_bf16_h8_kernel, dim3((unsigned)blocks, a->B, 3), dim3(256), 0, stream, jobs, a->H, a->dk);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
 }
 

@@ -197,3 +197,5 @@ size_t tpa_prefill_dense_bytes(int64_t B, int64_t lq, int64_t lk, int64_t H, int
 int tpa_prefill_wants_dense(int64_t lq, int64_t rk);
 // dense bf16 X[B, L, H, D] = (scale/R) sum_r a_r (x) b_r from bf16 factors
 int tpa_recon_dense_bf16(const TpaFactor* fa, const TpaFactor* fb, uint16_t* out, int B, int L, int H, int D, int R, float scale, hipStream_t stream);
+// dense Q (times q_scale), K, V of a forward call in one launch; TPA_ERR_UNSUPPORTED where the vectorised kernel does not apply
+int tpa_recon_dense_qkv_bf16(const TpaFwdArgs* a, uint16_t* qd, uint16_t* kd, uint16_t* vd, float q_scale, hipStream_t stream);

@@ -1178,9 +1178,12 @@ int tpa_prefill_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {
     uint16_t* kd = static_cast<uint16_t*>(a->workspace);
     uint16_t* vd = kd + kv_slot / 2;
     uint16_t* qd = vd + kv_slot / 2;
-    int rc = tpa_recon_dense_bf16(&a->ka, &a->kb, kd, a->B, a->lk, a->H, a->dk, a->rk, 1.f, stream);
-    if (rc == TPA_OK) rc = tpa_recon_dense_bf16(&a->va, &a->vb, vd, a->B, a->lk, a->H, a->dv, a->rk, 1.f, stream);
-    if (rc == TPA_OK) rc = tpa_recon_dense_bf16(&a->qa, &a->qb, qd, a->B, a->lq, a->H, a->dk, a->rq, a->sm_scale * kLog2e, stream);
+    int rc = tpa_recon_dense_qkv_bf16(a, qd, kd, vd, a->sm_scale * kLog2e, stream);
+    if (rc == TPA_ERR_UNSUPPORTED) {
+      rc = tpa_recon_dense_bf16(&a->ka, &a->kb, kd, a->B, a->lk, a->H, a->dk, a->rk, 1.f, stream);
+      if (rc == TPA_OK) rc = tpa_recon_dense_bf16(&a->va, &a->vb, vd, a->B, a->lk, a->H, a->dv, a->rk, 1.f, stream);
+      if (rc == TPA_OK) rc = tpa_recon_dense_bf16(&a->qa, &a->qb, qd, a->B, a->lq, a->H, a->dk, a->rq, a->sm_scale * kLog2e, stream);
+    }
     if (rc != TPA_OK) return rc;
     p.qb = TpaFactor{qd, a->lq * hd, hd, 0};
     p.kb = TpaFactor{kd, a->lk * hd, hd, 0};
