@@ -113,23 +113,29 @@ __global__ __launch_bounds__(256) void recon_bf16_h8_kernel(ReconJobs jobs, int 
   for (int i = 0; i < 8; ++i)
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[i][j] = 0.f;
-  u32x4 av = *reinterpret_cast<const u32x4*>(ap), bv = *reinterpret_cast<const u32x4*>(bp);
-  for (int r = 0; r < R; ++r) {
-    const u32x4 a_cur = av, b_cur = bv;
-    if (r + 1 < R) {  // the next rank's pieces are on their way during this rank's arithmetic
-      av = *reinterpret_cast<const u32x4*>(ap + (int64_t)(r + 1) * fa.stride_r);
-      bv = *reinterpret_cast<const u32x4*>(bp + (int64_t)(r + 1) * fb.stride_r);
-    }
-    float af[8], bf[8];
+  constexpr int G = 4;  // ranks whose loads are in flight together (the kernel is bound by their latency)
+  for (int r0 = 0; r0 < R; r0 += G) {
+    u32x4 av[G], bv[G];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      af[2 * j] = bf16lo_to_f32(a_cur[j]); af[2 * j + 1] = bf16hi_to_f32(a_cur[j]);
-      bf[2 * j] = bf16lo_to_f32(b_cur[j]); bf[2 * j + 1] = bf16hi_to_f32(b_cur[j]);
+    for (int u = 0; u < G; ++u) {
+      const int r = min(r0 + u, R - 1);
+      av[u] = *reinterpret_cast<const u32x4*>(ap + (int64_t)r * fa.stride_r);
+      bv[u] = *reinterpret_cast<const u32x4*>(bp + (int64_t)r * fb.stride_r);
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int u = 0; u < G; ++u) {
+      if (r0 + u >= R) break;
+      float af[8], bf[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc[i][j] += af[i] * bf[j];
+      for (int j = 0; j < 4; ++j) {
+        af[2 * j] = bf16lo_to_f32(av[u][j]); af[2 * j + 1] = bf16hi_to_f32(av[u][j]);
+        bf[2 * j] = bf16lo_to_f32(bv[u][j]); bf[2 * j + 1] = bf16hi_to_f32(bv[u][j]);
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] += af[i] * bf[j];
+    }
   }
   const float inv = scale / (float)R;
   uint16_t* op = out + (((int64_t)b * L + t) * H + 8 * g) * D + 8 * cc;

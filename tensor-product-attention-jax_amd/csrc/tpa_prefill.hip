@@ -1148,13 +1148,16 @@ size_t tpa_prefill_dense_bytes(int64_t B, int64_t lq, int64_t lk, int64_t H, int
   return slot(B * lq * H * D) + 2 * slot(B * lk * H * D);
 }
 
-// Whether reconstructing dense Q, K and V once (three HBM-bound launches) and running the plain
-// tile loader beats rebuilding every tile in the flash loop: from the second query block on.  The
-// loop over dense tiles overlaps the logits of one tile with the softmax of the one before and
-// has no rebuild in it; the reconstruction grows with the length only.
+// Whether reconstructing dense Q, K and V once (one HBM-bound launch) and running the plain tile
+// loader beats rebuilding every tile in the flash loop.  The loop over dense tiles overlaps the
+// logits of one tile with the softmax of the one before and has no rebuild in it; the
+// reconstruction grows with the length only.  Rank 2 has a tuned rebuild in the fused kernel:
+// measured at B * H = 64, D = 128 the two routes meet at 1024 rows (51 against 52 us) and the dense
+// one wins from 2048 on (105 against 115 us; 4096: 0.32 against 0.38 ms).  Other ranks loop over
+// the ranks per tile in the fused kernel: dense from the second query block on.
 int tpa_prefill_wants_dense(int64_t lq, int64_t rk) {
-  (void)rk;
-  return lq > tpa::kBQ;
+  if (rk != 2) return lq > tpa::kBQ;
+  return lq >= 2048;
 }
 
 int tpa_prefill_mfma_launch(const TpaFwdArgs* a, hipStream_t stream) {

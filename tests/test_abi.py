@@ -77,7 +77,8 @@ def test_size_queries_need_no_gpu():
     assert lib.tpa_fwd_workspace_bytes(8, 2048, 2048, 64, 64, 64, 16, 8) == 3 * 8 * 2048 * 64 * 64 * 2  # dense Q, K, V
     assert lib.tpa_fwd_workspace_bytes(4, 4096, 4096, 16, 128, 128, 6, 2) == 3 * 4 * 4096 * 16 * 128 * 2
     assert lib.tpa_fwd_workspace_bytes(1, 32768, 32768, 32, 128, 128, 6, 2) == 3 * 32768 * 32 * 128 * 2
-    assert lib.tpa_fwd_workspace_bytes(2, 256, 4096, 16, 128, 128, 6, 2) == 0   # one query block: the fused kernel
+    assert lib.tpa_fwd_workspace_bytes(2, 1024, 4096, 16, 128, 128, 6, 2) == 0   # rank 2 below 2048 rows: the fused kernel
+    assert lib.tpa_fwd_workspace_bytes(2, 257, 4096, 16, 128, 128, 6, 4) > 0    # other ranks: from the second query block on
     assert lib.tpa_fwd_workspace_bytes(2, 512, 512, 4, 48, 48, 6, 4) == 0        # not an MFMA head size
     # backward: dense Q, K, V and their gradients (fp32, each rounded up to 256 bytes) plus delta
     r = lambda n: (n + 255) // 256 * 256

@@ -222,7 +222,7 @@ def test_config2_full_size_sampled_rows_and_prefix(gpu):
 
     rows = np.array([0, 1, 63, 64, 255, 256, 1000, 2047, 2048, 4095])
     (tq, tk, tv), o, lse = sampled_rows_check(gpu, 4, 4096, 16, 128, 6, 2, True, rows, batches=[0, 3])
-    n = 1024
+    n = 2048  # long enough for the same route as the full call on either setting of the workspace
     h = 16
     o_p, lse_p = tpa.tpa_factors(
         tq[:, :n, :, :h], tq[:, :n, :, h:], tk[:, :n, :, :h], tk[:, :n, :, h:], tv[:, :n, :, :h], tv[:, :n, :, h:],
@@ -395,6 +395,50 @@ def test_mha_bf16_flash_vs_oracle(gpu, d, causal):
     o_ref, l_ref = orc.mha_forward(as_f64(q), as_f64(k), as_f64(v), bias, d**-0.5)
     o, (lse, *_) = _mha_fwd(q, k, v, None, d**-0.5, causal=causal, kernel=2)
     check(o, lse, o_ref, l_ref, BF16_TOL, dense_bounds(as_f64(q), as_f64(k), as_f64(v), d**-0.5))
+
+
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("lk", [192, 193, 256, 257, 320, 321, 449, 1000])
+def test_mha_pipelined_loop_boundaries(gpu, prefill_route, d, causal, lk):
+    """Dense flash attention at key counts around the entry and exit of the pipelined tile loop: it takes
+    the unmasked tiles 1 .. n-1 of a wave when there are at least two of them, enters with an odd tile and
+    leaves after an even or an odd number of iterations; under the causal mask every wave of a workgroup
+    has its own range."""
+    from tpa.mha import _mha_fwd
+
+    if prefill_route != "dense":
+        pytest.skip("one route: dense attention brings no workspace")
+    rng = np.random.Generator(np.random.Philox(lk))
+    b, h = 2, 2
+    lq = lk if causal else 300
+    q, k, v = (torch.from_numpy(rng.standard_normal((b, l, h, d), dtype=np.float32)).to(torch.bfloat16).to(gpu) for l in (lq, lk, lk))
+    bias = np.where(np.tril(np.ones((lq, lk), bool)), 0.0, -np.inf)[None].repeat(b, 0) if causal else None
+    o_ref, l_ref = orc.mha_forward(as_f64(q), as_f64(k), as_f64(v), bias, d**-0.5)
+    o, (lse, *_) = _mha_fwd(q, k, v, None, d**-0.5, causal=causal, kernel=2)
+    check(o, lse, o_ref, l_ref, BF16_TOL, dense_bounds(as_f64(q), as_f64(k), as_f64(v), d**-0.5))
+
+
+def test_mha_reference_moves_inside_the_pipelined_loop(gpu, prefill_route):
+    """Logits that grow along the keys (the row maximum leaves the slack of the running reference in tile
+    after tile): the rare path of the pipelined loop rescales the accumulators, the row sums and the logits
+    of the tile whose accumulation has already begun."""
+    from tpa.mha import _mha_fwd
+
+    if prefill_route != "dense":
+        pytest.skip("one route: dense attention brings no workspace")
+    rng = np.random.Generator(np.random.Philox(77))
+    b, h, d, lq, lk = 1, 2, 128, 256, 1024
+    q = rng.standard_normal((b, lq, h, d), dtype=np.float32)
+    k = rng.standard_normal((b, lk, h, d), dtype=np.float32)
+    v = rng.standard_normal((b, lk, h, d), dtype=np.float32)
+    # a component along which every query has a positive projection, growing with the key index
+    q[..., 0] = 4.0
+    k[..., 0] = np.linspace(0.0, 24.0, lk, dtype=np.float32)[None, :, None]
+    tq, tk, tv = (torch.from_numpy(x).to(torch.bfloat16).to(gpu) for x in (q, k, v))
+    o_ref, l_ref = orc.mha_forward(as_f64(tq), as_f64(tk), as_f64(tv), None, d**-0.5)
+    o, (lse, *_) = _mha_fwd(tq, tk, tv, None, d**-0.5, kernel=2)
+    check(o, lse, o_ref, l_ref, BF16_TOL, dense_bounds(as_f64(tq), as_f64(tk), as_f64(tv), d**-0.5))
 
 
 def test_mha_equals_tpa_on_reconstructed_kv(gpu):
