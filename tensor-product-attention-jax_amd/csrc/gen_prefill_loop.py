@@ -55,8 +55,9 @@ def O(db): return 80 + 16 * db                    # v[80:143]: O^T accumulators
 def Q(ks): return 144 + 4 * ks                    # v[144:175]: Q fragments
 def KREG(ps): return 176 + 4 * ps                 # v[176:183]: K rows on their way (one tuple per loader pass)
 def VREG(ps): return 184 + 4 * ps                 # v[184:191]: V rows
-RING_BUFS = [192, 196, 200]                       # v[192:203]: fragment buffers
-assert 1 <= LA < len(RING_BUFS)
+RING_BUFS = [192, 196, 200, 212]                  # v[192:203], v[212:215]: fragment buffers
+BATCH = int(os.environ.get("PF_BATCH", "1"))      # fragments fetched, and waited for, together
+assert 1 <= LA < len(RING_BUFS) and BATCH in (1, 2)
 MREF, LSUM, KFRAG0, VFRAG, KW0, VW, KVOFF, VVOFF = range(204, 212)   # v[204:219]: state / address tuple
 TA, TB, T0A, T1A, KFRAG, KW, RD, RAL, T0B, T1B = range(220, 230)        # v[220:229]: temporaries
 # s[32:47] scalar tuple
@@ -262,14 +263,20 @@ def load_groups():
     return g
 
 
-def frag_buf(f): return RING_BUFS[f % (LA + 1)]
+def frag_buf(f): return RING_BUFS[f % (LA + 1)] if BATCH == 1 else RING_BUFS[f % 4]
+
+def qk_of(f):
+    """(32-key block, k step) of S^T instruction f: the two blocks alternate, so that consecutive
+    matrix instructions accumulate into different tuples (back-to-back accumulation into one tuple
+    costs 37 cycles an instruction instead of 32)"""
+    return (f % 2, f // 2) if "qkchain" not in KO else divmod(f, NKS)
 
 def emit_frag_load(e, f, p):
     if "frag" in KO:
         return
     b = frag_buf(f)
     if f < 2 * NKS:                       # rows of K tile j+1
-        mb, kk = divmod(f, NKS)
+        mb, kk = qk_of(f)
         e.ins("ds_read_b128", vt(b), f"v{KFRAG} offset:{mb * 32 * KS * 2 + kk * 32}")
     else:                                 # columns of V tile j (buffer p)
         kk, db = divmod(f - 2 * NKS, NDB)
@@ -282,7 +289,7 @@ def emit_mfma(e, f, p):
         return
     b = frag_buf(f)
     if f < 2 * NKS:                       # logits of tile j+1 into the other set
-        mb, kk = divmod(f, NKS)
+        mb, kk = qk_of(f)
         s = S(1 - p, mb)
         e.ins("v_mfma_f32_32x32x16_bf16", vt(s, 16), vt(b), vt(Q(kk)), vt(NMREF, 16) if kk == 0 else vt(s, 16))
     else:                                 # O^T += V^T P^T of tile j
@@ -383,7 +390,7 @@ def half(e, p, rare):
     """iteration j with j & 1 == p"""
     e.ins("v_add_u32", f"v{KFRAG}", f"s{S_KR}", f"v{KFRAG0}")
     e.ins("v_add_u32", f"v{KW}", f"s{S_KWB}", f"v{KW0}")
-    for f in range(LA):
+    for f in range(LA if BATCH == 1 else 2):
         emit_frag_load(e, f, p)
     slots = [[] for _ in range(NF)]
     N_QK = 2 * NKS
@@ -408,10 +415,16 @@ def half(e, p, rare):
     if n_max:
         branch_slot = (n_max - 1) * (N_QK - 1) // len(ga.items)
         assert branch_slot < N_QK // 2     # before the first exponential of block 1
-        rare[p] = [mb for mb in range(2) if mb * NKS <= branch_slot]
+        rare[p] = sorted({qk_of(f)[0] for f in range(branch_slot + 1)})
     for f in range(NF):
-        if f + LA < NF:
-            emit_frag_load(e, f + LA, p)
+        if BATCH == 1:
+            if f + LA < NF:
+                emit_frag_load(e, f + LA, p)
+        elif f % 2 == 0:                 # the next pair on its way, then one wait for this pair
+            for g in (f + 2, f + 3):
+                if g < NF:
+                    emit_frag_load(e, g, p)
+            e._wait_for({f"v{frag_buf(g) + k}" for g in (f, f + 1) for k in range(4)})
         emit_mfma(e, f, p)
         for it in slots[f]:
             replay(e, it)
@@ -454,8 +467,9 @@ def main():
         for ln in lines:
             f.write(f'"{ln}\\n\\t"\n')
     # registers the loop uses beyond its operands
-    ring = [b + k for b in RING_BUFS[:LA + 1] for k in range(4)]
-    clob = [f"v{n}" for n in sorted(set(ring) | set(range(TA, T1B + 1)))]
+    ring = [b + k for b in (RING_BUFS[:LA + 1] if BATCH == 1 else RING_BUFS) for k in range(4)]
+    # (a buffer inside the state tuple v[204:219] is part of an in/out operand already)
+    clob = [f"v{n}" for n in sorted((set(ring) | set(range(TA, T1B + 1))) - set(range(204, 220)))]
     clob += [f"s{n}" for n in (S_T0, S_T1, S_SLACK)] + ["vcc", "scc", "memory"]
     with open(OUT.replace(".inc", "_clobbers.inc"), "w") as f:
         f.write("// generated by gen_prefill_loop.py: do not edit\n")
