@@ -75,7 +75,7 @@ def measured_traffic(workload):
     """HBM bytes per launch of the workload's kernels, read from the committed rocprofv3 counter summary
     (FETCH_SIZE / WRITE_SIZE in KiB per dispatch, one table row per kernel), each counter scaled by what it
     reads for the 1 GiB device copy in the same table.  None where the summary has no row for the kernels."""
-    kernels = {"c2": ["prefill_kernel<128, 0, false"], "c4": ["decode_kernel<128, 2, false, 1", "decode_merge_kernel<128, bf16"]}.get(workload)
+    kernels = {"c2": ["recon_bf16_h8_kernel", "prefill_kernel<128, 2, false, 1"], "c4": ["decode_kernel<128, 2, false, 1", "decode_merge_kernel<128, bf16"]}.get(workload)
     if not kernels or not os.path.exists(TRAFFIC_PROFILE):
         return None
     rows = {}
@@ -381,7 +381,8 @@ def main():
             value=r["tflops_wall"], unit="TFLOP/s", ms_per_step=r["wall_ms"],
             roofline=dict(bound="mfma", achieved=r["tflops_kernel"], peak=peak, unit="TFLOP/s",
                           frac=r["tflops_kernel"] / peak, traffic=measured_traffic(args.workload),
-                          kernel="prefill_f32_kernel" if f32 else ("decode_kernel + decode_merge_kernel per 64 query rows" if args.workload.endswith("n") else "prefill_kernel"),
+                          kernel="prefill_f32_kernel" if f32 else ("decode_kernel + decode_merge_kernel per 64 query rows" if args.workload.endswith("n")
+                                                                   else "prefill_kernel" if args.workload.endswith("u") else "recon_bf16_h8_kernel + prefill_kernel"),
                           ms_per_launch=r["kernel_ms"],
                           ms_per_launch_min=r["kernel_ms_min"], algorithmic_flops_per_launch=r["flops"]),
             config=dict(workload=f"{args.workload}: TPA prefill" + (", fp32 inputs" if f32 else "") + (", nomat" if args.workload.endswith("n") else ""), **r["shape"]),
