@@ -173,6 +173,76 @@ __global__ __launch_bounds__(256) void append_mfma_kernel(AppendParams p) {
   write_new_lengths(p);
 }
 
+// ---- bf16, at most 64 new tokens in all (a decode step): the call is one read of W, so the k
+// dimension is split over the eight waves of a workgroup that owns 16 output columns - enough
+// workgroups to pull W at the rate of the memory system, where 64 x 64 tiles would leave most of the
+// chip idle.  Operands go from global memory straight into v_mfma_f32_16x16x32_bf16 fragments (a lane
+// holds 8 consecutive k of one token / one row of W, which is how both arrays lie in memory); the
+// eight partial tiles meet in LDS and 128 threads finish one chunk of eight columns each.
+constexpr int kFewTokens = 64, kFewCols = 16, kFewWaves = 8;
+__global__ __launch_bounds__(kFewWaves * 64) void append_fewrows_kernel(AppendParams p) {
+  __shared__ __attribute__((aligned(16))) float part[kFewWaves][kFewTokens][kFewCols + 4];
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, r16 = l & 15, kg = l >> 4;
+  const int n0 = blockIdx.x * kFewCols;
+  const uint16_t* x = static_cast<const uint16_t*>(p.x);
+  const uint16_t* wt = static_cast<const uint16_t*>(p.w);
+  const int kw = p.K / kFewWaves, k_begin = w * kw;             // this wave's share of the contraction
+  const uint16_t* wrow = wt + (int64_t)min(n0 + r16, p.N - 1) * p.K + k_begin + 8 * kg;
+  const uint16_t* xrow[4];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb) xrow[mb] = x + (int64_t)min(16 * mb + r16, p.M - 1) * p.K + k_begin + 8 * kg;
+  const int nblk = (p.M + 15) / 16;                             // blocks of 16 tokens that exist
+  f32x4 acc[4];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  constexpr int U = 4;                                          // k steps of 32 whose loads are in flight together
+  for (int k0 = 0; k0 < kw; k0 += 32 * U) {
+    bf16x8 bq[U], a[U][4];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kk = min(k0 + 32 * u, kw - 32);
+      bq[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wrow + kk));
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+        if (mb < nblk) a[u][mb] = *reinterpret_cast<const bf16x8*>(xrow[mb] + kk);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (k0 + 32 * u >= kw) break;
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+        if (mb < nblk) acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][mb], bq[u], acc[mb], 0, 0, 0);
+    }
+  }
+  // acc[mb][v] = partial y[token 16 mb + 4 kg + v][column n0 + r16]
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) part[w][16 * mb + 4 * kg + v][r16] = acc[mb][v];
+  __syncthreads();
+  if (tid < kFewTokens * (kFewCols / 8)) {
+    const int m = tid >> 1, cc = tid & 1, c0 = n0 + 8 * cc;
+    if (m < p.M && c0 < p.N) {
+      float y[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) y[j] = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < kFewWaves; ++ww) {
+        const f32x4 lo = *reinterpret_cast<const f32x4*>(&part[ww][m][8 * cc]), hi = *reinterpret_cast<const f32x4*>(&part[ww][m][8 * cc + 4]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { y[j] += lo[j]; y[4 + j] += hi[j]; }
+      }
+      bool rotate; int j0, pos;
+      uint16_t* dst = chunk_destination<uint16_t>(p, m, c0, rotate, j0, pos);
+      if (dst) {
+        if (rotate) rotate_chunk(p, y, pos, j0);
+        store_chunk(dst, y);
+      }
+    }
+  }
+  write_new_lengths(p);
+}
+
 // ---- any dtype and shape: one thread per chunk of eight columns
 template <typename T>
 __global__ __launch_bounds__(256) void append_generic_kernel(AppendParams p) {
@@ -242,7 +312,9 @@ extern "C" int tpa_cache_append(const TpaAppendArgs* a, void* stream) {
   bool mfma = a->kernel != TPA_KERNEL_GENERIC && a->dtype == TPA_DTYPE_BF16 && a->d_model % kBK == 0 && aligned16(a->x) && aligned16(a->w);
   for (const TpaFactor* f : fs) mfma = mfma && chunk_ok(*f);
   if (a->kernel == TPA_KERNEL_MFMA && !mfma) return TPA_ERR_UNSUPPORTED;
-  if (mfma) {
+  if (mfma && p.M <= kFewTokens && a->d_model % (32 * kFewWaves) == 0) {
+    hipLaunchKernelGGL(append_fewrows_kernel, dim3((p.N + kFewCols - 1) / kFewCols), dim3(kFewWaves * 64), 0, s, p);
+  } else if (mfma) {
     dim3 grid((p.N + kBN - 1) / kBN, (p.M + kBM - 1) / kBM);
     if (grid.y > 65535) return TPA_ERR_SHAPE;
     hipLaunchKernelGGL(append_mfma_kernel, grid, dim3(256), 0, s, p);

@@ -34,7 +34,17 @@ def make_layer(seed, b, n, dm, h, d, rq, rk, dtype, gpu):
 
 
 @pytest.mark.parametrize("dtype,kernel", [(torch.bfloat16, 2), (torch.bfloat16, 1), (torch.float32, 0)])
-@pytest.mark.parametrize("b,n,dm,h,d,rq,rk", [(3, 5, 256, 16, 64, 6, 2), (2, 70, 128, 8, 128, 3, 4), (1, 1, 64, 32, 128, 6, 2)])
+@pytest.mark.parametrize(
+    "b,n,dm,h,d,rq,rk",
+    [
+        (3, 5, 256, 16, 64, 6, 2),     # 15 tokens: the decode-step kernel (k split over the waves), one k step per wave
+        (2, 70, 128, 8, 128, 3, 4),    # 140 tokens: 64 x 64 tiles
+        (1, 1, 64, 32, 128, 6, 2),     # d_model too short for the k split: tiles
+        (64, 1, 1024, 32, 128, 6, 2),  # a decode step of 64 sequences: all four blocks of 16 tokens
+        (7, 3, 512, 8, 64, 2, 1),      # 21 tokens: the second block of 16 is ragged
+        (5, 2, 256, 8, 64, 1, 1),      # 216 output columns: the last workgroup owns half a block of columns
+    ],
+)
 def test_append_matches_the_oracle(gpu, dtype, kernel, b, n, dm, h, d, rq, rk):
     x, w = make_layer(1, b, n, dm, h, d, rq, rk, dtype, gpu)
     cache_len = 96
