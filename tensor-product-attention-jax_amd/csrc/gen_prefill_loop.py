@@ -281,6 +281,9 @@ def emit_frag_load(e, f, p):
     else:                                 # columns of V tile j (buffer p)
         kk, db = divmod(f - 2 * NKS, NDB)
         off = p * VBUF + kk * 16 * VS * 2 + db * 64
+        if "vtr" in KO:                    # timing only: one plain 16-byte read in place of the two transposed ones
+            e.ins("ds_read_b128", vt(b), f"v{KFRAG} offset:{(db % 2) * 32 * KS * 2 + ((kk * NDB + db) % NKS) * 32}")
+            return
         e.ins("ds_read_b64_tr_b16", vt(b, 2), f"v{VFRAG} offset:{off}")
         e.ins("ds_read_b64_tr_b16", vt(b + 2, 2), f"v{VFRAG} offset:{off + 8 * VS * 2}")
 
