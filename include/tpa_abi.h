@@ -281,18 +281,20 @@ const char* tpa_strerror(int code);
  * tpa/tpa.py:492-543 for all batch entries at once (the reference vmaps it, tpa/tpa.py:144-163).
  * If `workspace` holds at least tpa_decode_workspace_bytes(...) bytes and the problem is a
  * decode (lq <= 16, lk >= 1024, no segment ids) that tpa_decode's kernel takes, the call is served by
- * it; if the rank of k, v is not 2 (or the sequence is long, 16384 rows and more) and `workspace`
- * holds tpa_fwd_workspace_bytes(...) bytes, K and V are reconstructed into it once.  Without a
- * workspace the same problems run on the fused prefill kernel.
+ * it; if `workspace` holds tpa_fwd_workspace_bytes(...) bytes and the problem is long enough for it to
+ * pay (rank 2: 2048 query rows and more; other ranks: more than 256), dense bf16 Q (times
+ * sm_scale * log2 e), K and V are reconstructed into it once and the prefill kernel runs its loop over
+ * dense tiles.  Without a workspace the same problems run on the fused prefill kernel, which rebuilds
+ * K / V tiles from the rank factors inside its loop.  The two routes round at the same points (Q, K, V,
+ * the probabilities and the output to bf16 once each) but are not bit-identical.
  */
 int tpa_fwd(const TpaFwdArgs* args, void* stream);
 
 /*
  * Bytes of optional workspace (256-byte aligned) with which tpa_fwd can pick a faster kernel for
  * this problem, 0 if none would be used: the split partials of the decode kernel (lq <= 16 over
- * a long cache), or room for dense bf16 K and V when the rank of k and v is not 2 or there are
- * 16384 query rows and more - then K and V are reconstructed once (tpa/tpa.py:364,417 do it per
- * query block) and the flash kernel runs with its plain tile loader.
+ * a long cache), or room for dense bf16 K, V [B, lk, H, D] and Q [B, lq, H, D] (the reference
+ * reconstructs them per pair of blocks, tpa/tpa.py:317,364,417).
  */
 size_t tpa_fwd_workspace_bytes(int32_t B, int32_t lq, int32_t lk, int32_t H, int32_t dk, int32_t dv, int32_t rq, int32_t rk);
 

@@ -178,7 +178,7 @@ def tpa_factors(
     lse = torch.empty((b, h, lq), dtype=torch.float32, device=device) if return_lse else None
     lib = _d.load_library()
     # hand the library the workspace with which it can pick its fastest kernel (split partials for
-    # a decode through this entry point, dense K and V for ranks other than 2); it decides whether
+    # a decode through this entry point, dense Q, K and V for prefills that are long enough); it decides whether
     # the problem qualifies
     ws, ws_ptr, ws_bytes = None, None, 0
     # (fp32 inputs: only the split-key decode kernel takes a workspace)
