@@ -152,11 +152,15 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(BwdParams p) {
   uint16_t* const lds_v = smem + 2 * kTile * S;  // [2][64][S]
   int32_t* const lds_seg = reinterpret_cast<int32_t*>(smem + 4 * kTile * S);  // [2][64]
 
+  // Workgroup ids are dealt round-robin to the 8 XCDs.  The dense arrays of one (batch, head) are what
+  // workgroups can share, so an XCD owns whole (batch, head) pairs and runs their blocks heaviest first,
+  // the same block of all its pairs side by side: neighbouring blocks of a pair walk the same tiles at
+  // about the same time and find them in that XCD's L2.
   const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
-  const int round = slot / p.H, h = slot % p.H;
-  const int pair = round * 8 + xcd_pair_slot(round, xcd, p.B);
-  if (pair >= p.npairs) return;
-  const int qblk = p.nblk - 1 - pair / p.B, b = pair % p.B;  // heaviest causal blocks first
+  const int per_xcd = (p.B * p.H + 7) / 8;
+  const int bh = (slot % per_xcd) * 8 + xcd;
+  if (bh >= p.B * p.H) return;
+  const int qblk = p.nblk - 1 - slot / per_xcd, b = bh / p.H, h = bh % p.H;  // heaviest causal blocks first
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
   const int lp = l & 15, dhalf = (l >> 4) & 1;
   const int q0 = qblk * kBQ, wrow0 = q0 + kWQ * w;
@@ -344,11 +348,12 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
   float* const lds_ndel = lds_nlse + 2 * kTile;                            // [2][64]  -delta
   int32_t* const lds_seg = reinterpret_cast<int32_t*>(lds_ndel + 2 * kTile);  // [2][64]
 
+  // (batch, head) pairs per XCD, blocks heaviest first: see bwd_dq_kernel
   const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
-  const int round = slot / p.H, h = slot % p.H;
-  const int pair = round * 8 + xcd_pair_slot(round, xcd, p.B);
-  if (pair >= p.npairs) return;
-  const int kblk = pair / p.B, b = pair % p.B;  // under the causal mask the first key blocks are the heaviest
+  const int per_xcd = (p.B * p.H + 7) / 8;
+  const int bh = (slot % per_xcd) * 8 + xcd;
+  if (bh >= p.B * p.H) return;
+  const int kblk = slot / per_xcd, b = bh / p.H, h = bh % p.H;  // under the causal mask the first key blocks are the heaviest
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
   const int lp = l & 15, dhalf = (l >> 4) & 1;
   const int k0 = kblk * kBK, wkey0 = k0 + kWK * w;
@@ -566,7 +571,7 @@ int launch_dq(const BwdParams& base, hipStream_t stream) {
   const size_t smem = (size_t)4 * kTile * tile_stride(D) * 2 + 2 * kTile * 4;
   static bool configured[kMaxDevices] = {};
   if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), smem); rc != TPA_OK) return rc;
-  hipLaunchKernelGGL(kern, dim3(((p.npairs + 7) / 8) * 8 * p.H), dim3(NW * 64), smem, stream, p);
+  hipLaunchKernelGGL(kern, dim3(((p.B * p.H + 7) / 8) * 8 * p.nblk), dim3(NW * 64), smem, stream, p);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
 }
 
@@ -579,7 +584,7 @@ int launch_dkv(const BwdParams& base, hipStream_t stream) {
   const size_t smem = (size_t)4 * kTile * tile_stride(D) * 2 + 6 * kTile * 4;
   static bool configured[kMaxDevices] = {};
   if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), smem); rc != TPA_OK) return rc;
-  hipLaunchKernelGGL(kern, dim3(((p.npairs + 7) / 8) * 8 * p.H), dim3(NW * 64), smem, stream, p);
+  hipLaunchKernelGGL(kern, dim3(((p.B * p.H + 7) / 8) * 8 * p.nblk), dim3(NW * 64), smem, stream, p);
   return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
 }
 

@@ -1188,3 +1188,48 @@ def test_ring_schedule_on_the_references_ring_grid(gpu, batch_size, rank_q, rank
     o_ref, _ = orc.tpa_reference(q, k, v, qseg, kvseg, h, sm_scale=1.0)
     np.testing.assert_array_equal(np.isnan(o_ring), np.isnan(o_ref))
     assert np.nanmax(np.abs(o_ring - o_ref), initial=0.0) <= F32_TOL
+
+
+# ---------------------------------------------------------------- the route through dense Q, K, V, at random
+@pytest.mark.parametrize("seed", range(24))
+def test_random_problems_on_the_dense_route(gpu, prefill_route, seed):
+    """Random prefills with key / value ranks other than 2 and more than one query block: with the workspace
+    they are reconstructed as dense Q, K, V and run the pipelined tile loop, whose entry, exit and per-wave
+    ranges depend on the lengths, the causal diagonal (with a random offset) and ragged per-sequence lengths.
+    Every fourth problem uses the bottom-right alignment over sequences of different lengths."""
+    from tpa import _dispatch as dd
+    from tpa import tpa
+
+    rng = np.random.default_rng(9000 + seed)
+    b = int(rng.integers(1, 4))
+    lq = int(rng.integers(257, 1400))
+    lk = int(rng.integers(200, 1900))
+    h, d = int(rng.integers(1, 4)) * 8, int(rng.choice([64, 128]))
+    rq, rk = int(rng.integers(1, 7)), int(rng.choice([1, 3, 4, 8]))
+    mode = seed % 4  # 0: no mask, 1: top-left causal + offset, 2: causal + offset + lengths, 3: bottom right + lengths
+    q, k, v = make_factors(9100 + seed, b, lq, lk, h, d, d, rq, rk, scale_by_rank=True)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    if prefill_route == "dense":
+        assert dd.load_library().tpa_fwd_workspace_bytes(b, lq, lk, h, d, d, rq, rk) > 0
+    sm_scale = d**-0.5
+    fq, fk, fv = as_f64(tq), as_f64(tk), as_f64(tv)
+    if mode == 0:
+        o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=sm_scale, kernel=2)
+        o_ref, l_ref = orc.tpa_reference(fq, fk, fv, None, None, h, sm_scale=sm_scale)
+    elif mode == 1:
+        offset = int(rng.integers(-200, lk))
+        o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=sm_scale, causal=True, kernel=2, causal_offset=offset)
+        o_ref, l_ref = _offset_reference(fq, fk, fv, h, sm_scale, offset)
+    else:
+        lengths = [int(x) for x in rng.integers(1, lk + 1, b)]
+        lengths[0] = lk
+        kvl = torch.tensor(lengths, dtype=torch.int32, device=gpu)
+        if mode == 2:
+            offset = int(rng.integers(0, lk))
+            o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=sm_scale, causal=True, kernel=2, causal_offset=offset, kv_lengths=kvl)
+            kvseg = (np.arange(lk)[None, :] >= np.asarray(lengths)[:, None]).astype(np.int32)  # padding keys carry id 1
+            o_ref, l_ref = _offset_reference(fq, fk, fv, h, sm_scale, offset, np.zeros((b, lq), np.int32), kvseg)
+        else:
+            o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=sm_scale, causal=tpa.CAUSAL_BOTTOM_RIGHT, kernel=2, kv_lengths=kvl)
+            o_ref, l_ref = _bottom_right_reference(fq, fk, fv, lengths, h, sm_scale, 0)
+    check(o, lse, o_ref, l_ref, BF16_TOL, bf16_bounds(tq, tk, tv, h, sm_scale))
