@@ -523,9 +523,24 @@ int tpa_bwd_t(const TpaBwdArgs* a, hipStream_t stream, bool mfma) {
       else
         hipLaunchKernelGGL((recon_kernel<T, uint16_t>), dim3(L, a->B), dim3(threads), 0, stream, fa, fb, out, L, a->H, D, R);
     };
-    recon16(a->qa, a->qb, q16, a->lq, a->dk, a->rq);
-    recon16(a->ka, a->kb, k16, a->lk, a->dk, a->rk);
-    recon16(a->va, a->vb, v16, a->lk, a->dv, a->rk);
+    // all three in one launch where the vectorised kernel applies (16-byte aligned factors, H % 8 == 0)
+    bool one_launch = sizeof(T) == 2 && a->H % 8 == 0 && a->dk % 8 == 0 && a->dk == a->dv;
+    const TpaFactor* fs[6] = {&a->qa, &a->qb, &a->ka, &a->kb, &a->va, &a->vb};
+    for (const TpaFactor* f : fs)
+      one_launch = one_launch && !(reinterpret_cast<uintptr_t>(f->ptr) & 15) && f->stride_b % 8 == 0 && f->stride_l % 8 == 0 && f->stride_r % 8 == 0;
+    const int lmax = a->lq > a->lk ? a->lq : a->lk;
+    const int64_t blocks = ((int64_t)lmax * (a->dk / 8) * (a->H / 8) + 255) / 256;
+    if (one_launch && blocks <= 2147483647LL) {
+      ReconJobs jobs{};
+      jobs.job[0] = ReconJob{a->qa, a->qb, q16, a->lq, a->rq, 1.f};
+      jobs.job[1] = ReconJob{a->ka, a->kb, k16, a->lk, a->rk, 1.f};
+      jobs.job[2] = ReconJob{a->va, a->vb, v16, a->lk, a->rk, 1.f};
+      hipLaunchKernelGGL(recon_bf16_h8_kernel, dim3((unsigned)blocks, a->B, 3), dim3(256), 0, stream, jobs, a->H, a->dk);
+    } else {
+      recon16(a->qa, a->qb, q16, a->lq, a->dk, a->rq);
+      recon16(a->ka, a->kb, k16, a->lk, a->dk, a->rk);
+      recon16(a->va, a->vb, v16, a->lk, a->dv, a->rk);
+    }
   } else {
     hipLaunchKernelGGL((recon_kernel<T, float>), dim3(a->lq, a->B), dim3(threads), 0, stream, a->qa, a->qb, qd, a->lq, a->H, a->dk, a->rq);
     hipLaunchKernelGGL((recon_kernel<T, float>), dim3(a->lk, a->B), dim3(threads), 0, stream, a->ka, a->kb, kd, a->lk, a->H, a->dk, a->rk);
