@@ -462,9 +462,107 @@ __global__ __launch_bounds__(256) void project_kernel(const float* dx, TpaFactor
   }
 }
 
+// The same projections for bf16 factors with H % 8 == 0 and (D / 8) (H / 8) a power of two up to 64,
+// without LDS: a thread owns the 8 x 8 piece dX[8 hg .. + 7][8 cc .. + 7] of one token (pieces of D
+// are the fastest thread index, so the 16 loads of a piece are coalesced 32-byte runs), multiplies it
+// with its 8 values of b (for da) and of a (for db) rank by rank, and the sums over d and over h are
+// reductions across the lanes that share a token: over the D / 8 neighbouring lanes with DPP adds,
+// over the H / 8 groups above them with lane exchanges.  Several tokens share a wave.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__global__ __launch_bounds__(256) void project_h8_kernel(const float* dx, TpaFactor fa, TpaFactor fb, TpaGrad ga, TpaGrad gb, int L, int H,
+                                                         int D, int R) {
+  const int cpr = D / 8, hgs = H / 8, tt = cpr * hgs;  // threads per token
+  const int64_t gtid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int cc = (int)(gtid % cpr), hg = (int)(gtid / cpr % hgs);
+  const int64_t tok = gtid / tt;
+  const bool live = tok < L;
+  const int64_t t = live ? tok : L - 1;  // lanes past the end idle along: the reductions need whole waves
+  const int b = blockIdx.y;
+  const float* xp = dx + (((int64_t)b * L + t) * H + 8 * hg) * D + 8 * cc;
+  const uint16_t* ap = static_cast<const uint16_t*>(fa.ptr) + b * fa.stride_b + t * fa.stride_l + 8 * hg;
+  const uint16_t* bp = static_cast<const uint16_t*>(fb.ptr) + b * fb.stride_b + t * fb.stride_l + 8 * cc;
+  float x[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const f32x4 lo = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xp + (int64_t)i * D));
+    const f32x4 hi = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xp + (int64_t)i * D + 4));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { x[i][j] = lo[j]; x[i][4 + j] = hi[j]; }
+  }
+  const float inv = 1.f / (float)R;
+  float* oa = ga.ptr + b * ga.stride_b + t * ga.stride_l + 8 * hg;
+  float* ob = gb.ptr + b * gb.stride_b + t * gb.stride_l + 8 * cc;
+  for (int r = 0; r < R; ++r) {
+    const u32x4 av = *reinterpret_cast<const u32x4*>(ap + (int64_t)r * fa.stride_r);
+    const u32x4 bv = *reinterpret_cast<const u32x4*>(bp + (int64_t)r * fb.stride_r);
+    float af[8], bf[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      af[2 * j] = bf16lo_to_f32(av[j]); af[2 * j + 1] = bf16hi_to_f32(av[j]);
+      bf[2 * j] = bf16lo_to_f32(bv[j]); bf[2 * j + 1] = bf16hi_to_f32(bv[j]);
+    }
+    float da[8], db[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc += x[i][j] * bf[j];
+      da[i] = acc;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc += x[i][j] * af[i];
+      db[j] = acc;
+    }
+    // da: sum over the cpr (8 or 16) neighbouring lanes of this (token, head group)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float v = da[i];
+      v = dpp_add<0xB1>(v);   // quad_perm [1, 0, 3, 2]
+      v = dpp_add<0x4E>(v);   // quad_perm [2, 3, 0, 1]
+      v = dpp_add<0x141>(v);  // row_half_mirror: the other quad of the same eight lanes
+      if (cpr == 16) v = dpp_add<0x140>(v);  // row_mirror: the other eight lanes of the row
+      da[i] = v;
+    }
+    // db: sum over the head groups, which lie cpr lanes apart
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float v = db[j];
+      for (int m = cpr; m < tt; m <<= 1) v += __shfl_xor(v, m, 64);
+      db[j] = v;
+    }
+    if (live && cc == 0) {
+      *reinterpret_cast<f32x4*>(oa + (int64_t)r * ga.stride_r) = f32x4{da[0] * inv, da[1] * inv, da[2] * inv, da[3] * inv};
+      *reinterpret_cast<f32x4*>(oa + (int64_t)r * ga.stride_r + 4) = f32x4{da[4] * inv, da[5] * inv, da[6] * inv, da[7] * inv};
+    }
+    if (live && hg == 0) {
+      *reinterpret_cast<f32x4*>(ob + (int64_t)r * gb.stride_r) = f32x4{db[0] * inv, db[1] * inv, db[2] * inv, db[3] * inv};
+      *reinterpret_cast<f32x4*>(ob + (int64_t)r * gb.stride_r + 4) = f32x4{db[4] * inv, db[5] * inv, db[6] * inv, db[7] * inv};
+    }
+  }
+}
+
 template <typename T>
 void launch_project(const float* dx, const TpaFactor& fa, const TpaFactor& fb, const TpaGrad& ga, const TpaGrad& gb, int B, int L,
                     int H, int D, int R, hipStream_t stream) {
+  if constexpr (sizeof(T) == 2) {
+    const int cpr = D / 8, hgs = H / 8, tt = cpr * hgs;
+    auto al16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
+    const bool fast = D % 8 == 0 && H % 8 == 0 && (cpr == 8 || cpr == 16) && tt <= 64 && (tt & (tt - 1)) == 0 && al16(dx) && al16(fa.ptr) &&
+                      al16(fb.ptr) && al16(ga.ptr) && al16(gb.ptr) && fa.stride_b % 8 == 0 && fa.stride_l % 8 == 0 && fa.stride_r % 8 == 0 &&
+                      fb.stride_b % 8 == 0 && fb.stride_l % 8 == 0 && fb.stride_r % 8 == 0 && ga.stride_b % 4 == 0 && ga.stride_l % 4 == 0 &&
+                      ga.stride_r % 4 == 0 && gb.stride_b % 4 == 0 && gb.stride_l % 4 == 0 && gb.stride_r % 4 == 0;
+    const int64_t blocks = ((int64_t)L * tt + 255) / 256;
+    if (fast && blocks <= 2147483647LL) {
+      hipLaunchKernelGGL(project_h8_kernel, dim3((unsigned)blocks, B), dim3(256), 0, stream, dx, fa, fb, ga, gb, L, H, D, R);
+      return;
+    }
+  }
   const size_t smem = ((size_t)H * (D + 4) + (size_t)R * D + (size_t)R * H) * sizeof(float);
   int dsh = 0;
   while ((1 << dsh) < D) ++dsh;

@@ -206,6 +206,12 @@ def _bf16_case(gpu, seed, b, lq, lk, h, d, rq, rk, seg, causal, kernel):
         (1, 700, 333, 2, 128, 2, 1, None),
         (2, 384, 384, 2, 64, 6, 2, 100),     # packed sequences
         (1, 640, 384, 2, 128, 2, 2, 77),     # rows whose segment has no key: no gradient from them
+        # head counts that are multiples of 8: the one-launch reconstruction and the lane-reduction projections
+        (1, 300, 300, 8, 128, 6, 2, None),   # 16 lanes per (token, head group), one group
+        (2, 200, 260, 16, 64, 3, 4, None),   # 8 lanes per group, two groups; lq != lk, ragged token count per wave
+        (1, 130, 131, 32, 128, 2, 2, None),  # four groups: a token fills a wave
+        (1, 100, 100, 64, 64, 2, 1, None),   # eight groups of eight lanes
+        (1, 100, 100, 64, 128, 2, 2, 50),    # more than a wave per token: the staged projection; packed
     ],
 )
 def test_backward_bf16_mfma_kernels(gpu, b, lq, lk, h, d, rq, rk, seg, causal):
