@@ -267,8 +267,11 @@ def run_append(torch, tpa, device, name, steps, warmup):
     caches = [torch.zeros((B, cache_len, rk, inner), dtype=torch.bfloat16, device=device) for inner in (H, D, H, D)]
     lengths = torch.full((B,), cache_len - n - 1, dtype=torch.int32, device=device)
 
+    ws_bytes = tpa.cache_append_workspace_bytes(B, n, dm, H, D, rq, rk)  # decode steps split the contraction over workgroups
+    ws = torch.empty(ws_bytes + 16, dtype=torch.uint8, device=device) if ws_bytes else None
+
     def step(i):
-        tpa.tpa_cache_append(x, w, cos, sin, *caches, lengths, rank_q=rq, kernel=2)
+        tpa.tpa_cache_append(x, w, cos, sin, *caches, lengths, rank_q=rq, kernel=2, workspace=ws)
 
     wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
     fl = 2.0 * B * n * dm * n_out

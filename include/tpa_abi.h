@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define TPA_ABI_VERSION 7
+#define TPA_ABI_VERSION 8
 
 /* element types of the factor / output arrays */
 enum { TPA_DTYPE_F32 = 0, TPA_DTYPE_BF16 = 1 };
@@ -262,13 +262,22 @@ typedef struct TpaAppendArgs {
   int32_t rope_len;           /* rows of the rotary tables: positions are clamped to rope_len - 1 */
   int32_t dtype;              /* TPA_DTYPE_*: element type of x, w, the q outputs and the cache */
   int32_t kernel;             /* TPA_KERNEL_*: the MFMA kernel takes bf16 with d_model % 64 == 0, H % 8 == 0, D % 8 == 0 */
+  void* workspace;            /* optional (NULL: none), 16-byte aligned: see tpa_cache_append_workspace_bytes */
+  size_t workspace_bytes;
 } TpaAppendArgs;
 
 /*
  * Projections to the rank factors, rotary embedding and append to the factored cache (see
- * TpaAppendArgs).  Enqueues one kernel on `stream`; needs no workspace.
+ * TpaAppendArgs).  Enqueues one kernel on `stream` and needs no workspace; a decode step (at most 64
+ * new tokens in all) that brings tpa_cache_append_workspace_bytes(...) bytes runs as two kernels that
+ * split the contraction over more workgroups (fp32 partial sums in the workspace, same results up to
+ * the order of the fp32 additions).
  */
 int tpa_cache_append(const TpaAppendArgs* args, void* stream);
+
+/* Bytes of optional workspace with which tpa_cache_append can split the contraction of a decode step
+   over workgroups, 0 if it would not use one (more than 64 new tokens, dtype or d_model not eligible). */
+size_t tpa_cache_append_workspace_bytes(int32_t B, int32_t n, int32_t d_model, int32_t H, int32_t D, int32_t rq, int32_t rk, int32_t dtype);
 
 /* ABI version of the loaded library (TPA_ABI_VERSION it was built with). */
 int tpa_abi_version(void);

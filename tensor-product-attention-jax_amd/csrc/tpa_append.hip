@@ -33,6 +33,8 @@ struct AppendParams {
   int B, n, K, H, D, rq, rk, cache_len, rope_len;
   int M, N;          // tokens (B * n), output columns
   int seg[7];        // first column of qa, qb, ka, kb, va, vb, and N
+  float* partial;    // decode-step kernel with the contraction split over workgroups: [slabs][kFewTokens][N] fp32
+  int slabs;
 };
 
 // Where chunk (token m, columns c0 .. c0 + 7) of y goes: the factor it belongs to, and the address
@@ -173,71 +175,121 @@ __global__ __launch_bounds__(256) void append_mfma_kernel(AppendParams p) {
   write_new_lengths(p);
 }
 
-// ---- bf16, at most 64 new tokens in all (a decode step): the call is one read of W, so the k
-// dimension is split over the eight waves of a workgroup that owns 16 output columns - enough
-// workgroups to pull W at the rate of the memory system, where 64 x 64 tiles would leave most of the
-// chip idle.  Operands go from global memory straight into v_mfma_f32_16x16x32_bf16 fragments (a lane
-// holds 8 consecutive k of one token / one row of W, which is how both arrays lie in memory); the
-// eight partial tiles meet in LDS and 128 threads finish one chunk of eight columns each.
-constexpr int kFewTokens = 64, kFewCols = 16, kFewWaves = 8;
+// ---- bf16, at most 64 new tokens in all (a decode step): the call is one read of W, and 64 x 64 tiles
+// would leave most of the chip idle.  Operands go from global memory straight into
+// v_mfma_f32_16x16x32_bf16 fragments (a lane holds 8 consecutive k of one token / one row of W, which
+// is how both arrays lie in memory); the eight waves of a workgroup split its share of k, their partial
+// tiles meet in LDS and one thread per chunk of eight columns finishes.
+// What bounds it: a wave ingests fragments as half cache lines (16 rows x 64 bytes per load
+// instruction), about 18 bytes per clock and CU, and every workgroup needs all 64 tokens of x for its
+// share of k.  Without a workspace a workgroup owns 16 columns and all of k (100 workgroups at 1600
+// columns; x alone is 512 KB per workgroup, 14 of the kernel's 22 us at d_model = 4096).  With a
+// workspace the contraction is also split over `slabs` workgroups (blockIdx.y) that own 64 columns
+// each: x is then read once per 64 columns and slab, the fp32 partial tiles go to the workspace and
+// append_finish_kernel adds them up and finishes.
+// U = k steps of 32 whose loads are in flight together, NCB = blocks of 16 columns per workgroup.
+constexpr int kFewTokens = 64, kFewWaves = 8;
+template <int U, int NCB>
 __global__ __launch_bounds__(kFewWaves * 64) void append_fewrows_kernel(AppendParams p) {
-  __shared__ __attribute__((aligned(16))) float part[kFewWaves][kFewTokens][kFewCols + 4];
+  constexpr int kCols = 16 * NCB;
+  extern __shared__ __attribute__((aligned(16))) float part_mem[];  // [kFewWaves][kFewTokens][kCols + 4]
+  auto part = [&](int ww, int m, int c) -> float& { return part_mem[(ww * kFewTokens + m) * (kCols + 4) + c]; };
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, r16 = l & 15, kg = l >> 4;
-  const int n0 = blockIdx.x * kFewCols;
+  const int n0 = blockIdx.x * kCols;
   const uint16_t* x = static_cast<const uint16_t*>(p.x);
   const uint16_t* wt = static_cast<const uint16_t*>(p.w);
-  const int kw = p.K / kFewWaves, k_begin = w * kw;             // this wave's share of the contraction
-  const uint16_t* wrow = wt + (int64_t)min(n0 + r16, p.N - 1) * p.K + k_begin + 8 * kg;
+  const int kw = p.K / (kFewWaves * p.slabs), k_begin = (blockIdx.y * kFewWaves + w) * kw;  // this wave's share of the contraction
+  const uint16_t* wrow[NCB];
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) wrow[cb] = wt + (int64_t)min(n0 + 16 * cb + r16, p.N - 1) * p.K + k_begin + 8 * kg;
   const uint16_t* xrow[4];
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb) xrow[mb] = x + (int64_t)min(16 * mb + r16, p.M - 1) * p.K + k_begin + 8 * kg;
-  const int nblk = (p.M + 15) / 16;                             // blocks of 16 tokens that exist
-  f32x4 acc[4];
-#pragma unroll
-  for (int mb = 0; mb < 4; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
-  constexpr int U = 4;                                          // k steps of 32 whose loads are in flight together
-  for (int k0 = 0; k0 < kw; k0 += 32 * U) {
-    bf16x8 bq[U], a[U][4];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int kk = min(k0 + 32 * u, kw - 32);
-      bq[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wrow + kk));
-#pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
-        if (mb < nblk) a[u][mb] = *reinterpret_cast<const bf16x8*>(xrow[mb] + kk);
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if (k0 + 32 * u >= kw) break;
-#pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
-        if (mb < nblk) acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][mb], bq[u], acc[mb], 0, 0, 0);
-    }
-  }
-  // acc[mb][v] = partial y[token 16 mb + 4 kg + v][column n0 + r16]
+  // (all four blocks of 16 tokens are always computed: rows past the last token repeat it and are dropped
+  // at the end - branches around the loads would keep them from being in flight together)
+  f32x4 acc[4][NCB];
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
-    for (int v = 0; v < 4; ++v) part[w][16 * mb + 4 * kg + v][r16] = acc[mb][v];
+    for (int cb = 0; cb < NCB; ++cb) acc[mb][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < kw; k0 += 32 * U) {
+    bf16x8 bq[U][NCB], a[U][4];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int cb = 0; cb < NCB; ++cb) bq[u][cb] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(wrow[cb] + k0 + 32 * u));
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) a[u][mb] = *reinterpret_cast<const bf16x8*>(xrow[mb] + k0 + 32 * u);
+    }
+    __builtin_amdgcn_sched_barrier(0);  // every load of the group is issued before the first matrix instruction waits
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) acc[mb][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][mb], bq[u][cb], acc[mb][cb], 0, 0, 0);
+  }
+  // acc[mb][cb][v] = partial y[token 16 mb + 4 kg + v][column n0 + 16 cb + r16]
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) part(w, 16 * mb + 4 * kg + v, 16 * cb + r16) = acc[mb][cb][v];
   __syncthreads();
-  if (tid < kFewTokens * (kFewCols / 8)) {
-    const int m = tid >> 1, cc = tid & 1, c0 = n0 + 8 * cc;
-    if (m < p.M && c0 < p.N) {
-      float y[8];
+  for (int idx = tid; idx < kFewTokens * (kCols / 8); idx += kFewWaves * 64) {
+    const int m = idx / (kCols / 8), cc = idx % (kCols / 8), c0 = n0 + 8 * cc;
+    if (m >= p.M || c0 >= p.N) continue;
+    float y[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) y[j] = 0.f;
+    for (int j = 0; j < 8; ++j) y[j] = 0.f;
 #pragma unroll
-      for (int ww = 0; ww < kFewWaves; ++ww) {
-        const f32x4 lo = *reinterpret_cast<const f32x4*>(&part[ww][m][8 * cc]), hi = *reinterpret_cast<const f32x4*>(&part[ww][m][8 * cc + 4]);
+    for (int ww = 0; ww < kFewWaves; ++ww) {
+      const f32x4 lo = *reinterpret_cast<const f32x4*>(&part(ww, m, 8 * cc)), hi = *reinterpret_cast<const f32x4*>(&part(ww, m, 8 * cc + 4));
 #pragma unroll
-        for (int j = 0; j < 4; ++j) { y[j] += lo[j]; y[4 + j] += hi[j]; }
-      }
-      bool rotate; int j0, pos;
-      uint16_t* dst = chunk_destination<uint16_t>(p, m, c0, rotate, j0, pos);
-      if (dst) {
-        if (rotate) rotate_chunk(p, y, pos, j0);
-        store_chunk(dst, y);
-      }
+      for (int j = 0; j < 4; ++j) { y[j] += lo[j]; y[4 + j] += hi[j]; }
+    }
+    if (p.partial) {  // this slab's share of the chunk; append_finish_kernel takes it from there
+      float* dst = p.partial + ((int64_t)blockIdx.y * kFewTokens + m) * p.N + c0;
+      *reinterpret_cast<f32x4*>(dst) = f32x4{y[0], y[1], y[2], y[3]};
+      *reinterpret_cast<f32x4*>(dst + 4) = f32x4{y[4], y[5], y[6], y[7]};
+      continue;
+    }
+    bool rotate; int j0, pos;
+    uint16_t* dst = chunk_destination<uint16_t>(p, m, c0, rotate, j0, pos);
+    if (dst) {
+      if (rotate) rotate_chunk(p, y, pos, j0);
+      store_chunk(dst, y);
+    }
+  }
+  if (!p.partial) write_new_lengths(p);  // (with partial sums the finishing kernel writes them)
+}
+
+// second kernel of the split decode step: eight lanes per chunk of eight columns, one per slab of k; they add
+// their partial sums with three exchanges and the first of them finishes the chunk
+__global__ __launch_bounds__(256) void append_finish_kernel(AppendParams p) {
+  const int idx = (blockIdx.x * 256 + threadIdx.x) >> 3, sl = threadIdx.x & 7, nchunks = p.N / 8;
+  const bool live = idx < p.M * nchunks;
+  const int m = live ? idx / nchunks : 0, c0 = live ? 8 * (idx % nchunks) : 0;
+  float y[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) y[j] = 0.f;
+  if (live && sl < p.slabs) {
+    const float* src = p.partial + ((int64_t)sl * kFewTokens + m) * p.N + c0;
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(src), hi = *reinterpret_cast<const f32x4*>(src + 4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { y[j] = lo[j]; y[4 + j] = hi[j]; }
+  }
+#pragma unroll
+  for (int off = 1; off < 8; off <<= 1)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) y[j] += __shfl_xor(y[j], off);
+  if (live && sl == 0) {
+    bool rotate; int j0, pos;
+    uint16_t* dst = chunk_destination<uint16_t>(p, m, c0, rotate, j0, pos);
+    if (dst) {
+      if (rotate) rotate_chunk(p, y, pos, j0);
+      store_chunk(dst, y);
     }
   }
   write_new_lengths(p);
@@ -272,10 +324,37 @@ __global__ __launch_bounds__(256) void append_generic_kernel(AppendParams p) {
 }
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
+
+// slabs of k that a split decode step uses: as many as 8, each a whole number of k steps per wave
+int few_slabs(int d_model) {
+  for (int sl = 8; sl > 1; sl >>= 1)
+    if (d_model % (32 * kFewWaves * sl) == 0) return sl;
+  return 1;
+}
+
+template <int U, int NCB>
+int launch_fewrows(const AppendParams& p, hipStream_t s) {
+  auto kern = append_fewrows_kernel<U, NCB>;
+  const size_t lds = (size_t)kFewWaves * kFewTokens * (16 * NCB + 4) * sizeof(float);
+  static bool configured[kMaxDevices] = {};
+  if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), lds); rc != TPA_OK) return rc;
+  hipLaunchKernelGGL(kern, dim3((p.N + 16 * NCB - 1) / (16 * NCB), p.slabs), dim3(kFewWaves * 64), lds, s, p);
+  return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
+}
 bool chunk_ok(const TpaFactor& f) { return aligned16(f.ptr) && f.stride_b % 8 == 0 && f.stride_l % 8 == 0 && f.stride_r % 8 == 0; }
 
 }  // namespace
 }  // namespace tpa
+
+extern "C" size_t tpa_cache_append_workspace_bytes(int32_t B, int32_t n, int32_t d_model, int32_t H, int32_t D, int32_t rq, int32_t rk, int32_t dtype) {
+  using namespace tpa;
+  if (B <= 0 || n <= 0 || d_model <= 0 || H <= 0 || D <= 0 || rq <= 0 || rk <= 0 || dtype != TPA_DTYPE_BF16) return 0;
+  if ((int64_t)B * n > kFewTokens || H % 8 != 0 || D % 8 != 0) return 0;
+  const int slabs = few_slabs(d_model);
+  if (slabs == 1) return 0;
+  const int64_t n_out = (int64_t)(rq + 2 * rk) * (H + D);
+  return (size_t)slabs * kFewTokens * n_out * sizeof(float);
+}
 
 extern "C" int tpa_cache_append(const TpaAppendArgs* a, void* stream) {
   using namespace tpa;
@@ -313,7 +392,16 @@ extern "C" int tpa_cache_append(const TpaAppendArgs* a, void* stream) {
   for (const TpaFactor* f : fs) mfma = mfma && chunk_ok(*f);
   if (a->kernel == TPA_KERNEL_MFMA && !mfma) return TPA_ERR_UNSUPPORTED;
   if (mfma && p.M <= kFewTokens && a->d_model % (32 * kFewWaves) == 0) {
-    hipLaunchKernelGGL(append_fewrows_kernel, dim3((p.N + kFewCols - 1) / kFewCols), dim3(kFewWaves * 64), 0, s, p);
+    const size_t need = tpa_cache_append_workspace_bytes(a->B, a->n, a->d_model, a->H, a->D, a->rq, a->rk, a->dtype);
+    const bool split = need && a->workspace && a->workspace_bytes >= need && aligned16(a->workspace);
+    p.slabs = split ? few_slabs(a->d_model) : 1;
+    p.partial = split ? static_cast<float*>(a->workspace) : nullptr;
+    const int steps = a->d_model / (32 * kFewWaves * p.slabs);  // k steps of 32 per wave
+    int rc;
+    if (split) rc = steps % 4 == 0 ? launch_fewrows<4, 4>(p, s) : steps % 2 == 0 ? launch_fewrows<2, 4>(p, s) : launch_fewrows<1, 4>(p, s);
+    else rc = steps % 4 == 0 ? launch_fewrows<4, 1>(p, s) : launch_fewrows<1, 1>(p, s);
+    if (rc != TPA_OK) return rc;
+    if (split) hipLaunchKernelGGL(append_finish_kernel, dim3((p.M * (p.N / 8) * 8 + 255) / 256), dim3(256), 0, s, p);
   } else if (mfma) {
     dim3 grid((p.N + kBN - 1) / kBN, (p.M + kBM - 1) / kBM);
     if (grid.y > 65535) return TPA_ERR_SHAPE;

@@ -22,7 +22,7 @@ KERNEL_AUTO = 0
 KERNEL_GENERIC = 1
 KERNEL_MFMA = 2
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 
 class TpaFactor(ctypes.Structure):
@@ -191,6 +191,8 @@ class TpaAppendArgs(ctypes.Structure):
         ("rope_len", ctypes.c_int32),
         ("dtype", ctypes.c_int32),
         ("kernel", ctypes.c_int32),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_size_t),
     ]
 
 
@@ -231,6 +233,8 @@ def load_library(path: str | None = None) -> ctypes.CDLL:
         lib.mha_fwd.argtypes = [ctypes.POINTER(MhaFwdArgs), ctypes.c_void_p]
         lib.tpa_cache_append.restype = ctypes.c_int
         lib.tpa_cache_append.argtypes = [ctypes.POINTER(TpaAppendArgs), ctypes.c_void_p]
+        lib.tpa_cache_append_workspace_bytes.restype = ctypes.c_size_t
+        lib.tpa_cache_append_workspace_bytes.argtypes = [ctypes.c_int32] * 8
         lib.tpa_decode_workspace_bytes.restype = ctypes.c_size_t
         lib.tpa_decode_workspace_bytes.argtypes = [ctypes.c_int32] * 6
         lib.tpa_decode_default_splits.restype = ctypes.c_int32

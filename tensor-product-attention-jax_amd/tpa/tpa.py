@@ -286,6 +286,8 @@ def tpa_cache_append(
     positions=None,
     page_table=None,
     kernel: int = _d.KERNEL_AUTO,
+    workspace: torch.Tensor | None = None,
+    use_workspace: bool | None = None,
 ):
     """The producer step for `n` new tokens per sequence (an addition: the reference takes the
     factors as given): y = x w^T gives the six rank factors of every token, the B factors of Q and
@@ -295,7 +297,10 @@ def tpa_cache_append(
     x[b, n, d_model]; w[rq*(h+d) + 2*rk*(h+d), d_model] (rows in the order qa, qb, ka, kb, va, vb,
     as torch.nn.Linear keeps its weight); rope_cos, rope_sin[rope_len, d/2] fp32; the cache arrays
     [b, cache_len, rk, h|d], or page pools [pages, page_size, rk, h|d] with `page_table`
-    [b, pages_per_seq]; `positions` [b, n] defaults to kv_lengths[b] + i.
+    [b, pages_per_seq]; `positions` [b, n] defaults to kv_lengths[b] + i.  A decode step (at most 64 new
+    tokens in all) is faster with scratch memory for partial sums: `workspace` (uint8, at least
+    `cache_append_workspace_bytes(...)`; a serving loop passes the same one every step) or, with
+    `use_workspace` (default: the module's `USE_WORKSPACE`), one allocated here.
     Returns (qa[b, n, rq, h], qb[b, n, rq, d], new_kv_lengths[b])."""
     device = _pick_device(x, w, ka, kb, va, vb)
     x, w, ka, kb, va, vb = (_as_device_tensor(t, device) for t in (x, w, ka, kb, va, vb))
@@ -330,6 +335,17 @@ def tpa_cache_append(
     qa = torch.empty((b, n, rq, h), dtype=dtype, device=device)
     qb = torch.empty((b, n, rq, d), dtype=dtype, device=device)
     new_len = torch.empty((b,), dtype=torch.int32, device=device)
+    lib = _d.load_library()
+    ws_ptr, ws_bytes = None, 0
+    if use_workspace is None:
+        use_workspace = USE_WORKSPACE
+    if workspace is None and use_workspace and kernel != _d.KERNEL_GENERIC:
+        need = lib.tpa_cache_append_workspace_bytes(b, n, d_model, h, d, rq, rk, _d.dtype_code(dtype))
+        if need:
+            workspace = torch.empty(need + 16, dtype=torch.uint8, device=device)
+    if workspace is not None:
+        pad = (-workspace.data_ptr()) % 16
+        ws_ptr, ws_bytes = workspace.data_ptr() + pad, workspace.numel() * workspace.element_size() - pad
     args = _d.TpaAppendArgs(
         x=x.data_ptr(), w=w.data_ptr(), rope_cos=cos.data_ptr(), rope_sin=sin.data_ptr(),
         positions=None if pos is None else pos.data_ptr(), kv_lengths=None if kvlen is None else kvlen.data_ptr(),
@@ -337,11 +353,15 @@ def tpa_cache_append(
         qa=_d.factor(qa), qb=_d.factor(qb), ka=_d.factor(ka), kb=_d.factor(kb), va=_d.factor(va), vb=_d.factor(vb),
         page_table=None if pt is None else pt.data_ptr(), page_size=int(page_size), pages_per_seq=int(pages_per_seq),
         B=b, n=n, d_model=d_model, H=h, D=d, rq=rq, rk=rk, cache_len=int(cache_len), rope_len=int(cos.shape[0]),
-        dtype=_d.dtype_code(dtype), kernel=int(kernel),
+        dtype=_d.dtype_code(dtype), kernel=int(kernel), workspace=ws_ptr, workspace_bytes=ws_bytes,
     )
     with torch.cuda.device(device):
-        _d.check("tpa_cache_append", _d.load_library().tpa_cache_append(args, _d.current_stream_ptr(device)))
+        _d.check("tpa_cache_append", lib.tpa_cache_append(args, _d.current_stream_ptr(device)))
     return qa, qb, new_len
+
+
+def cache_append_workspace_bytes(b: int, n: int, d_model: int, h: int, d: int, rq: int, rk: int, dtype=torch.bfloat16) -> int:
+    return int(_d.load_library().tpa_cache_append_workspace_bytes(b, n, d_model, h, d, rq, rk, _d.dtype_code(dtype)))
 
 
 def decode_workspace_bytes(b: int, lq: int, lk: int, h: int, dv: int, num_splits: int = 0) -> int:

@@ -43,15 +43,24 @@ def make_layer(seed, b, n, dm, h, d, rq, rk, dtype, gpu):
         (64, 1, 1024, 32, 128, 6, 2),  # a decode step of 64 sequences: all four blocks of 16 tokens
         (7, 3, 512, 8, 64, 2, 1),      # 21 tokens: the second block of 16 is ragged
         (5, 2, 256, 8, 64, 1, 1),      # 216 output columns: the last workgroup owns half a block of columns
+        (8, 2, 2048, 16, 128, 2, 2),   # with a workspace: 8 slabs of k, one k step per wave
+        (4, 9, 4096, 8, 64, 3, 1),     # 8 slabs, two k steps per wave; 200 columns: the last workgroup owns 8 of its 64
+        (2, 3, 1536, 8, 64, 2, 2),     # 2 slabs, three k steps per wave
     ],
 )
-def test_append_matches_the_oracle(gpu, dtype, kernel, b, n, dm, h, d, rq, rk):
+@pytest.mark.parametrize("use_workspace", [False, True])
+def test_append_matches_the_oracle(gpu, dtype, kernel, b, n, dm, h, d, rq, rk, use_workspace):
+    """With `use_workspace` a decode step whose d_model is a multiple of 512 runs as two kernels (partial sums of
+    2, 4 or 8 slabs of k in the workspace, then a finishing kernel); every other case ignores it."""
     x, w = make_layer(1, b, n, dm, h, d, rq, rk, dtype, gpu)
+    if use_workspace and kernel == 2 and b * n <= 64 and dm % 512 == 0:
+        slabs = next(sl for sl in (8, 4, 2) if dm % (256 * sl) == 0)
+        assert tpa.cache_append_workspace_bytes(b, n, dm, h, d, rq, rk) == slabs * 64 * (rq + 2 * rk) * (h + d) * 4
     cache_len = 96
     cos, sin = rope_tables(256, d)
     lengths = np.array([(7 * i + 3) % (cache_len - n - 1) for i in range(b)], dtype=np.int32)
     caches = [torch.full((b, cache_len, rk, inner), float("nan"), dtype=dtype, device=gpu) for inner in (h, d, h, d)]
-    qa, qb, new_len = tpa.tpa_cache_append(x, w, cos, sin, *caches, lengths, rank_q=rq, kernel=kernel)
+    qa, qb, new_len = tpa.tpa_cache_append(x, w, cos, sin, *caches, lengths, rank_q=rq, kernel=kernel, use_workspace=use_workspace)
     pos = lengths[:, None] + np.arange(n)[None, :]
     want = orc.tpa_append_reference(f64(x), f64(w), cos, sin, pos, h, d, rq, rk)
     rel = 2.0**-8 if dtype == torch.bfloat16 else 1e-5
