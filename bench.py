@@ -458,7 +458,7 @@ def main():
             unit="GB/s" if hbm else "TFLOP/s", ms_per_step=r["wall_ms"],
             roofline=dict(bound="hbm" if hbm else "mfma", achieved=ach, peak=PEAK_HBM_GBS if hbm else PEAK_BF16_TFLOPS,
                           unit="GB/s" if hbm else "TFLOP/s", frac=ach / (PEAK_HBM_GBS if hbm else PEAK_BF16_TFLOPS), traffic=None,
-                          kernel="append_mfma_kernel", ms_per_launch=r["kernel_ms"], ms_per_launch_min=r["kernel_ms_min"],
+                          kernel="append_fewrows_kernel + append_finish_kernel" if hbm else "append_gemm_kernel", ms_per_launch=r["kernel_ms"], ms_per_launch_min=r["kernel_ms_min"],
                           algorithmic_flops_per_launch=r["flops"], algorithmic_bytes_per_launch=r["bytes"]),
             config=dict(workload=f"{args.workload}: TPA cache append", **r["shape"]),
         )

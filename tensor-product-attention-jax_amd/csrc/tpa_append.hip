@@ -4,16 +4,31 @@
 // prefill kernels read.  The reference has no such step (its tests draw the factors at random,
 // tpa/tpa_test.py:86-91); the arithmetic follows arXiv 2501.06425, section 3.
 //
-// bf16: one workgroup computes a 64-token x 64-column tile of y with v_mfma_f32_32x32x16_bf16 (four
-// waves, one 32 x 32 block each; x and W tiles of 64 x 64 double buffered in LDS, the next tiles in
-// registers while the current ones are multiplied), stages the fp32 tile in LDS, and every thread
-// then finishes whole 16-byte chunks of eight columns: a chunk lies inside one rank row of one
-// factor (H and D are multiples of 8), so the rotation partners (2j, 2j+1) are inside it.
+// bf16, three kernels by the number of new tokens: 256 x 256 tiles once they fill the chip (a prefill
+// chunk), 64 x 64 tiles below that, and for a decode step (at most 64 tokens in all) a kernel that
+// splits the contraction instead of the tokens.  All of them compute with v_mfma_f32_*_bf16, stage the
+// fp32 results in LDS, and finish whole 16-byte chunks of eight columns: a chunk lies inside one rank
+// row of one factor (H and D are multiples of 8), so the rotation partners (2j, 2j+1) are inside it.
 // Any other dtype / shape: one thread per chunk of eight columns, fp32 arithmetic.
+#include <type_traits>
+#include <utility>
+
 #include "tpa_common.h"
 
 namespace tpa {
 namespace {
+
+// compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N-1>{})
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+template <int V>
+using IC = std::integral_constant<int, V>;
 
 constexpr int kBM = 64, kBN = 64, kBK = 64;
 constexpr int kXS = kBK + 8;   // LDS row stride of the x / W tiles (elements): 16-byte reads of 32 rows are conflict free
@@ -102,7 +117,8 @@ __device__ __forceinline__ void write_new_lengths(const AppendParams& p) {
     }
 }
 
-// ---- bf16 on the matrix cores
+// ---- bf16, 64 x 64 tiles: four waves, one 32 x 32 block each; x and W tiles of 64 x 64 double buffered in LDS,
+// the next tiles in registers while the current ones are multiplied
 __global__ __launch_bounds__(256) void append_mfma_kernel(AppendParams p) {
   __shared__ __attribute__((aligned(16))) uint16_t xs[2][kBM * kXS];
   __shared__ __attribute__((aligned(16))) uint16_t ws[2][kBN * kXS];
@@ -173,6 +189,217 @@ __global__ __launch_bounds__(256) void append_mfma_kernel(AppendParams p) {
     store_chunk(dst, y);
   }
   write_new_lengths(p);
+}
+
+// ---- bf16, many new tokens (a prefill chunk): 256 tokens x 256 columns of y per workgroup, four waves
+// (one per SIMD, 512 registers each: the 256 accumulators sit in AGPRs).  A wave owns 128 tokens x 128
+// columns = 4 x 4 blocks of v_mfma_f32_32x32x16_bf16, computed transposed (A = rows of W, B = tokens), so
+// that a lane ends up with runs of four consecutive columns of one token.  A k step reads 8 fragments for
+// 16 MFMAs (the 64 x 64 tiles above read 2 for 1, which is what bounds them; eight waves of 64 x 128 read
+// 6 for 8 and measured the same time as this form).  x and W tiles of 256 rows x 64 k are double buffered
+// in LDS (row stride 72 elements), raw buffer loads over the tile's rows only (rows past the end read as
+// zeros and are never stored).
+// One wave per SIMD has nobody to hide behind, so the order inside an iteration is fixed by hand:
+//   k step 0, 1: fragments of the next step requested, 16 MFMAs
+//   k step 2:    fragments of step 3 requested, 16 MFMAs with the stores of the next tile between them
+//   barrier
+//   k step 3:    fragments of the next tile's step 0 requested, 16 MFMAs with the loads of the tile after next
+// Epilogue: each wave stages its fp32 tile through its own quarter of the (now free) buffers, 64 tokens x 64
+// columns at a time, and finishes 16-byte chunks; everything that depends on the token alone (sequence,
+// position, cache row or page) is worked out once per workgroup into a small LDS table, everything that
+// depends on the column alone once per lane and piece.
+// Grid: linear ids are dealt to the 8 XCDs round robin, so the column tiles of one token tile get ids
+// that are 8 apart (same XCD: its L2 serves their x tiles).
+constexpr int kGM = 256, kGN = 256, kGK = 64, kGS = kGK + 8;
+constexpr int kGStage = (kGM + kGN) * kGS;            // elements per buffer
+constexpr int kGCS = 64 + 4;                          // row stride of a wave's staged fp32 piece
+constexpr size_t kGemmLds = 2 * kGStage * sizeof(uint16_t) + kGM * 5 * sizeof(int32_t);
+static_assert(64 * kGCS <= kGStage / 4 && kGStage % 16 == 0, "a wave's staged piece fits its slice");
+__global__ __launch_bounds__(256) void append_gemm_kernel(AppendParams p) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t gsm[];
+  int32_t* const table = reinterpret_cast<int32_t*>(gsm + 2 * kGStage);  // [5][kGM]: pos, b, i, cache row coordinates
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
+  const int wm = w >> 1, wn = w & 1;
+  const int ntn = (p.N + kGN - 1) / kGN, ntm = (p.M + kGM - 1) / kGM;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int tm = (slot / ntn) * 8 + xcd, tn = slot % ntn;
+  if (tm >= ntm) return;  // the grid is rounded up to whole groups of 8 token tiles
+  const int m0 = tm * kGM, n0 = tn * kGN;
+  const uint16_t* x = static_cast<const uint16_t*>(p.x);
+  const uint16_t* wt = static_cast<const uint16_t*>(p.w);
+
+  {  // what the epilogue needs to know about a token (one per thread)
+    const int m = min(m0 + tid, p.M - 1);
+    const int b = m / p.n, ii = m % p.n;
+    const int base_len = p.kvlen ? max(0, min(p.kvlen[b], p.cache_len)) : 0;
+    int pos = p.positions ? p.positions[(int64_t)b * p.n + ii] : base_len + ii;
+    pos = max(0, min(pos, p.rope_len - 1));
+    const int t = base_len + ii;
+    int ra = b, rb = t;
+    if (t >= p.cache_len) { ra = 0; rb = -1; }  // dropped
+    else if (p.page_table) { ra = p.page_table[(int64_t)b * p.pages_per_seq + t / p.page_size]; rb = t % p.page_size; }
+    table[tid] = pos; table[kGM + tid] = b; table[2 * kGM + tid] = ii; table[3 * kGM + tid] = ra; table[4 * kGM + tid] = rb;
+  }
+
+  // loader: thread -> chunk tid & 7 of rows (tid >> 3) + 32 q of x and of W
+  const int lrow = tid >> 3, lc = tid & 7;
+  constexpr int kRsrcFlags = 0x00020000;  // raw 32-bit data format
+  const __amdgpu_buffer_rsrc_t x_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(x + (int64_t)m0 * p.K), 0, min(kGM, p.M - m0) * p.K * 2, kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t w_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(wt + (int64_t)n0 * p.K), 0, min(kGN, p.N - n0) * p.K * 2, kRsrcFlags);
+  const int voff = (lrow * p.K + 8 * lc) * 2;
+  const int nk = p.K / kGK;
+  u32x4 xr[8], wr[8];
+  auto load = [&](int kt) __attribute__((always_inline)) {  // (tiles past the last repeat it: loaded, stored, never read)
+    const int k0 = min(kt, nk - 1) * kGK;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      xr[q] = __builtin_amdgcn_raw_buffer_load_b128(x_rs, voff, (32 * q * p.K + k0) * 2, 0);
+      wr[q] = __builtin_amdgcn_raw_buffer_load_b128(w_rs, voff, (32 * q * p.K + k0) * 2, 0);
+    }
+  };
+  auto stage = [&](int buf) __attribute__((always_inline)) {
+    uint16_t* xs = gsm + buf * kGStage + lrow * kGS + 8 * lc;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      *reinterpret_cast<u32x4*>(xs + 32 * q * kGS) = xr[q];
+      *reinterpret_cast<u32x4*>(xs + (kGM + 32 * q) * kGS) = wr[q];
+    }
+  };
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int cb = 0; cb < 4; ++cb)
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[cb][tb][v] = 0.f;
+  // (a wave whose columns all lie past the end multiplies zeros: with one wave per SIMD nobody would use the time)
+  bf16x8 fa[2][4], fb[2][4];
+  const int frag_x = (128 * wm + i) * kGS + 8 * g, frag_w = (kGM + 128 * wn + i) * kGS + 8 * g;
+  auto read_frags = [&](auto slot_c, int buf, auto ks_c) __attribute__((always_inline)) {
+    constexpr int sl = decltype(slot_c)::value, ks = decltype(ks_c)::value;
+    const uint16_t* base = gsm + buf * kGStage + 16 * ks;
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) fa[sl][cb] = *reinterpret_cast<const bf16x8*>(base + frag_w + 32 * cb * kGS);
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb) fb[sl][tb] = *reinterpret_cast<const bf16x8*>(base + frag_x + 32 * tb * kGS);
+  };
+  // acc[cb][tb][v] = y[token 128 wm + 32 tb + i][column 128 wn + 32 cb + 8 (v / 4) + 4 g + v % 4]
+  auto mfmas = [&](auto slot_c) __attribute__((always_inline)) {
+    constexpr int sl = decltype(slot_c)::value;
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb)
+#pragma unroll
+      for (int tb = 0; tb < 4; ++tb) acc[cb][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[sl][cb], fb[sl][tb], acc[cb][tb], 0, 0, 0);
+  };
+  load(0);
+  stage(0);
+  load(1);
+  __syncthreads();
+  read_frags(IC<0>{}, 0, IC<0>{});
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1, nxt = cur ^ 1;
+    read_frags(IC<1>{}, cur, IC<1>{});
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas(IC<0>{});
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(IC<0>{}, cur, IC<2>{});
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas(IC<1>{});
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(IC<1>{}, cur, IC<3>{});
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas(IC<0>{});
+    stage(nxt);
+#pragma unroll
+    for (int n = 0; n < 16; ++n) {  // one tile store behind every MFMA
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    read_frags(IC<0>{}, nxt, IC<0>{});
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas(IC<1>{});
+    load(kt + 2);
+#pragma unroll
+    for (int n = 0; n < 16; ++n) {  // one tile load behind every MFMA
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  __syncthreads();  // every wave has left the loop: the buffers are free
+
+  // ---- epilogue: pieces of 64 tokens x 64 columns through this wave's quarter of the buffers
+  float* const cs = reinterpret_cast<float*>(gsm) + w * (kGStage / 4);
+  const int cc = l & 7, trow = l >> 3;
+#pragma unroll
+  for (int ch = 0; ch < 2; ++ch) {
+    const int c0 = n0 + 128 * wn + 64 * ch + 8 * cc;
+    const bool col_ok = c0 < p.N;
+    // the column's side of the address: factor, rank row, element
+    int f = 0;
+#pragma unroll
+    for (int k = 1; k < 6; ++k) f += c0 >= p.seg[k];
+    const int width = (f & 1) ? p.D : p.H;
+    const int local = c0 - p.seg[f], r = local / width, e = local % width;
+    const bool rotate = f == 1 || f == 3;
+    auto pick = [&](auto get) __attribute__((always_inline)) {
+      return f == 0 ? get(p.qa) : f == 1 ? get(p.qb) : f == 2 ? get(p.ka) : f == 3 ? get(p.kb) : f == 4 ? get(p.va) : get(p.vb);
+    };
+    uint16_t* const base = static_cast<uint16_t*>(const_cast<void*>(pick([](const TpaFactor& t) { return t.ptr; }))) +
+                           (int64_t)r * pick([](const TpaFactor& t) { return t.stride_r; }) + e;
+    const int64_t sb = pick([](const TpaFactor& t) { return t.stride_b; });
+    const int64_t sl = pick([](const TpaFactor& t) { return t.stride_l; });
+    const int half_d = p.D / 2;
+#pragma unroll
+    for (int th = 0; th < 2; ++th) {
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int cq = 0; cq < 2; ++cq)
+#pragma unroll
+        for (int tq = 0; tq < 2; ++tq)
+#pragma unroll
+          for (int vq = 0; vq < 4; ++vq) {
+            const f32x16& t = acc[2 * ch + cq][2 * th + tq];
+            *reinterpret_cast<f32x4*>(cs + (32 * tq + i) * kGCS + 32 * cq + 8 * vq + 4 * g) = f32x4{t[4 * vq], t[4 * vq + 1], t[4 * vq + 2], t[4 * vq + 3]};
+          }
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own writes have landed
+      __builtin_amdgcn_wave_barrier();
+      if (!col_ok) continue;
+      // everything a pass fetches from memory first (row coordinates, angles), then the arithmetic and the stores
+      int64_t off[8];
+      f32x4 c4[8], s4[8];
+#pragma unroll
+      for (int pass = 0; pass < 8; ++pass) {
+        const int tl = 128 * wm + 64 * th + 8 * pass + trow;  // token within the workgroup's tile
+        const int ra = f < 2 ? table[kGM + tl] : table[3 * kGM + tl], rb = f < 2 ? table[2 * kGM + tl] : table[4 * kGM + tl];
+        off[pass] = m0 + tl < p.M && rb >= 0 ? ra * sb + rb * sl : -1;
+        if (rotate) {
+          const int64_t at = (int64_t)table[tl] * half_d + (e >> 1);
+          c4[pass] = *reinterpret_cast<const f32x4*>(p.cosv + at);
+          s4[pass] = *reinterpret_cast<const f32x4*>(p.sinv + at);
+        }
+      }
+#pragma unroll
+      for (int pass = 0; pass < 8; ++pass) {
+        if (off[pass] < 0) continue;
+        const float* src = cs + (8 * pass + trow) * kGCS + 8 * cc;
+        const f32x4 lo = *reinterpret_cast<const f32x4*>(src), hi = *reinterpret_cast<const f32x4*>(src + 4);
+        float y[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        if (rotate) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float a0 = y[2 * j], b0 = y[2 * j + 1];
+            y[2 * j] = a0 * c4[pass][j] - b0 * s4[pass][j];
+            y[2 * j + 1] = b0 * c4[pass][j] + a0 * s4[pass][j];
+          }
+        }
+        store_chunk(base + off[pass], y);
+      }
+    }
+  }
+  if (blockIdx.x == 0) write_new_lengths(p);
 }
 
 // ---- bf16, at most 64 new tokens in all (a decode step): the call is one read of W, and 64 x 64 tiles
@@ -325,6 +552,13 @@ __global__ __launch_bounds__(256) void append_generic_kernel(AppendParams p) {
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
 
+// 256 x 256 tiles pay once they fill the chip (256 CUs, one workgroup each); the rotation tables must allow
+// 16-byte reads of four angles
+bool gemm_tiles_pay(const AppendParams& p, const TpaAppendArgs* a) {
+  const int64_t tiles = (int64_t)((p.M + kGM - 1) / kGM) * ((p.N + kGN - 1) / kGN);
+  return tiles >= 192 && tiles < (1 << 28) && p.D % 8 == 0 && aligned16(a->rope_cos) && aligned16(a->rope_sin);
+}
+
 // slabs of k that a split decode step uses: as many as 8, each a whole number of k steps per wave
 int few_slabs(int d_model) {
   for (int sl = 8; sl > 1; sl >>= 1)
@@ -402,6 +636,11 @@ extern "C" int tpa_cache_append(const TpaAppendArgs* a, void* stream) {
     else rc = steps % 4 == 0 ? launch_fewrows<4, 1>(p, s) : launch_fewrows<1, 1>(p, s);
     if (rc != TPA_OK) return rc;
     if (split) hipLaunchKernelGGL(append_finish_kernel, dim3((p.M * (p.N / 8) * 8 + 255) / 256), dim3(256), 0, s, p);
+  } else if (mfma && gemm_tiles_pay(p, a)) {
+    const int ntn = (p.N + kGN - 1) / kGN, ntm = (p.M + kGM - 1) / kGM;
+    static bool configured[kMaxDevices] = {};
+    if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(append_gemm_kernel), kGemmLds); rc != TPA_OK) return rc;
+    hipLaunchKernelGGL(append_gemm_kernel, dim3((ntm + 7) / 8 * 8 * ntn), dim3(256), kGemmLds, s, p);
   } else if (mfma) {
     dim3 grid((p.N + kBN - 1) / kBN, (p.M + kBM - 1) / kBM);
     if (grid.y > 65535) return TPA_ERR_SHAPE;

@@ -156,3 +156,46 @@ def test_append_contiguous_and_paged_caches_hold_the_same_rows(gpu):
     for c, p_ in zip(cont, pool):
         gathered = p_[table.long()].reshape(b, cache_len, rk, -1)  # [b, pages, page_size, rk, x] -> [b, cache_len, rk, x]
         assert torch.equal(gathered, c)
+
+
+@pytest.mark.parametrize(
+    "b,n,dm,h,d,rq,rk",
+    [
+        (3, 2731, 128, 32, 128, 6, 2),  # 8193 tokens: the last token tile holds one; 1600 columns: the last column tile a quarter
+        (2, 4900, 64, 32, 96, 6, 2),    # 1280 columns = five whole column tiles; one k step
+        (5, 2000, 192, 16, 128, 7, 1),  # 1296 columns: rank rows and factors change inside a wave's 64-column pieces
+    ],
+)
+@pytest.mark.parametrize("paged", [False, True])
+def test_prefill_chunks_take_the_large_tiles(gpu, b, n, dm, h, d, rq, rk, paged):
+    """Enough new tokens to fill the chip with 256 x 256 tiles (the kernel a prefill chunk gets): every output
+    against the oracle, ragged last tiles in both directions, tokens past the capacity dropped, contiguous
+    and paged caches, explicit positions."""
+    x, w = make_layer(11, b, n, dm, h, d, rq, rk, torch.bfloat16, gpu)
+    page_size = 64
+    cache_len = (n + 5 + page_size - 1) // page_size * page_size
+    cos, sin = rope_tables(cache_len + 7, d)
+    lengths = np.array([(3 * i) % 7 for i in range(b)], dtype=np.int32)
+    lengths[-1] = cache_len - n + 2  # the last two tokens of the last sequence do not fit
+    rng = np.random.default_rng(12)
+    pos = (lengths[:, None] + np.arange(n)[None, :] + rng.integers(0, 3, size=(b, 1))).astype(np.int32)
+    if paged:
+        pages_per_seq = cache_len // page_size
+        table = torch.from_numpy(rng.permutation(b * pages_per_seq).astype(np.int32)).reshape(b, pages_per_seq).to(gpu)
+        caches = [torch.full((b * pages_per_seq, page_size, rk, inner), float("nan"), dtype=torch.bfloat16, device=gpu) for inner in (h, d, h, d)]
+    else:
+        table = None
+        caches = [torch.full((b, cache_len, rk, inner), float("nan"), dtype=torch.bfloat16, device=gpu) for inner in (h, d, h, d)]
+    qa, qb, new_len = tpa.tpa_cache_append(x, w, cos, sin, *caches, lengths, rank_q=rq, positions=pos, page_table=table, kernel=2)
+    want = orc.tpa_append_reference(f64(x), f64(w), cos, sin, np.minimum(pos, cos.shape[0] - 1), h, d, rq, rk)
+    rel = 2.0**-8
+    for name, got in (("qa", qa), ("qb", qb)):
+        assert np.abs(f64(got) - want[name]).max() <= rel * np.abs(want[name]).max(), name
+    for name, cache in zip(("ka", "kb", "va", "vb"), caches):
+        c = f64(cache[table.long()].reshape(b, cache_len, rk, -1) if paged else cache)
+        for bi in range(b):
+            fits = min(n, cache_len - lengths[bi])
+            rows = c[bi, lengths[bi] : lengths[bi] + fits]
+            assert np.abs(rows - want[name][bi, :fits]).max() <= rel * np.abs(want[name]).max(), (name, bi)
+            assert np.isnan(c[bi, : lengths[bi]]).all() and np.isnan(c[bi, lengths[bi] + fits :]).all(), (name, bi)
+    assert new_len.cpu().tolist() == [min(int(l) + n, cache_len) for l in lengths]
