@@ -71,6 +71,25 @@ COPY_BYTES = 1 << 30  # --workload copy: bytes read (and bytes written) by each 
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "prefill_c2_decode_c4_hbm_bytes.txt")
 
 
+def mfma_sustained_rate():
+    """TFLOP/s that back-to-back bf16 MFMAs on N(0, 1) operands sustain on this device, all CUs busy, nothing
+    else running: the stand-alone yardstick built beside the library (csrc/mfma_rate.hip), run as a child
+    process.  The published peak stays the roofline's `peak`; this says how much of it the matrix cores
+    deliver on non-zero data under the device's power limit.  None if the program is missing or fails."""
+    import subprocess
+
+    exe = os.path.join(ROOT, "tensor-product-attention-jax_amd", "lib", "mfma_rate")
+    if not os.access(exe, os.X_OK):
+        log(f"[bench] {exe} not built: no sustained MFMA rate")
+        return None
+    try:
+        out = subprocess.run([exe, "2", "0", "256", "8192"], capture_output=True, text=True, timeout=120, check=True).stdout
+        return float(json.loads(out.strip().splitlines()[-1])["tflops"])
+    except Exception as e:  # a yardstick, not part of the measurement
+        log(f"[bench] mfma_rate failed: {e}")
+        return None
+
+
 def measured_traffic(workload):
     """HBM bytes per launch of the workload's kernels, read from the committed rocprofv3 counter summary
     (FETCH_SIZE / WRITE_SIZE in KiB per dispatch, one table row per kernel), each counter scaled by what it
@@ -492,6 +511,14 @@ def main():
             config=dict(workload=f"{args.workload}: TPA decode over the factored KV cache" +
                         (", fp32 cache" if args.workload in F32_WORKLOADS else ""), **d["shape"]),
         )
+    roof = result.get("roofline", {})
+    if roof.get("bound") == "mfma" and args.workload not in F32_WORKLOADS:
+        rate = mfma_sustained_rate()
+        if rate:
+            log(f"[bench] back-to-back bf16 MFMAs on N(0,1) operands sustain {rate:.0f} TFLOP/s on this device ({rate / PEAK_BF16_TFLOPS:.2f} of the published peak)")
+            roof["mfma_sustained"] = dict(value=rate, unit="TFLOP/s", frac_of_peak=rate / PEAK_BF16_TFLOPS,
+                                          achieved_over_sustained=roof["achieved"] / rate,
+                                          how="mfma_rate 2 0 256 8192: 8 independent v_mfma_f32_32x32x16_bf16 chains per wave, 2 waves per SIMD, 256 workgroups, no memory traffic")
     result.update(
         n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True, scaling="weak",
         vs_baseline=None, dtype="f32" if args.workload in F32_WORKLOADS else "bf16", data="synthetic",
