@@ -90,6 +90,34 @@ def mfma_sustained_rate():
         return None
 
 
+def hbm_sustained_rates():
+    """GB/s that a plain read (16-byte non-temporal loads) and a plain copy of 2 GiB buffers sustain on this device:
+    the stand-alone yardstick built beside the library (csrc/hbm_rate.hip), run as a child process.  None if the
+    program is missing or fails."""
+    import subprocess
+
+    exe = os.path.join(ROOT, "tensor-product-attention-jax_amd", "lib", "hbm_rate")
+    if not os.access(exe, os.X_OK):
+        log(f"[bench] {exe} not built: no sustained HBM rates")
+        return None
+    try:
+        out = subprocess.run([exe, "2048"], capture_output=True, text=True, timeout=120, check=True).stdout
+        line = json.loads(out.strip().splitlines()[-1])
+        return float(line["read_gbs"]), float(line["copy_gbs"])
+    except Exception as e:  # a yardstick, not part of the measurement
+        log(f"[bench] hbm_rate failed: {e}")
+        return None
+
+
+def add_hbm_sustained(roof):
+    rates = hbm_sustained_rates()
+    if rates:
+        log(f"[bench] a plain read sustains {rates[0]:.0f} GB/s on this device, a plain copy {rates[1]:.0f} GB/s (read + written)")
+        roof["hbm_sustained"] = dict(read=rates[0], copy=rates[1], unit="GB/s", frac_of_peak_read=rates[0] / PEAK_HBM_GBS,
+                                     achieved_over_sustained_read=roof["achieved"] / rates[0],
+                                     how="hbm_rate 2048: 2 GiB buffers, 16-byte loads (non-temporal for the read), 2 in flight per lane, 768 workgroups of 256")
+
+
 def measured_traffic(workload):
     """HBM bytes per launch of the workload's kernels, read from the committed rocprofv3 counter summary
     (FETCH_SIZE / WRITE_SIZE in KiB per dispatch, one table row per kernel), each counter scaled by what it
@@ -422,6 +450,7 @@ def main():
                               algorithmic_bytes_per_launch=d["bytes"]),
                 config=dict(workload="c4: TPA decode over the factored KV cache", **d["shape"]),
             )
+            add_hbm_sustained(result["decode"]["roofline"])
             log("[bench] dense decode at the c4 shape")
             from tpa import mha
 
@@ -512,6 +541,8 @@ def main():
                         (", fp32 cache" if args.workload in F32_WORKLOADS else ""), **d["shape"]),
         )
     roof = result.get("roofline", {})
+    if roof.get("bound") == "hbm" and kind == "decode":
+        add_hbm_sustained(roof)
     if roof.get("bound") == "mfma" and args.workload not in F32_WORKLOADS:
         rate = mfma_sustained_rate()
         if rate:
