@@ -75,9 +75,13 @@ ffi::Error fill(TpaFwdArgs* a, const ffi::AnyBuffer& q, const ffi::AnyBuffer& k,
 
 // workspace: an extra u8 result of max(tpa_fwd_workspace_bytes(...), 1) bytes allocated by XLA (256-byte aligned,
 // as XLA's buffers are), with which tpa_fwd picks the split-key decode kernel or the dense-K/V route where
-// they are faster; a one-byte buffer keeps every call on the fused prefill kernel
-void attach_workspace(TpaFwdArgs* a, ffi::Result<ffi::AnyBuffer>& workspace) {
-  const size_t need = tpa_fwd_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dk, a->dv, a->rq, a->rk);
+// they are faster; a one-byte buffer keeps every call on the fused prefill kernel.  `nomat` is the reference's
+// static of that name (tpa/tpa.py:250): the evaluation order that never forms K or V, which needs the
+// workspace of tpa_fwd_nomat_workspace_bytes(...) instead.
+void attach_workspace(TpaFwdArgs* a, ffi::Result<ffi::AnyBuffer>& workspace, bool nomat) {
+  a->nomat = nomat ? 1 : 0;
+  const size_t need = nomat ? tpa_fwd_nomat_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dk, a->dv, a->rq, a->rk)
+                            : tpa_fwd_workspace_bytes(a->B, a->lq, a->lk, a->H, a->dk, a->dv, a->rq, a->rk);
   if (need && workspace->size_bytes() >= need) {
     a->workspace = workspace->untyped_data();
     a->workspace_bytes = workspace->size_bytes();
@@ -91,10 +95,10 @@ bool seg_ok(const ffi::Buffer<ffi::DataType::S32>& ids, int64_t b, int64_t l) {
 
 ffi::Error TpaFwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v,
                       ffi::Result<ffi::AnyBuffer> o, ffi::Result<ffi::AnyBuffer> lse,
-                      ffi::Result<ffi::AnyBuffer> workspace, int32_t num_heads, float sm_scale, bool causal) {
+                      ffi::Result<ffi::AnyBuffer> workspace, int32_t num_heads, float sm_scale, bool causal, bool nomat) {
   TpaFwdArgs a;
   if (ffi::Error e = fill(&a, q, k, v, o, lse, num_heads, sm_scale, causal); e.failure()) return e;
-  attach_workspace(&a, workspace);
+  attach_workspace(&a, workspace, nomat);
   const int rc = tpa_fwd(&a, stream);
   return rc == TPA_OK ? ffi::Error::Success() : fail(rc);
 }
@@ -102,12 +106,12 @@ ffi::Error TpaFwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ff
 ffi::Error TpaFwdSegImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v,
                          ffi::Buffer<ffi::DataType::S32> q_segment_ids, ffi::Buffer<ffi::DataType::S32> kv_segment_ids,
                          ffi::Result<ffi::AnyBuffer> o, ffi::Result<ffi::AnyBuffer> lse,
-                         ffi::Result<ffi::AnyBuffer> workspace, int32_t num_heads, float sm_scale, bool causal) {
+                         ffi::Result<ffi::AnyBuffer> workspace, int32_t num_heads, float sm_scale, bool causal, bool nomat) {
   TpaFwdArgs a;
   if (ffi::Error e = fill(&a, q, k, v, o, lse, num_heads, sm_scale, causal); e.failure()) return e;
   if (!seg_ok(q_segment_ids, a.B, a.lq) || !seg_ok(kv_segment_ids, a.B, a.lk))
     return ffi::Error::InvalidArgument("segment ids must be s32 [b, lq] and [b, lk]");
-  attach_workspace(&a, workspace);
+  attach_workspace(&a, workspace, nomat);
   a.q_segment_ids = q_segment_ids.typed_data();
   a.kv_segment_ids = kv_segment_ids.typed_data();
   const int rc = tpa_fwd(&a, stream);
@@ -241,7 +245,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(TpaFwd, TpaFwdImpl,
                                   .Ctx<ffi::PlatformStream<hipStream_t>>()
                                   .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
                                   .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
-                                  .Attr<int32_t>("num_heads").Attr<float>("sm_scale").Attr<bool>("causal"));
+                                  .Attr<int32_t>("num_heads").Attr<float>("sm_scale").Attr<bool>("causal").Attr<bool>("nomat"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(TpaFwdSeg, TpaFwdSegImpl,
                               ffi::Ffi::Bind()
@@ -249,7 +253,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(TpaFwdSeg, TpaFwdSegImpl,
                                   .Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>().Arg<ffi::AnyBuffer>()
                                   .Arg<ffi::Buffer<ffi::DataType::S32>>().Arg<ffi::Buffer<ffi::DataType::S32>>()
                                   .Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>().Ret<ffi::AnyBuffer>()
-                                  .Attr<int32_t>("num_heads").Attr<float>("sm_scale").Attr<bool>("causal"));
+                                  .Attr<int32_t>("num_heads").Attr<float>("sm_scale").Attr<bool>("causal").Attr<bool>("nomat"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(TpaDecode, TpaDecodeImpl,
                               ffi::Ffi::Bind()
