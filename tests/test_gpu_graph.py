@@ -1,87 +1,70 @@
-"""The library's launches inside a captured HIP graph (what a serving loop does with the decode
-step): the C ABI only enqueues kernels on the stream it is given - no allocation, no memset, no
-synchronisation - so a capture records them, and every replay must equal the eager call on the
-inputs of that moment.  Replays alternate with eager work and synchronisations.
-"""
+"""The entry points only enqueue kernels on the caller's stream (no allocation, no synchronisation, no memset), so a
+caller may record them into a HIP graph: prefill, decode and the producer step captured once and replayed, with
+eager work and synchronisations between the replays, give the eager results bit for bit every time."""
 
-import numpy as np
 import pytest
 import torch
 
 from conftest import make_factors
+from test_gpu_parity import split, to_gpu
 
 pytestmark = pytest.mark.gpu
 
 
-def _capture(gpu, fn):
-    """Warm up on a side stream (first-use set-up of the kernels happens outside the capture), then capture fn."""
-    side = torch.cuda.Stream(device=gpu)
-    side.wait_stream(torch.cuda.current_stream(gpu))
-    with torch.cuda.stream(side):
-        fn()
-    torch.cuda.current_stream(gpu).wait_stream(side)
-    torch.cuda.synchronize(gpu)
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        out = fn()
-    return graph, out
-
-
-def _same(x, y):
-    return torch.equal(torch.nan_to_num(x.float(), nan=7.0), torch.nan_to_num(y.float(), nan=7.0))
-
-
-@pytest.mark.parametrize("lq,causal", [(1, False), (4, 2)])
-def test_decode_replays_in_a_graph(gpu, lq, causal):
+@pytest.mark.parametrize("rk", [2, 4])  # rank 4: the prefill goes through dense Q, K, V (two launches)
+def test_prefill_decode_and_append_replay_from_a_graph(gpu, rk):
     from tpa import tpa
 
-    b, lk, h, d, rq, rk = 4, 2048, 16, 128, 6, 2
-    q, k, v = make_factors(170, b, lq, lk, h, d, d, rq, rk, scale_by_rank=True)
-    bf = lambda x: torch.from_numpy(x).to(gpu).to(torch.bfloat16)
-    tq, tk, tv = bf(q), bf(k), bf(v)
-    ops = [t.contiguous() for x in (tq, tk, tv) for t in (x[..., :h], x[..., h:])]
-    lengths = torch.tensor([lk, 1500, 700, 64], dtype=torch.int32, device=gpu)
-    ws = torch.empty(tpa.decode_workspace_bytes(b, lq, lk, h, d) + 256, dtype=torch.uint8, device=gpu)
-    call = lambda: tpa.tpa_decode(*ops, sm_scale=d**-0.5, workspace=ws, kernel=2, kv_lengths=lengths, causal=causal)
-    graph, (o_g, lse_g) = _capture(gpu, call)
-    gen = torch.Generator(device=gpu)
-    gen.manual_seed(171)
-    for rep in range(4):
-        # the serving loop's own work between replays: new queries, one more token in every cache
-        ops[0].copy_(torch.randn(ops[0].shape, generator=gen, device=gpu))
-        ops[1].copy_(torch.randn(ops[1].shape, generator=gen, device=gpu))
-        lengths.add_(torch.tensor([0, 1, 1, 1], dtype=torch.int32, device=gpu))
+    b, t, h, d, rq = 2, 640, 8, 128, 6
+    q, k, v = make_factors(3, b, t, t, h, d, d, rq, rk, scale_by_rank=True)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    qa, qb, ka, kb, va, vb = split(tq, tk, tv, h)
+    scale = d**-0.5
+    # decode: the last token of q against all keys; producer step: four new tokens per sequence into a cache
+    dq = (qa[:, -1:].contiguous(), qb[:, -1:].contiguous())
+    lk_dec = 2048
+    _, kd, vd = make_factors(4, b, 1, lk_dec, h, d, d, rq, rk, scale_by_rank=True)
+    dk_, dv_ = (to_gpu(x, torch.bfloat16, gpu) for x in (kd, vd))
+    dka, dkb, dva, dvb = dk_[..., :h].contiguous(), dk_[..., h:].contiguous(), dv_[..., :h].contiguous(), dv_[..., h:].contiguous()
+    ws = torch.empty(max(tpa.decode_workspace_bytes(b, 1, lk_dec, h, d), 16), dtype=torch.uint8, device=gpu)
+    dm, n_new, cache_len = 256, 4, 64
+    g = torch.Generator(device=gpu)
+    g.manual_seed(5)
+    x = torch.randn((b, n_new, dm), generator=g, device=gpu).to(torch.bfloat16)
+    w = (torch.randn(((rq + 2 * rk) * (h + d), dm), generator=g, device=gpu) / dm**0.5).to(torch.bfloat16)
+    ang = torch.arange(cache_len, device=gpu, dtype=torch.float32)[:, None] * (10000.0 ** (-torch.arange(0, d, 2, device=gpu, dtype=torch.float32) / d))[None]
+    cos, sin = torch.cos(ang).contiguous(), torch.sin(ang).contiguous()
+    lengths = torch.tensor([3, 17], dtype=torch.int32, device=gpu)
+
+    def work(caches):
+        o, lse = tpa.tpa_factors(qa, qb, ka, kb, va, vb, sm_scale=scale, causal=True, kernel=2)
+        od, lsed = tpa.tpa_decode(*dq, dka, dkb, dva, dvb, sm_scale=scale, workspace=ws, kernel=2)
+        aq, bq, new_len = tpa.tpa_cache_append(x, w, cos, sin, *caches, lengths, rank_q=rq, kernel=2)
+        return o, lse, od, lsed, aq, bq, new_len
+
+    new_caches = lambda: [torch.zeros((b, cache_len, rk, inner), dtype=torch.bfloat16, device=gpu) for inner in (h, d, h, d)]
+    eager_caches = new_caches()
+    eager = work(eager_caches)
+    torch.cuda.synchronize()
+
+    graph_caches = new_caches()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        work(graph_caches)  # warm up on the capture stream (library set-up, allocator)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            captured = work(graph_caches)
+    torch.cuda.synchronize()
+    for replay in range(3):
+        for c in graph_caches:
+            c.fill_(float("nan"))  # eager work between the replays; every replay has to write the rows again
+        torch.cuda.synchronize()
         graph.replay()
-        torch.cuda.synchronize(gpu)
-        o_e, lse_e = call()
-        torch.cuda.synchronize(gpu)
-        assert _same(o_g, o_e) and torch.equal(lse_g, lse_e), rep
-
-
-def test_prefill_and_backward_replay_in_a_graph(gpu):
-    from tpa import tpa
-
-    b, t, h, d = 2, 512, 4, 128
-    q, k, v = make_factors(172, b, t, t, h, d, d, 6, 2, scale_by_rank=True)
-    bf = lambda x: torch.from_numpy(x).to(gpu).to(torch.bfloat16)
-    ops = [p.contiguous() for x in (bf(q), bf(k), bf(v)) for p in (x[..., :h], x[..., h:])]
-    do = torch.randn((b, t, h, d), device=gpu).to(torch.bfloat16)
-    bws = torch.empty(tpa.bwd_workspace_bytes(b, t, t, h, d, d) + 256, dtype=torch.uint8, device=gpu)
-
-    def call():
-        o, lse = tpa.tpa_factors(*ops, sm_scale=d**-0.5, causal=True, kernel=2)
-        grads = tpa.tpa_factors_bwd(*ops, None, None, o, lse, do, d**-0.5, True, workspace=bws, kernel=2)
-        return (o, lse) + tuple(grads)
-
-    graph, outs_g = _capture(gpu, call)
-    gen = torch.Generator(device=gpu)
-    gen.manual_seed(173)
-    for rep in range(3):
-        for x in ops:
-            x.copy_(torch.randn(x.shape, generator=gen, device=gpu) * 0.5)
-        graph.replay()
-        torch.cuda.synchronize(gpu)
-        outs_e = call()
-        torch.cuda.synchronize(gpu)
-        for g_, e_ in zip(outs_g, outs_e):
-            assert _same(g_, e_), rep
+        torch.cuda.synchronize()
+        for name, got, want in zip(("o", "lse", "o_decode", "lse_decode", "qa", "qb", "new_lengths"), captured, eager):
+            assert torch.equal(got, want), (replay, name)
+        for got, want in zip(graph_caches, eager_caches):
+            for bi in range(b):
+                lo = int(lengths[bi])
+                assert torch.equal(got[bi, lo : lo + n_new], want[bi, lo : lo + n_new]), replay
