@@ -24,7 +24,8 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points():
     names = declared_functions()
     for f in ("tpa_fwd", "tpa_decode", "mha_fwd", "tpa_decode_workspace_bytes", "tpa_strerror", "tpa_abi_version",
-              "tpa_bwd", "mha_bwd", "tpa_bwd_workspace_bytes", "mha_bwd_workspace_bytes"):
+              "tpa_bwd", "mha_bwd", "tpa_bwd_workspace_bytes", "mha_bwd_workspace_bytes", "tpa_cache_append",
+              "tpa_cache_append_workspace_bytes", "tpa_fwd_nomat_workspace_bytes", "tpa_decode_noalloc"):
         assert f in names, names
 
 
@@ -64,6 +65,8 @@ def test_struct_layout_matches_the_c_compiler(tmp_path):
 
 
 def test_size_queries_need_no_gpu():
+    import torch
+
     from tpa import _dispatch
 
     lib = _dispatch.load_library()
@@ -87,6 +90,18 @@ def test_size_queries_need_no_gpu():
     assert lib.mha_bwd_workspace_bytes(2, 10, 7, 3, 5, 6, 0) == r(nd)
     assert lib.mha_bwd_workspace_bytes(2, 10, 7, 3, 5, 6, 1) == r(nd) + r(nq) + r(nk) + r(nv)
     assert lib.tpa_bwd_workspace_bytes(2, 0, 7, 3, 5, 6) == 0
+    # producer step: partial sums of a decode step whose contraction is split over 2, 4 or 8 slabs of d_model
+    bf16, f32 = _dispatch.dtype_code(torch.bfloat16), _dispatch.dtype_code(torch.float32)
+    n_out = (6 + 2 * 2) * (32 + 128)
+    assert lib.tpa_cache_append_workspace_bytes(64, 1, 4096, 32, 128, 6, 2, bf16) == 8 * 64 * n_out * 4
+    assert lib.tpa_cache_append_workspace_bytes(8, 2, 1024, 32, 128, 6, 2, bf16) == 4 * 64 * n_out * 4
+    assert lib.tpa_cache_append_workspace_bytes(8, 2, 1536, 32, 128, 6, 2, bf16) == 2 * 64 * n_out * 4
+    assert lib.tpa_cache_append_workspace_bytes(8, 2, 256, 32, 128, 6, 2, bf16) == 0    # d_model too short to split
+    assert lib.tpa_cache_append_workspace_bytes(65, 1, 4096, 32, 128, 6, 2, bf16) == 0  # more than 64 new tokens
+    assert lib.tpa_cache_append_workspace_bytes(64, 1, 4096, 32, 128, 6, 2, f32) == 0
+    # nomat: the split-key kernels' partials for one window of 64 query rows
+    assert lib.tpa_fwd_nomat_workspace_bytes(2, 200, 4096, 8, 64, 64, 6, 2) == lib.tpa_decode_workspace_bytes(2, 64, 4096, 8, 64, 0)
+    assert lib.tpa_fwd_nomat_workspace_bytes(2, 200, 4096, 2, 3, 5, 6, 2) == 0
 
 
 def test_null_and_shape_errors_are_reported_before_any_launch():
