@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2u|c3|c3u|c4|c4pg|c4s|c5|c5u|c2n|c5n|c2f|c3f|c2fb|c4f|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|ap1|ap2|copy] [--no-cpu] [--no-decode] [--no-backward]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2u|c3|c3u|c4|c4pg|c4s|c5|c5u|c2n|c5n|c2f|c3f|c2fb|c4f|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|ap1|ap2|ap3|copy] [--no-cpu] [--no-decode] [--no-backward]
 
 A step is one forward pass over one batch of synthetic, seeded inputs that are resident in HBM
 before the timed region starts.  The default workload is the prefill configuration the headline
@@ -64,6 +64,7 @@ WORKLOADS = {
     # one decode step of the c4 batch, and a prefill chunk of 4096 tokens for four sequences
     "ap1": ("append", 64, 1, 8192, 32, 128, 6, 2, False),
     "ap2": ("append", 4, 4096, 8192, 32, 128, 6, 2, False),
+    "ap3": ("append", 4, 512, 8192, 32, 128, 6, 2, False),     # a chunk of 2048 tokens: 128 x 128 tiles
 }
 F32_WORKLOADS = ("c2f", "c3f", "c2fb", "c4f")
 COPY_BYTES = 1 << 30  # --workload copy: bytes read (and bytes written) by each plain copy launch
@@ -506,7 +507,7 @@ def main():
             unit="GB/s" if hbm else "TFLOP/s", ms_per_step=r["wall_ms"],
             roofline=dict(bound="hbm" if hbm else "mfma", achieved=ach, peak=PEAK_HBM_GBS if hbm else PEAK_BF16_TFLOPS,
                           unit="GB/s" if hbm else "TFLOP/s", frac=ach / (PEAK_HBM_GBS if hbm else PEAK_BF16_TFLOPS), traffic=None,
-                          kernel="append_fewrows_kernel + append_finish_kernel" if hbm else "append_gemm_kernel", ms_per_launch=r["kernel_ms"], ms_per_launch_min=r["kernel_ms_min"],
+                          kernel="append_fewrows_kernel + append_finish_kernel" if hbm else ("append_gemm_kernel<2>" if args.workload == "ap3" else "append_gemm_kernel<4>"), ms_per_launch=r["kernel_ms"], ms_per_launch_min=r["kernel_ms_min"],
                           algorithmic_flops_per_launch=r["flops"], algorithmic_bytes_per_launch=r["bytes"]),
             config=dict(workload=f"{args.workload}: TPA cache append", **r["shape"]),
         )

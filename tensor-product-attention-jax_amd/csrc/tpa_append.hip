@@ -210,12 +210,21 @@ __global__ __launch_bounds__(256) void append_mfma_kernel(AppendParams p) {
 // depends on the column alone once per lane and piece.
 // Grid: linear ids are dealt to the 8 XCDs round robin, so the column tiles of one token tile get ids
 // that are 8 apart (same XCD: its L2 serves their x tiles).
-constexpr int kGM = 256, kGN = 256, kGK = 64, kGS = kGK + 8;
-constexpr int kGStage = (kGM + kGN) * kGS;            // elements per buffer
+// WB = blocks of 32 per wave and dimension: 4 (the tile described above) or 2 (128 x 128 tiles, a wave owns
+// 64 x 64, 4 fragment reads per 4 MFMAs, two workgroups per CU) for chunks too small to fill the chip with the large tiles.
+constexpr int kGK = 64, kGS = kGK + 8;
 constexpr int kGCS = 64 + 4;                          // row stride of a wave's staged fp32 piece
-constexpr size_t kGemmLds = 2 * kGStage * sizeof(uint16_t) + kGM * 5 * sizeof(int32_t);
-static_assert(64 * kGCS <= kGStage / 4 && kGStage % 16 == 0, "a wave's staged piece fits its slice");
+template <int WB>
+struct GemmTile {
+  static constexpr int kM = 64 * WB, kN = 64 * WB;    // tokens, columns per workgroup
+  static constexpr int kStage = (kM + kN) * kGS;      // elements per buffer
+  static constexpr size_t kLds = 2 * kStage * sizeof(uint16_t) + kM * 5 * sizeof(int32_t);
+  static_assert(64 * kGCS <= kStage / 4 && kStage % 16 == 0, "a wave's staged piece fits its slice");
+};
+template <int WB>
 __global__ __launch_bounds__(256) void append_gemm_kernel(AppendParams p) {
+  constexpr int kGM = GemmTile<WB>::kM, kGN = GemmTile<WB>::kN, kGStage = GemmTile<WB>::kStage;
+  constexpr int kWT = 32 * WB;                        // tokens / columns per wave
   extern __shared__ __attribute__((aligned(16))) uint16_t gsm[];
   int32_t* const table = reinterpret_cast<int32_t*>(gsm + 2 * kGStage);  // [5][kGM]: pos, b, i, cache row coordinates
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
@@ -228,7 +237,7 @@ __global__ __launch_bounds__(256) void append_gemm_kernel(AppendParams p) {
   const uint16_t* x = static_cast<const uint16_t*>(p.x);
   const uint16_t* wt = static_cast<const uint16_t*>(p.w);
 
-  {  // what the epilogue needs to know about a token (one per thread)
+  if (tid < kGM) {  // what the epilogue needs to know about a token (one per thread)
     const int m = min(m0 + tid, p.M - 1);
     const int b = m / p.n, ii = m % p.n;
     const int base_len = p.kvlen ? max(0, min(p.kvlen[b], p.cache_len)) : 0;
@@ -248,11 +257,12 @@ __global__ __launch_bounds__(256) void append_gemm_kernel(AppendParams p) {
   const __amdgpu_buffer_rsrc_t w_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(wt + (int64_t)n0 * p.K), 0, min(kGN, p.N - n0) * p.K * 2, kRsrcFlags);
   const int voff = (lrow * p.K + 8 * lc) * 2;
   const int nk = p.K / kGK;
-  u32x4 xr[8], wr[8];
+  constexpr int NLD = 2 * WB;  // 16-byte chunks of x and of W per thread and tile
+  u32x4 xr[NLD], wr[NLD];
   auto load = [&](int kt) __attribute__((always_inline)) {  // (tiles past the last repeat it: loaded, stored, never read)
     const int k0 = min(kt, nk - 1) * kGK;
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
+    for (int q = 0; q < NLD; ++q) {
       xr[q] = __builtin_amdgcn_raw_buffer_load_b128(x_rs, voff, (32 * q * p.K + k0) * 2, 0);
       wr[q] = __builtin_amdgcn_raw_buffer_load_b128(w_rs, voff, (32 * q * p.K + k0) * 2, 0);
     }
@@ -260,36 +270,36 @@ __global__ __launch_bounds__(256) void append_gemm_kernel(AppendParams p) {
   auto stage = [&](int buf) __attribute__((always_inline)) {
     uint16_t* xs = gsm + buf * kGStage + lrow * kGS + 8 * lc;
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
+    for (int q = 0; q < NLD; ++q) {
       *reinterpret_cast<u32x4*>(xs + 32 * q * kGS) = xr[q];
       *reinterpret_cast<u32x4*>(xs + (kGM + 32 * q) * kGS) = wr[q];
     }
   };
-  f32x16 acc[4][4];
+  f32x16 acc[WB][WB];
 #pragma unroll
-  for (int cb = 0; cb < 4; ++cb)
+  for (int cb = 0; cb < WB; ++cb)
 #pragma unroll
-    for (int tb = 0; tb < 4; ++tb)
+    for (int tb = 0; tb < WB; ++tb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[cb][tb][v] = 0.f;
   // (a wave whose columns all lie past the end multiplies zeros: with one wave per SIMD nobody would use the time)
-  bf16x8 fa[2][4], fb[2][4];
-  const int frag_x = (128 * wm + i) * kGS + 8 * g, frag_w = (kGM + 128 * wn + i) * kGS + 8 * g;
+  bf16x8 fa[2][WB], fb[2][WB];
+  const int frag_x = (kWT * wm + i) * kGS + 8 * g, frag_w = (kGM + kWT * wn + i) * kGS + 8 * g;
   auto read_frags = [&](auto slot_c, int buf, auto ks_c) __attribute__((always_inline)) {
     constexpr int sl = decltype(slot_c)::value, ks = decltype(ks_c)::value;
     const uint16_t* base = gsm + buf * kGStage + 16 * ks;
 #pragma unroll
-    for (int cb = 0; cb < 4; ++cb) fa[sl][cb] = *reinterpret_cast<const bf16x8*>(base + frag_w + 32 * cb * kGS);
+    for (int cb = 0; cb < WB; ++cb) fa[sl][cb] = *reinterpret_cast<const bf16x8*>(base + frag_w + 32 * cb * kGS);
 #pragma unroll
-    for (int tb = 0; tb < 4; ++tb) fb[sl][tb] = *reinterpret_cast<const bf16x8*>(base + frag_x + 32 * tb * kGS);
+    for (int tb = 0; tb < WB; ++tb) fb[sl][tb] = *reinterpret_cast<const bf16x8*>(base + frag_x + 32 * tb * kGS);
   };
-  // acc[cb][tb][v] = y[token 128 wm + 32 tb + i][column 128 wn + 32 cb + 8 (v / 4) + 4 g + v % 4]
+  // acc[cb][tb][v] = y[token kWT wm + 32 tb + i][column kWT wn + 32 cb + 8 (v / 4) + 4 g + v % 4]
   auto mfmas = [&](auto slot_c) __attribute__((always_inline)) {
     constexpr int sl = decltype(slot_c)::value;
 #pragma unroll
-    for (int cb = 0; cb < 4; ++cb)
+    for (int cb = 0; cb < WB; ++cb)
 #pragma unroll
-      for (int tb = 0; tb < 4; ++tb) acc[cb][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[sl][cb], fb[sl][tb], acc[cb][tb], 0, 0, 0);
+      for (int tb = 0; tb < WB; ++tb) acc[cb][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[sl][cb], fb[sl][tb], acc[cb][tb], 0, 0, 0);
   };
   load(0);
   stage(0);
@@ -311,9 +321,9 @@ __global__ __launch_bounds__(256) void append_gemm_kernel(AppendParams p) {
     mfmas(IC<0>{});
     stage(nxt);
 #pragma unroll
-    for (int n = 0; n < 16; ++n) {  // one tile store behind every MFMA
+    for (int n = 0; n < WB * WB; ++n) {  // the tile stores spread behind the MFMAs
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x200, 2 * NLD / (WB * WB), 0);
     }
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
@@ -322,9 +332,9 @@ __global__ __launch_bounds__(256) void append_gemm_kernel(AppendParams p) {
     mfmas(IC<1>{});
     load(kt + 2);
 #pragma unroll
-    for (int n = 0; n < 16; ++n) {  // one tile load behind every MFMA
+    for (int n = 0; n < WB * WB; ++n) {  // the tile loads spread behind the MFMAs
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 2 * NLD / (WB * WB), 0);
     }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -334,8 +344,8 @@ __global__ __launch_bounds__(256) void append_gemm_kernel(AppendParams p) {
   float* const cs = reinterpret_cast<float*>(gsm) + w * (kGStage / 4);
   const int cc = l & 7, trow = l >> 3;
 #pragma unroll
-  for (int ch = 0; ch < 2; ++ch) {
-    const int c0 = n0 + 128 * wn + 64 * ch + 8 * cc;
+  for (int ch = 0; ch < WB / 2; ++ch) {
+    const int c0 = n0 + kWT * wn + 64 * ch + 8 * cc;
     const bool col_ok = c0 < p.N;
     // the column's side of the address: factor, rank row, element
     int f = 0;
@@ -353,7 +363,7 @@ __global__ __launch_bounds__(256) void append_gemm_kernel(AppendParams p) {
     const int64_t sl = pick([](const TpaFactor& t) { return t.stride_l; });
     const int half_d = p.D / 2;
 #pragma unroll
-    for (int th = 0; th < 2; ++th) {
+    for (int th = 0; th < WB / 2; ++th) {
       __builtin_amdgcn_wave_barrier();
 #pragma unroll
       for (int cq = 0; cq < 2; ++cq)
@@ -372,7 +382,7 @@ __global__ __launch_bounds__(256) void append_gemm_kernel(AppendParams p) {
       f32x4 c4[8], s4[8];
 #pragma unroll
       for (int pass = 0; pass < 8; ++pass) {
-        const int tl = 128 * wm + 64 * th + 8 * pass + trow;  // token within the workgroup's tile
+        const int tl = kWT * wm + 64 * th + 8 * pass + trow;  // token within the workgroup's tile
         const int ra = f < 2 ? table[kGM + tl] : table[3 * kGM + tl], rb = f < 2 ? table[2 * kGM + tl] : table[4 * kGM + tl];
         off[pass] = m0 + tl < p.M && rb >= 0 ? ra * sb + rb * sl : -1;
         if (rotate) {
@@ -552,11 +562,24 @@ __global__ __launch_bounds__(256) void append_generic_kernel(AppendParams p) {
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
 
-// 256 x 256 tiles pay once they fill the chip (256 CUs, one workgroup each); the rotation tables must allow
-// 16-byte reads of four angles
+// 256 x 256 tiles (WB = 4) pay once they fill three quarters of the chip (256 CUs, one workgroup each), 128 x 128
+// tiles (WB = 2) from half of it; the rotation tables must allow 16-byte reads of four angles
+template <int WB>
 bool gemm_tiles_pay(const AppendParams& p, const TpaAppendArgs* a) {
-  const int64_t tiles = (int64_t)((p.M + kGM - 1) / kGM) * ((p.N + kGN - 1) / kGN);
-  return tiles >= 192 && tiles < (1 << 28) && p.D % 8 == 0 && aligned16(a->rope_cos) && aligned16(a->rope_sin);
+  constexpr int kM = GemmTile<WB>::kM, kN = GemmTile<WB>::kN;
+  const int64_t tiles = (int64_t)((p.M + kM - 1) / kM) * ((p.N + kN - 1) / kN);
+  return tiles >= (WB == 4 ? 192 : 128) && tiles < (1 << 28) && p.D % 8 == 0 && aligned16(a->rope_cos) && aligned16(a->rope_sin);
+}
+
+template <int WB>
+int launch_gemm(const AppendParams& p, hipStream_t s) {
+  constexpr int kM = GemmTile<WB>::kM, kN = GemmTile<WB>::kN;
+  const int ntn = (p.N + kN - 1) / kN, ntm = (p.M + kM - 1) / kM;
+  auto kern = append_gemm_kernel<WB>;
+  static bool configured[kMaxDevices] = {};
+  if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), GemmTile<WB>::kLds); rc != TPA_OK) return rc;
+  hipLaunchKernelGGL(kern, dim3((ntm + 7) / 8 * 8 * ntn), dim3(256), GemmTile<WB>::kLds, s, p);
+  return hipGetLastError() == hipSuccess ? TPA_OK : TPA_ERR_LAUNCH;
 }
 
 // slabs of k that a split decode step uses: as many as 8, each a whole number of k steps per wave
@@ -636,11 +659,10 @@ extern "C" int tpa_cache_append(const TpaAppendArgs* a, void* stream) {
     else rc = steps % 4 == 0 ? launch_fewrows<4, 1>(p, s) : launch_fewrows<1, 1>(p, s);
     if (rc != TPA_OK) return rc;
     if (split) hipLaunchKernelGGL(append_finish_kernel, dim3((p.M * (p.N / 8) * 8 + 255) / 256), dim3(256), 0, s, p);
-  } else if (mfma && gemm_tiles_pay(p, a)) {
-    const int ntn = (p.N + kGN - 1) / kGN, ntm = (p.M + kGM - 1) / kGM;
-    static bool configured[kMaxDevices] = {};
-    if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(append_gemm_kernel), kGemmLds); rc != TPA_OK) return rc;
-    hipLaunchKernelGGL(append_gemm_kernel, dim3((ntm + 7) / 8 * 8 * ntn), dim3(256), kGemmLds, s, p);
+  } else if (mfma && gemm_tiles_pay<4>(p, a)) {
+    if (int rc = launch_gemm<4>(p, s); rc != TPA_OK) return rc;
+  } else if (mfma && gemm_tiles_pay<2>(p, a)) {
+    if (int rc = launch_gemm<2>(p, s); rc != TPA_OK) return rc;
   } else if (mfma) {
     dim3 grid((p.N + kBN - 1) / kBN, (p.M + kBM - 1) / kBM);
     if (grid.y > 65535) return TPA_ERR_SHAPE;

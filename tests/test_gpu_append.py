@@ -164,11 +164,13 @@ def test_append_contiguous_and_paged_caches_hold_the_same_rows(gpu):
         (3, 2731, 128, 32, 128, 6, 2),  # 8193 tokens: the last token tile holds one; 1600 columns: the last column tile a quarter
         (2, 4900, 64, 32, 96, 6, 2),    # 1280 columns = five whole column tiles; one k step
         (5, 2000, 192, 16, 128, 7, 1),  # 1296 columns: rank rows and factors change inside a wave's 64-column pieces
+        (2, 1025, 128, 32, 128, 6, 2),  # 2050 tokens: too few for the 256 x 256 tiles, enough for the 128 x 128 ones
+        (3, 700, 64, 16, 128, 6, 2),    # 128 x 128 tiles: 1440 columns (the last tile a quarter), one k step
     ],
 )
 @pytest.mark.parametrize("paged", [False, True])
 def test_prefill_chunks_take_the_large_tiles(gpu, b, n, dm, h, d, rq, rk, paged):
-    """Enough new tokens to fill the chip with 256 x 256 tiles (the kernel a prefill chunk gets): every output
+    """Enough new tokens to fill the chip with 256 x 256 or 128 x 128 tiles (the kernels a prefill chunk gets): every output
     against the oracle, ragged last tiles in both directions, tokens past the capacity dropped, contiguous
     and paged caches, explicit positions."""
     x, w = make_layer(11, b, n, dm, h, d, rq, rk, torch.bfloat16, gpu)
