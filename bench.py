@@ -175,10 +175,28 @@ def decode_bytes(B, lq, lk, H, D, rq, rk, elem=2):
     return cache + qf + out
 
 
-def time_steps(torch, fn, steps, warmup):
-    """Returns (wall ms per step over the whole timed region, mean ms per launch from events)."""
-    for _ in range(warmup):
-        fn(0)
+PREHEAT_S = 0.4  # seconds of the step itself, untimed, before the counted warm-up (see time_steps)
+
+
+def time_steps(torch, fn, steps, warmup, preheat_s=None):
+    """Times `steps` calls of fn after `warmup` untimed ones.  Returns a dict: wall ms per step over the
+    whole timed region, and mean / median / min ms per step from events on the launch stream.
+
+    Before the counted warm-up the step is repeated for `preheat_s` seconds (untimed, reported): the first
+    workload of a process otherwise meets a device that has not settled yet - lazily loaded code objects,
+    first-touch page mappings of fresh allocations, and a clock that the power management has not yet
+    brought to what it holds under this load - and a few warm-up steps of 0.3 ms do not cover that."""
+    preheat_s = PREHEAT_S if preheat_s is None else preheat_s
+    t0 = time.perf_counter()
+    n_pre = 0
+    while time.perf_counter() - t0 < preheat_s:
+        for _ in range(8):
+            fn(n_pre)
+            n_pre += 1
+        torch.cuda.synchronize()
+    pre_ms = (time.perf_counter() - t0) * 1e3
+    for i in range(warmup):
+        fn(i)
     torch.cuda.synchronize()
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
@@ -190,7 +208,17 @@ def time_steps(torch, fn, steps, warmup):
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     ev = [s.elapsed_time(e) for s, e in zip(starts, ends)]
-    return wall_ms, sum(ev) / len(ev), min(ev)
+    srt = sorted(ev)
+    med = srt[len(srt) // 2] if len(srt) % 2 else 0.5 * (srt[len(srt) // 2 - 1] + srt[len(srt) // 2])
+    log("[bench]   per-step event ms: " + " ".join(f"{x:.4f}" for x in ev))
+    return dict(wall_ms=wall_ms, kernel_ms=sum(ev) / len(ev), kernel_ms_median=med, kernel_ms_min=srt[0],
+                preheat=dict(seconds=pre_ms / 1e3, steps=n_pre))
+
+
+def launch_times(r):
+    """event times per step for a roofline object: mean (what `achieved` is computed from), median, fastest"""
+    return dict(ms_per_launch=r["kernel_ms"], ms_per_launch_median=r["kernel_ms_median"], ms_per_launch_min=r["kernel_ms_min"],
+                preheat=r["preheat"])
 
 
 def run_prefill(torch, tpa, device, name, steps, warmup):
@@ -209,11 +237,12 @@ def run_prefill(torch, tpa, device, name, steps, warmup):
     def step(i):
         out["o"], out["lse"] = tpa.tpa_factors(*x, seg, seg, sm_scale=scale, causal=causal, kernel=2, use_workspace=use_ws, nomat=nomat)
 
-    wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
+    t = time_steps(torch, step, steps, warmup)
+    wall_ms, ev_ms, ev_min, ev_med = t["wall_ms"], t["kernel_ms"], t["kernel_ms_min"], t["kernel_ms_median"]
     # packed: only pairs inside a document count
     fl = prefill_flops(B * (lq // doc), doc, doc, H, D, causal) if doc else prefill_flops(B, lq, lk, H, D, causal)
     return dict(
-        wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, flops=fl,
+        wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, kernel_ms_median=ev_med, preheat=t["preheat"], flops=fl,
         tflops_wall=fl / wall_ms / 1e9, tflops_kernel=fl / ev_ms / 1e9,
         shape=dict(B=B, lq=lq, lk=lk, H=H, D=D, rank_q=rq, rank_k=rk, causal=causal, **({"document_len": doc} if doc else {})),
         inputs=x, out=out,
@@ -232,10 +261,11 @@ def run_dense_prefill(torch, mha, device, name, steps, warmup):
     def step(i):
         mha._mha_fwd(q, k, v, None, scale, causal=causal, kernel=2)
 
-    wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
+    t = time_steps(torch, step, steps, warmup)
+    wall_ms, ev_ms, ev_min, ev_med = t["wall_ms"], t["kernel_ms"], t["kernel_ms_min"], t["kernel_ms_median"]
     fl = prefill_flops(B, lq, lk, H, D, causal)
     return dict(
-        wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, flops=fl,
+        wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, kernel_ms_median=ev_med, preheat=t["preheat"], flops=fl,
         tflops_wall=fl / wall_ms / 1e9, tflops_kernel=fl / ev_ms / 1e9,
         shape=dict(B=B, lq=lq, lk=lk, H=H, D=D, causal=causal),
     )
@@ -260,11 +290,12 @@ def run_backward(torch, tpa, device, name, steps, warmup):
     def step(i):
         tpa.tpa_factors_bwd(*x, seg, seg, o, lse, do, scale, causal, grads=grads, workspace=ws, kernel=2)
 
-    wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
+    t = time_steps(torch, step, steps, warmup)
+    wall_ms, ev_ms, ev_min, ev_med = t["wall_ms"], t["kernel_ms"], t["kernel_ms_min"], t["kernel_ms_median"]
     # five contractions against the forward's two; packed: only pairs inside a document count
     fl = 2.5 * (prefill_flops(B * (lq // doc), doc, doc, H, D, causal) if doc else prefill_flops(B, lq, lk, H, D, causal))
     return dict(
-        wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, flops=fl,
+        wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, kernel_ms_median=ev_med, preheat=t["preheat"], flops=fl,
         tflops_wall=fl / wall_ms / 1e9, tflops_kernel=fl / ev_ms / 1e9,
         shape=dict(B=B, lq=lq, lk=lk, H=H, D=D, rank_q=rq, rank_k=rk, causal=causal, **({"document_len": doc} if doc else {})),
     )
@@ -291,10 +322,11 @@ def run_decode(torch, tpa, device, name, steps, warmup):
     def step(i):
         out["o"], out["lse"] = tpa.tpa_decode(*xs[i & 1], sm_scale=scale, workspace=ws, kernel=2, page_table=table, causal=causal)
 
-    wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
+    t = time_steps(torch, step, steps, warmup)
+    wall_ms, ev_ms, ev_min, ev_med = t["wall_ms"], t["kernel_ms"], t["kernel_ms_min"], t["kernel_ms_median"]
     nbytes = decode_bytes(B, lq, lk, H, D, rq, rk, elem=4 if f32 else 2)
     return dict(
-        wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, bytes=nbytes,
+        wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, kernel_ms_median=ev_med, preheat=t["preheat"], bytes=nbytes,
         gbs_wall=nbytes / wall_ms / 1e6, gbs_kernel=nbytes / ev_ms / 1e6,
         shape=dict(B=B, lq=lq, lk=lk, H=H, D=D, rank_q=rq, rank_k=rk), inputs=xs[0], out=out,
     )
@@ -321,10 +353,11 @@ def run_append(torch, tpa, device, name, steps, warmup):
     def step(i):
         tpa.tpa_cache_append(x, w, cos, sin, *caches, lengths, rank_q=rq, kernel=2, workspace=ws)
 
-    wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
+    t = time_steps(torch, step, steps, warmup)
+    wall_ms, ev_ms, ev_min, ev_med = t["wall_ms"], t["kernel_ms"], t["kernel_ms_min"], t["kernel_ms_median"]
     fl = 2.0 * B * n * dm * n_out
     nbytes = (B * n * dm + n_out * dm + B * n * n_out) * 2
-    return dict(wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, flops=fl, bytes=nbytes,
+    return dict(wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, kernel_ms_median=ev_med, preheat=t["preheat"], flops=fl, bytes=nbytes,
                 shape=dict(B=B, new_tokens=n, d_model=dm, H=H, D=D, rank_q=rq, rank_k=rk, outputs=n_out))
 
 
@@ -345,9 +378,10 @@ def run_dense_decode(torch, mha, device, name, steps, warmup):
         k, v = kvs[i & 1]
         mha._mha_fwd(q, k, v, None, scale, kernel=2)
 
-    wall_ms, ev_ms, ev_min = time_steps(torch, step, steps, warmup)
+    t = time_steps(torch, step, steps, warmup)
+    wall_ms, ev_ms, ev_min, ev_med = t["wall_ms"], t["kernel_ms"], t["kernel_ms_min"], t["kernel_ms_median"]
     nbytes = 2 * B * lk * H * D * 2 + B * lq * H * D * 2 * 2 + B * H * lq * 4
-    return dict(wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, bytes=nbytes, gbs_kernel=nbytes / ev_ms / 1e6)
+    return dict(wall_ms=wall_ms, kernel_ms=ev_ms, kernel_ms_min=ev_min, kernel_ms_median=ev_med, preheat=t["preheat"], bytes=nbytes, gbs_kernel=nbytes / ev_ms / 1e6)
 
 
 def cpu_baseline_prefill(torch, inputs, shape, budget_s=12.0):
@@ -389,18 +423,22 @@ def cpu_baseline_prefill(torch, inputs, shape, budget_s=12.0):
 
 
 def main():
+    global PREHEAT_S
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["copy"],
                     help="copy = a plain device copy of known size, the yardstick for the HBM byte counters")
+    ap.add_argument("--preheat", type=float, default=PREHEAT_S,
+                    help="seconds of untimed repetitions of a workload's step before its counted warm-up (0 = none)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the secondary decode measurement")
     ap.add_argument("--no-backward", action="store_true", help="skip the secondary backward measurement")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives are built); use --gpus 1")
+    PREHEAT_S = max(0.0, args.preheat)
 
     import torch
 
@@ -413,7 +451,8 @@ def main():
     if args.workload == "copy":
         src = torch.empty(COPY_BYTES, dtype=torch.uint8, device=device).random_(0, 255)
         dst = torch.empty_like(src)
-        wall_ms, ev_ms, ev_min = time_steps(torch, lambda i: dst.copy_(src), args.steps, args.warmup)
+        t = time_steps(torch, lambda i: dst.copy_(src), args.steps, args.warmup)
+        wall_ms, ev_ms = t["wall_ms"], t["kernel_ms"]
         print(json.dumps(dict(metric="plain device copy", value=2 * COPY_BYTES / ev_ms / 1e6, unit="GB/s",
                               bytes_read_per_launch=COPY_BYTES, bytes_written_per_launch=COPY_BYTES,
                               ms_per_step=wall_ms, ms_per_launch=ev_ms, n_gpus=1, steps=args.steps,
@@ -434,8 +473,7 @@ def main():
                           frac=r["tflops_kernel"] / peak, traffic=measured_traffic(args.workload),
                           kernel="prefill_f32_kernel" if f32 else ("decode_kernel + decode_merge_kernel per 64 query rows" if args.workload.endswith("n")
                                                                    else "prefill_kernel" if args.workload.endswith("u") else "recon_bf16_h8_kernel + prefill_kernel"),
-                          ms_per_launch=r["kernel_ms"],
-                          ms_per_launch_min=r["kernel_ms_min"], algorithmic_flops_per_launch=r["flops"]),
+                          **launch_times(r), algorithmic_flops_per_launch=r["flops"]),
             config=dict(workload=f"{args.workload}: TPA prefill" + (", fp32 inputs" if f32 else "") + (", nomat" if args.workload.endswith("n") else ""), **r["shape"]),
         )
         if not args.no_decode and not f32:
@@ -447,7 +485,7 @@ def main():
                 roofline=dict(bound="hbm", achieved=d["gbs_kernel"], peak=PEAK_HBM_GBS, unit="GB/s",
                               frac=d["gbs_kernel"] / PEAK_HBM_GBS, traffic=measured_traffic("c4"),
                               kernel="decode_kernel + decode_merge_kernel",
-                              ms_per_launch=d["kernel_ms"], ms_per_launch_min=d["kernel_ms_min"],
+                              **launch_times(d),
                               algorithmic_bytes_per_launch=d["bytes"]),
                 config=dict(workload="c4: TPA decode over the factored KV cache", **d["shape"]),
             )
@@ -469,7 +507,7 @@ def main():
                 roofline=dict(bound="mfma", achieved=bw["tflops_kernel"], peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
                               frac=bw["tflops_kernel"] / PEAK_BF16_TFLOPS, traffic=None,
                               kernel="recon + delta + bwd_dq_kernel + bwd_dkv_kernel + project (whole call)",
-                              ms_per_launch=bw["kernel_ms"], ms_per_launch_min=bw["kernel_ms_min"],
+                              **launch_times(bw),
                               algorithmic_flops_per_launch=bw["flops"]),
                 config=dict(workload="c2b: TPA backward", **bw["shape"]),
             )
@@ -491,7 +529,7 @@ def main():
             metric="dense flash attention forward throughput", value=r["tflops_wall"], unit="TFLOP/s", ms_per_step=r["wall_ms"],
             roofline=dict(bound="mfma", achieved=r["tflops_kernel"], peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
                           frac=r["tflops_kernel"] / PEAK_BF16_TFLOPS, traffic=None, kernel="prefill_kernel (dense loader)",
-                          ms_per_launch=r["kernel_ms"], ms_per_launch_min=r["kernel_ms_min"],
+                          **launch_times(r),
                           algorithmic_flops_per_launch=r["flops"]),
             config=dict(workload=f"{args.workload}: dense flash attention (tpa/mha.py) at the prefill shape", **r["shape"]),
         )
@@ -507,7 +545,7 @@ def main():
             unit="GB/s" if hbm else "TFLOP/s", ms_per_step=r["wall_ms"],
             roofline=dict(bound="hbm" if hbm else "mfma", achieved=ach, peak=PEAK_HBM_GBS if hbm else PEAK_BF16_TFLOPS,
                           unit="GB/s" if hbm else "TFLOP/s", frac=ach / (PEAK_HBM_GBS if hbm else PEAK_BF16_TFLOPS), traffic=None,
-                          kernel="append_fewrows_kernel + append_finish_kernel" if hbm else ("append_gemm_kernel<2>" if args.workload == "ap3" else "append_gemm_kernel<4>"), ms_per_launch=r["kernel_ms"], ms_per_launch_min=r["kernel_ms_min"],
+                          kernel="append_fewrows_kernel + append_finish_kernel" if hbm else ("append_gemm_kernel<2>" if args.workload == "ap3" else "append_gemm_kernel<4>"), **launch_times(r),
                           algorithmic_flops_per_launch=r["flops"], algorithmic_bytes_per_launch=r["bytes"]),
             config=dict(workload=f"{args.workload}: TPA cache append", **r["shape"]),
         )
@@ -523,7 +561,7 @@ def main():
                           frac=r["tflops_kernel"] / peak, traffic=None,
                           kernel=("recon + delta + bwd_f32_dq_kernel + bwd_f32_dkv_kernel + project (whole call)" if f32 else
                                   "recon + delta + bwd_dq_kernel + bwd_dkv_kernel + project (whole call)"),
-                          ms_per_launch=r["kernel_ms"], ms_per_launch_min=r["kernel_ms_min"],
+                          **launch_times(r),
                           algorithmic_flops_per_launch=r["flops"]),
             config=dict(workload=f"{args.workload}: TPA backward" + (", fp32 inputs" if f32 else ""), **r["shape"]),
         )
@@ -536,7 +574,7 @@ def main():
             roofline=dict(bound="hbm", achieved=d["gbs_kernel"], peak=PEAK_HBM_GBS, unit="GB/s",
                           frac=d["gbs_kernel"] / PEAK_HBM_GBS, traffic=measured_traffic(args.workload),
                           kernel=("decode_f32_kernel" if args.workload in F32_WORKLOADS else "decode_kernel") + " + decode_merge_kernel",
-                          ms_per_launch=d["kernel_ms"], ms_per_launch_min=d["kernel_ms_min"],
+                          **launch_times(d),
                           algorithmic_bytes_per_launch=d["bytes"]),
             config=dict(workload=f"{args.workload}: TPA decode over the factored KV cache" +
                         (", fp32 cache" if args.workload in F32_WORKLOADS else ""), **d["shape"]),
@@ -555,6 +593,13 @@ def main():
         n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True, scaling="weak",
         vs_baseline=None, dtype="f32" if args.workload in F32_WORKLOADS else "bf16", data="synthetic",
     )
+    # the yardstick children have been waited for (subprocess.run); release the device memory before the line is
+    # printed, so that the process is gone right after it
+    r = d = bw = None
+    import gc
+
+    gc.collect()
+    torch.cuda.empty_cache()
     print(json.dumps(result), flush=True)
 
 
