@@ -123,17 +123,20 @@ typedef struct TpaFwdArgs {
      it meets (tpa/ring_tpa.py:73-79 calls the block function with local indices only).  Rows that see no key
      end as NaN / -inf like any other empty row.  tpa_fwd and tpa_decode; ignored when causal == 0. */
   int32_t causal_offset;
-  /* tpa_fwd only; replaces the static `nomat` of the reference kernel (tpa/tpa.py:250, 333-359, 398-413).  Non-zero:
-     never form K or V.  The logits come from the rank-space identity x = (sm_scale / (rq rk)) sum_{r,s}
-     (qa_r . ka_s restricted to the head)(qb_r . kb_s), whose (qb_r . kb_s) table is shared by every head, and
-     o = (1/rk) sum_s (sum_k p_k va_s[k]) vb_s likewise.  Query rows are served in windows of at most 64 by the
-     split-key kernels of tpa_decode, which need args.workspace >= tpa_fwd_nomat_workspace_bytes(...) (else
-     TPA_ERR_WORKSPACE) and the shapes those kernels take (dk == dv in {64, 128}, rk a power of two <= 32, no
-     segment ids; bf16 also H % 8 == 0 and 16-byte aligned factors); any other problem runs the generic kernel
-     (TPA_ERR_UNSUPPORTED with kernel == TPA_KERNEL_MFMA).  The result is the same function of the inputs as with
-     nomat == 0 (tpa/tpa_test.py:122-190 runs one grid over both), in another order of operations.  Never chosen
-     by the library itself: on matrix cores it is the faster route only for a few query rows over a long
-     cache, which is what tpa_decode is. */
+  /* tpa_fwd only; stands where the reference kernel has its static `nomat` (tpa/tpa.py:250).  Non-zero: never form
+     K or V.  What runs is the split-key kernels of tpa_decode over windows of at most 64 query rows (two launches
+     per window): per head they form Qm[h] = (1/rq) sum_r qa_r[h] qb_r once, the logits are
+     (sm_scale / rk) sum_s ka_s[h] (kb_s . Qm[h]) and o = (1/rk) sum_s (sum_k p_k va_s[k, h]) vb_s, so every head
+     shares one pass over the kb / vb rows.  This is NOT the reference's form of the logits
+     (tpa/tpa.py:333-359: a table bb = qb_r . kb_s per rank pair that all heads of a block share, combined with
+     qa_r ka_s per head): Q is still formed per head here and no rank-pair table exists; the reference's form is
+     not implemented.  The o side is the reference's (tpa/tpa.py:398-413).  Needs args.workspace >=
+     tpa_fwd_nomat_workspace_bytes(...) (else TPA_ERR_WORKSPACE) and the shapes those kernels take (dk == dv in
+     {64, 128}, rk a power of two <= 32, no segment ids; bf16 also H % 8 == 0 and 16-byte aligned factors); any
+     other problem runs the generic kernel (TPA_ERR_UNSUPPORTED with kernel == TPA_KERNEL_MFMA).  The result is
+     the same function of the inputs as with nomat == 0 (tpa/tpa_test.py:122-190 runs one grid over both), in
+     another order of operations.  Never chosen by the library itself: on matrix cores it is the faster route
+     only for a few query rows over a long cache, which is what tpa_decode is. */
   int32_t nomat;
 } TpaFwdArgs;
 
@@ -257,7 +260,8 @@ typedef struct TpaAppendArgs {
   TpaFactor ka, kb, va, vb;   /* the cache, [B, cache_len, rk, H|D] or page pools (ptr is written through) */
   const int32_t* page_table;  /* as in TpaFwdArgs, or NULL */
   int32_t page_size, pages_per_seq;
-  int32_t B, n, d_model, H, D, rq, rk;
+  int32_t B, n, d_model, H, D, rq, rk;  /* H % 8 == 0 and D % 8 == 0 for every kernel of this call (outputs are written
+                                           in 16-byte chunks of 8 columns that must not straddle two arrays), else TPA_ERR_SHAPE */
   int32_t cache_len;          /* token capacity of one sequence (paged: pages_per_seq * page_size) */
   int32_t rope_len;           /* rows of the rotary tables: positions are clamped to rope_len - 1 */
   int32_t dtype;              /* TPA_DTYPE_*: element type of x, w, the q outputs and the cache */

@@ -9,11 +9,14 @@ reference, all on purpose:
   * the logsumexp residual is fp32 (the reference keeps it in the input dtype, tpa/tpa.py:530);
   * sequence lengths need not be multiples of the block sizes (tpa/tpa.py:489-490 asserts that);
     `block_sizes` is accepted and ignored because the kernels fix their own tiles;
-  * `nomat` picks an evaluation order, as in the reference (tpa/tpa.py:333-359,398-413), and
-    changes no result: `nomat=True` runs the kernels that never form K or V (the split-key
-    decode kernels, over windows of 64 query rows) wherever they take the problem, and the
-    plain kernel elsewhere; the default rebuilds K/V tiles in LDS, which is the faster order on
-    matrix cores except for a few query rows over a long cache (`tpa_decode`);
+  * `nomat` picks an evaluation order, as in the reference (tpa/tpa.py:250), and changes no
+    result: `nomat=True` runs the kernels that never form K or V (the split-key decode kernels,
+    over windows of 64 query rows, two launches per window) wherever they take the problem, and
+    the plain kernel elsewhere.  Those kernels form Q per head and share one pass over the kb / vb
+    rows between the heads; the reference's rank-pair table bb = qb_r . kb_s shared by the heads
+    (tpa/tpa.py:333-359) is not what they compute and is not implemented.  The default rebuilds
+    K/V tiles in LDS, which is the faster order on matrix cores except for a few query rows over
+    a long cache (`tpa_decode`);
   * `interpret=True` (the Pallas CPU interpreter upstream) selects the plain fp32-arithmetic
     kernel instead of the MFMA kernels; `debug` is ignored;
   * the backward pass (tpa/tpa.py:168-214,546-995) goes through dense Q, K, V and dense gradients
