@@ -391,26 +391,27 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   using IsK = std::integral_constant<bool, false>;
   using IsV = std::integral_constant<bool, true>;
 
-  // Head factors (LOAD_TPA_R2): threads 0..255 (waves 0-3) fetch one value a[matrix][token][rank]
-  // each, matrix = tid / 128 (0: K of tile kt, 1: V of tile vt), token = (tid / 2) % 64, rank = tid % 2,
-  // and park it in a register until it is stored into an LDS slot one iteration later.
+  // Head factors (LOAD_TPA_R2): a thread fetches one value a[matrix][token][rank], matrix = (tid % 256) / 128
+  // (0: K of tile kt, 1: V of tile vt), token = (tid / 2) % 64, rank = tid % 2, and parks it in a register
+  // until it is stored into an LDS slot one iteration later.  Waves 4-7 repeat what waves 0-3 do (same
+  // values to the same addresses), so that the eight waves run one instruction stream.
   uint32_t a_pending = 0;
-  const int a_mat = tid / (2 * kTK), a_tok = (tid >> 1) % kTK, a_rank = tid & 1;
+  const int a_idx = tid & (4 * kTK - 1);
+  const int a_mat = a_idx / (2 * kTK), a_tok = (a_idx >> 1) % kTK, a_rank = a_idx & 1;
   const int ka_bytes = ((lk_r - 1) * p.ka.stride_l + p.ka.stride_r + 1) * 2, va_bytes = ((lk_r - 1) * p.va.stride_l + p.va.stride_r + 1) * 2;
   const __amdgpu_buffer_rsrc_t ka_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(ka_b), 0, ka_bytes, kRsrcFlags);
   const __amdgpu_buffer_rsrc_t va_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(va_b), 0, va_bytes, kRsrcFlags);
   const int ka_voff = (a_tok * p.ka.stride_l + a_rank * p.ka.stride_r) * 2, va_voff = (a_tok * p.va.stride_l + a_rank * p.va.stride_r) * 2;
   auto issue_a = [&](int kt, int vt) __attribute__((always_inline)) {
     if constexpr (LOADER != LOAD_TPA_R2) return;
-    if (tid >= 4 * kTK) return;
-    // waves 0, 1 fetch K's head factors, waves 2, 3 V's (uniform per wave); tokens past the end read as 0
+    // waves 0, 1 (4, 5) fetch K's head factors, waves 2, 3 (6, 7) V's (uniform per wave); tokens past the end read as 0
     if (a_mat == 0) a_pending = __builtin_amdgcn_raw_buffer_load_b16(ka_rs, ka_voff, kt * kTK * p.ka.stride_l * 2, 0);
     else a_pending = __builtin_amdgcn_raw_buffer_load_b16(va_rs, va_voff, vt * kTK * p.va.stride_l * 2, 0);
   };
   auto store_a = [&](int slot_idx) __attribute__((always_inline)) {
     if constexpr (LOADER != LOAD_TPA_R2) return;
     // stored halved (exact in bf16): the 1/R of the reconstruction with R = 2
-    if (tid < 4 * kTK) lds_a(slot_idx)[tid] = (uint16_t)(pack_bf16(bf16lo_to_f32(a_pending) * 0.5f, 0.f));
+    lds_a(slot_idx)[a_idx] = (uint16_t)(pack_bf16(bf16lo_to_f32(a_pending) * 0.5f, 0.f));
   };
 
   // Key segment ids (packed sequences, tpa/tpa.py:369-375): the threads of one wave (wave 4 where
@@ -866,7 +867,8 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
 
   // ---- plain iteration: first tile, masked tiles, tiles a row block skips, last tile.
   // `mask_c` = the row blocks of this wave that take part (bit r); `part_c` = 0: the whole tile, 1: its
-  // logits only (they stay in s), 2: the rest of a tile whose logits are in s already.
+  // logits only (they stay in s), 2: the rest of a tile whose logits are in s already, 3: the logits of
+  // its first 32 keys only, 4: the rest of a tile whose first 32 logits are in s already.
   auto cold_compute = [&](int j, auto mask_c, auto part_c) __attribute__((always_inline)) {
     constexpr int M = decltype(mask_c)::value, PART = decltype(part_c)::value;
     const uint16_t* ks = lds_k(j % 3);
@@ -875,21 +877,24 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
     // while the softmax runs); not with the any-rank loader, whose kernel got slower with it
     constexpr int LA = LOADER == LOAD_TPA_ANY ? 0 : 3;
     bf16x8 fr[N_MFMA];
-    constexpr int FIRST = PART == 2 ? N_QK : 0, END = PART == 1 ? N_QK : N_MFMA;  // fragments this call uses
+    // fragments this call uses (0 .. N_QK - 1: K rows, the first NKS of them those of keys 0-31), and which of
+    // them belong to the logits
+    constexpr int FIRST = PART == 2 ? N_QK : PART == 4 ? NKS : 0, END = PART == 1 ? N_QK : PART == 3 ? NKS : N_MFMA;
+    constexpr int QK_END = PART == 3 ? NKS : N_QK;
     static_for<LA>([&](auto n_c) __attribute__((always_inline)) {
       constexpr int n = FIRST + decltype(n_c)::value;
       if constexpr (n < END) fr[n] = load_frag(IC<n>{}, ks, vs);
     });
     if constexpr (PART != 2) {
-      static_for<N_QK>([&](auto n_c) __attribute__((always_inline)) {
-        constexpr int n = decltype(n_c)::value;
+      static_for<QK_END - FIRST>([&](auto n_c) __attribute__((always_inline)) {
+        constexpr int n = FIRST + decltype(n_c)::value;
         if constexpr (n + LA < END) fr[n + LA] = load_frag(IC<n + LA>{}, ks, vs);
         static_for<RB>([&](auto r_c) __attribute__((always_inline)) {
-          if constexpr ((M >> decltype(r_c)::value) & 1) mfma_with(n_c, r_c, fr[n]);
+          if constexpr ((M >> decltype(r_c)::value) & 1) mfma_with(IC<n>{}, r_c, fr[n]);
         });
       });
     }
-    if constexpr (PART != 1) {
+    if constexpr (PART != 1 && PART != 3) {
       static_for<RB>([&](auto r_c) __attribute__((always_inline)) {
         if constexpr ((M >> decltype(r_c)::value) & 1) do_softmax(j, r_c);
       });
@@ -956,10 +961,9 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
   // tiles, tiles past this wave's causal range, the last tile).  Three separate loops rather than
   // a branch inside one: every wave passes the same number of barriers either way.
   auto tail = [&](int j) __attribute__((always_inline)) {
-    if (w < 4) {  // head factors: publish those of K tile j+3 / V tile j+2, fetch those of K tile j+4 / V tile j+3
-      store_a((j + 1) & 1);
-      issue_a(min(j + 4, last), min(j + 3, last));
-    }
+    // head factors: publish those of K tile j+3 / V tile j+2, fetch those of K tile j+4 / V tile j+3
+    store_a((j + 1) & 1);
+    issue_a(min(j + 4, last), min(j + 3, last));
     // key segment ids (one wave): publish those of tile j+1, fetch those of tile j+2
     store_seg((j + 1) & 1);
     issue_seg(min(j + 2, last));
@@ -1053,6 +1057,97 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
       s[0][0] = odd ? sb0 : sa0;
       s[0][1] = odd ? sb1 : sa1;
       cold_compute(j, IC<1>{}, IC<2>{});
+      advance_tiles(j);
+      tail(j);
+      ++j;
+    }
+  } else if constexpr (LOADER == LOAD_TPA_R2 && !SEG) {
+    // Unmasked tiles 1 .. hot_end - 1 pipelined in blocks of 32 keys: a block's softmax runs beside the
+    // logits of the next block, its O^T beside the rebuild of the tiles ahead.  The logits of the first 32
+    // keys of tile 1 are computed here; the loop (generated by gen_prefill_loop.py, which documents the
+    // register assignment) runs iterations 1 .. hot_end - 2 - everything advance_tiles() and tail() do
+    // included - and leaves the logits of the first 32 keys of tile hot_end - 1, which is finished here.
+    if (hot_end >= 3) {
+      cold_compute(1, IC<1>{}, IC<3>{});
+      auto cat4 = [](const u32x4& a0, const u32x4& a1, const u32x4& a2, const u32x4& a3) __attribute__((always_inline)) -> u32x16 {
+        const u32x8 lo = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+        const u32x8 hi = __builtin_shufflevector(a2, a3, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+      };
+      auto qv = [&](int ks) __attribute__((always_inline)) { return __builtin_bit_cast(u32x4, qf[0][ks]); };
+      const u32x16 qp0 = cat4(qv(0), qv(1), qv(2), qv(3));
+      const u32x16 qp1 = NKS > 4 ? cat4(qv(NKS > 4 ? 4 : 0), qv(NKS > 4 ? 5 : 0), qv(NKS > 4 ? 6 : 0), qv(NKS > 4 ? 7 : 0)) : qp0;
+      // rows in flight: (pass, rank) tuples of four registers
+      u32x16 kv_k = cat4(kreg[0][0], kreg[0][1], kreg[NPASS - 1][0], kreg[NPASS - 1][1]);
+      u32x16 kv_v = cat4(vreg[0][0], vreg[0][1], vreg[NPASS - 1][0], vreg[NPASS - 1][1]);
+      f32x16 set0 = s[0][0], set1 = {};
+      const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t*)smem;
+      u32x16 st16 = {};
+      st16[0] = __float_as_uint(mref[0]); st16[1] = __float_as_uint(lsum[0]);
+      st16[2] = lds0 + 2 * (L::k_off(0) + i * KS + 8 * g);                                                   // K fragment rows
+      st16[3] = lds0 + 2 * (L::v_off(0) + (4 * g + (lp >> 2)) * VS + 16 * dhalf + 4 * (lp & 3));             // V fragment columns
+      st16[4] = lds0 + 2 * (L::k_off(0) + lt * KS + 8 * lc);                                                 // this thread's chunk of a K tile
+      st16[5] = lds0 + 2 * (L::v_off(0) + lt * VS + 8 * lc);                                                 // ... of a V tile
+      st16[6] = kvoff; st16[7] = vvoff;
+      st16[8] = lds0 + 2 * L::a_off(0) + 4 * lt;                                                             // head factor pairs of this thread's tokens
+      st16[9] = lds0 + 2 * (L::a_off(0) + a_idx);                                                            // where this thread's head factor goes
+      st16[10] = a_mat ? va_voff : ka_voff;
+      st16[11] = a_pending;
+      auto uni = [](uint32_t x) __attribute__((always_inline)) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); };
+      u32x16 sc16 = {};
+      sc16[0] = 1; sc16[1] = uni(hot_end - 1); sc16[2] = uni(last);
+      sc16[3] = uni(kTK * p.kb.stride_l * 2); sc16[4] = uni(kTK * p.vb.stride_l * 2);
+      sc16[5] = uni(TPP * p.kb.stride_l * 2); sc16[6] = uni(TPP * p.vb.stride_l * 2);
+      sc16[7] = 1 * L::kK * 2; sc16[8] = 2 * L::kK * 2; sc16[9] = 0;  // K buffers of tiles 1 and 2, and the one tile 3 goes to
+      sc16[10] = uni(p.kb.stride_r * 2); sc16[11] = uni(p.vb.stride_r * 2);
+      sc16[12] = uni(kTK * (a_mat ? p.va.stride_l : p.ka.stride_l) * 2);
+      sc16[13] = uni(a_mat ? 3 : 4);
+      auto rsrc_words = [&](const uint16_t* base, int bytes) __attribute__((always_inline)) -> u32x4 {
+        const uint64_t a64 = reinterpret_cast<uint64_t>(base);
+        return u32x4{uni((uint32_t)a64), uni((uint32_t)(a64 >> 32) & 0xffffu), uni((uint32_t)bytes), (uint32_t)kRsrcFlags};
+      };
+      const u32x4 kbr = rsrc_words(kb_b, k_rows_bytes), vbr = rsrc_words(vb_b, v_rows_bytes);
+      const u32x4 abr = rsrc_words(a_mat ? va_b : ka_b, a_mat ? va_bytes : ka_bytes);
+      if constexpr (D == 128) {
+        asm volatile(
+#include "gen/prefill_loop_128_r2.inc"
+            : "+{v[0:15]}"(set0), "+{v[16:31]}"(set1), "+{v[32:47]}"(nmref[0]),
+              "+{v[48:63]}"(o[0][0]), "+{v[64:79]}"(o[0][1]), "+{v[80:95]}"(o[0][NDB > 2 ? 2 : 0]), "+{v[96:111]}"(o[0][NDB > 2 ? 3 : 0]),
+              "+{v[144:159]}"(kv_k), "+{v[160:175]}"(kv_v), "+{v[188:203]}"(st16), "+{s[32:47]}"(sc16)
+            : "{v[112:127]}"(qp0), "{v[128:143]}"(qp1), "{s[48:51]}"(kbr), "{s[52:55]}"(vbr), "{s[56:59]}"(abr)
+            :
+#include "gen/prefill_loop_128_r2_clobbers.inc"
+        );
+      } else {
+        u32x8 kv_k8 = __builtin_shufflevector(kv_k, kv_k, 0, 1, 2, 3, 4, 5, 6, 7);
+        u32x8 kv_v8 = __builtin_shufflevector(kv_v, kv_v, 0, 1, 2, 3, 4, 5, 6, 7);
+        asm volatile(
+#include "gen/prefill_loop_64_r2.inc"
+            : "+{v[0:15]}"(set0), "+{v[16:31]}"(set1), "+{v[32:47]}"(nmref[0]),
+              "+{v[48:63]}"(o[0][0]), "+{v[64:79]}"(o[0][1]),
+              "+{v[144:151]}"(kv_k8), "+{v[160:167]}"(kv_v8), "+{v[188:203]}"(st16), "+{s[32:47]}"(sc16)
+            : "{v[112:127]}"(qp0), "{s[48:51]}"(kbr), "{s[52:55]}"(vbr), "{s[56:59]}"(abr)
+            :
+#include "gen/prefill_loop_64_r2_clobbers.inc"
+        );
+        kv_k = __builtin_shufflevector(kv_k8, kv_k8, 0, 1, 2, 3, 4, 5, 6, 7, 0, 1, 2, 3, 4, 5, 6, 7);
+        kv_v = __builtin_shufflevector(kv_v8, kv_v8, 0, 1, 2, 3, 4, 5, 6, 7, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
+      kreg[0][0] = __builtin_shufflevector(kv_k, kv_k, 0, 1, 2, 3);
+      kreg[0][1] = __builtin_shufflevector(kv_k, kv_k, 4, 5, 6, 7);
+      vreg[0][0] = __builtin_shufflevector(kv_v, kv_v, 0, 1, 2, 3);
+      vreg[0][1] = __builtin_shufflevector(kv_v, kv_v, 4, 5, 6, 7);
+      if constexpr (NPASS > 1) {
+        kreg[NPASS - 1][0] = __builtin_shufflevector(kv_k, kv_k, 8, 9, 10, 11);
+        kreg[NPASS - 1][1] = __builtin_shufflevector(kv_k, kv_k, 12, 13, 14, 15);
+        vreg[NPASS - 1][0] = __builtin_shufflevector(kv_v, kv_v, 8, 9, 10, 11);
+        vreg[NPASS - 1][1] = __builtin_shufflevector(kv_v, kv_v, 12, 13, 14, 15);
+      }
+      mref[0] = __uint_as_float(st16[0]); lsum[0] = __uint_as_float(st16[1]);
+      a_pending = st16[11];
+      j = hot_end - 1;
+      s[0][0] = set0;
+      cold_compute(j, IC<1>{}, IC<4>{});
       advance_tiles(j);
       tail(j);
       ++j;
