@@ -638,8 +638,10 @@ __global__ __launch_bounds__((8 / RB) * 64) void prefill_kernel(PrefillParams pp
     const bool up = seen[r] && tmax > kSlack;         // rare: the row's max left the slack
     if (__any(first || up)) {
       // a first tile sets the reference (nothing accumulated yet, so nothing to rescale); later
-      // the references move up and O and the row sums are rescaled
-      const float delta = first ? tmax : (up ? tmax : 0.f);
+      // the references move up and O and the row sums are rescaled.  The reference is always a whole
+      // number: every exponent 2^(x - mref) then has the mantissa of 2^x itself, so which tile set or
+      // moved the reference changes no rounding of P (and all rescaling is by exact powers of two)
+      const float delta = (first || up) ? __builtin_ceilf(tmax) : 0.f;
       const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);
       mref[r] += delta;
       refresh_nmref(r_c);

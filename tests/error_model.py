@@ -68,21 +68,128 @@ def round_bf16(x):
     return u.view(np.float32).astype(np.float64)
 
 
-def emulate_bf16_prefill(q, k, v, num_heads, sm_scale, causal=False):
-    """The rounding points of the bf16 prefill kernel in numpy (float64 between them): bf16 of the
-    pre-scaled Q, of K, V, P and of the output.  -> (o[b,lq,h,dv], lse[b,lq,h])"""
-    q, k, v = (np.asarray(x, dtype=np.float64) for x in (q, k, v))
-    rec = lambda x: np.matmul(np.swapaxes(x[..., :num_heads], 2, 3), x[..., num_heads:]) / x.shape[2]
-    log2e = 1.4426950408889634
-    qs = round_bf16(rec(q) * (sm_scale * log2e))
-    kk, vv = round_bf16(rec(k)), round_bf16(rec(v))
-    x = np.einsum("bqhd,bkhd->bhqk", qs, kk)  # log2 domain
+def truncate_bf16(x):
+    """float64/float32 array -> bfloat16 by dropping the low 16 bits of the float32 (round toward zero)."""
+    u = np.asarray(x, dtype=np.float32).view(np.uint32) & np.uint32(0xFFFF0000)
+    return u.view(np.float32).astype(np.float64)
+
+
+def bf16_ulp(x):
+    """spacing of bfloat16 (8 significand bits) at |x|; the spacing at the smallest normal number below it"""
+    ax = np.maximum(np.abs(np.asarray(x, dtype=np.float64)), 2.0**-126)
+    return 2.0 ** (np.floor(np.log2(ax)) - 7)
+
+
+LOG2E_F32 = float(np.float32(1.4426950408889634))
+
+
+def emulate_bf16_attention(qd, kd, vd, sm_scale, bias=None, q_prescaled=False, faults=(), reference_shift=0):
+    """The rounding points of the bf16 matrix-core prefill kernels in numpy, float64 between them, on dense
+    qd[b,lq,h,d], kd[b,lk,h,d], vd[b,lk,h,dv] (float64, not yet rounded):
+
+        Q' = bf16(Q * sm_scale * log2 e)   K' = bf16(K)   V' = bf16(V)
+        x  = Q' . K' (+ bias, 0 / -inf)                       the exponent, base 2
+        p  = 2^(x - m),  m a WHOLE number (here: ceil of the row maximum)
+        l  = sum_k p_k (unrounded)          P = bf16(p)
+        o  = bf16( (sum_k P_k V'_k) / l )   lse = (m + log2 l) / log2 e
+
+    Because m is a whole number, P has the mantissa of bf16(2^x) whatever m is: the kernels' choice of
+    reference (the first tile's maximum rounded up, moved by whole numbers) changes no bit of P, so this
+    emulation and a kernel differ only by fp32 summation order, the fp32 accuracy of exp2 and rare double
+    roundings - a few output elements in a thousand, by one bf16 spacing.
+
+    `faults` injects mistakes for the tests of the gate itself: "p_twice" rounds P a second time at another
+    scale, "p_trunc" truncates P instead of rounding it, "q_unscaled_round" rounds Q before the scale factor
+    is applied and again after.
+
+    -> (o[b,lq,h,dv] (bf16 values), lse[b,lq,h], slack[b,lq,h,dv]): slack is what an output element may move
+    by before its last rounding without any rounding point being wrong: TIGHT_REL of sum_k p_k |V'_k| / l (fp32
+    summation order), plus one bf16 spacing (2^-7 of the value at most) of the row's largest p_k / l times the largest |V'| of the column
+    (the rounding of one P or V' element flipped, because an exponent or a reconstructed value that lies on a
+    rounding boundary in float64 lies beside it in fp32; with many keys of similar weight this is nothing,
+    with one dominant key it is the spacing of V')"""
+    qd, kd, vd = (np.asarray(x, dtype=np.float64) for x in (qd, kd, vd))
+    c = 1.0 if q_prescaled else float(np.float32(np.float32(sm_scale) * np.float32(LOG2E_F32)))
+    if "q_unscaled_round" in faults:
+        qd = round_bf16(qd)
+    qs, kk, vv = round_bf16(qd * c), round_bf16(kd), round_bf16(vd)
+    x = np.matmul(np.transpose(qs, (0, 2, 1, 3)), np.transpose(kk, (0, 2, 3, 1)))  # b h lq lk
+    if bias is not None:
+        x = x + np.asarray(bias, dtype=np.float64)[:, None, :, :]
+    with np.errstate(invalid="ignore", divide="ignore", over="ignore"):
+        m = np.ceil(x.max(-1, keepdims=True)) + int(reference_shift)  # any whole number gives the same bits
+        p = np.exp2(x - m)  # a row without a visible key: -inf - -inf = NaN, as the kernels give
+        l = p.sum(-1, keepdims=True)
+        if "p_trunc" in faults:
+            pr = truncate_bf16(p)
+        elif "p_twice" in faults:
+            pr = round_bf16(round_bf16(p * 0.75) / 0.75)
+        else:
+            pr = round_bf16(p)
+        vt = np.transpose(vv, (0, 2, 1, 3))  # b h lk dv
+        o = np.matmul(pr, vt) / l
+        slack = TIGHT_REL * np.matmul(p, np.abs(vt)) / l + 2.0**-7 * (p.max(-1, keepdims=True) / l) * np.abs(vt).max(-2, keepdims=True)
+        lse = np.where(np.isneginf(m[..., 0]), -np.inf, (m[..., 0] + np.log2(l[..., 0])) / LOG2E_F32)
+    o = np.transpose(o, (0, 2, 1, 3))
+    return round_bf16(o), np.transpose(lse, (0, 2, 1)), np.transpose(slack, (0, 2, 1, 3))
+
+
+def reconstruct_dense(x, num_heads):
+    """concatenated factors x[b,l,r,h+d] -> (1/R) sum_r a_r (x) b_r as [b,l,h,d], exact in float64"""
+    x = np.asarray(x, dtype=np.float64)
+    return np.matmul(np.swapaxes(x[..., :num_heads], 2, 3), x[..., num_heads:]) / x.shape[2]
+
+
+def emulate_bf16_prefill(q, k, v, num_heads, sm_scale, causal=False, bias=None, faults=(), reference_shift=0):
+    """emulate_bf16_attention on concatenated factors q[b,lq,rq,h+dk], k[b,lk,rk,h+dk], v[b,lk,rk,h+dv] (the
+    bf16 values the kernel reads): Q, K and V are reconstructed exactly and rounded once, as both prefill
+    routes do.  `bias` [b,lq,lk] of 0 / -inf is added to a top-left causal mask where `causal` is set.
+    -> (o, lse[b,lq,h], slack)"""
+    qd, kd, vd = (reconstruct_dense(x, num_heads) for x in (q, k, v))
     if causal:
-        lq, lk = x.shape[-2:]
-        x = np.where(np.tril(np.ones((lq, lk), bool)), x, -np.inf)
-    m = x.max(-1, keepdims=True)
-    p = np.exp2(x - m)
-    l = p.sum(-1, keepdims=True)
-    o = np.einsum("bhqk,bkhd->bqhd", round_bf16(p), vv) / np.transpose(l, (0, 2, 1, 3))
-    lse = (m[..., 0] + np.log2(l[..., 0])) / log2e
-    return round_bf16(o), np.transpose(lse, (0, 2, 1))
+        lq, lk = qd.shape[1], kd.shape[1]
+        tri = np.where(np.tril(np.ones((lq, lk), bool)), 0.0, -np.inf)[None]
+        bias = tri if bias is None else np.asarray(bias, dtype=np.float64) + tri
+    return emulate_bf16_attention(qd, kd, vd, sm_scale, bias=bias, faults=faults, reference_shift=reference_shift)
+
+
+# The gate that holds a bf16 kernel to its emulation: per output element two bf16 spacings (a flipped last
+# rounding, and the neighbouring value where the element sits at a power of two) plus the emulation's slack
+# (fp32 summation order, one flipped P or V' rounding), at most TIGHT_FRAC of the elements different at all,
+# and the logsumexp within TIGHT_LSE (+ its own fp32 rounding).  Measured on the GPU over benchmark-like,
+# sharp, packed and high-rank problems on both prefill routes: 0.002 - 0.17 % of the elements differ,
+# logsumexp by at most 7e-5; a second rounding of P, a truncated P or Q rounded before its scale factor make
+# 9 - 65 % of the elements differ (tests/test_error_model.py).
+TIGHT_SPACINGS = 2.0
+TIGHT_REL = 1e-4
+TIGHT_FRAC = 0.01
+TIGHT_LSE = 2e-4
+
+
+def tight_violations(o, lse_blh, o_emu, lse_emu, slack):
+    """-> list of strings, empty if (o, lse) agree with the emulation (see TIGHT_*).  All arrays float64;
+    o / o_emu hold bf16 values."""
+    bad = []
+    o, o_emu = np.asarray(o, dtype=np.float64), np.asarray(o_emu, dtype=np.float64)
+    if not np.array_equal(np.isnan(o), np.isnan(o_emu)):
+        return ["NaN rows differ"]
+    if not np.array_equal(np.isneginf(lse_blh), np.isneginf(lse_emu)):
+        return ["-inf logsumexp rows differ"]
+    ok = ~np.isnan(o_emu)
+    if ok.any():
+        d = np.abs(np.where(ok, o - o_emu, 0.0))
+        tol = np.where(ok, TIGHT_SPACINGS * np.maximum(bf16_ulp(o_emu), bf16_ulp(o)) + np.nan_to_num(slack), np.inf)
+        worst = (d / tol).max()
+        if worst > 1.0:
+            bad.append(f"an output element is {worst:.2f} x ({TIGHT_SPACINGS:.0f} bf16 spacings + slack) away from the emulation")
+        frac = (d > 0).sum() / ok.sum()
+        if frac > TIGHT_FRAC:
+            bad.append(f"{100 * frac:.1f} % of the output elements differ from the emulation (gate {100 * TIGHT_FRAC:.0f} %)")
+    okl = ~np.isneginf(lse_emu)
+    if okl.any():
+        with np.errstate(invalid="ignore"):
+            dl = np.abs(np.where(okl, lse_blh - lse_emu, 0.0))
+        told = TIGHT_LSE + 1e-6 * np.abs(np.where(okl, lse_emu, 0.0))
+        if (dl > told).any():
+            bad.append(f"logsumexp off by {dl.max():.2e} (gate {TIGHT_LSE:.0e})")
+    return bad

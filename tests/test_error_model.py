@@ -6,7 +6,7 @@ import numpy as np
 import torch
 
 from conftest import bf16_round, make_factors
-from error_model import emulate_bf16_prefill, round_bf16, tpa_bounds
+from error_model import emulate_bf16_prefill, round_bf16, tight_violations, tpa_bounds
 from oracle import tpa_oracle as orc
 
 
@@ -21,7 +21,7 @@ def _errors(seed, b, lq, lk, h, d, rq, rk, scaled, causal):
     q, k, v = (bf16_round(x) for x in make_factors(seed, b, lq, lk, h, d, d, rq, rk, scale_by_rank=scaled))
     scale = d**-0.5
     o_ref, l_ref = orc.tpa_reference(q, k, v, None, None, h, sm_scale=scale, causal=causal)
-    o, l = emulate_bf16_prefill(q, k, v, h, scale, causal)
+    o, l, _ = emulate_bf16_prefill(q, k, v, h, scale, causal)
     lse_b, o_b = tpa_bounds(q, k, v, h, scale)
     return np.abs(o - o_ref).max(-1), np.abs(l - l_ref), o_b, lse_b
 
@@ -48,3 +48,39 @@ def test_bound_stays_inside_the_absolute_gates_on_benchmark_like_inputs():
     q, k, v = (bf16_round(x) for x in make_factors(2, 1, 128, 256, 4, 128, 128, 6, 2, scale_by_rank=True))
     lse_f, o_f = tpa_bounds(q, k, v, 4, 128**-0.5, form="factored")
     assert (lse_f >= lse_b).all() and (o_f >= o_b).all()
+
+
+CASES = {  # seed, b, lq, lk, h, d, rq, rk, factors scaled by 1/sqrt(R), causal
+    "sharp": (1, 2, 96, 160, 4, 128, 1, 2, False, True),
+    "benchmark-like": (2, 1, 128, 256, 4, 128, 6, 2, True, True),
+}
+
+
+def test_tight_gate_rejects_one_extra_rounding():
+    """The gate that holds the GPU kernels to the emulation (tests/test_gpu_parity.py: check_tight) fails an
+    emulation with one mistake in its rounding points: P rounded twice, P truncated, Q rounded before its
+    scale factor is applied.  The unmodified emulation passes against itself trivially; what the GPU kernels
+    measure against it is written beside the TIGHT_* constants."""
+    for name, (seed, b, lq, lk, h, d, rq, rk, scaled, causal) in CASES.items():
+        q, k, v = (bf16_round(x) for x in make_factors(seed, b, lq, lk, h, d, d, rq, rk, scale_by_rank=scaled))
+        o, l, slack = emulate_bf16_prefill(q, k, v, h, d**-0.5, causal)
+        assert not tight_violations(o, l, o, l, slack)
+        for fault in ("p_twice", "p_trunc", "q_unscaled_round"):
+            o2, l2, _ = emulate_bf16_prefill(q, k, v, h, d**-0.5, causal, faults=(fault,))
+            assert tight_violations(o2, l2, o, l, slack), (name, fault)
+
+
+def test_whole_number_reference_changes_no_bit():
+    """P = bf16(2^(x - m)) has the same mantissa for every whole number m, so neither the output nor any
+    rounding depends on which whole number the kernels use as the softmax reference: the emulation with the
+    reference three above the row maximum returns the same bits."""
+    seed, b, lq, lk, h, d, rq, rk, scaled, causal = CASES["sharp"]
+    q, k, v = (bf16_round(x) for x in make_factors(seed, b, lq, lk, h, d, d, rq, rk, scale_by_rank=scaled))
+    o, l, _ = emulate_bf16_prefill(q, k, v, h, d**-0.5, causal)
+    o3, l3, _ = emulate_bf16_prefill(q, k, v, h, d**-0.5, causal, reference_shift=3)
+    np.testing.assert_array_equal(o, o3)
+    np.testing.assert_allclose(l, l3, rtol=0, atol=1e-12)
+    # a reference that is not a whole number does change roundings of P
+    import error_model as em
+
+    assert em.round_bf16(2.0**-0.37 * 1.2345) != em.round_bf16(1.2345) * 2.0**-0.37

@@ -13,7 +13,7 @@ import pytest
 import torch
 
 from conftest import make_factors, segment_ids
-from error_model import dense_bounds, tpa_bounds
+from error_model import dense_bounds, emulate_bf16_attention, emulate_bf16_prefill, tight_violations, tpa_bounds
 from oracle import tpa_oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -69,6 +69,34 @@ def check(o, lse_bhl, o_ref, lse_ref_blh, tol, bounds=None):
     with np.errstate(invalid="ignore"):  # -inf minus -inf on rows without a visible key
         excess = np.where(okl, np.abs(lse - lse_ref_blh) - lse_bound, 0.0)
     assert excess.max(initial=0.0) <= 0.0, f"logsumexp error exceeds its bound by {excess.max():.3e}"
+
+
+def visible_bias(b, lq, lk, qseg=None, kvseg=None, causal=False, offset=0, lengths=None, bottom_right=False):
+    """Additive bias [b, lq, lk] of 0 / -inf for the masks the kernels take: segment ids, `key <= query +
+    offset` (per batch entry counted from the end of its keys with `bottom_right`), keys beyond lengths[b]."""
+    vis = np.ones((b, lq, lk), dtype=bool)
+    if qseg is not None:
+        vis &= np.asarray(qseg)[:, :, None] == np.asarray(kvseg)[:, None, :]
+    kk, qq = np.arange(lk)[None, None, :], np.arange(lq)[None, :, None]
+    n = np.full(b, lk) if lengths is None else np.minimum(np.asarray(lengths), lk)
+    if lengths is not None:
+        vis &= kk < n[:, None, None]
+    if causal:
+        off = offset + (n - lq if bottom_right else np.zeros(b, dtype=np.int64))
+        vis &= kk <= qq + off[:, None, None]
+    return np.where(vis, 0.0, -np.inf)
+
+
+def check_tight(o, lse_bhl, tq, tk, tv, h, sm_scale, bias=None):
+    """The bf16 matrix-core prefill kernels against the numpy emulation of their rounding points
+    (tests/error_model.py: emulate_bf16_prefill): at most two bf16 spacings plus fp32 summation noise per
+    output element, at most 1 % of the elements different at all, logsumexp within 2e-4.  Both prefill routes
+    round at the same points, so one emulation serves both.  The worst-case law of check() stays the bound a
+    caller can rely on; this gate is what catches a kernel that got a few times less accurate."""
+    fq, fk, fv = (np.nan_to_num(as_f64(t)) for t in (tq, tk, tv))
+    o_e, l_e, slack = emulate_bf16_prefill(fq, fk, fv, h, sm_scale, bias=bias)
+    bad = tight_violations(as_f64(o), as_f64(lse_bhl).transpose(0, 2, 1), o_e, l_e, slack)
+    assert not bad, "; ".join(bad)
 
 
 # ---------------------------------------------------------------- the reference's forward grid
@@ -168,6 +196,7 @@ def test_prefill_bf16_mfma(gpu, d, causal, b, lq, lk, h, rq, rk):
     (tq, tk, tv), o, lse = run_bf16(gpu, q, k, v, h, scale, causal)
     o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h, sm_scale=scale, causal=causal)
     check(o, lse, o_ref, l_ref, BF16_TOL, bf16_bounds(tq, tk, tv, h, scale))
+    check_tight(o, lse, tq, tk, tv, h, scale, visible_bias(b, lq, lk, causal=causal))
 
 
 @pytest.mark.parametrize("causal", [False, True])
@@ -179,6 +208,7 @@ def test_prefill_bf16_sharp_softmax(gpu, causal):
     (tq, tk, tv), o, lse = run_bf16(gpu, q, k, v, h, d**-0.5, causal)
     o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h, sm_scale=d**-0.5, causal=causal)
     check(o, lse, o_ref, l_ref, BF16_TOL, bf16_bounds(tq, tk, tv, h, d**-0.5))
+    check_tight(o, lse, tq, tk, tv, h, d**-0.5, visible_bias(b, t, t, causal=causal))
     rel = np.abs(as_f64(o) - o_ref).max() / np.abs(o_ref).max()
     assert rel < 2e-2
 
@@ -395,6 +425,10 @@ def test_mha_bf16_flash_vs_oracle(gpu, d, causal):
     o_ref, l_ref = orc.mha_forward(as_f64(q), as_f64(k), as_f64(v), bias, d**-0.5)
     o, (lse, *_) = _mha_fwd(q, k, v, None, d**-0.5, causal=causal, kernel=2)
     check(o, lse, o_ref, l_ref, BF16_TOL, dense_bounds(as_f64(q), as_f64(k), as_f64(v), d**-0.5))
+    # the dense kernel's rounding points: Q once after the scale factor, P, the output
+    o_e, l_e, slack = emulate_bf16_attention(as_f64(q), as_f64(k), as_f64(v), d**-0.5, bias=bias)
+    bad = tight_violations(as_f64(o), as_f64(lse).transpose(0, 2, 1), o_e, l_e, slack)
+    assert not bad, "; ".join(bad)
 
 
 @pytest.mark.parametrize("d", [128, 64])
@@ -579,6 +613,7 @@ def test_prefill_reference_moves_on_unmasked_tiles(gpu, d, causal, where):
     (tq, tk, tv), o, lse = run_bf16(gpu, q, k, v, h, scale, causal)
     o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h, sm_scale=scale, causal=causal)
     check(o, lse, o_ref, l_ref, BF16_TOL, bf16_bounds(tq, tk, tv, h, scale))
+    check_tight(o, lse, tq, tk, tv, h, scale, visible_bias(b, t, t, causal=causal))
 
 
 # ---------------------------------------------------------------- packed sequences through the MFMA prefill kernel
@@ -603,6 +638,7 @@ def test_prefill_bf16_segment_ids(gpu, b, lq, lk, h, d, rk, seg, causal):
     o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), tqs, tks, d**-0.5, causal, 2)
     o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), qseg, kvseg, h, sm_scale=d**-0.5, causal=causal)
     check(o, lse, o_ref, l_ref, BF16_TOL, bf16_bounds(tq, tk, tv, h, d**-0.5))
+    check_tight(o, lse, tq, tk, tv, h, d**-0.5, visible_bias(b, lq, lk, qseg, kvseg, causal))
     if lq > lk:
         assert np.isnan(o_ref).any()  # the case really has empty rows
 
@@ -673,6 +709,7 @@ def test_random_shapes_bf16_mfma(gpu, seed):
     o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), tqs, tks, d**-0.5, causal, 2)
     o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), qseg, kvseg, h, sm_scale=d**-0.5, causal=causal)
     check(o, lse, o_ref, l_ref, BF16_TOL, bf16_bounds(tq, tk, tv, h, d**-0.5))
+    check_tight(o, lse, tq, tk, tv, h, d**-0.5, visible_bias(b, lq, lk, qseg, kvseg, causal))
 
 
 def _id_pattern(name, b, lq, lk):
@@ -837,6 +874,8 @@ def test_prefill_with_per_sequence_key_lengths(gpu, kernel, dt, causal):
     o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), None, None, d**-0.5, causal, kernel, kv_lengths=lengths)
     o_ref, l_ref = _varlen_reference(as_f64(tq), np.nan_to_num(as_f64(tk)), np.nan_to_num(as_f64(tv)), lengths, h, d**-0.5, causal)
     check(o, lse, o_ref, l_ref, BF16_TOL if dt == torch.bfloat16 else F32_TOL, bf16_bounds(tq, tk, tv, h, d**-0.5))
+    if dt == torch.bfloat16:
+        check_tight(o, lse, tq, tk, tv, h, d**-0.5, visible_bias(b, lq, lk, causal=causal, lengths=lengths))
 
 
 @pytest.mark.parametrize("d,rk,page_size", [(128, 2, 16), (128, 2, 256), (64, 4, 8), (64, 1, 32)])
@@ -990,6 +1029,8 @@ def test_causal_offset(gpu, dt, kernel, b, lq, lk, h, d, rq, rk, offset, seg):
     o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), qseg, kvseg, sm_scale=sm_scale, causal=True, kernel=kernel, causal_offset=offset)
     o_ref, l_ref = _offset_reference(as_f64(tq), as_f64(tk), as_f64(tv), h, sm_scale, offset, qseg, kvseg)
     check(o, lse, o_ref, l_ref, F32_TOL if dt == torch.float32 else BF16_TOL, bf16_bounds(tq, tk, tv, h, sm_scale))
+    if dt == torch.bfloat16 and kernel == 2:
+        check_tight(o, lse, tq, tk, tv, h, sm_scale, visible_bias(b, lq, lk, qseg, kvseg, True, offset))
 
 
 def test_causal_offset_rows_equal_the_tail_of_the_full_causal_call(gpu):
@@ -1233,3 +1274,7 @@ def test_random_problems_on_the_dense_route(gpu, prefill_route, seed):
             o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=sm_scale, causal=tpa.CAUSAL_BOTTOM_RIGHT, kernel=2, kv_lengths=kvl)
             o_ref, l_ref = _bottom_right_reference(fq, fk, fv, lengths, h, sm_scale, 0)
     check(o, lse, o_ref, l_ref, BF16_TOL, bf16_bounds(tq, tk, tv, h, sm_scale))
+    bias = [None, lambda: visible_bias(b, lq, lk, causal=True, offset=offset),
+            lambda: visible_bias(b, lq, lk, causal=True, offset=offset, lengths=lengths),
+            lambda: visible_bias(b, lq, lk, causal=True, lengths=lengths, bottom_right=True)][mode]
+    check_tight(o, lse, tq, tk, tv, h, sm_scale, bias() if bias else None)
