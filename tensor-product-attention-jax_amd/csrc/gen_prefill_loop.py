@@ -694,7 +694,8 @@ def main():
             f.write(f'"{ln}\\n\\t"\n')
     # registers the loop uses beyond its operands (the state tuple is an in/out operand)
     ring = [b + k for b in RING_BUFS for k in range(4)]
-    clob = [f"v{n}" for n in sorted((set(ring) | set(TEMPS)) - set(STATE))]
+    named = set().union(*(regs_of(ln) for ln in lines))     # a head size with one loader pass leaves some unused
+    clob = [f"v{n}" for n in sorted((set(ring) | set(TEMPS)) - set(STATE)) if f"v{n}" in named]
     clob += [f"s{n}" for n in S_CLOB] + ["vcc", "scc", "memory"]
     with open(OUT.replace(".inc", "_clobbers.inc"), "w") as f:
         f.write("// generated by gen_prefill_loop.py: do not edit\n")
