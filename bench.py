@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2u|c3|c3u|c4|c4pg|c4s|c5|c5u|c2n|c5n|c2f|c3f|c2fb|c4f|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|ap1|ap2|ap3|copy] [--no-cpu] [--no-decode] [--no-backward]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2u|c3|c3u|c4|c4pg|c4s|c5|c5u|c2n|c5n|c5r|c5rn|c5rp|c2f|c3f|c2fb|c4f|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|ap1|ap2|ap3|copy] [--no-cpu] [--no-decode] [--no-backward]
 
 A step is one forward pass over one batch of synthetic, seeded inputs that are resident in HBM
 before the timed region starts.  The default workload is the prefill configuration the headline
@@ -41,6 +41,11 @@ WORKLOADS = {
     # nomat=True (tpa/tpa.py:250): the order of operations that never forms K or V, at the c2 and c5 shapes
     "c2n": ("prefill", 4, 4096, 4096, 16, 128, 6, 2, True),
     "c5n": ("prefill", 8, 2048, 2048, 64, 64, 16, 8, False),
+    # the c5 shape with the benchmark ranks 6 / 2: the default route (c5r), the split-key order (c5rn) and the
+    # reference's rank-pair tables, tpa/tpa.py:333-359 (c5rp)
+    "c5r": ("prefill", 8, 2048, 2048, 64, 64, 6, 2, False),
+    "c5rn": ("prefill", 8, 2048, 2048, 64, 64, 6, 2, False),
+    "c5rp": ("prefill", 8, 2048, 2048, 64, 64, 6, 2, False),
     "c4": ("decode", 64, 1, 8192, 32, 128, 6, 2, False),
     "c4pg": ("decode", 64, 1, 8192, 32, 128, 6, 2, False),  # the c4 cache as a pool of shuffled 64-token pages
     "c4s": ("decode", 64, 4, 8192, 32, 128, 6, 2, True),  # four appended tokens per sequence, each masked to its predecessors
@@ -232,7 +237,7 @@ def run_prefill(torch, tpa, device, name, steps, warmup):
         seg = (torch.arange(lq, device=device, dtype=torch.int32) // doc).repeat(B, 1).contiguous()
 
     use_ws = not name.endswith("u")
-    nomat = name.endswith("n")
+    nomat = "pairs" if name.endswith("rp") else name.endswith("n")
 
     def step(i):
         out["o"], out["lse"] = tpa.tpa_factors(*x, seg, seg, sm_scale=scale, causal=causal, kernel=2, use_workspace=use_ws, nomat=nomat)
@@ -471,10 +476,10 @@ def main():
             value=r["tflops_wall"], unit="TFLOP/s", ms_per_step=r["wall_ms"],
             roofline=dict(bound="mfma", achieved=r["tflops_kernel"], peak=peak, unit="TFLOP/s",
                           frac=r["tflops_kernel"] / peak, traffic=measured_traffic(args.workload),
-                          kernel="prefill_f32_kernel" if f32 else ("decode_kernel + decode_merge_kernel per 64 query rows" if args.workload.endswith("n")
+                          kernel="prefill_f32_kernel" if f32 else ("nomat_pairs_kernel" if args.workload.endswith("rp") else "decode_kernel + decode_merge_kernel per 64 query rows" if args.workload.endswith("n")
                                                                    else "prefill_kernel" if args.workload.endswith("u") else "recon_bf16_h8_kernel + prefill_kernel"),
                           **launch_times(r), algorithmic_flops_per_launch=r["flops"]),
-            config=dict(workload=f"{args.workload}: TPA prefill" + (", fp32 inputs" if f32 else "") + (", nomat" if args.workload.endswith("n") else ""), **r["shape"]),
+            config=dict(workload=f"{args.workload}: TPA prefill" + (", fp32 inputs" if f32 else "") + (", nomat (rank-pair tables)" if args.workload.endswith("rp") else ", nomat" if args.workload.endswith("n") else ""), **r["shape"]),
         )
         if not args.no_decode and not f32:
             log("[bench] decode c4")

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define TPA_ABI_VERSION 8
+#define TPA_ABI_VERSION 9
 
 /* element types of the factor / output arrays */
 enum { TPA_DTYPE_F32 = 0, TPA_DTYPE_BF16 = 1 };
@@ -58,6 +58,11 @@ enum {
 #define TPA_CAUSAL_NONE 0
 #define TPA_CAUSAL_TOP_LEFT 1     /* the reference's mask (tpa/tpa.py:377-379) */
 #define TPA_CAUSAL_BOTTOM_RIGHT 2 /* an addition: see TpaFwdArgs.causal_offset */
+
+/* TpaFwdArgs.nomat */
+#define TPA_NOMAT_OFF 0
+#define TPA_NOMAT_SPLIT_KEYS 1
+#define TPA_NOMAT_RANK_PAIRS 2
 
 /*
  * One factor array: A factors a[b, l, r, h] or B factors b[b, l, r, d].  The innermost
@@ -123,20 +128,21 @@ typedef struct TpaFwdArgs {
      it meets (tpa/ring_tpa.py:73-79 calls the block function with local indices only).  Rows that see no key
      end as NaN / -inf like any other empty row.  tpa_fwd and tpa_decode; ignored when causal == 0. */
   int32_t causal_offset;
-  /* tpa_fwd only; stands where the reference kernel has its static `nomat` (tpa/tpa.py:250).  Non-zero: never form
-     K or V.  What runs is the split-key kernels of tpa_decode over windows of at most 64 query rows (two launches
-     per window): per head they form Qm[h] = (1/rq) sum_r qa_r[h] qb_r once, the logits are
-     (sm_scale / rk) sum_s ka_s[h] (kb_s . Qm[h]) and o = (1/rk) sum_s (sum_k p_k va_s[k, h]) vb_s, so every head
-     shares one pass over the kb / vb rows.  This is NOT the reference's form of the logits
-     (tpa/tpa.py:333-359: a table bb = qb_r . kb_s per rank pair that all heads of a block share, combined with
-     qa_r ka_s per head): Q is still formed per head here and no rank-pair table exists; the reference's form is
-     not implemented.  The o side is the reference's (tpa/tpa.py:398-413).  Needs args.workspace >=
-     tpa_fwd_nomat_workspace_bytes(...) (else TPA_ERR_WORKSPACE) and the shapes those kernels take (dk == dv in
-     {64, 128}, rk a power of two <= 32, no segment ids; bf16 also H % 8 == 0 and 16-byte aligned factors); any
-     other problem runs the generic kernel (TPA_ERR_UNSUPPORTED with kernel == TPA_KERNEL_MFMA).  The result is
-     the same function of the inputs as with nomat == 0 (tpa/tpa_test.py:122-190 runs one grid over both), in
-     another order of operations.  Never chosen by the library itself: on matrix cores it is the faster route
-     only for a few query rows over a long cache, which is what tpa_decode is. */
+  /* tpa_fwd only; stands where the reference kernel has its static `nomat` (tpa/tpa.py:250): never form K or V.
+     The result is the same function of the inputs as with nomat == 0 (tpa/tpa_test.py:122-190 runs one grid over
+     both), in another order of operations.  Never chosen by the library itself.
+     TPA_NOMAT_SPLIT_KEYS (1): the split-key kernels of tpa_decode over windows of at most 64 query rows (two
+       launches per window).  Per head they form Qm[h] = (1/rq) sum_r qa_r[h] qb_r once, the logits are
+       (sm_scale / rk) sum_s ka_s[h] (kb_s . Qm[h]) and o = (1/rk) sum_s (sum_k p_k va_s[k, h]) vb_s
+       (tpa/tpa.py:398-413), so every head shares one pass over the kb / vb rows; Q is still formed per head.
+       Needs args.workspace >= tpa_fwd_nomat_workspace_bytes(...) (else TPA_ERR_WORKSPACE) and the shapes those
+       kernels take (dk == dv in {64, 128}, rk a power of two <= 32, no segment ids; bf16 also H % 8 == 0 and
+       16-byte aligned factors).  The faster of the two; it is what tpa_decode is.
+     TPA_NOMAT_RANK_PAIRS (2): the reference's own arithmetic (tpa/tpa.py:333-359): a table bb = kb_s . qb_r per
+       rank pair and block of keys that the heads of a workgroup share, combined per head with qa_r ka_s; neither
+       Q nor K nor V is formed.  One launch, no workspace; bf16, dk == dv in {64, 128}, rq in {1, 6},
+       rk in {1, 2, 4}, no segment ids, 16-byte aligned B factors and output.
+     Any other problem runs the generic kernel (TPA_ERR_UNSUPPORTED with kernel == TPA_KERNEL_MFMA). */
   int32_t nomat;
 } TpaFwdArgs;
 

@@ -113,6 +113,11 @@ int tpa_fwd(const TpaFwdArgs* a, void* stream) {
   if (rc != TPA_OK) return rc;
   if (a->page_table) return TPA_ERR_UNSUPPORTED;  // paged caches are read by tpa_decode only
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (a->nomat == TPA_NOMAT_RANK_PAIRS) {
+    if (a->kernel != TPA_KERNEL_GENERIC && tpa_nomat_pairs_supported(a)) return tpa_nomat_pairs_launch(a, s);
+    if (a->kernel == TPA_KERNEL_MFMA) return TPA_ERR_UNSUPPORTED;
+    return tpa_generic_launch(a, s);
+  }
   if (a->nomat) return tpa_fwd_nomat(a, s);
   // few query tokens over a long cache (the reference's decode is this same call with lq = 1,
   // tpa/tpa.py:485): split over keys, if the caller brought the workspace for it

@@ -171,6 +171,8 @@ int tpa_prefill_f32_supported(const TpaFwdArgs* a);
 int tpa_prefill_f32_launch(const TpaFwdArgs* a, hipStream_t stream);
 int mha_prefill_f32_supported(const MhaFwdArgs* a);
 int mha_prefill_f32_launch(const MhaFwdArgs* a, hipStream_t stream);
+int tpa_nomat_pairs_supported(const TpaFwdArgs* a);
+int tpa_nomat_pairs_launch(const TpaFwdArgs* a, hipStream_t stream);
 int tpa_decode_mfma_supported(const TpaFwdArgs* a);
 int tpa_decode_mfma_launch(const TpaFwdArgs* a, hipStream_t stream);
 int tpa_decode_f32_supported(const TpaFwdArgs* a);

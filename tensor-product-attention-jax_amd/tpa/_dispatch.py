@@ -22,7 +22,7 @@ KERNEL_AUTO = 0
 KERNEL_GENERIC = 1
 KERNEL_MFMA = 2
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 
 class TpaFactor(ctypes.Structure):

@@ -13,8 +13,9 @@ reference, all on purpose:
     result: `nomat=True` runs the kernels that never form K or V (the split-key decode kernels,
     over windows of 64 query rows, two launches per window) wherever they take the problem, and
     the plain kernel elsewhere.  Those kernels form Q per head and share one pass over the kb / vb
-    rows between the heads; the reference's rank-pair table bb = qb_r . kb_s shared by the heads
-    (tpa/tpa.py:333-359) is not what they compute and is not implemented.  The default rebuilds
+    rows between the heads.  `tpa_factors(nomat="pairs")` runs the reference's own arithmetic: a
+    table bb = qb_r . kb_s per rank pair shared by the heads of a workgroup, combined per head with
+    qa_r ka_s (tpa/tpa.py:333-359; csrc/tpa_nomat.hip); it is the slowest of the three.  The default rebuilds
     K/V tiles in LDS, which is the faster order on matrix cores except for a few query rows over
     a long cache (`tpa_decode`);
   * `interpret=True` (the Pallas CPU interpreter upstream) selects the plain fp32-arithmetic
@@ -74,6 +75,10 @@ def _lse_accum(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
 
 
 CAUSAL_BOTTOM_RIGHT = 2  # value of `causal`: the last query aligned with the last key of each batch entry
+# `nomat` of tpa_factors: True / 1 = the split-key kernels over windows of query rows, "pairs" / 2 = the
+# reference's own arithmetic, a table per rank pair shared by the heads of a workgroup (tpa/tpa.py:333-359)
+NOMAT_SPLIT_KEYS = 1
+NOMAT_RANK_PAIRS = 2
 
 
 def _causal_code(causal) -> int:
@@ -185,7 +190,10 @@ def tpa_factors(
     # the problem qualifies
     ws, ws_ptr, ws_bytes = None, None, 0
     # (fp32 inputs: only the split-key decode kernel takes a workspace)
-    if nomat:
+    nomat = NOMAT_RANK_PAIRS if nomat in ("pairs", NOMAT_RANK_PAIRS) and nomat is not True else int(bool(nomat))
+    if nomat == NOMAT_RANK_PAIRS:
+        pass  # one launch, no workspace
+    elif nomat:
         # the split partials of the non-materialising kernels: required, not optional
         need = lib.tpa_fwd_nomat_workspace_bytes(b, lq, lk, h, dk, dv, rq, rk) if kernel != _d.KERNEL_GENERIC else 0
         if need:
@@ -207,7 +215,7 @@ def tpa_factors(
         dtype=_d.dtype_code(dtype), sm_scale=float(sm_scale), causal=_causal_code(causal), kernel=int(kernel),
         workspace=ws_ptr, workspace_bytes=ws_bytes, num_splits=0,
         kv_lengths=kvlen.data_ptr() if kvlen is not None else None,
-        causal_offset=int(causal_offset), nomat=int(bool(nomat)),
+        causal_offset=int(causal_offset), nomat=nomat,
     )
     with torch.cuda.device(device):
         _d.check("tpa_fwd", lib.tpa_fwd(args, _d.current_stream_ptr(device)))

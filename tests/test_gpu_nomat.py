@@ -1,11 +1,13 @@
-"""`nomat=True`: the evaluation order that never forms K or V (tpa/tpa.py:250,333-359,398-413).
+"""`nomat`: the evaluation orders that never form K or V (tpa/tpa.py:250,333-359,398-413).
 
 The reference runs one test grid over nomat in {False, True} against the same dense reference
 (tpa/tpa_test.py:60-125): the switch changes the order of operations, never the function.  Here
 it selects the split-key kernels over windows of 64 query rows; `kernel=2` (matrix-core kernels
 only, no fallback) makes a test fail with an error if anything else would have served the call.
 Tolerances as in tests/test_gpu_parity.py: fp32 1e-4 / 1e-3, bf16 the per-row bounds of
-tests/error_model.py in their `factored` form (these kernels round Q only).
+tests/error_model.py in their `factored` form (these kernels round Q only).  `nomat="pairs"`
+selects the reference's own arithmetic instead (a table per rank pair shared by the heads of a
+workgroup, csrc/tpa_nomat.hip), which rounds nothing before the probabilities; same tests, same bounds.
 """
 
 import numpy as np
@@ -136,6 +138,98 @@ def test_config5_full_size_against_the_materialising_route(gpu):
     tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
     o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=d**-0.5, kernel=MFMA_ONLY, nomat=True)
     rows = np.array([0, 63, 64, 1023, 2047])
+    for bi in (0, 7):
+        sl = slice(bi, bi + 1)
+        o_ref, l_ref = orc.tpa_reference_rows(as_f64(tq[sl]), as_f64(tk[sl]), as_f64(tv[sl]), None, None, h, rows, sm_scale=d**-0.5, causal=False, dtype=np.float32)
+        assert np.abs(as_f64(o[sl][:, rows]) - o_ref).max() <= BF16_TOL
+        assert np.abs(as_f64(lse[sl][:, :, rows]).transpose(0, 2, 1) - l_ref).max() <= LSE_TOL
+    o_m, lse_m = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=d**-0.5)
+    assert (o.float() - o_m.float()).abs().max().item() <= BF16_TOL
+    assert (lse - lse_m).abs().max().item() <= LSE_TOL
+
+
+# ---------------------------------------------------------------- nomat="pairs": the reference's rank-pair tables
+@pytest.mark.parametrize("rank_q", [1, 6])
+@pytest.mark.parametrize("rank_k", [1, 2, 4])
+@pytest.mark.parametrize(
+    "batch_size,lq,lk,h,d",
+    [
+        (1, 8, 8, 8, 64),
+        (2, 1024, 128, 8, 64),
+        (2, 128, 1024, 8, 128),
+        (1, 1024, 1024, 16, 64),
+        (1, 300, 333, 3, 128),   # ragged lengths, a head block that is not full
+    ],
+)
+def test_reference_grid_shapes_with_rank_pair_tables(gpu, batch_size, rank_q, rank_k, lq, lk, h, d):
+    """The lengths, batch sizes and ranks of the reference's grid (tpa/tpa_test.py:60-76) through the kernel that
+    computes what the reference's nomat branch computes (tpa/tpa.py:333-359, 398-413)."""
+    from tpa import tpa
+
+    q, k, v = make_factors(0, batch_size, lq, lk, h, d, d, rank_q, rank_k, dist="uniform")
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h)
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=1.0, kernel=MFMA_ONLY, nomat="pairs")
+    check(o, lse, o_ref, l_ref, BF16_TOL, bf16_bounds(tq, tk, tv, h, 1.0, form="factored"))
+    # the three evaluation orders agree
+    lb, ob = bf16_bounds(tq, tk, tv, h, 1.0, form="factored")
+    for other in (False, True):
+        o_m, lse_m = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=1.0, nomat=other)
+        assert (o.float() - o_m.float()).abs().max().item() <= 2 * ob.max()
+        assert (lse - lse_m).abs().max().item() <= 2 * lb.max()
+
+
+@pytest.mark.parametrize("lq,lk,causal_offset", [(130, 130, 0), (257, 400, 143), (100, 300, -20), (65, 64, 3), (600, 600, -259)])
+def test_rank_pair_tables_under_a_causal_mask(gpu, lq, lk, causal_offset):
+    """Diagonal blocks, an offset between query and key positions, rows that see no key (NaN / -inf)."""
+    from tpa import tpa
+
+    b, h, d, rq, rk = 2, 8, 64, 6, 2
+    q, k, v = make_factors(5, b, lq, lk, h, d, d, rq, rk, scale_by_rank=True)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    o_ref, l_ref = _offset_reference(as_f64(tq), as_f64(tk), as_f64(tv), h, d**-0.5, causal_offset)
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=d**-0.5, causal=True, kernel=MFMA_ONLY, causal_offset=causal_offset, nomat="pairs")
+    check(o, lse, o_ref, l_ref, BF16_TOL, bf16_bounds(tq, tk, tv, h, d**-0.5, form="factored"))
+
+
+def test_rank_pair_tables_on_a_ragged_batch(gpu):
+    from tpa import tpa
+
+    b, lq, lk, h, d, rq, rk = 4, 150, 500, 8, 128, 6, 2
+    lengths = [500, 151, 320, 0]
+    q, k, v = make_factors(9, b, lq, lk, h, d, d, rq, rk, scale_by_rank=True)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    kvl = torch.tensor(lengths, dtype=torch.int32, device=gpu)
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=d**-0.5, causal=tpa.CAUSAL_BOTTOM_RIGHT, kernel=MFMA_ONLY, kv_lengths=kvl, nomat="pairs")
+    o_ref, l_ref = _bottom_right_reference(as_f64(tq), as_f64(tk), as_f64(tv), lengths, h, d**-0.5, 0)
+    check(o, lse, o_ref, l_ref, BF16_TOL, bf16_bounds(tq, tk, tv, h, d**-0.5, form="factored"))
+
+
+def test_rank_pair_tables_where_no_instance_exists(gpu):
+    """Other ranks, fp32 or segment ids: the plain kernel serves the call (same results); matrix cores only is refused."""
+    from tpa import _dispatch as dd
+    from tpa import tpa
+
+    b, lq, lk, h, d = 1, 96, 200, 8, 64
+    q, k, v = make_factors(3, b, lq, lk, h, d, d, 3, 2, scale_by_rank=True)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h, sm_scale=d**-0.5)
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=d**-0.5, nomat="pairs")
+    check(o, lse, o_ref, l_ref, BF16_TOL, bf16_bounds(tq, tk, tv, h, d**-0.5, form="factored"))
+    with pytest.raises(dd.TpaError):
+        tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=d**-0.5, kernel=MFMA_ONLY, nomat="pairs")
+
+
+def test_rank_pair_tables_at_the_config5_shape(gpu):
+    """B=8, T=2048, H=64, D=64 with the ranks 6 / 2 the kernel is instantiated for: sampled rows against the oracle,
+    the whole output against the default route (which forms K and V)."""
+    from tpa import tpa
+
+    b, t, h, d, rq, rk = 8, 2048, 64, 64, 6, 2
+    q, k, v = make_factors(0, b, t, t, h, d, d, rq, rk, scale_by_rank=True)
+    tq, tk, tv = (to_gpu(x, torch.bfloat16, gpu) for x in (q, k, v))
+    o, lse = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=d**-0.5, kernel=MFMA_ONLY, nomat="pairs")
+    rows = np.array([0, 31, 32, 255, 256, 1023, 2047])
     for bi in (0, 7):
         sl = slice(bi, bi + 1)
         o_ref, l_ref = orc.tpa_reference_rows(as_f64(tq[sl]), as_f64(tk[sl]), as_f64(tv[sl]), None, None, h, rows, sm_scale=d**-0.5, causal=False, dtype=np.float32)
