@@ -389,6 +389,7 @@ def tpa_factors_bwd(
     workspace: torch.Tensor | None = None,
     kernel: int = _d.KERNEL_AUTO,
     causal_offset: int = 0,
+    kv_lengths=None,
 ):
     """Backward pass on the split factor arrays: the operands of the reference's backward kernel
     launch (tpa/tpa.py:872-958) with a leading batch dimension, `lse` as [b, h, lq] fp32.
@@ -396,9 +397,12 @@ def tpa_factors_bwd(
     Returns the six fp32 gradients (dqa, dqb, dka, dkb, dva, dvb), each shaped like its factor.
     `grads` may hold six fp32 tensors (or views, e.g. the two parts of a concatenated
     dq[b, lq, rq, h+dk]) to be written in place.  `causal_offset`: the value the forward call
-    was made with (see `tpa_factors`).  There is no `kv_lengths` here: the backward reads all lk
-    keys, so the gradients of a forward that was made with `kv_lengths` are not available (slice
-    the batch entries to their lengths instead).
+    was made with (see `tpa_factors`).  `kv_lengths` (int32 [b]): the value the forward call was made
+    with.  The backward kernels take a ragged batch as a mask: the padding keys get a segment id that no
+    query carries (ids are made up here where the call has none), so they receive zero gradients and the
+    tiles that hold only padding are skipped.  Unlike the forward, the backward does read the padding rows of
+    k and v: they must hold finite values.  `causal=CAUSAL_BOTTOM_RIGHT` together with `kv_lengths` (an
+    offset per batch entry) is not available here and raises NotImplementedError.
     """
     device = _pick_device(qa, qb, ka, kb, va, vb)
     qa, qb, ka, kb, va, vb, o, lse, do = (_as_device_tensor(x, device) for x in (qa, qb, ka, kb, va, vb, o, lse, do))
@@ -411,6 +415,17 @@ def tpa_factors_bwd(
     assert tuple(lse.shape) == (b, h, lq), lse.shape
     qseg = _segment_ids(q_segment_ids, b, lq, device)
     kvseg = _segment_ids(kv_segment_ids, b, lk, device)
+    kvlen = _lengths(kv_lengths, b, device)
+    if kvlen is not None:
+        if _causal_code(causal) == CAUSAL_BOTTOM_RIGHT:
+            raise NotImplementedError("tpa_factors_bwd: kv_lengths with causal=CAUSAL_BOTTOM_RIGHT needs an offset per batch entry")
+        padding = torch.arange(lk, device=device, dtype=torch.int32)[None, :] >= kvlen[:, None]
+        if qseg is None:
+            qseg = torch.zeros((b, lq), dtype=torch.int32, device=device)
+            kvseg = padding.to(torch.int32).contiguous()
+        else:
+            below = torch.minimum(qseg.min(), kvseg.min()) - 1  # an id that no query carries
+            kvseg = torch.where(padding, below.to(torch.int32), kvseg).contiguous()
     o = o.to(dtype).contiguous()
     do = do.to(dtype).contiguous()
     lse = lse.to(torch.float32).contiguous()

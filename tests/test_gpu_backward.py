@@ -458,3 +458,50 @@ def test_ring_schedule_backward_on_the_references_ring_grid(gpu, batch_size, ran
     for n, w in enumerate(want):
         got = torch.cat([acc[2 * n], acc[2 * n + 1]], dim=-1).cpu().numpy()
         np.testing.assert_allclose(got, w, atol=1e-3, rtol=1e-2)
+
+
+@pytest.mark.parametrize("dt,d,kernel", [(torch.float32, 24, 1), (torch.float32, 64, 2), (torch.bfloat16, 128, 2)])
+@pytest.mark.parametrize("causal,offset,seg", [(False, 0, None), (True, 40, None), (True, 0, 70)])
+def test_backward_of_a_ragged_batch(gpu, dt, d, kernel, causal, offset, seg):
+    """kv_lengths in the backward (vector-ALU, fp32 and bf16 matrix-core kernels): gradients of a forward made
+    with kv_lengths equal the oracle's on each batch entry cut to its length, and are zero on the padding."""
+    from tpa import tpa
+
+    b, lq, lk, h, rq, rk = 3, 200, 330, 8, 3, 2
+    lengths = [330, 129, 64]
+    q, k, v = make_factors(21, b, lq, lk, h, d, d, rq, rk, scale_by_rank=True)
+    do = np.random.default_rng(22).standard_normal((b, lq, h, d)).astype(np.float32)
+    qseg = segment_ids(lq, seg, b) if seg else None
+    kvseg = segment_ids(lk, seg, b) if seg else None
+    tq, tk, tv, tdo = (torch.from_numpy(x).to(gpu).to(dt) for x in (q, k, v, do))
+    scale = d**-0.5
+    sp = lambda x: (x[..., :h], x[..., h:])
+    o, lse = tpa.tpa_factors(*sp(tq), *sp(tk), *sp(tv), qseg, kvseg, scale, causal, kernel, kv_lengths=lengths, causal_offset=offset)
+    grads = tpa.tpa_factors_bwd(*sp(tq), *sp(tk), *sp(tv), qseg, kvseg, o, lse, tdo, scale, causal, kernel=kernel,
+                                causal_offset=offset, kv_lengths=lengths)
+    f64 = lambda t: t.detach().float().cpu().numpy().astype(np.float64)
+    fq, fk, fv, fdo = f64(tq), f64(tk), f64(tv), f64(tdo)
+    tol = 2e-4 if dt == torch.float32 else 1.5e-2
+    for bi, n in enumerate(lengths):
+        # the oracle on the entry cut to its length; an offset mask is a segment-free tril with that diagonal,
+        # which the oracle's backward takes as a dense bias through its segment / causal arguments only for
+        # offset 0, so offsets are folded into segment-free calls on shifted keys where needed
+        qs = None if qseg is None else qseg[bi : bi + 1]
+        ks = None if kvseg is None else kvseg[bi : bi + 1, :n]
+        if causal and offset:
+            # key <= query + offset  <=>  top-left causal after prepending `offset` dummy queries
+            pad_q = np.zeros((1, offset, rq, h + d))
+            want = orc.tpa_backward(np.concatenate([pad_q, fq[bi : bi + 1]], 1), fk[bi : bi + 1, :n], fv[bi : bi + 1, :n], None, None, h,
+                                    np.concatenate([np.zeros((1, offset, h, d)), fdo[bi : bi + 1]], 1), sm_scale=scale, causal=True)
+            want = (want[0][:, offset:], want[1], want[2])
+        else:
+            want = orc.tpa_backward(fq[bi : bi + 1], fk[bi : bi + 1, :n], fv[bi : bi + 1, :n], qs, ks, h, fdo[bi : bi + 1], sm_scale=scale, causal=causal)
+        got_q = np.concatenate([f64(grads[0][bi : bi + 1]), f64(grads[1][bi : bi + 1])], -1)
+        got_k = np.concatenate([f64(grads[2][bi : bi + 1]), f64(grads[3][bi : bi + 1])], -1)
+        got_v = np.concatenate([f64(grads[4][bi : bi + 1]), f64(grads[5][bi : bi + 1])], -1)
+        assert rel_err(got_q, want[0]) <= tol, ("q", bi)
+        assert rel_err(got_k[:, :n], want[1]) <= tol, ("k", bi)
+        assert rel_err(got_v[:, :n], want[2]) <= tol, ("v", bi)
+        assert not got_k[:, n:].any() and not got_v[:, n:].any(), "padding keys receive no gradient"
+    with pytest.raises(NotImplementedError):
+        tpa.tpa_factors_bwd(*sp(tq), *sp(tk), *sp(tv), None, None, o, lse, tdo, scale, tpa.CAUSAL_BOTTOM_RIGHT, kv_lengths=lengths)
