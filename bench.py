@@ -124,11 +124,19 @@ def add_hbm_sustained(roof):
                                      how="hbm_rate 2048: 2 GiB buffers, 16-byte loads (non-temporal for the read), 2 in flight per lane, 768 workgroups of 256")
 
 
+TRAFFIC_KERNELS = {  # workload -> the kernels of one step, as rocprofv3 prints the start of their names
+    "c2": ["recon_bf16_h8_kernel", "prefill_kernel<128, 2, false>"],
+    "c2u": ["prefill_kernel<128, 0, false>"],
+    "c4": ["decode_kernel<128, 2, false, 1>", "decode_merge_kernel<128, bf16"],
+}
+
+
 def measured_traffic(workload):
     """HBM bytes per launch of the workload's kernels, read from the committed rocprofv3 counter summary
     (FETCH_SIZE / WRITE_SIZE in KiB per dispatch, one table row per kernel), each counter scaled by what it
-    reads for the 1 GiB device copy in the same table.  None where the summary has no row for the kernels."""
-    kernels = {"c2": ["recon_bf16_h8_kernel", "prefill_kernel<128, 2, false, 1"], "c4": ["decode_kernel<128, 2, false, 1", "decode_merge_kernel<128, bf16"]}.get(workload)
+    reads for the 1 GiB device copy in the same table.  None where the summary has no row for the kernels.
+    This is a figure from the profile run named in the summary's header, not from the run that prints it."""
+    kernels = TRAFFIC_KERNELS.get(workload)
     if not kernels or not os.path.exists(TRAFFIC_PROFILE):
         return None
     rows = {}
@@ -138,12 +146,24 @@ def measured_traffic(workload):
             if line.strip().startswith(k):
                 nums = [float(x) for x in parts if x.replace(".", "", 1).isdigit() and "." in x]
                 if len(nums) >= 2:
-                    rows[k] = nums[:2]
+                    rows[k] = nums[-2:]
     if "__amd_rocclr_copyBuffer" not in rows or any(k not in rows for k in kernels):
         return None
     kib = COPY_BYTES / 1024
     fetch_scale, write_scale = kib / rows["__amd_rocclr_copyBuffer"][0], kib / rows["__amd_rocclr_copyBuffer"][1]
     return sum(fetch_scale * rows[k][0] + write_scale * rows[k][1] for k in kernels) * 1024
+
+
+def traffic_source():
+    """where `roofline.traffic` comes from: the summary file and the source commit its header names"""
+    commit = None
+    if os.path.exists(TRAFFIC_PROFILE):
+        for line in open(TRAFFIC_PROFILE):
+            if "git commit" in line:
+                commit = line.split("git commit")[1].split()[0].strip(".,;:()")
+                break
+    return dict(file=os.path.relpath(TRAFFIC_PROFILE, ROOT), source_commit=commit,
+                how="rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a 1 GiB device copy; not measured in this run")
 
 
 def log(*a):
@@ -476,6 +496,7 @@ def main():
             value=r["tflops_wall"], unit="TFLOP/s", ms_per_step=r["wall_ms"],
             roofline=dict(bound="mfma", achieved=r["tflops_kernel"], peak=peak, unit="TFLOP/s",
                           frac=r["tflops_kernel"] / peak, traffic=measured_traffic(args.workload),
+                          **({"traffic_source": traffic_source()} if measured_traffic(args.workload) else {}),
                           kernel="prefill_f32_kernel" if f32 else ("nomat_pairs_kernel" if args.workload.endswith("rp") else "decode_kernel + decode_merge_kernel per 64 query rows" if args.workload.endswith("n")
                                                                    else "prefill_kernel" if args.workload.endswith("u") else "recon_bf16_h8_kernel + prefill_kernel"),
                           **launch_times(r), algorithmic_flops_per_launch=r["flops"]),
@@ -489,6 +510,7 @@ def main():
                 metric="TPA decode effective HBM bandwidth", value=d["gbs_wall"], unit="GB/s", ms_per_step=d["wall_ms"],
                 roofline=dict(bound="hbm", achieved=d["gbs_kernel"], peak=PEAK_HBM_GBS, unit="GB/s",
                               frac=d["gbs_kernel"] / PEAK_HBM_GBS, traffic=measured_traffic("c4"),
+                              **({"traffic_source": traffic_source()} if measured_traffic("c4") else {}),
                               kernel="decode_kernel + decode_merge_kernel",
                               **launch_times(d),
                               algorithmic_bytes_per_launch=d["bytes"]),
@@ -578,6 +600,7 @@ def main():
             metric="TPA decode effective HBM bandwidth", value=d["gbs_wall"], unit="GB/s", ms_per_step=d["wall_ms"],
             roofline=dict(bound="hbm", achieved=d["gbs_kernel"], peak=PEAK_HBM_GBS, unit="GB/s",
                           frac=d["gbs_kernel"] / PEAK_HBM_GBS, traffic=measured_traffic(args.workload),
+                          **({"traffic_source": traffic_source()} if measured_traffic(args.workload) else {}),
                           kernel=("decode_f32_kernel" if args.workload in F32_WORKLOADS else "decode_kernel") + " + decode_merge_kernel",
                           **launch_times(d),
                           algorithmic_bytes_per_launch=d["bytes"]),
