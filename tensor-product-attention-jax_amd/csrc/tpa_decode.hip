@@ -305,8 +305,12 @@ __global__ __launch_bounds__(kWaves * 64) void decode_kernel(DecodeParams p) {
       }
       tmax = halves_max(tmax);
       // finite with one query row (row0 itself is always inside its keys); a row that sees fewer
-      // keys than its neighbour can meet a block with none of its keys, before any or after all
-      const float m_new = fmaxf(m[r], tmax);
+      // keys than its neighbour can meet a block with none of its keys, before any or after all.
+      // The reference is a whole number (the running maximum rounded up): 2^(s - m) then has the same
+      // significand whatever m is, so the bf16 rounding of P' below does not depend on how the keys are
+      // split over waves and ranges, and every rescaling factor (here, in the wave merge, in the merge of
+      // the key ranges) is an exact power of two
+      const float m_new = fmaxf(m[r], __builtin_ceilf(tmax));
       const float m_use = NQ > 1 && m_new == -INFINITY ? 0.f : m_new;
       if (__any(m_new > m[r])) {
         const float alpha = __builtin_amdgcn_exp2f(m[r] - m_use);

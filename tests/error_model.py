@@ -153,6 +153,54 @@ def emulate_bf16_prefill(q, k, v, num_heads, sm_scale, causal=False, bias=None, 
     return emulate_bf16_attention(qd, kd, vd, sm_scale, bias=bias, faults=faults, reference_shift=reference_shift)
 
 
+def emulate_bf16_decode(q, k, v, num_heads, sm_scale, bias=None, faults=()):
+    """The rounding points of the bf16 split-key decode kernels in numpy, float64 between them, on concatenated
+    factors q[b,lq,rq,h+d], k[b,lk,rk,h+d], v[b,lk,rk,h+dv] (the bf16 values the kernel reads).  The cache
+    factors are used as they are; K and V are never formed:
+
+        Qm[h]  = bf16( (sm_scale log2 e / (rq rk)) * sum_r qa_r[h] qb_r )          the only rounding of the query
+        x[h,t] = sum_j ka_j[t,h] (Qm[h] . kb_j[t])  (+ bias, 0 / -inf)             the exponent, base 2
+        p      = 2^(x - m),  m a WHOLE number (ceil of the row maximum);  l = sum_t p (unrounded)
+        P'_j   = bf16( p * va_j[t,h] )                                              one rounding per (key, rank)
+        o      = bf16( (sum_t sum_j P'_j vb_j[t]) / (rk l) )       lse = (m + log2 l) / log2 e
+
+    With m a whole number P' has the same significand whatever m is, so the split of the keys over waves and
+    ranges changes no bit of it.  `faults`: "p_before_av" rounds p and then the product again, "p_trunc"
+    truncates P', "q_unscaled_round" rounds the query sum before the scale factor and again after.
+    -> (o[b,lq,h,dv], lse[b,lq,h], slack[b,lq,h,dv]) as emulate_bf16_attention."""
+    q, k, v = (np.asarray(x, dtype=np.float64) for x in (q, k, v))
+    h = num_heads
+    rq, rk = q.shape[2], k.shape[2]
+    c = float(np.float32(np.float32(np.float32(sm_scale) * np.float32(LOG2E_F32)) / (np.float32(rq) * np.float32(rk))))
+    qsum = np.einsum("blrh,blrd->blhd", q[..., :h], q[..., h:])
+    if "q_unscaled_round" in faults:
+        qsum = round_bf16(qsum)
+    qm = round_bf16(qsum * c)  # b lq h d
+    t = np.einsum("bqhd,bkjd->bhqkj", qm, k[..., h:])  # Qm . kb_j
+    x = np.einsum("bhqkj,bkjh->bhqk", t, k[..., :h])
+    if bias is not None:
+        x = x + np.asarray(bias, dtype=np.float64)[:, None, :, :]
+    with np.errstate(invalid="ignore", divide="ignore", over="ignore"):
+        m = np.ceil(x.max(-1, keepdims=True))
+        p = np.exp2(x - m)
+        l = p.sum(-1, keepdims=True)
+        va = np.transpose(v[..., :h], (0, 3, 1, 2))[:, :, None]  # b h 1 lk rk
+        pa = p[..., None] * va  # b h lq lk rk
+        if "p_trunc" in faults:
+            pr = truncate_bf16(pa)
+        elif "p_before_av" in faults:
+            pr = round_bf16(round_bf16(p)[..., None] * va)
+        else:
+            pr = round_bf16(pa)
+        vb = v[..., h:]  # b lk rk dv
+        o = np.einsum("bhqkj,bkjd->bhqd", pr, vb) / (rk * l)
+        mass = np.einsum("bhqkj,bkjd->bhqd", np.abs(pa), np.abs(vb)) / (rk * l)
+        one = 2.0**-7 * (np.abs(pa).max(axis=(-1, -2))[..., None] / l) * np.abs(vb).max(axis=(1, 2))[:, None, None, :] / rk
+        slack = TIGHT_REL * mass + one
+        lse = np.where(np.isneginf(m[..., 0]), -np.inf, (m[..., 0] + np.log2(l[..., 0])) / LOG2E_F32)
+    return round_bf16(np.transpose(o, (0, 2, 1, 3))), np.transpose(lse, (0, 2, 1)), np.transpose(slack, (0, 2, 1, 3))
+
+
 # The gate that holds a bf16 kernel to its emulation: per output element two bf16 spacings (a flipped last
 # rounding, and the neighbouring value where the element sits at a power of two) plus the emulation's slack
 # (fp32 summation order, one flipped P or V' rounding), at most TIGHT_FRAC of the elements different at all,

@@ -84,3 +84,30 @@ def test_whole_number_reference_changes_no_bit():
     import error_model as em
 
     assert em.round_bf16(2.0**-0.37 * 1.2345) != em.round_bf16(1.2345) * 2.0**-0.37
+
+
+DECODE_CASES = {  # seed, b, lq, lk, h, d, rq, rk, factors scaled by 1/sqrt(R)
+    "sharp": (3, 2, 2, 300, 8, 128, 1, 2, False),
+    "benchmark-like": (4, 2, 1, 700, 8, 128, 6, 2, True),
+    "rank 4, head size 64": (5, 1, 3, 257, 16, 64, 6, 4, True),
+}
+
+
+def test_decode_emulation_follows_the_oracle_and_its_gate_rejects_one_extra_rounding():
+    """The decode twin of the tight gate: the split-key kernels round the folded query once and every
+    (probability x head factor of V) product once; the emulation of exactly that stays inside the worst-case
+    law against the float64 oracle, and the gate that compares the GPU kernels with it fails an emulation that
+    rounds p before the product, truncates the product, or rounds the query sum before its scale factor."""
+    from error_model import emulate_bf16_decode
+
+    for name, (seed, b, lq, lk, h, d, rq, rk, scaled) in DECODE_CASES.items():
+        q, k, v = (bf16_round(x) for x in make_factors(seed, b, lq, lk, h, d, d, rq, rk, scale_by_rank=scaled))
+        scale = d**-0.5
+        o, l, slack = emulate_bf16_decode(q, k, v, h, scale)
+        o_ref, l_ref = orc.tpa_reference(q, k, v, None, None, h, sm_scale=scale)
+        lse_b, o_b = tpa_bounds(q, k, v, h, scale, form="factored")
+        assert (np.abs(o - o_ref).max(-1) <= o_b).all() and (np.abs(l - l_ref) <= lse_b).all(), name
+        assert not tight_violations(o, l, o, l, slack)
+        for fault in ("p_before_av", "p_trunc", "q_unscaled_round"):
+            o2, l2, _ = emulate_bf16_decode(q, k, v, h, scale, faults=(fault,))
+            assert tight_violations(o2, l2, o, l, slack), (name, fault)

@@ -13,7 +13,7 @@ import pytest
 import torch
 
 from conftest import make_factors, segment_ids
-from error_model import dense_bounds, emulate_bf16_attention, emulate_bf16_prefill, tight_violations, tpa_bounds
+from error_model import dense_bounds, emulate_bf16_attention, emulate_bf16_decode, emulate_bf16_prefill, tight_violations, tpa_bounds
 from oracle import tpa_oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -95,6 +95,16 @@ def check_tight(o, lse_bhl, tq, tk, tv, h, sm_scale, bias=None):
     caller can rely on; this gate is what catches a kernel that got a few times less accurate."""
     fq, fk, fv = (np.nan_to_num(as_f64(t)) for t in (tq, tk, tv))
     o_e, l_e, slack = emulate_bf16_prefill(fq, fk, fv, h, sm_scale, bias=bias)
+    bad = tight_violations(as_f64(o), as_f64(lse_bhl).transpose(0, 2, 1), o_e, l_e, slack)
+    assert not bad, "; ".join(bad)
+
+
+def check_tight_decode(o, lse_bhl, tq, tk, tv, h, sm_scale, bias=None):
+    """The bf16 split-key decode kernels against the emulation of their rounding points (the folded query
+    once, every probability x head-factor product once, the output once; tests/error_model.py:
+    emulate_bf16_decode), to the same gate as check_tight."""
+    fq, fk, fv = (np.nan_to_num(as_f64(t)) for t in (tq, tk, tv))
+    o_e, l_e, slack = emulate_bf16_decode(fq, fk, fv, h, sm_scale, bias=bias)
     bad = tight_violations(as_f64(o), as_f64(lse_bhl).transpose(0, 2, 1), o_e, l_e, slack)
     assert not bad, "; ".join(bad)
 
@@ -309,6 +319,7 @@ def test_decode_bf16_mfma(gpu, d, b, lq, lk, h, rq, rk):
     (tq, tk, tv), o, lse = run_decode(gpu, q, k, v, h, scale)
     o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h, sm_scale=scale)
     check(o, lse, o_ref, l_ref, BF16_TOL, bf16_bounds(tq, tk, tv, h, scale, form="factored"))
+    check_tight_decode(o, lse, tq, tk, tv, h, scale)
 
 
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
@@ -325,6 +336,8 @@ def test_decode_high_ranks(gpu, dt, d, rk, h, lk):
     o, lse = tpa.tpa_decode(*split(tq, tk, tv, h), sm_scale=d**-0.5, kv_lengths=lengths, kernel=2)
     o_ref, l_ref = _varlen_reference(as_f64(tq), as_f64(tk), as_f64(tv), lengths.tolist(), h, d**-0.5, False)
     check(o, lse, o_ref, l_ref, BF16_TOL if dt == torch.bfloat16 else F32_TOL, bf16_bounds(tq, tk, tv, h, d**-0.5, form="factored"))
+    if dt == torch.bfloat16:
+        check_tight_decode(o, lse, tq, tk, tv, h, d**-0.5, visible_bias(b, 1, lk, lengths=lengths.tolist()))
 
 
 def test_decode_sharp_softmax_and_split_invariance(gpu):
@@ -334,6 +347,7 @@ def test_decode_sharp_softmax_and_split_invariance(gpu):
     results = []
     for s in (1, 2, 3, 8):
         (tq, tk, tv), o, lse = run_decode(gpu, q, k, v, h, scale, num_splits=s)
+        check_tight_decode(o, lse, tq, tk, tv, h, scale)  # unscaled factors: a sharp softmax
         results.append((as_f64(o), as_f64(lse)))
     o_ref, l_ref = orc.tpa_reference(as_f64(tq), as_f64(tk), as_f64(tv), None, None, h, sm_scale=scale)
     for o, lse in results:
@@ -367,6 +381,7 @@ def test_config4_full_size_decode(gpu):
         o_ref, l_ref = orc.tpa_reference(as_f64(tq[sl]), as_f64(tk[sl]), as_f64(tv[sl]), None, None, h, sm_scale=scale, dtype=np.float32)
         assert np.abs(as_f64(o[sl]) - o_ref).max() <= BF16_TOL
         assert np.abs(as_f64(lse[sl]).transpose(0, 2, 1) - l_ref).max() <= LSE_TOL
+        check_tight_decode(o[sl], lse[sl], tq[sl], tk[sl], tv[sl], h, scale)
     # the generic kernel on the same inputs (no MFMA, no split) agrees
     from tpa import tpa
 
@@ -856,6 +871,7 @@ def test_decode_with_per_sequence_cache_lengths(gpu, d, rk, h):
     o, lse = tpa.tpa_decode(*tpa_split(tq, tk, tv, h), sm_scale=d**-0.5, kv_lengths=torch.tensor(lengths, dtype=torch.int32), kernel=2)
     o_ref, l_ref = _varlen_reference(as_f64(tq), np.nan_to_num(as_f64(tk)), np.nan_to_num(as_f64(tv)), lengths, h, d**-0.5, False)
     check(o, lse, o_ref, l_ref, BF16_TOL, bf16_bounds(tq, tk, tv, h, d**-0.5, form="factored"))
+    check_tight_decode(o, lse, tq, tk, tv, h, d**-0.5, visible_bias(b, 1, lk, lengths=lengths))
 
 
 @pytest.mark.parametrize("causal", [False, True])
@@ -909,6 +925,8 @@ def test_decode_over_a_paged_cache(gpu, dt, d, rk, page_size):
     assert torch.equal(o1, o2) and torch.equal(l1, l2)
     o_ref, l_ref = _varlen_reference(as_f64(tq), as_f64(tk), as_f64(tv), lengths, h, d**-0.5, False)
     check(o1, l1, o_ref, l_ref, BF16_TOL if dt == torch.bfloat16 else F32_TOL, bf16_bounds(tq, tk, tv, h, d**-0.5, form="factored"))
+    if dt == torch.bfloat16:
+        check_tight_decode(o1, l1, tq, tk, tv, h, d**-0.5, visible_bias(b, 1, lk, lengths=lengths))
 
 
 def test_paged_cache_is_refused_where_no_kernel_reads_it(gpu):
@@ -1081,6 +1099,8 @@ def test_decode_with_a_causal_limit_per_query_row(gpu, dt, b, lq, lk, h, d, rq, 
         o_ref, l_ref = _offset_reference(fq, fk, fv, h, sm_scale, offset, np.zeros((b, lq), np.int32), kvseg)
     tol = F32_TOL if dt == torch.float32 else BF16_TOL
     check(o, lse, o_ref, l_ref, tol, bf16_bounds(tq, tk, tv, h, sm_scale, form="factored"))
+    if dt == torch.bfloat16:
+        check_tight_decode(o, lse, tq, tk, tv, h, sm_scale, visible_bias(b, lq, lk, causal=True, offset=offset, lengths=lengths))
     o2, lse2 = tpa.tpa_factors(*split(tq, tk, tv, h), sm_scale=sm_scale, causal=True, kernel=2, kv_lengths=kvl, causal_offset=offset,
                                use_workspace=True)  # with it this entry point reaches the same split-key kernel
     assert torch.equal(torch.nan_to_num(o2.float(), nan=7.0), torch.nan_to_num(o.float(), nan=7.0)) and torch.equal(lse2, lse)
