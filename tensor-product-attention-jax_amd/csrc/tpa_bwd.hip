@@ -113,7 +113,11 @@ __global__ __launch_bounds__(256) void recon_bf16_h8_kernel(ReconJobs jobs, int 
   for (int i = 0; i < 8; ++i)
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[i][j] = 0.f;
-  constexpr int G = 4;  // ranks whose loads are in flight together (the kernel is bound by their latency)
+  // Two ranks per step of the inner product: the head factors of ranks (r, r + 1) and the b elements of the
+  // same two ranks are paired into packed bf16 words (16 byte permutes per pair of ranks), and one dot
+  // instruction then adds a_r[h] b_r[d] + a_r+1[h] b_r+1[d] to the accumulator - half the instructions of
+  // unpacking both and multiplying in fp32, which is what bounds this kernel from rank 8 on.
+  constexpr int G = 4;  // ranks whose loads are in flight together (at low ranks the kernel is bound by their latency)
   for (int r0 = 0; r0 < R; r0 += G) {
     u32x4 av[G], bv[G];
 #pragma unroll
@@ -121,20 +125,24 @@ __global__ __launch_bounds__(256) void recon_bf16_h8_kernel(ReconJobs jobs, int 
       const int r = min(r0 + u, R - 1);
       av[u] = *reinterpret_cast<const u32x4*>(ap + (int64_t)r * fa.stride_r);
       bv[u] = *reinterpret_cast<const u32x4*>(bp + (int64_t)r * fb.stride_r);
+      if (r0 + u >= R) av[u] = u32x4{0u, 0u, 0u, 0u};  // past the last rank: weight zero
     }
 #pragma unroll
-    for (int u = 0; u < G; ++u) {
+    for (int u = 0; u < G; u += 2) {
       if (r0 + u >= R) break;
-      float af[8], bf[8];
+      uint32_t apair[8], bpair[8];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        af[2 * j] = bf16lo_to_f32(av[u][j]); af[2 * j + 1] = bf16hi_to_f32(av[u][j]);
-        bf[2 * j] = bf16lo_to_f32(bv[u][j]); bf[2 * j + 1] = bf16hi_to_f32(bv[u][j]);
+        apair[2 * j] = __builtin_amdgcn_perm(av[u + 1][j], av[u][j], 0x05040100u);      // (a_r[2j], a_r+1[2j])
+        apair[2 * j + 1] = __builtin_amdgcn_perm(av[u + 1][j], av[u][j], 0x07060302u);  // (a_r[2j+1], a_r+1[2j+1])
+        bpair[2 * j] = __builtin_amdgcn_perm(bv[u + 1][j], bv[u][j], 0x05040100u);
+        bpair[2 * j + 1] = __builtin_amdgcn_perm(bv[u + 1][j], bv[u][j], 0x07060302u);
       }
 #pragma unroll
       for (int i = 0; i < 8; ++i)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[i][j] += af[i] * bf[j];
+        for (int j = 0; j < 8; ++j)
+          acc[i][j] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, apair[i]), __builtin_bit_cast(bf16x2, bpair[j]), acc[i][j], false);
     }
   }
   const float inv = scale / (float)R;
