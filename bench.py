@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the TPA forward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2u|c3|c3u|c4|c4pg|c4s|c5|c5u|c2n|c5n|c5r|c5rn|c5rp|c2f|c3f|c2fb|c4f|c2m|c3m|c5m|c2p|c3p|c2b|c3b|c2pb|ap1|ap2|ap3|copy] [--no-cpu] [--no-decode] [--no-backward]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2u|c3|c3u|c4|c4pg|c4s|c5|c5u|c2n|c5n|c5r|c5rn|c5rp|c2f|c3f|c2fb|c4f|c2m|c3m|c5m|c2p|c3p|c2pu|c3pu|c2b|c3b|c2pb|ap1|ap2|ap3|copy] [--no-cpu] [--no-decode] [--no-backward]
 
 A step is one forward pass over one batch of synthetic, seeded inputs that are resident in HBM
 before the timed region starts.  The default workload is the prefill configuration the headline
@@ -60,6 +60,8 @@ WORKLOADS = {
     "c2pb": ("backward", 4, 4096, 4096, 16, 128, 6, 2, True),   # packed documents, as c2p
     "c2p": ("prefill", 4, 4096, 4096, 16, 128, 6, 2, True),
     "c3p": ("prefill", 1, 32768, 32768, 32, 128, 6, 2, True),
+    "c2pu": ("prefill", 4, 4096, 4096, 16, 128, 6, 2, True),     # packed documents without a workspace: the fused kernel
+    "c3pu": ("prefill", 1, 32768, 32768, 32, 128, 6, 2, True),
     # fp32 inputs (the reference's default dtype) at the c2 shape and at a quarter of c3's length: the fp32 MFMA kernel
     "c2f": ("prefill", 4, 4096, 4096, 16, 128, 6, 2, True),
     "c3f": ("prefill", 1, 16384, 16384, 32, 128, 6, 2, True),
@@ -185,7 +187,7 @@ def make_inputs(torch, device, B, lq, lk, H, D, rq, rk, seed, dtype=None):
     )
 
 
-DOC_LEN = {"c2p": 1024, "c3p": 4096, "c2pb": 1024}
+DOC_LEN = {"c2p": 1024, "c3p": 4096, "c2pb": 1024, "c2pu": 1024, "c3pu": 4096}
 
 
 def prefill_flops(B, lq, lk, H, D, causal):

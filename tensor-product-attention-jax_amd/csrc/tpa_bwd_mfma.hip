@@ -116,10 +116,17 @@ __device__ __forceinline__ void id_window(const int32_t* mine, int n_mine, const
                                           int tid, int& first, int& last) {
   if (tid == 0) { red[0] = INT32_MAX; red[1] = INT32_MIN; red[2] = INT32_MAX; red[3] = -1; }
   __syncthreads();
-  for (int t = tid; t < n_mine; t += NT) {
-    const int32_t sid = mine[t];
-    __hip_atomic_fetch_min(&red[0], sid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    __hip_atomic_fetch_max(&red[1], sid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  {  // one atomic per wave: the lanes' values are reduced in registers first
+    int32_t smin = INT32_MAX, smax = INT32_MIN;
+    for (int t = tid; t < n_mine; t += NT) {
+      const int32_t sid = mine[t];
+      smin = min(smin, sid); smax = max(smax, sid);
+    }
+    smin = wave_min(smin); smax = wave_max(smax);
+    if ((tid & 63) == 0 && smin <= smax) {
+      __hip_atomic_fetch_min(&red[0], smin, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_fetch_max(&red[1], smax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
   }
   __syncthreads();
   const int32_t lo_id = red[0], hi_id = red[1];
@@ -128,7 +135,8 @@ __device__ __forceinline__ void id_window(const int32_t* mine, int n_mine, const
     const int32_t sid = other[t];
     if (sid >= lo_id && sid <= hi_id) { lo = min(lo, t); hi = max(hi, t); }
   }
-  if (hi >= 0) {
+  lo = wave_min(lo); hi = wave_max(hi);
+  if ((tid & 63) == 0 && hi >= 0) {
     __hip_atomic_fetch_min(&red[2], lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     __hip_atomic_fetch_max(&red[3], hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   }

@@ -73,6 +73,24 @@ __device__ __forceinline__ float halves_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// Minimum / maximum / sum of an int over the 64 lanes of a wave (every lane gets the result): what goes into a
+// shared-memory atomic should be one value per wave - atomics of all lanes on one address are served one by one.
+__device__ __forceinline__ int wave_min(int x) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) x = min(x, __shfl_xor(x, m, 64));
+  return x;
+}
+__device__ __forceinline__ int wave_max(int x) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) x = max(x, __shfl_xor(x, m, 64));
+  return x;
+}
+__device__ __forceinline__ int wave_sum(int x) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) x += __shfl_xor(x, m, 64);
+  return x;
+}
+
 // Q fragments from rank factors: qf[ks] = bf16( scale * sum_r a[r] * b[r][16 ks + 0..7] ), where
 // `ap` points at this lane's a[0] (rank stride a_stride) and `bp` at b[0][this lane's first
 // element] (rank stride b_stride).  Ranks are taken G at a time with all 16-byte loads of the
