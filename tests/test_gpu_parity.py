@@ -4,8 +4,9 @@ Tolerances: fp32 outputs max-abs <= 1e-4, logsumexp <= 1e-3.  The reference's ow
 (tpa/tpa_test.py:60-125) uses rtol = atol = 1e-3 on fp32; it is run here at the tighter 1e-4.
 bf16 kernels: the five benchmark configurations are held to the absolute bf16 outputs <= 2e-2,
 logsumexp <= 1e-3; every other bf16 case to the per-row bound that the kernels' bf16 rounding
-points imply for its inputs (tests/error_model.py: |dlogit| <= 2^-8 sm_scale sum_d |q_d||k_d|),
-a few 1e-3 on the logsumexp for benchmark-like inputs and 1e-1 for sharp softmaxes.
+points imply for its inputs (tests/error_model.py: |dlogit| <= 2^-7 sm_scale sum_d |q_d||k_d|),
+up to 1e-2 on the logsumexp for benchmark-like inputs and 2e-1 for sharp softmaxes; the bf16 matrix-core
+kernels are also held to the emulation of their rounding points, to two bf16 spacings (check_tight).
 """
 
 import numpy as np

@@ -1,0 +1,141 @@
+"""Seeded random problems through tpa_factors / tpa_factors_bwd with `kernel = AUTO`, against the oracle.
+
+The parametrised tests elsewhere walk the shapes the kernels were written for; these walk shapes nobody
+picked: lengths that are not multiples of anything, head counts and head sizes on and off the matrix-core
+kernels' grid, every mask the interface takes (segment ids in runs of random length, causal with an offset,
+per-sequence key lengths, bottom-right alignment) in random combination, with and without the optional
+workspace, both storage types.  Whatever kernel the dispatcher picks must meet the same bounds as in
+tests/test_gpu_parity.py: fp32 1e-4 / 1e-3, bf16 the per-row bound of its rounding points.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import make_factors
+from error_model import tpa_bounds
+from oracle import tpa_oracle as orc
+from test_gpu_parity import BF16_TOL, F32_TOL, as_f64, check, split, to_gpu, visible_bias
+
+pytestmark = pytest.mark.gpu
+
+
+def _runs(rng, b, length, mean_run):
+    """ids [b, length] in runs of random length (non-decreasing: packed documents)"""
+    out = np.zeros((b, length), np.int32)
+    for i in range(b):
+        pos, sid = 0, int(rng.integers(0, 3))
+        while pos < length:
+            n = int(rng.integers(1, 2 * mean_run))
+            out[i, pos : pos + n] = sid
+            pos += n
+            sid += int(rng.integers(1, 3))
+    return out
+
+
+def _problem(rng):
+    mfma_grid = rng.random() < 0.75
+    d = int(rng.choice([64, 128])) if mfma_grid else int(rng.choice([8, 24, 40, 72, 96]))
+    dv = d if mfma_grid or rng.random() < 0.5 else int(rng.choice([16, 48, 80]))
+    h = int(rng.choice([8, 16, 24, 32, 40])) if mfma_grid else int(rng.choice([1, 3, 5, 12]))
+    b = int(rng.integers(1, 4))
+    lq = int(rng.choice([1, 2, 5, 17, 64, 100, 129, 256, 300, 511, 640]))
+    lk = int(rng.choice([1, 7, 63, 64, 65, 200, 257, 512, 700, 1100, 2050]))
+    rq, rk = int(rng.choice([1, 2, 3, 6])), int(rng.choice([1, 2, 3, 4, 8]))
+    dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float32
+    mask = rng.choice(["none", "causal", "causal_offset", "bottom_right", "segments", "segments_causal", "lengths"])
+    return dict(b=b, lq=lq, lk=lk, h=h, d=d, dv=dv, rq=rq, rk=rk, dtype=dtype, mask=str(mask), ws=bool(rng.random() < 0.5),
+                sharp=bool(rng.random() < 0.2))
+
+
+def _masks(rng, c):
+    b, lq, lk = c["b"], c["lq"], c["lk"]
+    qseg = kvseg = lengths = None
+    causal, offset = False, 0
+    m = c["mask"]
+    if m in ("causal", "segments_causal"):
+        causal = True
+    if m == "causal_offset":
+        causal, offset = True, int(rng.integers(-3, max(lk - lq, 0) + 4))
+    if m == "bottom_right":
+        causal = 2
+        lengths = [int(x) for x in rng.integers(min(lq, lk), lk + 1, size=b)]
+    if m == "lengths":
+        lengths = [int(x) for x in rng.integers(0, lk + 1, size=b)]
+        lengths[0] = lk
+    if m.startswith("segments"):
+        # one run pattern cut to both lengths, so that queries and keys of a document line up as in a packed batch
+        ids = _runs(rng, b, max(lq, lk), int(rng.choice([20, 90, 300])))
+        qseg, kvseg = ids[:, :lq].copy(), ids[:, :lk].copy()
+    bias = visible_bias(b, lq, lk, qseg, kvseg, causal=bool(causal), offset=offset, lengths=lengths, bottom_right=causal == 2)
+    return qseg, kvseg, lengths, causal, offset, bias
+
+
+@pytest.mark.parametrize("seed", range(160))
+def test_random_forward_problem(gpu, seed):
+    from tpa import tpa
+
+    rng = np.random.default_rng(1000 + seed)
+    c = _problem(rng)
+    b, lq, lk, h, d, dv, rq, rk, dtype = (c[k] for k in ("b", "lq", "lk", "h", "d", "dv", "rq", "rk", "dtype"))
+    q, k, v = make_factors(seed, b, lq, lk, h, d, dv, rq, rk, scale_by_rank=not c["sharp"])
+    qseg, kvseg, lengths, causal, offset, bias = _masks(rng, c)
+    tq, tk, tv = (to_gpu(x, dtype, gpu) for x in (q, k, v))
+    sm_scale = d**-0.5
+    o, lse = tpa.tpa_factors(
+        *split(tq, tk, tv, h),
+        None if qseg is None else torch.from_numpy(qseg).to(gpu), None if kvseg is None else torch.from_numpy(kvseg).to(gpu),
+        sm_scale, causal, use_workspace=c["ws"], kv_lengths=lengths, causal_offset=offset,
+    )
+    fq, fk, fv = as_f64(tq), as_f64(tk), as_f64(tv)
+    dense = [orc.reconstruct(*orc.split_factors(x, h)) for x in (fq, fk, fv)]
+    o_ref, l_ref = orc.mha_forward(*dense, bias=bias, sm_scale=sm_scale)
+    bf16 = dtype == torch.bfloat16
+    # which kernel ran is the dispatcher's business: the factored bound covers the split-key kernels too
+    bounds = tpa_bounds(fq, fk, fv, h, sm_scale, form="factored") if bf16 else None
+    check(o, lse, o_ref, l_ref, BF16_TOL if bf16 else F32_TOL, bounds)
+
+
+@pytest.mark.parametrize("seed", range(64))
+def test_random_backward_problem(gpu, seed):
+    from tpa import tpa
+
+    rng = np.random.default_rng(5000 + seed)
+    c = _problem(rng)
+    c["lq"], c["lk"] = min(c["lq"], 300), min(c["lk"], 700)  # the oracle's backward holds [b, h, lq, lk] several times over
+    if c["mask"] == "bottom_right":
+        c["mask"] = "causal_offset"  # the backward takes lengths with top-left alignment only
+    b, lq, lk, h, d, dv, rq, rk, dtype = (c[k] for k in ("b", "lq", "lk", "h", "d", "dv", "rq", "rk", "dtype"))
+    q, k, v = make_factors(seed, b, lq, lk, h, d, dv, rq, rk, scale_by_rank=True)
+    qseg, kvseg, lengths, causal, offset, bias = _masks(rng, c)
+    tq, tk, tv = (to_gpu(x, dtype, gpu) for x in (q, k, v))
+    sm_scale = d**-0.5
+    tqs = None if qseg is None else torch.from_numpy(qseg).to(gpu)
+    tks = None if kvseg is None else torch.from_numpy(kvseg).to(gpu)
+    fs = split(tq, tk, tv, h)
+    o, lse = tpa.tpa_factors(*fs, tqs, tks, sm_scale, causal, kv_lengths=lengths, causal_offset=offset)
+    do = torch.from_numpy(np.random.default_rng(seed).standard_normal((b, lq, h, dv)).astype(np.float32)).to(dtype).to(gpu)
+    grads = tpa.tpa_factors_bwd(*fs, tqs, tks, o, lse, do, sm_scale, causal, kv_lengths=lengths, causal_offset=offset)
+    # oracle: gradients of sum(o * do) through the dense attention with the same additive bias, projected onto the factors
+    fq, fk, fv = as_f64(tq), as_f64(tk), as_f64(tv)
+    (qa, qb), (ka, kb), (va, vb) = (orc.split_factors(x, h) for x in (fq, fk, fv))
+    dq, dk, dv_ = orc.mha_backward(orc.reconstruct(qa, qb), orc.reconstruct(ka, kb), orc.reconstruct(va, vb), bias, sm_scale, as_f64(do))
+    want = []
+    for dx, (a, bb) in ((dq, (qa, qb)), (dk, (ka, kb)), (dv_, (va, vb))):
+        want += list(orc.project_to_factors(np.nan_to_num(dx), a, bb))
+    # bf16 matrix-core kernels: dense Q, K, V, P and dS are rounded to bf16, so the probabilities carry the relative
+    # error E that the forward's error law gives the exponent (tests/error_model.py; 3e-3 for benchmark-like
+    # inputs, 0.1 where low ranks make the softmax sharp), and the gradients inherit it: 2e-2 + 2 E of the largest
+    # entry.  fp32: 3e-4.  A gradient array that is exactly zero (a row that sees a single key has p = 1 and
+    # dS = 0, so nothing reaches q and k) is held against a fiftieth of the largest entry of all six instead of
+    # against itself.
+    if dtype == torch.bfloat16:
+        tol = 2e-2 + 2.0 * float(tpa_bounds(fq, fk, fv, h, sm_scale)[0].max())
+    else:
+        tol = 3e-4
+    floor = 0.02 * max(np.abs(w).max() for w in want)
+    for name, g, w in zip(("dqa", "dqb", "dka", "dkb", "dva", "dvb"), grads, want):
+        g = as_f64(g)
+        assert np.isfinite(g).all(), name
+        scale = max(np.abs(w).max(), floor, 1e-30)
+        assert np.abs(g - w).max() <= tol * scale, (name, float(np.abs(g - w).max() / scale), tol, c)
