@@ -139,3 +139,96 @@ def test_random_backward_problem(gpu, seed):
         assert np.isfinite(g).all(), name
         scale = max(np.abs(w).max(), floor, 1e-30)
         assert np.abs(g - w).max() <= tol * scale, (name, float(np.abs(g - w).max() / scale), tol, c)
+
+
+@pytest.mark.parametrize("seed", range(64))
+def test_random_decode_problem(gpu, seed):
+    """tpa_decode with whatever the interface takes: several query rows, key ranges, ragged and paged caches,
+    a causal limit per row (offset or aligned with the end of each cache)."""
+    from tpa import tpa
+
+    rng = np.random.default_rng(9000 + seed)
+    b, lq = int(rng.integers(1, 6)), int(rng.choice([1, 1, 2, 3, 4, 7]))
+    h, d = int(rng.choice([8, 16, 32, 40, 64])), int(rng.choice([64, 128]))
+    rq, rk = int(rng.choice([1, 2, 6])), int(rng.choice([1, 2, 4, 8]))
+    dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float32
+    paged = rng.random() < 0.4
+    page_size = int(rng.choice([32, 64, 256])) if paged else 0
+    lk = int(rng.choice([2, 5, 8, 17, 33])) * page_size if paged else int(rng.choice([37, 300, 1024, 1500, 4100]))
+    q, k, v = make_factors(seed, b, lq, lk, h, d, d, rq, rk, scale_by_rank=rng.random() < 0.8)
+    tq, tk, tv = (to_gpu(x, dtype, gpu) for x in (q, k, v))
+    lengths = None
+    if rng.random() < 0.6:
+        lengths = [int(x) for x in rng.integers(lq, lk + 1, size=b)]
+    mode = str(rng.choice(["none", "offset", "bottom_right"]))
+    causal, offset = False, 0
+    if mode == "offset":
+        causal, offset = True, lk - lq - int(rng.integers(0, 4))
+    if mode == "bottom_right":
+        causal = 2
+    qa, qb, ka, kb, va, vb = split(tq, tk, tv, h)
+    table = None
+    if paged:
+        pps = lk // page_size
+        npages = b * pps + 3
+        table = torch.from_numpy(rng.permutation(npages)[: b * pps].astype(np.int32)).reshape(b, pps).to(gpu)
+        pool = lambda x: torch.full((npages, page_size) + tuple(x.shape[2:]), float("nan"), dtype=x.dtype, device=gpu).index_copy_(
+            0, table.reshape(-1).long(), x.reshape(b * pps, page_size, *x.shape[2:]))
+        ka, kb, va, vb = (pool(x) for x in (ka, kb, va, vb))
+    sm_scale = d**-0.5
+    o, lse = tpa.tpa_decode(qa, qb, ka, kb, va, vb, sm_scale=sm_scale, num_splits=int(rng.choice([0, 0, 1, 3, 9])),
+                            kv_lengths=lengths, page_table=table, causal=causal, causal_offset=offset)
+    bias = visible_bias(b, lq, lk, causal=bool(causal), offset=offset, lengths=lengths, bottom_right=causal == 2)
+    fq, fk, fv = as_f64(tq), as_f64(tk), as_f64(tv)
+    dense = [orc.reconstruct(*orc.split_factors(x, h)) for x in (fq, fk, fv)]
+    o_ref, l_ref = orc.mha_forward(*dense, bias=bias, sm_scale=sm_scale)
+    bf16 = dtype == torch.bfloat16
+    check(o, lse, o_ref, l_ref, BF16_TOL if bf16 else F32_TOL, tpa_bounds(fq, fk, fv, h, sm_scale, form="factored") if bf16 else None)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_append_problem(gpu, seed):
+    """tpa_cache_append on layers and batches nobody picked: every output factor against the oracle, the rest of
+    the cache untouched, tokens past the capacity dropped; contiguous and paged caches, given positions."""
+    from test_gpu_append import f64, make_layer, rope_tables
+    from tpa import tpa
+
+    rng = np.random.default_rng(13000 + seed)
+    b, n = int(rng.integers(1, 9)), int(rng.choice([1, 1, 2, 3, 7, 16, 33, 70, 129, 300, 1100]))
+    dm = int(rng.choice([64, 128, 192, 256, 512, 1024, 1536]))
+    h, d = int(rng.choice([8, 16, 24, 32])), int(rng.choice([64, 96, 128]))
+    rq, rk = int(rng.choice([1, 2, 3, 6])), int(rng.choice([1, 2, 4]))
+    dtype = torch.bfloat16 if rng.random() < 0.75 else torch.float32
+    x, w = make_layer(seed, b, n, dm, h, d, rq, rk, dtype, gpu)
+    page_size = int(rng.choice([8, 16, 64]))
+    cache_len = (n + int(rng.integers(0, 40)) + page_size - 1) // page_size * page_size
+    cos, sin = rope_tables(cache_len + 9, d)
+    lengths = rng.integers(0, max(cache_len - n, 0) + 1, size=b).astype(np.int32)
+    if rng.random() < 0.3:
+        lengths[-1] = min(max(cache_len - n + 2, 0), cache_len)  # the last tokens of the last sequence do not fit
+    pos = None
+    if rng.random() < 0.4:
+        pos = (lengths[:, None] + np.arange(n)[None, :] + rng.integers(0, 5, size=(b, 1))).astype(np.int32)
+    paged = rng.random() < 0.5
+    if paged:
+        pps = cache_len // page_size
+        table = torch.from_numpy(rng.permutation(b * pps + 2)[: b * pps].astype(np.int32)).reshape(b, pps).to(gpu)
+        caches = [torch.full((b * pps + 2, page_size, rk, inner), float("nan"), dtype=dtype, device=gpu) for inner in (h, d, h, d)]
+    else:
+        table = None
+        caches = [torch.full((b, cache_len, rk, inner), float("nan"), dtype=dtype, device=gpu) for inner in (h, d, h, d)]
+    qa, qb, new_len = tpa.tpa_cache_append(x, w, cos, sin, *caches, lengths, rank_q=rq, positions=pos, page_table=table,
+                                           use_workspace=bool(rng.random() < 0.5))
+    used = pos if pos is not None else lengths[:, None] + np.arange(n)[None, :]
+    want = orc.tpa_append_reference(f64(x), f64(w), cos, sin, np.minimum(used, cos.shape[0] - 1), h, d, rq, rk)
+    rel = 2.0**-8 if dtype == torch.bfloat16 else 1e-5
+    for name, got in (("qa", qa), ("qb", qb)):
+        assert np.abs(f64(got) - want[name]).max() <= rel * np.abs(want[name]).max(), name
+    for name, cache in zip(("ka", "kb", "va", "vb"), caches):
+        c = f64(cache[table.long()].reshape(b, cache_len, rk, -1) if paged else cache)
+        for bi in range(b):
+            fits = max(min(n, cache_len - int(lengths[bi])), 0)
+            rows = c[bi, lengths[bi] : lengths[bi] + fits]
+            assert np.abs(rows - want[name][bi, :fits]).max(initial=0.0) <= rel * np.abs(want[name]).max(), (name, bi)
+            assert np.isnan(c[bi, : lengths[bi]]).all() and np.isnan(c[bi, lengths[bi] + fits :]).all(), (name, bi)
+    assert new_len.cpu().tolist() == [min(int(l) + n, cache_len) for l in lengths]
