@@ -232,3 +232,51 @@ def test_random_append_problem(gpu, seed):
             assert np.abs(rows - want[name][bi, :fits]).max(initial=0.0) <= rel * np.abs(want[name]).max(), (name, bi)
             assert np.isnan(c[bi, : lengths[bi]]).all() and np.isnan(c[bi, lengths[bi] + fits :]).all(), (name, bi)
     assert new_len.cpu().tolist() == [min(int(l) + n, cache_len) for l in lengths]
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_dense_attention_problem(gpu, seed):
+    """mha (tpa/mha.py) forward and backward: head sizes on and off the matrix-core grid, dk != dv, a dense bias
+    with -inf entries (rows without any visible key among them) or the causal flag, few rows over many keys."""
+    from error_model import dense_bounds
+    from tpa import mha
+
+    rng = np.random.default_rng(17000 + seed)
+    b, h = int(rng.integers(1, 4)), int(rng.choice([1, 2, 4, 8, 16]))
+    lq = int(rng.choice([1, 3, 16, 65, 128, 200, 384]))
+    lk = int(rng.choice([1, 9, 64, 100, 257, 640, 1500]))
+    mfma_grid = rng.random() < 0.7
+    dk = int(rng.choice([64, 128])) if mfma_grid else int(rng.choice([8, 24, 40, 96]))
+    dv = dk if mfma_grid or rng.random() < 0.5 else int(rng.choice([16, 48, 72]))
+    dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float32
+    mode = str(rng.choice(["none", "causal", "bias"]))
+    g = np.random.Generator(np.random.Philox(seed))
+    q, k, v, do = (g.standard_normal(s, dtype=np.float32) for s in ((b, lq, h, dk), (b, lk, h, dk), (b, lk, h, dv), (b, lq, h, dv)))
+    bias = None
+    if mode == "bias":
+        bias = g.standard_normal((b, lq, lk), dtype=np.float32)
+        bias[g.random((b, lq, lk)) < 0.3] = -np.inf
+        bias[:, lq // 2] = -np.inf  # a row that sees nothing
+    sm_scale = dk**-0.5
+    tq, tk, tv, tdo = (to_gpu(x, dtype, gpu) for x in (q, k, v, do))
+    o, res = mha._mha_fwd(tq, tk, tv, None if bias is None else torch.from_numpy(bias).to(gpu), sm_scale, causal=mode == "causal")
+    lse = res[0]
+    fq, fk, fv = as_f64(tq), as_f64(tk), as_f64(tv)
+    full_bias = np.zeros((b, lq, lk)) if bias is None else bias.astype(np.float64)
+    if mode == "causal":
+        full_bias = full_bias + visible_bias(b, lq, lk, causal=True)
+    o_ref, l_ref = orc.mha_forward(fq, fk, fv, bias=full_bias, sm_scale=sm_scale)
+    bf16 = dtype == torch.bfloat16
+    check(o, lse, o_ref, l_ref, BF16_TOL if bf16 else F32_TOL, dense_bounds(fq, fk, fv, sm_scale) if bf16 else None)
+    dq, dk_, dv_, _, _ = mha._mha_bwd(res, tdo)
+    want = orc.mha_backward(fq, fk, fv, full_bias, sm_scale, as_f64(tdo))
+    tol = 2e-2 + 2.0 * float(dense_bounds(fq, fk, fv, sm_scale)[0].max()) if bf16 else 3e-4
+    # a gradient that is exactly zero (one visible key: p = 1, dS = p (dp - delta) = 0) comes out as the rounding of
+    # o inside delta, 2^-8 of |dp| - with these unscaled N(0, 1) inputs a few percent of the largest gradient
+    floor = 0.1 * max(np.abs(w).max() for w in want)
+    for name, got, w in zip(("dq", "dk", "dv"), (dq, dk_, dv_), want):
+        got = as_f64(got)
+        assert np.isfinite(got).all(), name
+        scale = max(np.abs(w).max(), floor, 1e-30)
+        # (gradients come back in the input dtype: a bf16 rounding of their own on top)
+        assert np.abs(got - w).max() <= (tol + (2.0**-8 if bf16 else 0.0)) * scale, (name, float(np.abs(got - w).max() / scale), tol)
