@@ -471,8 +471,10 @@ __global__ __launch_bounds__(256) void project_kernel(const float* dx, TpaFactor
 }
 
 // The same projections for bf16 factors with H % 8 == 0 and (D / 8) (H / 8) a power of two up to 64,
-// without LDS: a thread owns the 8 x 8 piece dX[8 hg .. + 7][8 cc .. + 7] of one token (pieces of D
-// are the fastest thread index, so the 16 loads of a piece are coalesced 32-byte runs), multiplies it
+// without LDS: a thread owns an 8 x 8 piece of one token's dX, rows 8 hg .. 8 hg + 7, columns 4 cc .. 4 cc + 3 of
+// the lower and of the upper half of D (pieces of D are the fastest thread index, so each of the 16 loads of a
+// piece reads whole contiguous half rows across the lanes: 12 % faster than 8 consecutive columns per thread,
+// where one load instruction touched every other 16 bytes), multiplies it
 // with its 8 values of b (for da) and of a (for db) rank by rank, and the sums over d and over h are
 // reductions across the lanes that share a token: over the D / 8 neighbouring lanes with DPP adds,
 // over the H / 8 groups above them with lane exchanges.  Several tokens share a wave.
@@ -489,23 +491,26 @@ __global__ __launch_bounds__(256) void project_h8_kernel(const float* dx, TpaFac
   const bool live = tok < L;
   const int64_t t = live ? tok : L - 1;  // lanes past the end idle along: the reductions need whole waves
   const int b = blockIdx.y;
-  const float* xp = dx + (((int64_t)b * L + t) * H + 8 * hg) * D + 8 * cc;
+  const int dh = D / 2;  // a thread's eight columns: 4 cc .. 4 cc + 3 and the same in the upper half of the row
+  const float* xp = dx + (((int64_t)b * L + t) * H + 8 * hg) * D + 4 * cc;
   const uint16_t* ap = static_cast<const uint16_t*>(fa.ptr) + b * fa.stride_b + t * fa.stride_l + 8 * hg;
-  const uint16_t* bp = static_cast<const uint16_t*>(fb.ptr) + b * fb.stride_b + t * fb.stride_l + 8 * cc;
+  const uint16_t* bp = static_cast<const uint16_t*>(fb.ptr) + b * fb.stride_b + t * fb.stride_l + 4 * cc;
   float x[8][8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const f32x4 lo = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xp + (int64_t)i * D));
-    const f32x4 hi = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xp + (int64_t)i * D + 4));
+    const f32x4 hi = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(xp + (int64_t)i * D + dh));
 #pragma unroll
     for (int j = 0; j < 4; ++j) { x[i][j] = lo[j]; x[i][4 + j] = hi[j]; }
   }
   const float inv = 1.f / (float)R;
   float* oa = ga.ptr + b * ga.stride_b + t * ga.stride_l + 8 * hg;
-  float* ob = gb.ptr + b * gb.stride_b + t * gb.stride_l + 8 * cc;
+  float* ob = gb.ptr + b * gb.stride_b + t * gb.stride_l + 4 * cc;
   for (int r = 0; r < R; ++r) {
     const u32x4 av = *reinterpret_cast<const u32x4*>(ap + (int64_t)r * fa.stride_r);
-    const u32x4 bv = *reinterpret_cast<const u32x4*>(bp + (int64_t)r * fb.stride_r);
+    const u32x2 bl = *reinterpret_cast<const u32x2*>(bp + (int64_t)r * fb.stride_r);
+    const u32x2 bh = *reinterpret_cast<const u32x2*>(bp + (int64_t)r * fb.stride_r + dh);
+    const u32x4 bv = u32x4{bl[0], bl[1], bh[0], bh[1]};
     float af[8], bf[8];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -550,7 +555,7 @@ __global__ __launch_bounds__(256) void project_h8_kernel(const float* dx, TpaFac
     }
     if (live && hg == 0) {
       *reinterpret_cast<f32x4*>(ob + (int64_t)r * gb.stride_r) = f32x4{db[0] * inv, db[1] * inv, db[2] * inv, db[3] * inv};
-      *reinterpret_cast<f32x4*>(ob + (int64_t)r * gb.stride_r + 4) = f32x4{db[4] * inv, db[5] * inv, db[6] * inv, db[7] * inv};
+      *reinterpret_cast<f32x4*>(ob + (int64_t)r * gb.stride_r + dh) = f32x4{db[4] * inv, db[5] * inv, db[6] * inv, db[7] * inv};
     }
   }
 }
