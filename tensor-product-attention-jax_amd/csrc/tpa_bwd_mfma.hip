@@ -15,7 +15,7 @@
 //
 //   bwd_dkv_kernel  one workgroup = 32 keys per wave of one head, lane = key
 //     S  = Q K^T              A = Q rows (LDS),      B = K (registers, pre-scaled), addend -lse[row]
-//     dP = dO V^T             A = dO rows (LDS),     B = V (registers),             addend -delta[row]
+//     dP = dO V^T             A = dO rows (LDS),     B = V (registers; at D = 128 a per-lane LDS slot), addend -delta[row]
 //     dV^T += dO^T P          A = dO^T (transposed LDS reads), B = P
 //     dK^T += Q^T dS          A = Q^T  (transposed LDS reads), B = dS
 //
@@ -69,6 +69,14 @@ constexpr int kRsrcFlags = 0x00020000;  // raw 32-bit data format
 // consecutive rows) and transposed (8-byte reads of 4 consecutive rows); no padding serves both
 // without bank conflicts, these leave the row reads conflict-free and the transposed ones two-way.
 constexpr int tile_stride(int d) { return d == 128 ? d + 24 : d + 8; }
+
+// dK/dV kernel at D = 128: K, V and both accumulators of a wave's 32 keys are 192 of its 256 registers, and
+// with S, dP, the rows on their way to LDS and the addresses the compiler spilled 26 of them and reloaded 15
+// per tile (scratch reads in the loop: 4.2 M wave-level loads per launch at B = 4, T = 4096, H = 16).  The V
+// fragments therefore live in LDS - each lane parks its own eight 16-byte B operands once and reads them back
+// where dP = dO V^T needs them (one more 16-byte LDS read per matrix instruction of that product; LDS was busy
+// a third of the time).  No scratch is left, and the kernel takes 14 % less (0.666 -> 0.575 ms at that shape).
+constexpr bool dkv_v_in_lds(int d) { return d == 128; }
 
 // A-operand fragment of rows 32 mb .. 32 mb + 31 of a row-major tile (row stride S elements),
 // contraction columns 16 kk .. 16 kk + 15: lane (i, g) reads 8 elements of row 32 mb + i.
@@ -360,6 +368,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
   float* const lds_nlse = reinterpret_cast<float*>(smem + 4 * kTile * S);  // [2][64]  -lse * log2(e), -inf for dead rows
   float* const lds_ndel = lds_nlse + 2 * kTile;                            // [2][64]  -delta
   int32_t* const lds_seg = reinterpret_cast<int32_t*>(lds_ndel + 2 * kTile);  // [2][64]
+  u32x4* const lds_vf = reinterpret_cast<u32x4*>(lds_seg + 2 * kTile);  // [NW][NB][NKS][64 lanes]: V of the wave's keys as B operands
 
   // (batch, head) pairs per XCD, blocks heaviest first: see bwd_dq_kernel
   const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
@@ -374,7 +383,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
   const int k0 = kblk * kBK, wkey0 = k0 + kWK * w;
   const float c = p.sm_scale * kLog2e;
 
-  bf16x8 kf[NB][NKS], vf[NB][NKS];
+  constexpr bool VLDS = dkv_v_in_lds(D);
+  bf16x8 kf[NB][NKS], vf[VLDS ? 1 : NB][VLDS ? 1 : NKS];
   int32_t kseg[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
@@ -388,7 +398,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) sc[j] = pack_bf16(bf16lo_to_f32(raw[j]) * c, bf16hi_to_f32(raw[j]) * c);
       kf[nb][ks] = __builtin_bit_cast(bf16x8, sc);
-      vf[nb][ks] = *reinterpret_cast<const bf16x8*>(vp + 16 * ks + 8 * g);
+      if constexpr (VLDS) lds_vf[((w * NB + nb) * NKS + ks) * 64 + l] = *reinterpret_cast<const u32x4*>(vp + 16 * ks + 8 * g);
+      else vf[nb][ks] = *reinterpret_cast<const bf16x8*>(vp + 16 * ks + 8 * g);
     }
     kseg[nb] = SEG ? p.kvseg[(int64_t)b * p.lk + key_ld] : 0;
   }
@@ -490,11 +501,22 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, kf[nb][kk], s[nb], 0, 0, 0);
       });
+      // (the address passes through an empty asm per row block: the compiler would otherwise keep the fragments
+      // of the first block for the second, which is the register pressure this is meant to take away)
+      const u32x4* vf_base = lds_vf + w * NB * NKS * 64 + l;
+      asm volatile("" : "+v"(vf_base));
       static_for<NKS>([&](auto kk_c) __attribute__((always_inline)) {
         constexpr int kk = decltype(kk_c)::value;
         const bf16x8 a = rows_frag<S>(gs, mb, kk, i, g);
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) dp[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, vf[nb][kk], dp[nb], 0, 0, 0);
+        for (int nb = 0; nb < NB; ++nb) {
+          if constexpr (VLDS) {
+            const bf16x8 vfrag = __builtin_bit_cast(bf16x8, vf_base[(nb * NKS + kk) * 64]);
+            dp[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, vfrag, dp[nb], 0, 0, 0);
+          } else {
+            dp[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, vf[nb][kk], dp[nb], 0, 0, 0);
+          }
+        }
       });
       bf16x8 pf[NB][2], df[NB][2];
 #pragma unroll
@@ -616,7 +638,7 @@ int launch_dkv(const BwdParams& base, hipStream_t stream) {
   const int64_t nwg = (int64_t)((per_xcd + p.pair_group - 1) / p.pair_group) * p.pair_group * p.nblk * 8;
   if (nwg > 2147483647LL) return TPA_ERR_SHAPE;
   auto kern = bwd_dkv_kernel<D, NW, NB, SEG>;
-  const size_t smem = (size_t)4 * kTile * tile_stride(D) * 2 + 6 * kTile * 4;
+  const size_t smem = (size_t)4 * kTile * tile_stride(D) * 2 + 6 * kTile * 4 + (dkv_v_in_lds(D) ? (size_t)NW * NB * (D / 16) * 64 * 16 : 0);
   static bool configured[kMaxDevices] = {};
   if (int rc = raise_lds_limit(configured, reinterpret_cast<const void*>(kern), smem); rc != TPA_OK) return rc;
   hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(NW * 64), smem, stream, p);
@@ -625,8 +647,8 @@ int launch_dkv(const BwdParams& base, hipStream_t stream) {
 
 template <int D>
 int launch_both(const BwdParams& p, hipStream_t stream) {
-  // dK/dV: 8 waves of 32 keys.  (64 keys per wave would halve the LDS reads per MFMA, which bound
-  // this kernel, but its 384 stationary registers at D = 128 leave the compiler spilling.)
+  // dK/dV: 8 waves of 32 keys.  (64 keys per wave would halve the LDS reads per MFMA, but its 384
+  // stationary registers at D = 128 leave the compiler spilling.)
   // (measured at D = 128: the dQ kernel with 4 waves of 64 rows, one wave per SIMD and 512 registers, takes
   // 922 us where 8 waves of 32 rows take 401 us)
   constexpr int NW = 8, NB = 1;
