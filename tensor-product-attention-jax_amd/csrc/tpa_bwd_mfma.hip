@@ -276,18 +276,28 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(BwdParams p) {
       f32x16 s[NB], dp[NB];
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) { s[nb] = nlse[nb]; dp[nb] = ndelta[nb]; }
+      // The two chains are independent: they alternate, and their operands are requested two steps ahead.  The
+      // order is pinned (left alone, the compiler runs one chain after the other and reads each operand right
+      // before the instruction that takes it: 1 % of the call at B = 4, T = 4096, H = 16, more where blocks are long).
+      __builtin_amdgcn_sched_barrier(0);
       static_for<NKS>([&](auto kk_c) __attribute__((always_inline)) {
         constexpr int kk = decltype(kk_c)::value;
         const bf16x8 a = rows_frag<S>(ks, mb, kk, i, g);
+        const bf16x8 a2 = rows_frag<S>(vs, mb, kk, i, g);
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[nb][kk], s[nb], 0, 0, 0);
+        for (int nb = 0; nb < NB; ++nb) {
+          s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[nb][kk], s[nb], 0, 0, 0);
+          dp[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a2, gf[nb][kk], dp[nb], 0, 0, 0);
+        }
       });
-      static_for<NKS>([&](auto kk_c) __attribute__((always_inline)) {
-        constexpr int kk = decltype(kk_c)::value;
-        const bf16x8 a = rows_frag<S>(vs, mb, kk, i, g);
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) dp[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, gf[nb][kk], dp[nb], 0, 0, 0);
-      });
+      for (int n = 0; n < NKS - 2; ++n) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * NB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4 * NB, 0);
+      __builtin_amdgcn_sched_barrier(0);
       bf16x8 df[NB][2];
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
@@ -495,29 +505,39 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkv_kernel(BwdParams p) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) { s[nb][4 * vq + e] = a[e]; dp[nb][4 * vq + e] = d4[e]; }
       }
+      // the two independent chains alternate with their operands requested ahead, in a pinned order (see bwd_dq_kernel);
+      // the index of the parked V fragments passes through an empty asm per row block: the compiler would otherwise keep
+      // the first block's fragments for the second, which is the register pressure parking them is meant to take away
+      int vf_idx = w * NB * NKS * 64 + l;  // (the index, not the pointer: a pointer out of an asm has lost its address space)
+      asm volatile("" : "+v"(vf_idx));
+      __builtin_amdgcn_sched_barrier(0);
       static_for<NKS>([&](auto kk_c) __attribute__((always_inline)) {
         constexpr int kk = decltype(kk_c)::value;
         const bf16x8 a = rows_frag<S>(qs, mb, kk, i, g);
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, kf[nb][kk], s[nb], 0, 0, 0);
-      });
-      // (their index passes through an empty asm per row block: the compiler would otherwise keep the fragments
-      // of the first block for the second, which is the register pressure this is meant to take away)
-      int vf_idx = w * NB * NKS * 64 + l;  // (the index, not the pointer: a pointer out of an asm has lost its address space)
-      asm volatile("" : "+v"(vf_idx));
-      static_for<NKS>([&](auto kk_c) __attribute__((always_inline)) {
-        constexpr int kk = decltype(kk_c)::value;
-        const bf16x8 a = rows_frag<S>(gs, mb, kk, i, g);
+        const bf16x8 a2 = rows_frag<S>(gs, mb, kk, i, g);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
+          s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, kf[nb][kk], s[nb], 0, 0, 0);
           if constexpr (VLDS) {
             const bf16x8 vfrag = __builtin_bit_cast(bf16x8, lds_vf[vf_idx + (nb * NKS + kk) * 64]);
-            dp[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, vfrag, dp[nb], 0, 0, 0);
+            dp[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a2, vfrag, dp[nb], 0, 0, 0);
           } else {
-            dp[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, vf[nb][kk], dp[nb], 0, 0, 0);
+            dp[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a2, vf[nb][kk], dp[nb], 0, 0, 0);
           }
         }
       });
+      {
+        constexpr int RD = VLDS ? 2 + NB : 2;  // LDS reads per step
+        constexpr int AHEAD = VLDS ? 1 : 2;    // steps whose operands are in flight (registers decide)
+        __builtin_amdgcn_sched_group_barrier(0x100, AHEAD * RD, 0);
+#pragma unroll
+        for (int n = 0; n < NKS - AHEAD; ++n) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 2 * NB, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, RD, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * AHEAD * NB, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
       bf16x8 pf[NB][2], df[NB][2];
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
